@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X array-op hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-suite] [--no-cpu]
+
+Headline (the JSON line's `value`): f32 GEMM TFLOP/s at M=N=K=4096, C = A·B, operands seeded
+U(-1,1) and resident in HBM before the timed region.  One step = one pass of the kernel.
+The same line carries
+  roofline     - the GEMM kernel against the fp32 matrix peak, from HIP-event timing of the same
+                 launches on the stream they run on;
+  cpu_baseline - the CPU oracle's sgemm (a restatement of the reference's CPU path) timed on this
+                 host's cores on one pass of the same 4096^3 product;
+  suite        - the other workloads of the metric: A·Bᵀ / Aᵀ·B, the reductions, softmax fwd/bwd,
+                 transpose, the fused elementwise chain (GB/s of ALGORITHMIC bytes against 8 TB/s)
+                 and MLP training steps/s.
+Only one GPU is used; --gpus above 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
+HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
+SEED = 0x51CED
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def timed(ctx, fn, steps, warmup):
+    """(wall ms per step with sync on both sides, HIP-event ms per launch)."""
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    e0, e1 = ctx.event(), ctx.event()
+    t0 = time.perf_counter()
+    ctx.record(e0)
+    for _ in range(steps):
+        fn()
+    ctx.record(e1)
+    ctx.sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    ev = ctx.elapsed_ms(e0, e1) / steps
+    ctx.lib.slhip_event_destroy(e0)
+    ctx.lib.slhip_event_destroy(e1)
+    return wall, ev
+
+
+def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0):
+    a = ctx.uniform(m * k, -1, 1, 0, SEED)
+    b = ctx.uniform(k * n, -1, 1, 1, SEED)
+    c = ctx.zeros(m * n)
+    fn = lambda: ctx.call("slhip_sgemm", ta, tb, m, n, k, a.ptr, b.ptr, c.ptr, beta)
+    wall, ev = timed(ctx, fn, steps, warmup)
+    for x in (a, b, c):
+        x.free()
+    flop = 2.0 * m * n * k
+    return {"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
+            "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS}
+
+
+def bw_entry(name, algo_bytes, wall, ev):
+    gbs = algo_bytes / ev / 1e6
+    return {"op": name, "algorithmic_bytes": algo_bytes, "ms_wall": wall, "ms_kernel": ev, "GBps": gbs,
+            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+
+
+def bench_bandwidth_suite(ctx, steps, warmup):
+    out = []
+    R = C = 16384
+    n = R * C
+    x = ctx.uniform(n, -10, 10, 0, SEED)
+    vec_c, vec_r, one = ctx.empty(C), ctx.empty(R), ctx.empty(1)
+    y = ctx.empty(n)
+    for name, outbuf, olen in [("sum_rows", vec_c, C), ("sum_cols", vec_r, R), ("max_rows", vec_c, C),
+                               ("max_cols", vec_r, R)]:
+        fn = lambda name=name, outbuf=outbuf: ctx.call("slhip_" + name, R, C, x.ptr, outbuf.ptr)
+        w, e = timed(ctx, fn, steps, warmup)
+        out.append(bw_entry("%s [16384x16384]" % name, 4 * n + 4 * olen, w, e))
+        log(out[-1])
+    w, e = timed(ctx, lambda: ctx.call("slhip_mean", n, x.ptr, one.ptr), steps, warmup)
+    out.append(bw_entry("mean [2^28]", 4 * n + 4, w, e)); log(out[-1])
+    w, e = timed(ctx, lambda: ctx.call("slhip_transpose", R, C, x.ptr, y.ptr, 0.0), steps, warmup)
+    out.append(bw_entry("transpose [16384x16384]", 8 * n, w, e)); log(out[-1])
+    # degenerate 1-D shapes of the same tensor
+    N1 = 1 << 28
+    for name, rows, cols, olen in [("sum_cols", 1, N1, 1), ("sum_rows", N1, 1, 1), ("max_cols", 1, N1, 1),
+                                   ("max_rows", N1, 1, 1)]:
+        fn = lambda name=name, rows=rows, cols=cols: ctx.call("slhip_" + name, rows, cols, x.ptr, one.ptr)
+        w, e = timed(ctx, fn, steps, warmup)
+        out.append(bw_entry("%s [%dx%d]" % (name, rows, cols), 4 * n + 4 * olen, w, e)); log(out[-1])
+    # softmax forward / backward, [32768 x 4096] and the row-length sweep at 2^27 elements
+    for rows, cols in [(32768, 4096), (1 << 20, 128), (1 << 17, 1024), (1 << 13, 16384)]:
+        ne = rows * cols
+        xs, g, s = x.view(0, ne), x.view(ne, ne), y.view(0, ne)
+        xg = y.view(ne, ne)
+        w, e = timed(ctx, lambda: ctx.call("slhip_softmax", rows, cols, xs.ptr, s.ptr), steps, warmup)
+        out.append(bw_entry("softmax fwd [%dx%d]" % (rows, cols), 8 * ne, w, e)); log(out[-1])
+        w, e = timed(ctx, lambda: ctx.call("slhip_softmax_grad", rows, cols, xg.ptr, s.ptr, g.ptr, 0.0), steps, warmup)
+        out.append(bw_entry("softmax bwd [%dx%d]" % (rows, cols), 12 * ne, w, e)); log(out[-1])
+        if cols == 4096:
+            o1 = vec_c.view(0, cols)
+            w, e = timed(ctx, lambda: ctx.call("slhip_max_rows", rows, cols, xs.ptr, o1.ptr), steps, warmup)
+            out.append(bw_entry("max_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
+            w, e = timed(ctx, lambda: ctx.call("slhip_sum_rows", rows, cols, xs.ptr, o1.ptr), steps, warmup)
+            out.append(bw_entry("sum_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
+    # fused elementwise chain on 2^28 elements per tensor: 4 reads + 1 write
+    bb, cc, dd = ctx.uniform(n, -10, 10, 2, SEED), ctx.uniform(n, -10, 10, 3, SEED), ctx.uniform(n, -10, 10, 4, SEED)
+    w, e = timed(ctx, lambda: ctx.call("slhip_ew_chain", n, x.ptr, bb.ptr, cc.ptr, dd.ptr, y.ptr), steps, warmup)
+    out.append(bw_entry("ew_chain ((a+b)*c-d)^2^2 [2^28]", 20 * n, w, e)); log(out[-1])
+    w, e = timed(ctx, lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n), steps, warmup)
+    out.append(bw_entry("device copy [1 GiB] (achievable line)", 8 * n, w, e)); log(out[-1])
+    for b in (x, y, bb, cc, dd, vec_c, vec_r, one):
+        b.free()
+    return out
+
+
+def bench_mlp(ctx, steps_c5, steps_c1):
+    try:
+        from sliced_amd import host
+    except Exception as e:  # the host layer is optional for the kernel benchmark
+        return {"skipped": "host layer not built: %s" % e}
+    return host.bench_mlp(steps_c5, steps_c1)
+
+
+def cpu_baseline(m, n, k):
+    import oracle
+    cores = oracle.max_threads()
+    oracle.set_threads(cores)
+    rs = np.random.RandomState(1)
+    a = rs.uniform(-1, 1, m * k).astype(np.float32)
+    b = rs.uniform(-1, 1, k * n).astype(np.float32)
+    oracle.gemm(64, 64, 64, a[:4096], b[:4096])        # load + warm
+    t0 = time.perf_counter()
+    oracle.gemm(m, n, k, a, b)
+    dt = time.perf_counter() - t0
+    res = {"value": 2.0 * m * n * k / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+           "sample": "one pass of the same %dx%dx%d f32 product by the CPU oracle's blocked sgemm "
+                     "(sequential-k f32, no FMA), %.2f s on %d threads" % (m, n, k, dt, cores)}
+    oracle.set_threads(1)
+    ms = 1024
+    t0 = time.perf_counter()
+    oracle.gemm(ms, ms, ms, a[:ms * ms], b[:ms * ms])
+    dt1 = time.perf_counter() - t0
+    res["single_thread_TFLOPs_at_1024"] = 2.0 * ms ** 3 / dt1 / 1e12
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-suite", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--size", type=int, default=4096)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus %d refused); the hot path has no "
+              "multi-GPU leg" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from sliced_amd.device import Context
+    ctx = Context(0)
+    log("device:", ctx.name())
+    M = N = K = args.size
+
+    head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup)
+    log("gemm NN", head)
+    suite = {}
+    if not args.no_suite:
+        suite["gemm_4096"] = {"A*B": head,
+                              "A*Bt": bench_gemm(ctx, M, N, K, 0, 1, args.steps, args.warmup),
+                              "At*B": bench_gemm(ctx, M, N, K, 1, 0, args.steps, args.warmup)}
+        log(suite["gemm_4096"])
+        sweep = {}
+        for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (8192,) * 3, (8192, 2048, 784), (784, 2048, 8192)]:
+            st = max(3, args.steps // 4) if m >= 8192 and k >= 8192 else args.steps
+            for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
+                r = bench_gemm(ctx, m, n, k, ta, tb, st, 2)
+                sweep["%dx%dx%d %s" % (m, n, k, form)] = {"tflops": r["tflops_kernel"], "frac": r["frac_of_peak"]}
+                log(m, n, k, form, sweep["%dx%dx%d %s" % (m, n, k, form)])
+        suite["gemm_sweep"] = sweep
+        suite["bandwidth"] = bench_bandwidth_suite(ctx, max(5, args.steps // 2), 2)
+        suite["mlp"] = bench_mlp(ctx, 50, 200)
+        log(suite["mlp"])
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(M, N, K)
+        log("cpu", cpu)
+
+    line = {
+        "metric": "f32 GEMM TFLOP/s @4096^3",
+        "value": head["tflops_wall"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_wall"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
+                   "kernel": "gemm_kernel<false,false> 128x128x16 tiles, v_mfma_f32_32x32x2_f32"},
+        "roofline": {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": head["frac_of_peak"], "traffic": None},
+        "cpu_baseline": cpu,
+        "suite": suite,
+    }
+    print(json.dumps(line))
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,215 @@
+/* sliced_hip.h — C ABI of the MI355X (gfx950) backend for sliced's array-op hot path.
+ *
+ * These are the entry points a `HIP<Mods>` device in the reference's host language would bind
+ * (one per method of the op traits under src/ops2/ of the reference, plus the runtime calls
+ * its custos-style device layer needs).  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a SLHIP_E* code or a positive hipError_t otherwise;
+ *     slhip_last_error_string() describes the last failure on the calling thread;
+ *   - all matrices are f32, row-major, contiguous (len = rows * cols), as in the reference;
+ *   - data pointers are DEVICE pointers; a context owns one in-order HIP stream and every op
+ *     is asynchronous on it.  Only slhip_memcpy_d2h, slhip_sync and slhip_event_elapsed_ms
+ *     wait;
+ *   - a context is used from one host thread at a time (the reference's devices are
+ *     single-threaded, RefCell-style);
+ *   - the library never allocates inside an op call: partial results of the two-stage
+ *     reductions and of split-K GEMM live in a workspace that slhip_init allocates once;
+ *   - no aliasing between inputs and outputs unless a comment allows it.
+ *
+ * Naming trap kept from the reference: *_rows reduces OVER the rows (output length = cols),
+ * *_cols reduces OVER the columns (output length = rows).
+ */
+#ifndef SLICED_HIP_H
+#define SLICED_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct slhip_ctx slhip_ctx;
+typedef struct slhip_event slhip_event;
+
+enum {
+  SLHIP_OK = 0,
+  SLHIP_EINVAL = -1,     /* null pointer, zero/overflowing dims, unknown op code */
+  SLHIP_ENODEVICE = -2,  /* no HIP device / wrong architecture */
+  SLHIP_EWORKSPACE = -3, /* request does not fit the context workspace */
+  SLHIP_EALIAS = -4      /* forbidden overlap of operands */
+};
+
+/* BinaryElementWise op codes (reference: src/ops2/binary_ew/mod.rs:55-100). */
+enum { SLHIP_ADD = 0, SLHIP_SUB = 1, SLHIP_MUL = 2, SLHIP_DIV = 3 };
+
+/* apply_fn / add_unary_grad op codes (reference call sites: src/ops.rs:36-41 square,
+ * :65-72 pow, :423 clip, :438 exp; src/matrix.rs:181-187 relu; examples/nn.rs:137 -ln,
+ * :151 neg-div). p and q are the scalar parameters: pow exponent, clip bounds, scale factor. */
+enum {
+  SLHIP_SQUARE = 0,
+  SLHIP_POW = 1,
+  SLHIP_RELU = 2,
+  SLHIP_EXP = 3,
+  SLHIP_CLIP = 4,
+  SLHIP_NEG_LN = 5,
+  SLHIP_SCALE = 6,
+  SLHIP_NEG_DIV = 7
+};
+
+/* ---------------------------------------------------------------- runtime ----------
+ * Replaces what the reference gets from custos' device layer (not in its tree): Alloc,
+ * WriteBuf/Read, ClearBuf and the in-order queue (usage: src/ops2/gemm/cpu_stack.rs:35-43
+ * retrieve + add_op; examples/sine_net.rs:124 device construction). */
+int32_t slhip_init(int32_t device_ordinal, slhip_ctx** ctx);
+/* Same, but ops run on a stream the caller owns (e.g. a framework's current stream). */
+int32_t slhip_init_on_stream(int32_t device_ordinal, void* hip_stream, slhip_ctx** ctx);
+int32_t slhip_destroy(slhip_ctx* ctx);
+const char* slhip_last_error_string(void);
+int32_t slhip_device_name(slhip_ctx* ctx, char* buf, size_t buflen);
+int32_t slhip_stream(slhip_ctx* ctx, void** hip_stream);
+size_t slhip_workspace_bytes(slhip_ctx* ctx);
+
+int32_t slhip_malloc(slhip_ctx* ctx, size_t bytes, void** dptr);
+int32_t slhip_free(slhip_ctx* ctx, void* dptr);
+int32_t slhip_memcpy_h2d(slhip_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int32_t slhip_memcpy_d2h(slhip_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes); /* waits */
+int32_t slhip_memcpy_d2d(slhip_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
+int32_t slhip_memset(slhip_ctx* ctx, void* dptr, int32_t byte_value, size_t bytes);
+int32_t slhip_fill(slhip_ctx* ctx, size_t n, float value, float* x);
+int32_t slhip_sync(slhip_ctx* ctx);
+
+/* HIP events on the context's stream, for timing kernels where they run. */
+int32_t slhip_event_create(slhip_ctx* ctx, slhip_event** ev);
+int32_t slhip_event_record(slhip_ctx* ctx, slhip_event* ev);
+int32_t slhip_event_elapsed_ms(slhip_event* start, slhip_event* stop, float* ms); /* waits for stop */
+int32_t slhip_event_destroy(slhip_event* ev);
+
+/* Seeded counter-based uniform fill: x[i] = lo + (hi-lo) * u(seed, tag, i), u a 24-bit
+ * fraction from splitmix64((seed ^ (tag << 40)) + i).  Replaces RandOp::rand
+ * (src/rawops/cpu/rand.rs:7-12), whose generator is unseeded. */
+int32_t slhip_rand_uniform(slhip_ctx* ctx, uint64_t seed, uint64_t tag, float lo, float hi, size_t n,
+                           float* x);
+
+/* ---------------------------------------------------------------- GEMM -------------
+ * C[m×n] = op(A)·op(B) + beta·C.  trans_a: A is stored k×m; trans_b: B is stored n×k.
+ * Replaces GenericBlas::{gemm, gemmT, Tgemm} as called at src/ops2/gemm/cpu_stack.rs:39 and
+ * src/ops2/gemm/grad/cpu_stack.rs:36,39:
+ *     gemm (m,n,k,a,b,c) = slhip_sgemm(ctx,0,0,m,n,k,a,b,c,0)
+ *     gemmT(m,n,k,a,b,c) = slhip_sgemm(ctx,0,1,m,n,k,a,b,c,0)
+ *     Tgemm(m,n,k,a,b,c) = slhip_sgemm(ctx,1,0,m,n,k,a,b,c,0)
+ * beta = 0 is `Set`, beta = 1 is `Assign` (src/assign_or_set.rs; src/ops2/gemm/opencl.rs:138-139).
+ * C must not overlap A or B. */
+int32_t slhip_sgemm(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
+                    const float* a, const float* b, float* c, float beta);
+
+/* Gemm::gemm (src/ops2/gemm/mod.rs:21-32), trait argument order (m, k, n). */
+int32_t slhip_gemm(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,
+                   float* out);
+
+/* GemmGrad::gemm_grad (src/ops2/gemm/grad.rs:15-29; CPU body src/ops2/gemm/grad/cpu_stack.rs:24-41):
+ * lhs_grad[m×k] = out_grad·rhsᵀ, rhs_grad[k×n] = lhsᵀ·out_grad.  A NULL grad pointer means the
+ * operand does not require a gradient and that product is skipped.  beta 0 = SET (CPU
+ * behaviour), 1 = accumulate (OpenCL behaviour, src/ops2/gemm/grad/opencl.rs:20,33). */
+int32_t slhip_gemm_grad(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,
+                        float* lhs_grad, float* rhs_grad, const float* out_grad, float beta);
+
+/* Linear forward of the examples (examples/sine_net.rs:32-40: gemm + add_row_mut, optionally
+ * followed by Matrix::relu, src/matrix.rs:169-190) in one kernel: out = relu?(x[m×k]·w[k×n] + bias[n]).
+ * pre_act (may be NULL) receives the value before relu, which the relu gradient needs. */
+int32_t slhip_linear_fwd(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w,
+                         const float* bias, int32_t relu, float* pre_act, float* out);
+
+/* ---------------------------------------------------------------- reductions -------
+ * SumRows/SumCols (src/ops2/sum/mod.rs:19-25), MaxRows/MaxCols (src/ops2/max/mod.rs:20-26),
+ * MeanRows/MeanCols/Mean (src/ops2/mean/mod.rs:15-45), Sum/Max scalars
+ * (src/ops2/sum/cpu.rs:18-20, src/ops2/max/cpu.rs:23-25).  `out` is overwritten. */
+int32_t slhip_sum_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*cols*/);
+int32_t slhip_sum_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*rows*/);
+int32_t slhip_max_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*cols*/);
+int32_t slhip_max_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*rows*/);
+int32_t slhip_mean_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*cols*/);
+int32_t slhip_mean_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*rows*/);
+int32_t slhip_sum(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);
+int32_t slhip_max(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);
+int32_t slhip_mean(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);
+
+/* Backward traits (src/ops2/sum/grad.rs, src/ops2/max/grad.rs, src/ops2/mean/grad.rs); every
+ * one accumulates into x_grad (`+=`), as the CPU bodies do.
+ *   sum_rows_grad : x_grad[r,c] += out_grad[c]            (src/ops2/sum/grad/cpu.rs:41-48)
+ *   sum_cols_grad : x_grad[r,c] += out_grad[r]            (:50-56)
+ *   max_rows_grad : every r with x[r,c] == out[c] gets out_grad[c]   (src/ops2/max/grad/cpu.rs:40-55)
+ *   max_cols_grad : only the FIRST c with x[r,c] == out[r] gets out_grad[r]   (:57-69)
+ *   mean_rows_grad: x_grad[r,c] += (cols/len)·out_grad[c] (src/ops2/mean/grad/cpu.rs:43-54)
+ *   mean_cols_grad: x_grad[r,c] += out_grad[r]/cols       (:56-63) */
+int32_t slhip_sum_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad);
+int32_t slhip_sum_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad);
+int32_t slhip_max_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* out, const float* x,
+                            float* x_grad, const float* out_grad);
+int32_t slhip_max_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* out, const float* x,
+                            float* x_grad, const float* out_grad);
+int32_t slhip_mean_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad);
+int32_t slhip_mean_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad);
+
+/* ---------------------------------------------------------------- softmax ----------
+ * Softmax::softmax(samples, features, x) (src/ops2/softmax/mod.rs:16-18; CPU body
+ * src/ops2/softmax/cpu.rs:11-16 = max_cols, sub_cols, exp, sum_cols, div_cols) as ONE pass.
+ * SoftmaxGrad::softmax_grad (src/ops2/softmax/grad.rs:15-24; CPU body
+ * src/ops2/softmax/grad/cpu.rs:24-61 builds the Jacobian per sample): x_grad = s·(g − <s,g>),
+ * beta 0 = SET (CPU behaviour), 1 = accumulate. out may alias x; x_grad may alias out_grad. */
+int32_t slhip_softmax(slhip_ctx* ctx, size_t samples, size_t features, const float* x, float* out);
+int32_t slhip_softmax_grad(slhip_ctx* ctx, size_t samples, size_t features, float* x_grad,
+                           const float* out, const float* out_grad, float beta);
+
+/* ---------------------------------------------------------------- transpose --------
+ * Transpose::transpose(rows, cols, x) (src/ops2/transpose/mod.rs:17-21; slice_transpose
+ * src/ops2/transpose/cpu.rs:10-25): out[c·rows + r] = x[r·cols + c].  beta 0 = `Set`, 1 = `Assign`
+ * (+=, the OpenCL transpose_grad, src/ops2/transpose/grad/opencl.rs:21).  TranposeGrad is
+ * slhip_transpose(ctx, cols, rows, out_grad, x_grad, beta) (src/ops.rs:210-217). */
+int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, float beta);
+
+/* ---------------------------------------------------------------- row op (bias) ----
+ * RowOp::{add_row, add_row_mut} (src/ops2/row_op/mod.rs:17-47): out[r,c] = lhs[r,c] + rhs[c];
+ * out == lhs is the in-place add_row_mut.
+ * RowOpGrad::add_row_grad (src/ops2/row_op/grad/cpu.rs:54-64): lhs_grad is OVERWRITTEN with
+ * out_grad (skipped when NULL or the same pointer), rhs_grad[c] += Σ_r out_grad[r,c].
+ * RowOpGrad::add_row_mut_grad (:42-50): rhs_grad[c] += Σ_r out_grad[r,c]. */
+int32_t slhip_add_row(slhip_ctx* ctx, size_t rows, size_t cols, const float* lhs, const float* rhs, float* out);
+int32_t slhip_add_row_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* lhs_grad, float* rhs_grad,
+                           const float* out_grad);
+int32_t slhip_add_row_mut_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* rhs_grad, const float* out_grad);
+
+/* ---------------------------------------------------------------- elementwise ------
+ * BinaryElementWise::{add,sub,mul,div} (src/ops2/binary_ew/mod.rs:55-100) and
+ * BinaryElementWiseGrad with the closures of BinaryOpsMayGrad (src/ops.rs:115-171;
+ * slice_binary_grad src/ops2/binary_ew/grad/cpu_stack.rs:40-60): lg += dL·g, rg += dR·g.
+ * A NULL lg or rg skips that side.  out may alias l or r. */
+int32_t slhip_ew_binary(slhip_ctx* ctx, int32_t op, size_t n, const float* l, const float* r, float* out);
+int32_t slhip_ew_binary_grad(slhip_ctx* ctx, int32_t op, size_t n, const float* l, const float* r, float* lg,
+                             float* rg, const float* g);
+/* apply_fn / add_unary_grad: out[i] = f(x[i]); x_grad[i] += f'(x[i])·out_grad[i]. out may alias x. */
+int32_t slhip_ew_unary(slhip_ctx* ctx, int32_t op, float p, float q, size_t n, const float* x, float* out);
+int32_t slhip_ew_unary_grad(slhip_ctx* ctx, int32_t op, float p, size_t n, const float* x, float* x_grad,
+                            const float* out_grad);
+/* The chain of the elementwise workload, ((a+b)*c − d) -> pow 2 -> square, fused into one pass
+ * (same ops as examples/chained_perf.rs:86-90 chains: add, mul, sub, pow, square). */
+int32_t slhip_ew_chain(slhip_ctx* ctx, size_t n, const float* a, const float* b, const float* c,
+                       const float* d, float* out);
+
+/* ---------------------------------------------------------------- training helpers -
+ * Host loops of the examples that a device-resident training loop needs as kernels.
+ *   sgd_step : p[i] -= g[i]·lr                       (examples/sine_net.rs:105-116)
+ *   cce      : loss[r] = −ln Σ_c clip(p,1e-7,1−1e-7)·t (examples/nn.rs:124-138)
+ *   cce_grad : grad = (−(t/p))/rows                  (examples/nn.rs:140-152)
+ *   onehot   : out[r·classes + (size_t)cls[r]] = 1, rest 0 (src/ops2/onehot/cpu.rs:40-44) */
+int32_t slhip_sgd_step(slhip_ctx* ctx, size_t n, float* p, const float* g, float lr);
+int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets, float* loss);
+int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
+                       float* grad);
+int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLICED_HIP_H */

@@ -1,0 +1,105 @@
+// Shared definitions of the gfx950 backend: context, error plumbing, launch helpers and the
+// wave64 reduction primitives used by every bandwidth kernel.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/sliced_hip.h"
+
+#define SLHIP_API extern "C" __attribute__((visibility("default")))
+
+struct slhip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  bool owns_stream = false;
+  void* workspace = nullptr;     // partials of two-stage reductions and split-K GEMM
+  size_t workspace_bytes = 0;
+  int num_cu = 256;
+  char name[64] = {0};
+};
+
+struct slhip_event {
+  hipEvent_t ev;
+};
+
+namespace slhip {
+
+constexpr int WAVE = 64;
+constexpr size_t DEFAULT_WORKSPACE_BYTES = size_t(256) << 20;
+
+void set_error(const char* fmt, ...);
+int32_t hip_fail(hipError_t e, const char* what);
+
+#define SLHIP_CHECK_HIP(expr)                                   \
+  do {                                                          \
+    hipError_t _e = (expr);                                     \
+    if (_e != hipSuccess) return slhip::hip_fail(_e, #expr);    \
+  } while (0)
+
+#define SLHIP_REQUIRE(cond, msg)                                \
+  do {                                                          \
+    if (!(cond)) {                                              \
+      slhip::set_error("%s: %s", __func__, msg);                \
+      return SLHIP_EINVAL;                                      \
+    }                                                           \
+  } while (0)
+
+// rows*cols with overflow check; false on overflow or zero.
+inline bool checked_len(size_t rows, size_t cols, size_t* len) {
+  if (rows == 0 || cols == 0) return false;
+  if (rows > SIZE_MAX / cols) return false;
+  *len = rows * cols;
+  return *len <= (SIZE_MAX / sizeof(float));
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int32_t post_launch() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return hip_fail(e, "kernel launch");
+  return SLHIP_OK;
+}
+
+inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ------------------------------------------------------------------ device helpers
+struct SumOp {
+  static __device__ __forceinline__ float identity() { return 0.0f; }
+  static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+struct MaxOp {
+  static __device__ __forceinline__ float identity() { return -__builtin_huge_valf(); }
+  static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
+};
+
+// Butterfly reduction over `width` adjacent lanes (power of two, <= 64) of a wave64.
+template <class Op, int width = WAVE>
+__device__ __forceinline__ float wave_reduce(float v) {
+#pragma unroll
+  for (int off = width / 2; off > 0; off >>= 1) v = Op::apply(v, __shfl_xor(v, off, WAVE));
+  return v;
+}
+
+// Block-wide reduction; every thread receives the result. `smem` holds >= blockDim.x/64 floats.
+template <class Op>
+__device__ __forceinline__ float block_reduce(float v, float* smem) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + WAVE - 1) >> 6;
+  v = wave_reduce<Op>(v);
+  if (nw == 1) return v;
+  __syncthreads();  // smem may still be read from a previous call
+  if (lane == 0) smem[wid] = v;
+  __syncthreads();
+  float r = lane < nw ? smem[lane] : Op::identity();
+  r = wave_reduce<Op>(r);
+  return r;
+}
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+
+}  // namespace slhip

@@ -1,0 +1,439 @@
+// Streaming kernels: binary / unary elementwise ops and their gradients, the fused elementwise
+// chain, bias broadcast (row op), broadcast gradients of the reductions, SGD, cce, onehot.
+//
+// All of them are HBM-bound: one pass, float4 accesses, grid-stride over a grid sized to keep
+// every CU full.  Arithmetic is unfused f32 (the file is compiled with -ffp-contract=off) so
+// each op rounds exactly like the reference's scalar Rust loops.
+#include "common.hpp"
+
+namespace slhip {
+
+constexpr int EW_BLOCK = 256;
+
+inline unsigned ew_grid(const slhip_ctx* ctx, size_t work_items) {
+  size_t need = (work_items + EW_BLOCK - 1) / EW_BLOCK;
+  size_t cap = (size_t)ctx->num_cu * 16;
+  if (need < 1) need = 1;
+  return (unsigned)(need < cap ? need : cap);
+}
+
+// Generic elementwise driver.  F::apply(const float in[NIN], float io[NOUT]) computes one
+// element: io[] holds the current value of each output on entry when F::READS_OUT is set.
+template <int NIN, int NOUT, class F>
+struct EwArgs {
+  const float* in[NIN > 0 ? NIN : 1];
+  float* out[NOUT];
+  F f;
+};
+
+template <int NIN, int NOUT, class F, bool VEC>
+__global__ __launch_bounds__(EW_BLOCK) void ew_kernel(size_t n, EwArgs<NIN, NOUT, F> a) {
+  const size_t tid = (size_t)blockIdx.x * EW_BLOCK + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * EW_BLOCK;
+  size_t done = 0;
+  if (VEC) {
+    const size_t n4 = n >> 2;
+    for (size_t i = tid; i < n4; i += stride) {
+      float4 vin[NIN > 0 ? NIN : 1];
+      float4 vout[NOUT];
+#pragma unroll
+      for (int j = 0; j < NIN; ++j) vin[j] = ld4(a.in[j] + 4 * i);
+      if (F::READS_OUT) {
+#pragma unroll
+        for (int j = 0; j < NOUT; ++j) vout[j] = ld4(a.out[j] + 4 * i);
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float si[NIN > 0 ? NIN : 1], so[NOUT];
+#pragma unroll
+        for (int j = 0; j < NIN; ++j) si[j] = (&vin[j].x)[c];
+#pragma unroll
+        for (int j = 0; j < NOUT; ++j) so[j] = F::READS_OUT ? (&vout[j].x)[c] : 0.0f;
+        a.f.apply(si, so);
+#pragma unroll
+        for (int j = 0; j < NOUT; ++j) (&vout[j].x)[c] = so[j];
+      }
+#pragma unroll
+      for (int j = 0; j < NOUT; ++j) st4(a.out[j] + 4 * i, vout[j]);
+    }
+    done = n4 << 2;
+  }
+  for (size_t i = done + tid; i < n; i += stride) {
+    float si[NIN > 0 ? NIN : 1], so[NOUT];
+#pragma unroll
+    for (int j = 0; j < NIN; ++j) si[j] = a.in[j][i];
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) so[j] = F::READS_OUT ? a.out[j][i] : 0.0f;
+    a.f.apply(si, so);
+#pragma unroll
+    for (int j = 0; j < NOUT; ++j) a.out[j][i] = so[j];
+  }
+}
+
+template <int NIN, int NOUT, class F>
+int32_t ew_launch(slhip_ctx* ctx, size_t n, EwArgs<NIN, NOUT, F> a) {
+  if (n == 0) return SLHIP_OK;
+  bool vec = true;
+  for (int j = 0; j < NIN; ++j) vec = vec && aligned16(a.in[j]);
+  for (int j = 0; j < NOUT; ++j) vec = vec && aligned16(a.out[j]);
+  if (vec) {
+    unsigned grid = ew_grid(ctx, (n >> 2) + 1);
+    hipLaunchKernelGGL((ew_kernel<NIN, NOUT, F, true>), dim3(grid), dim3(EW_BLOCK), 0, ctx->stream, n, a);
+  } else {
+    unsigned grid = ew_grid(ctx, n);
+    hipLaunchKernelGGL((ew_kernel<NIN, NOUT, F, false>), dim3(grid), dim3(EW_BLOCK), 0, ctx->stream, n, a);
+  }
+  return post_launch();
+}
+
+// ------------------------------------------------------------------ functors
+template <int OP>
+struct BinF {
+  static constexpr bool READS_OUT = false;
+  __device__ __forceinline__ void apply(const float* in, float* o) const {
+    float a = in[0], b = in[1];
+    o[0] = OP == SLHIP_ADD ? a + b : OP == SLHIP_SUB ? a - b : OP == SLHIP_MUL ? a * b : a / b;
+  }
+};
+
+// in: l, r, g ; out: lg and/or rg (WHICH: 1 = lhs only, 2 = rhs only, 3 = both -> out[0]=lg, out[1]=rg)
+template <int OP, int WHICH>
+struct BinGradF {
+  static constexpr bool READS_OUT = true;
+  __device__ __forceinline__ void apply(const float* in, float* o) const {
+    float l = in[0], r = in[1], g = in[2];
+    float dl, dr;
+    if (OP == SLHIP_ADD) { dl = 1.0f; dr = 1.0f; }
+    else if (OP == SLHIP_SUB) { dl = 1.0f; dr = -1.0f; }
+    else if (OP == SLHIP_MUL) { dl = r; dr = l; }
+    else { dl = 1.0f / r; dr = -l / (r * r); }
+    if (WHICH == 1) o[0] += dl * g;
+    else if (WHICH == 2) o[0] += dr * g;
+    else { o[0] += dl * g; o[1] += dr * g; }
+  }
+};
+
+__device__ __forceinline__ float pow_ref(float x, float p) {
+  // powf proper: integer exponents of negative bases must not become NaN
+  return powf(x, p);
+}
+
+template <int OP>
+struct UnF {
+  static constexpr bool READS_OUT = false;
+  float p, q;
+  __device__ __forceinline__ void apply(const float* in, float* o) const {
+    float x = in[0];
+    switch (OP) {
+      case SLHIP_SQUARE: o[0] = x * x; break;
+      case SLHIP_POW: o[0] = pow_ref(x, p); break;
+      case SLHIP_RELU: o[0] = (x >= 0.0f ? 1.0f : 0.0f) * x; break;  // -0.0 for x<0, as geq(0)*x
+      case SLHIP_EXP: o[0] = expf(x); break;
+      case SLHIP_CLIP: o[0] = fminf(fmaxf(x, p), q); break;
+      case SLHIP_NEG_LN: o[0] = -logf(x); break;
+      case SLHIP_SCALE: o[0] = x * p; break;
+      default: o[0] = (-x) / p; break;
+    }
+  }
+};
+
+// in: x, g ; out: x_grad (+=)
+template <int OP>
+struct UnGradF {
+  static constexpr bool READS_OUT = true;
+  float p;
+  __device__ __forceinline__ void apply(const float* in, float* o) const {
+    float x = in[0], g = in[1], d;
+    switch (OP) {
+      case SLHIP_SQUARE: d = x * 2.0f; break;
+      case SLHIP_POW: d = pow_ref(x, p - 1.0f) * p; break;
+      case SLHIP_RELU: d = x >= 0.0f ? 1.0f : 0.0f; break;
+      case SLHIP_EXP: d = expf(x); break;
+      default: d = p; break;  // SLHIP_SCALE
+    }
+    o[0] += d * g;
+  }
+};
+
+struct ChainF {  // ((a+b)*c - d) -> pow 2 -> square
+  static constexpr bool READS_OUT = false;
+  __device__ __forceinline__ void apply(const float* in, float* o) const {
+    float t = (in[0] + in[1]) * in[2] - in[3];
+    float u = pow_ref(t, 2.0f);
+    o[0] = u * u;
+  }
+};
+
+struct SgdF {  // p -= g * lr
+  static constexpr bool READS_OUT = true;
+  float lr;
+  __device__ __forceinline__ void apply(const float* in, float* o) const { o[0] -= in[0] * lr; }
+};
+
+struct CceGradF {  // (-(t/p)) / rows ; in: p, t
+  static constexpr bool READS_OUT = false;
+  float rows;
+  __device__ __forceinline__ void apply(const float* in, float* o) const { o[0] = (-(in[1] / in[0])) / rows; }
+};
+
+// ------------------------------------------------------------------ broadcast kernels
+// MODE 0: out[r,c]  = lhs[r,c] + v[c]          (add_row / add_row_mut)
+// MODE 1: xg[r,c]  += s * v[c]                  (sum_rows_grad s=1, mean_rows_grad s=cols/len)
+// MODE 2: xg[r,c]  += v[r] (already scaled)     (sum_cols_grad; mean_cols_grad with DIV)
+// MODE 3: xg[r,c]  += (x[r,c]==v[c]) ? g[c] : 0 (max_rows_grad; v = out)
+// One block row-slab per blockIdx.y, columns across x; float4 when cols % 4 == 0.
+template <int MODE, bool VEC, bool DIVCOLS>
+__global__ __launch_bounds__(256) void bcast_kernel(size_t rows, size_t cols, const float* __restrict__ a,
+                                                    const float* __restrict__ v, const float* __restrict__ g,
+                                                    float* out, float s) {
+  constexpr int V = VEC ? 4 : 1;
+  const size_t colsv = cols / V;
+  const size_t total = rows * colsv;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  // (row, column-vector) of this thread's element, advanced incrementally: one division per
+  // thread instead of one per element.
+  const size_t i0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t sr = stride / colsv, sc = stride - sr * colsv;
+  size_t r = i0 / colsv, cv = i0 - r * colsv;
+  for (size_t i = i0; i < total; i += stride, r += sr, cv += sc) {
+    if (cv >= colsv) { cv -= colsv; ++r; }
+    const size_t c = cv * V;
+    const size_t off = r * cols + c;
+    float vv[4], o[4], av[4], gv[4];
+    if (VEC) {
+      float4 t;
+      if (MODE == 0 || MODE == 3) { t = ld4(a + off); av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w; }
+      if (MODE != 0) { t = ld4(out + off); o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w; }
+      if (MODE == 2) { vv[0] = vv[1] = vv[2] = vv[3] = DIVCOLS ? v[r] / s : v[r]; }
+      else { t = ld4(v + c); vv[0] = t.x; vv[1] = t.y; vv[2] = t.z; vv[3] = t.w; }
+      if (MODE == 3) { t = ld4(g + c); gv[0] = t.x; gv[1] = t.y; gv[2] = t.z; gv[3] = t.w; }
+    } else {
+      if (MODE == 0 || MODE == 3) av[0] = a[off];
+      if (MODE != 0) o[0] = out[off];
+      vv[0] = MODE == 2 ? (DIVCOLS ? v[r] / s : v[r]) : v[c];
+      if (MODE == 3) gv[0] = g[c];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      if (MODE == 0) o[j] = av[j] + vv[j];
+      else if (MODE == 1) o[j] += s * vv[j];
+      else if (MODE == 2) o[j] += vv[j];
+      else if (av[j] == vv[j]) o[j] += gv[j];
+    }
+    if (VEC) st4(out + off, make_float4(o[0], o[1], o[2], o[3]));
+    else out[off] = o[0];
+  }
+}
+
+template <int MODE, bool DIVCOLS = false>
+int32_t bcast_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* a, const float* v, const float* g,
+                     float* out, float s) {
+  bool vec = (cols % 4 == 0) && aligned16(out) && (MODE == 2 || aligned16(v)) &&
+             ((MODE != 0 && MODE != 3) || aligned16(a)) && (MODE != 3 || aligned16(g));
+  size_t total = rows * (vec ? cols / 4 : cols);
+  unsigned grid = ew_grid(ctx, total);
+  if (vec)
+    hipLaunchKernelGGL((bcast_kernel<MODE, true, DIVCOLS>), dim3(grid), dim3(256), 0, ctx->stream, rows, cols, a, v,
+                       g, out, s);
+  else
+    hipLaunchKernelGGL((bcast_kernel<MODE, false, DIVCOLS>), dim3(grid), dim3(256), 0, ctx->stream, rows, cols, a, v,
+                       g, out, s);
+  return post_launch();
+}
+
+// cce: one thread per row (rows are short: the class count)
+__global__ void cce_kernel(size_t rows, size_t cols, const float* __restrict__ p, const float* __restrict__ t,
+                           float* __restrict__ loss) {
+  size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const float lo = (float)1e-7, hi = (float)(1.0 - 1e-7);
+  float s = 0.0f;
+  for (size_t c = 0; c < cols; ++c) s += fminf(fmaxf(p[r * cols + c], lo), hi) * t[r * cols + c];
+  loss[r] = -logf(s);
+}
+
+__global__ void onehot_kernel(size_t n, size_t classes, const float* __restrict__ cls, float* __restrict__ out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * classes) return;
+  size_t r = i / classes, c = i - r * classes;
+  out[i] = ((size_t)cls[r] == c) ? 1.0f : 0.0f;
+}
+
+}  // namespace slhip
+
+using namespace slhip;
+
+// ---------------------------------------------------------------------------- C ABI
+SLHIP_API int32_t slhip_ew_binary(slhip_ctx* ctx, int32_t op, size_t n, const float* l, const float* r, float* out) {
+  SLHIP_REQUIRE(ctx && l && r && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+#define SL_BIN(OP)                                   \
+  case OP: {                                         \
+    EwArgs<2, 1, BinF<OP>> a{{l, r}, {out}, {}};     \
+    return ew_launch(ctx, n, a);                     \
+  }
+  switch (op) {
+    SL_BIN(SLHIP_ADD) SL_BIN(SLHIP_SUB) SL_BIN(SLHIP_MUL) SL_BIN(SLHIP_DIV)
+    default: break;
+  }
+#undef SL_BIN
+  set_error("slhip_ew_binary: unknown op %d", op);
+  return SLHIP_EINVAL;
+}
+
+template <int OP>
+static int32_t bin_grad(slhip_ctx* ctx, size_t n, const float* l, const float* r, float* lg, float* rg,
+                        const float* g) {
+  if (lg && rg) {
+    EwArgs<3, 2, BinGradF<OP, 3>> a{{l, r, g}, {lg, rg}, {}};
+    return ew_launch(ctx, n, a);
+  } else if (lg) {
+    EwArgs<3, 1, BinGradF<OP, 1>> a{{l, r, g}, {lg}, {}};
+    return ew_launch(ctx, n, a);
+  } else if (rg) {
+    EwArgs<3, 1, BinGradF<OP, 2>> a{{l, r, g}, {rg}, {}};
+    return ew_launch(ctx, n, a);
+  }
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_ew_binary_grad(slhip_ctx* ctx, int32_t op, size_t n, const float* l, const float* r,
+                                       float* lg, float* rg, const float* g) {
+  SLHIP_REQUIRE(ctx && l && r && g, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  if (lg && lg == rg) {
+    set_error("slhip_ew_binary_grad: lhs_grad and rhs_grad alias");
+    return SLHIP_EALIAS;
+  }
+  switch (op) {
+    case SLHIP_ADD: return bin_grad<SLHIP_ADD>(ctx, n, l, r, lg, rg, g);
+    case SLHIP_SUB: return bin_grad<SLHIP_SUB>(ctx, n, l, r, lg, rg, g);
+    case SLHIP_MUL: return bin_grad<SLHIP_MUL>(ctx, n, l, r, lg, rg, g);
+    case SLHIP_DIV: return bin_grad<SLHIP_DIV>(ctx, n, l, r, lg, rg, g);
+    default: break;
+  }
+  set_error("slhip_ew_binary_grad: unknown op %d", op);
+  return SLHIP_EINVAL;
+}
+
+SLHIP_API int32_t slhip_ew_unary(slhip_ctx* ctx, int32_t op, float p, float q, size_t n, const float* x, float* out) {
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+#define SL_UN(OP)                                    \
+  case OP: {                                         \
+    EwArgs<1, 1, UnF<OP>> a{{x}, {out}, {p, q}};     \
+    return ew_launch(ctx, n, a);                     \
+  }
+  switch (op) {
+    SL_UN(SLHIP_SQUARE) SL_UN(SLHIP_POW) SL_UN(SLHIP_RELU) SL_UN(SLHIP_EXP) SL_UN(SLHIP_CLIP)
+    SL_UN(SLHIP_NEG_LN) SL_UN(SLHIP_SCALE) SL_UN(SLHIP_NEG_DIV)
+    default: break;
+  }
+#undef SL_UN
+  set_error("slhip_ew_unary: unknown op %d", op);
+  return SLHIP_EINVAL;
+}
+
+SLHIP_API int32_t slhip_ew_unary_grad(slhip_ctx* ctx, int32_t op, float p, size_t n, const float* x, float* x_grad,
+                                      const float* out_grad) {
+  SLHIP_REQUIRE(ctx && x && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+#define SL_UNG(OP)                                              \
+  case OP: {                                                    \
+    EwArgs<2, 1, UnGradF<OP>> a{{x, out_grad}, {x_grad}, {p}};  \
+    return ew_launch(ctx, n, a);                                \
+  }
+  switch (op) {
+    SL_UNG(SLHIP_SQUARE) SL_UNG(SLHIP_POW) SL_UNG(SLHIP_RELU) SL_UNG(SLHIP_EXP) SL_UNG(SLHIP_SCALE)
+    default: break;
+  }
+#undef SL_UNG
+  set_error("slhip_ew_unary_grad: op %d has no gradient", op);
+  return SLHIP_EINVAL;
+}
+
+SLHIP_API int32_t slhip_ew_chain(slhip_ctx* ctx, size_t n, const float* a, const float* b, const float* c,
+                                 const float* d, float* out) {
+  SLHIP_REQUIRE(ctx && a && b && c && d && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  EwArgs<4, 1, ChainF> args{{a, b, c, d}, {out}, {}};
+  return ew_launch(ctx, n, args);
+}
+
+SLHIP_API int32_t slhip_sgd_step(slhip_ctx* ctx, size_t n, float* p, const float* g, float lr) {
+  SLHIP_REQUIRE(ctx && p && g, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  EwArgs<1, 1, SgdF> a{{g}, {p}, {lr}};
+  return ew_launch(ctx, n, a);
+}
+
+SLHIP_API int32_t slhip_add_row(slhip_ctx* ctx, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                                float* out) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && lhs && rhs && out, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<0>(ctx, rows, cols, lhs, rhs, nullptr, out, 0.0f);
+}
+
+SLHIP_API int32_t slhip_sum_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<1>(ctx, rows, cols, nullptr, out_grad, nullptr, x_grad, 1.0f);
+}
+
+SLHIP_API int32_t slhip_mean_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<1>(ctx, rows, cols, nullptr, out_grad, nullptr, x_grad, (float)cols / (float)len);
+}
+
+SLHIP_API int32_t slhip_sum_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<2>(ctx, rows, cols, nullptr, out_grad, nullptr, x_grad, 1.0f);
+}
+
+SLHIP_API int32_t slhip_mean_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<2, true>(ctx, rows, cols, nullptr, out_grad, nullptr, x_grad, (float)cols);
+}
+
+SLHIP_API int32_t slhip_max_rows_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* out, const float* x,
+                                      float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && out && x && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return bcast_launch<3>(ctx, rows, cols, x, out, out_grad, x_grad, 0.0f);
+}
+
+SLHIP_API int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
+                            float* loss) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && preds && targets && loss, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  hipLaunchKernelGGL(cce_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, ctx->stream, rows, cols, preds, targets,
+                     loss);
+  return post_launch();
+}
+
+SLHIP_API int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
+                                 float* grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && preds && targets && grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  EwArgs<2, 1, CceGradF> a{{preds, targets}, {grad}, {(float)rows}};
+  return ew_launch(ctx, len, a);
+}
+
+SLHIP_API int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* out) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && cls && out, "null argument");
+  SLHIP_REQUIRE(checked_len(n, classes, &len), "bad dims");
+  hipLaunchKernelGGL(onehot_kernel, dim3(ceil_div(len, 256)), dim3(256), 0, ctx->stream, n, classes, cls, out);
+  return post_launch();
+}

@@ -1,0 +1,458 @@
+// Row / column reductions (sum, max, mean), the scalar reductions, the bias gradient and the
+// first-tie max gradient.  All HBM-bound: every input element is read exactly once with
+// float4 loads; partial results of the two-stage forms live in the context workspace.
+//
+// Naming (kept from the reference): *_cols reduces along the contiguous axis (one value per
+// row); *_rows reduces along the strided axis (one value per column).
+#include "common.hpp"
+
+namespace slhip {
+
+// How a finished value is written: out = v*scale (+ out if accumulate).
+struct Finalize {
+  float scale;     // 1 for sum/max, 1/n for means (applied as a division to match the reference)
+  int divide;      // 1: out = v / scale_div
+  int accumulate;  // 1: out += v
+};
+__device__ __forceinline__ void finalize_store(float* p, float v, Finalize f) {
+  if (f.divide) v = v / f.scale;
+  if (f.accumulate) v = *p + v;
+  *p = v;
+}
+
+// ---------------------------------------------------------------------------------------
+// Contiguous-axis reduction.  TPR lanes (power of two <= 64) or a whole block (TPR == 0) own one
+// row segment; gridDim.y = number of segments a row is split into (partials when > 1).
+// ---------------------------------------------------------------------------------------
+template <class Op, bool VEC, int TPR>
+__global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols, const float* __restrict__ x,
+                                                        float* __restrict__ out, Finalize fin) {
+  __shared__ float smem[8];
+  constexpr int V = VEC ? 4 : 1;
+  constexpr int LANES = TPR == 0 ? 256 : TPR;
+  constexpr int ROWS_PER_BLOCK = TPR == 0 ? 1 : 256 / TPR;
+  const size_t colsv = cols / V;
+  const unsigned nseg = gridDim.y, seg = blockIdx.y;
+  const size_t seg_len = (colsv + nseg - 1) / nseg;
+  const size_t cbeg = (size_t)seg * seg_len;
+  const size_t cend = cbeg + seg_len < colsv ? cbeg + seg_len : colsv;
+  const int lane = TPR == 0 ? threadIdx.x : (threadIdx.x % LANES);
+  const size_t row = (size_t)blockIdx.x * ROWS_PER_BLOCK + (TPR == 0 ? 0 : threadIdx.x / LANES);
+  const bool active = row < rows;
+
+  float a0 = Op::identity(), a1 = Op::identity(), a2 = Op::identity(), a3 = Op::identity();
+  if (active) {
+    const float* xr = x + row * cols;
+    size_t c = cbeg + lane;
+    if (VEC) {
+      for (; c + 3 * LANES < cend; c += 4 * LANES) {
+        float4 v0 = ld4(xr + 4 * c), v1 = ld4(xr + 4 * (c + LANES)), v2 = ld4(xr + 4 * (c + 2 * LANES)),
+               v3 = ld4(xr + 4 * (c + 3 * LANES));
+        a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
+        a1 = Op::apply(a1, Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)));
+        a2 = Op::apply(a2, Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)));
+        a3 = Op::apply(a3, Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)));
+      }
+      for (; c < cend; c += LANES) {
+        float4 v0 = ld4(xr + 4 * c);
+        a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
+      }
+    } else {
+      for (; c + 3 * LANES < cend; c += 4 * LANES) {
+        a0 = Op::apply(a0, xr[c]);
+        a1 = Op::apply(a1, xr[c + LANES]);
+        a2 = Op::apply(a2, xr[c + 2 * LANES]);
+        a3 = Op::apply(a3, xr[c + 3 * LANES]);
+      }
+      for (; c < cend; c += LANES) a0 = Op::apply(a0, xr[c]);
+    }
+  }
+  float v = Op::apply(Op::apply(a0, a1), Op::apply(a2, a3));
+  if (TPR == 0) {
+    v = block_reduce<Op>(v, smem);
+    if (threadIdx.x == 0) {
+      if (nseg > 1) out[row * nseg + seg] = v;
+      else finalize_store(out + row, v, fin);
+    }
+  } else {
+    v = wave_reduce<Op, (TPR > 0 ? TPR : 1)>(v);
+    if (active && lane == 0) {
+      if (nseg > 1) out[row * nseg + seg] = v;
+      else finalize_store(out + row, v, fin);
+    }
+  }
+}
+
+template <class Op, bool VEC>
+static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, unsigned nseg,
+                                Finalize fin) {
+  const size_t colsv = cols / (VEC ? 4 : 1);
+  const size_t per_seg = (colsv + nseg - 1) / nseg;
+  // lanes per row: about 4 vectors per lane, a whole block once a segment is long
+  int tpr;
+  if (per_seg >= 1024) tpr = 0;
+  else {
+    tpr = 1;
+    while (tpr < 64 && (size_t)tpr * 4 < per_seg) tpr <<= 1;
+  }
+#define SL_RR(T)                                                                                              \
+  case T: {                                                                                                   \
+    unsigned rpb = T == 0 ? 1 : 256 / (T == 0 ? 1 : T);                                                       \
+    dim3 grid(ceil_div(rows, rpb), nseg);                                                                     \
+    hipLaunchKernelGGL((rowreduce_kernel<Op, VEC, T>), grid, dim3(256), 0, ctx->stream, rows, cols, x, out, fin); \
+    break;                                                                                                    \
+  }
+  switch (tpr) {
+    SL_RR(0) SL_RR(1) SL_RR(2) SL_RR(4) SL_RR(8) SL_RR(16) SL_RR(32) SL_RR(64)
+  }
+#undef SL_RR
+  return post_launch();
+}
+
+// out[r] = reduce over the contiguous axis.
+template <class Op>
+static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
+  // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
+  if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, rows * sizeof(float));
+  const bool vec = (cols % 4 == 0) && aligned16(x);
+  const size_t colsv = cols / (vec ? 4 : 1);
+  // few long rows: split every row so the whole chip is busy
+  unsigned nseg = 1;
+  const size_t want_blocks = (size_t)ctx->num_cu * 8;
+  if (rows < want_blocks && colsv >= 8192) {
+    size_t s = (want_blocks + rows - 1) / rows;
+    size_t max_s = colsv / 2048;  // each segment keeps >= 2048 vectors
+    if (s > max_s) s = max_s;
+    if (s > 1) nseg = (unsigned)s;
+  }
+  if (nseg == 1) return vec ? rowreduce_launch<Op, true>(ctx, rows, cols, x, out, 1, fin)
+                            : rowreduce_launch<Op, false>(ctx, rows, cols, x, out, 1, fin);
+  if (rows * nseg * sizeof(float) > ctx->workspace_bytes) {
+    set_error("reduce over columns: %zu x %u partials exceed the workspace", rows, nseg);
+    return SLHIP_EWORKSPACE;
+  }
+  float* part = (float*)ctx->workspace;
+  Finalize none{1.0f, 0, 0};
+  int32_t rc = vec ? rowreduce_launch<Op, true>(ctx, rows, cols, x, part, nseg, none)
+                   : rowreduce_launch<Op, false>(ctx, rows, cols, x, part, nseg, none);
+  if (rc) return rc;
+  return rowreduce_launch<Op, false>(ctx, rows, nseg, part, out, 1, fin);
+}
+
+// ---------------------------------------------------------------------------------------
+// Strided-axis reduction, stage 1.  The matrix is viewed as rows x colsv vectors; thread t owns
+// column vector (t % colsv) and the rows g, g+G, g+2G, ... with g = t / colsv, so that one sweep
+// of the whole grid reads one contiguous span of G rows.  Result: partial[g, :] (G x cols).
+// ---------------------------------------------------------------------------------------
+template <class Op, bool VEC>
+__global__ __launch_bounds__(256) void colreduce_kernel(size_t rows, size_t cols, size_t G,
+                                                        const float* __restrict__ x, float* __restrict__ part) {
+  constexpr int V = VEC ? 4 : 1;
+  const size_t colsv = cols / V;
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= colsv * G) return;
+  const size_t g = t / colsv, cv = t - g * colsv;
+  const size_t step = G * cols;  // elements between two rows of this thread
+  const float* p = x + g * cols + cv * V;
+  size_t r = g;
+  if (VEC) {
+    float4 a0 = make_float4(Op::identity(), Op::identity(), Op::identity(), Op::identity());
+    float4 a1 = a0, a2 = a0, a3 = a0;
+#define SL_ACC(A, Q) A.x = Op::apply(A.x, Q.x); A.y = Op::apply(A.y, Q.y); A.z = Op::apply(A.z, Q.z); A.w = Op::apply(A.w, Q.w);
+    for (; r + 3 * G < rows; r += 4 * G, p += 4 * step) {
+      float4 v0 = ld4(p), v1 = ld4(p + step), v2 = ld4(p + 2 * step), v3 = ld4(p + 3 * step);
+      SL_ACC(a0, v0) SL_ACC(a1, v1) SL_ACC(a2, v2) SL_ACC(a3, v3)
+    }
+    for (; r < rows; r += G, p += step) {
+      float4 v0 = ld4(p);
+      SL_ACC(a0, v0)
+    }
+    SL_ACC(a0, a1) SL_ACC(a2, a3) SL_ACC(a0, a2)
+#undef SL_ACC
+    st4(part + g * cols + cv * 4, a0);
+  } else {
+    float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
+    for (; r + 3 * G < rows; r += 4 * G, p += 4 * step) {
+      a0 = Op::apply(a0, p[0]);
+      a1 = Op::apply(a1, p[step]);
+      a2 = Op::apply(a2, p[2 * step]);
+      a3 = Op::apply(a3, p[3 * step]);
+    }
+    for (; r < rows; r += G, p += step) a0 = Op::apply(a0, p[0]);
+    part[g * cols + cv] = Op::apply(Op::apply(a0, a1), Op::apply(a2, a3));
+  }
+}
+
+// Stage 2 (also the only stage for short matrices): a block owns CW adjacent columns, its
+// 256/CW row-lanes stride over the rows and combine through LDS.
+template <class Op, int CW>
+__global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_t cols, const float* __restrict__ x,
+                                                              float* __restrict__ out, Finalize fin) {
+  constexpr int RL = 256 / CW;
+  __shared__ float sm[256];
+  const int cx = threadIdx.x % CW, ry = threadIdx.x / CW;
+  const size_t c = (size_t)blockIdx.x * CW + cx;
+  float a0 = Op::identity(), a1 = a0;
+  if (c < cols) {
+    size_t r = ry;
+    for (; r + RL < rows; r += 2 * RL) {
+      a0 = Op::apply(a0, x[r * cols + c]);
+      a1 = Op::apply(a1, x[(r + RL) * cols + c]);
+    }
+    for (; r < rows; r += RL) a0 = Op::apply(a0, x[r * cols + c]);
+  }
+  sm[threadIdx.x] = Op::apply(a0, a1);
+  __syncthreads();
+#pragma unroll
+  for (int s = RL / 2; s > 0; s >>= 1) {
+    if (ry < s) sm[threadIdx.x] = Op::apply(sm[threadIdx.x], sm[threadIdx.x + s * CW]);
+    __syncthreads();
+  }
+  if (ry == 0 && c < cols) finalize_store(out + c, sm[cx], fin);
+}
+
+template <class Op>
+static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out,
+                                      Finalize fin) {
+  if (cols >= 64 && rows <= 64) {
+    hipLaunchKernelGGL((colreduce_final_kernel<Op, 64>), dim3(ceil_div(cols, 64)), dim3(256), 0, ctx->stream, rows,
+                       cols, x, out, fin);
+  } else if (cols >= 16) {
+    hipLaunchKernelGGL((colreduce_final_kernel<Op, 16>), dim3(ceil_div(cols, 16)), dim3(256), 0, ctx->stream, rows,
+                       cols, x, out, fin);
+  } else if (cols >= 4) {
+    hipLaunchKernelGGL((colreduce_final_kernel<Op, 4>), dim3(ceil_div(cols, 4)), dim3(256), 0, ctx->stream, rows,
+                       cols, x, out, fin);
+  } else {
+    hipLaunchKernelGGL((colreduce_final_kernel<Op, 1>), dim3(ceil_div(cols, 1)), dim3(256), 0, ctx->stream, rows,
+                       cols, x, out, fin);
+  }
+  return post_launch();
+}
+
+// ---------------------------------------------------------------------------------------
+// Whole-buffer reduction: per-block partials, then one block.
+// ---------------------------------------------------------------------------------------
+template <class Op, bool VEC>
+__global__ __launch_bounds__(256) void fullreduce_kernel(size_t n, const float* __restrict__ x,
+                                                         float* __restrict__ part) {
+  __shared__ float smem[8];
+  const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
+  size_t done = 0;
+  if (VEC) {
+    const size_t n4 = n >> 2;
+    size_t i = tid;
+    for (; i + 3 * stride < n4; i += 4 * stride) {
+      float4 v0 = ld4(x + 4 * i), v1 = ld4(x + 4 * (i + stride)), v2 = ld4(x + 4 * (i + 2 * stride)),
+             v3 = ld4(x + 4 * (i + 3 * stride));
+      a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
+      a1 = Op::apply(a1, Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)));
+      a2 = Op::apply(a2, Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)));
+      a3 = Op::apply(a3, Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)));
+    }
+    for (; i < n4; i += stride) {
+      float4 v0 = ld4(x + 4 * i);
+      a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
+    }
+    done = n4 << 2;
+  }
+  for (size_t i = done + tid; i < n; i += stride) a0 = Op::apply(a0, x[i]);
+  float v = block_reduce<Op>(Op::apply(Op::apply(a0, a1), Op::apply(a2, a3)), smem);
+  if (threadIdx.x == 0) part[blockIdx.x] = v;
+}
+
+template <class Op>
+__global__ __launch_bounds__(1024) void fullreduce_final_kernel(size_t n, const float* __restrict__ part,
+                                                                float* __restrict__ out, Finalize fin) {
+  __shared__ float smem[16];
+  float a = Op::identity();
+  for (size_t i = threadIdx.x; i < n; i += 1024) a = Op::apply(a, part[i]);
+  a = block_reduce<Op>(a, smem);
+  if (threadIdx.x == 0) finalize_store(out, a, fin);
+}
+
+template <class Op>
+static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin) {
+  const bool vec = aligned16(x);
+  size_t items = vec ? (n >> 2) + 1 : n;
+  size_t blocks = (items + 256 * 8 - 1) / (256 * 8);
+  size_t cap = (size_t)ctx->num_cu * 8;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  float* part = (float*)ctx->workspace;
+  if (vec)
+    hipLaunchKernelGGL((fullreduce_kernel<Op, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
+  else
+    hipLaunchKernelGGL((fullreduce_kernel<Op, false>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
+  int32_t rc = post_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL((fullreduce_final_kernel<Op>), dim3(1), dim3(1024), 0, ctx->stream, blocks, part, out, fin);
+  return post_launch();
+}
+
+// out[c] = reduce over the strided axis.
+template <class Op>
+static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
+  if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin);
+  // one row: the reduction over rows is that row itself
+  if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, cols * sizeof(float));
+  const bool vec = (cols % 4 == 0) && aligned16(x);
+  const size_t colsv = cols / (vec ? 4 : 1);
+  // number of row groups: fill the chip (about 2048 threads per CU) but keep >= 16 rows per thread
+  const size_t target_threads = (size_t)ctx->num_cu * 2048;
+  size_t G = (target_threads + colsv - 1) / colsv;
+  if (G > rows / 16) G = rows / 16;
+  const size_t ws_floats = ctx->workspace_bytes / sizeof(float);
+  if (G > 1 && G * cols > ws_floats) G = ws_floats / cols;
+  if (G <= 1) return colreduce_final_launch<Op>(ctx, rows, cols, x, out, fin);
+  float* part = (float*)ctx->workspace;
+  const size_t threads = colsv * G;
+  if (vec)
+    hipLaunchKernelGGL((colreduce_kernel<Op, true>), dim3(ceil_div(threads, 256)), dim3(256), 0, ctx->stream, rows,
+                       cols, G, x, part);
+  else
+    hipLaunchKernelGGL((colreduce_kernel<Op, false>), dim3(ceil_div(threads, 256)), dim3(256), 0, ctx->stream, rows,
+                       cols, G, x, part);
+  int32_t rc = post_launch();
+  if (rc) return rc;
+  return colreduce_final_launch<Op>(ctx, G, cols, part, out, fin);
+}
+
+// ---------------------------------------------------------------------------------------
+// max_cols_grad: the FIRST column equal to the row maximum receives out_grad[row].
+// LANES lanes scan one row; the smallest matching index wins.
+// ---------------------------------------------------------------------------------------
+template <int TPR>
+__global__ __launch_bounds__(256) void max_cols_grad_kernel(size_t rows, size_t cols, const float* __restrict__ out,
+                                                            const float* __restrict__ x, float* __restrict__ x_grad,
+                                                            const float* __restrict__ out_grad) {
+  __shared__ unsigned long long smin;
+  constexpr int LANES = TPR == 0 ? 256 : TPR;
+  constexpr int RPB = TPR == 0 ? 1 : 256 / TPR;
+  const int lane = TPR == 0 ? threadIdx.x : threadIdx.x % LANES;
+  const size_t row = (size_t)blockIdx.x * RPB + (TPR == 0 ? 0 : threadIdx.x / LANES);
+  const unsigned long long NONE = ~0ull;
+  unsigned long long best = NONE;
+  if (TPR == 0) {
+    if (threadIdx.x == 0) smin = NONE;
+    __syncthreads();
+  }
+  if (row < rows) {
+    const float m = out[row];
+    const float* xr = x + row * cols;
+    // lanes interleave, so the first hit of a lane is its smallest index
+    for (size_t c = lane; c < cols; c += LANES)
+      if (xr[c] == m) { best = c; break; }
+  }
+  if (TPR == 0) {
+    if (best != NONE) atomicMin(&smin, best);
+    __syncthreads();
+    if (threadIdx.x == 0 && row < rows && smin != NONE) x_grad[row * cols + smin] += out_grad[row];
+  } else {
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) {
+      unsigned long long o = __shfl_xor(best, off, WAVE);
+      best = o < best ? o : best;
+    }
+    if (row < rows && lane == 0 && best != NONE) x_grad[row * cols + best] += out_grad[row];
+  }
+}
+
+}  // namespace slhip
+
+using namespace slhip;
+
+#define SL_DIMS_OK()                                           \
+  size_t len;                                                  \
+  SLHIP_REQUIRE(ctx && x && out, "null argument");             \
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");    \
+  (void)len;
+
+SLHIP_API int32_t slhip_sum_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_cols<SumOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_max_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_cols<MaxOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_mean_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_cols<SumOp>(ctx, rows, cols, x, out, Finalize{(float)cols, 1, 0});
+}
+SLHIP_API int32_t slhip_sum_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_rows<SumOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_max_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_rows<MaxOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_mean_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  return reduce_rows<SumOp>(ctx, rows, cols, x, out, Finalize{(float)rows, 1, 0});
+}
+
+SLHIP_API int32_t slhip_sum(slhip_ctx* ctx, size_t n, const float* x, float* out) {
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  return reduce_all<SumOp>(ctx, n, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_max(slhip_ctx* ctx, size_t n, const float* x, float* out) {
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  return reduce_all<MaxOp>(ctx, n, x, out, Finalize{1.0f, 0, 0});
+}
+SLHIP_API int32_t slhip_mean(slhip_ctx* ctx, size_t n, const float* x, float* out) {
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  SLHIP_REQUIRE(n > 0, "empty buffer");
+  return reduce_all<SumOp>(ctx, n, x, out, Finalize{(float)n, 1, 0});
+}
+
+// rhs_grad[c] += sum over rows of out_grad[r, c]
+SLHIP_API int32_t slhip_add_row_mut_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* rhs_grad,
+                                         const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && rhs_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  return reduce_rows<SumOp>(ctx, rows, cols, out_grad, rhs_grad, Finalize{1.0f, 0, 1});
+}
+
+SLHIP_API int32_t slhip_add_row_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* lhs_grad, float* rhs_grad,
+                                     const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && rhs_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  if (lhs_grad && lhs_grad != out_grad) {
+    int32_t rc = slhip_memcpy_d2d(ctx, lhs_grad, out_grad, len * sizeof(float));
+    if (rc) return rc;
+  }
+  return reduce_rows<SumOp>(ctx, rows, cols, out_grad, rhs_grad, Finalize{1.0f, 0, 1});
+}
+
+SLHIP_API int32_t slhip_max_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* out, const float* x,
+                                      float* x_grad, const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && out && x && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  int tpr;
+  if (cols >= 4096) tpr = 0;
+  else {
+    tpr = 1;
+    while (tpr < 64 && (size_t)tpr * 8 < cols) tpr <<= 1;
+  }
+#define SL_MCG(T)                                                                                          \
+  case T: {                                                                                                \
+    unsigned rpb = T == 0 ? 1 : 256 / (T == 0 ? 1 : T);                                                    \
+    hipLaunchKernelGGL((max_cols_grad_kernel<T>), dim3(ceil_div(rows, rpb)), dim3(256), 0, ctx->stream,    \
+                       rows, cols, out, x, x_grad, out_grad);                                              \
+    break;                                                                                                 \
+  }
+  switch (tpr) {
+    SL_MCG(0) SL_MCG(1) SL_MCG(2) SL_MCG(4) SL_MCG(8) SL_MCG(16) SL_MCG(32) SL_MCG(64)
+  }
+#undef SL_MCG
+  return post_launch();
+}

@@ -1,0 +1,236 @@
+// Row-wise softmax, forward and backward, as single-pass kernels: a row is loaded once into
+// registers (float4 per lane), reduced with wave64 shuffles (plus LDS across waves for long
+// rows), and written once.  Forward moves 8 B/element, backward 12 B/element (+4 when it
+// accumulates) - the algorithmic minimum.
+//
+// The reference builds the forward from five passes (max_cols, sub_cols, exp, sum_cols,
+// div_cols) and the backward from a per-sample Jacobian; the arithmetic per element is the
+// same: e = exp(x - max); out = e / sum(e);  x_grad = s * (g - <s, g>).
+#include "common.hpp"
+
+namespace slhip {
+
+// Reduce over the LANES threads that share a row (LANES <= 64: shuffles; else: whole block).
+template <class Op, int LANES>
+__device__ __forceinline__ float row_reduce(float v, float* smem) {
+  if (LANES <= 64) return wave_reduce<Op, (LANES <= 64 ? LANES : 64)>(v);
+  return block_reduce<Op>(v, smem);
+}
+
+template <bool VEC, int LANES, int ITEMS>
+__global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(size_t rows, size_t cols,
+                                                                                const float* __restrict__ x,
+                                                                                float* __restrict__ out) {
+  __shared__ float smem[16];
+  constexpr int V = VEC ? 4 : 1;
+  constexpr int RPB = LANES <= 64 ? 256 / LANES : 1;
+  const size_t colsv = cols / V;
+  const int lane = threadIdx.x % LANES;
+  const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / LANES;
+  const bool active = row < rows;
+  const float NEG_INF = -__builtin_huge_valf();
+
+  float v[ITEMS][V];
+  float m = NEG_INF;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const size_t c = (size_t)lane + (size_t)j * LANES;
+    if (active && c < colsv) {
+      if (VEC) {
+        float4 t = ld4(x + row * cols + 4 * c);
+        v[j][0] = t.x; v[j][V > 1 ? 1 : 0] = t.y; v[j][V > 1 ? 2 : 0] = t.z; v[j][V > 1 ? 3 : 0] = t.w;
+      } else {
+        v[j][0] = x[row * cols + c];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < V; ++q) v[j][q] = NEG_INF;
+    }
+#pragma unroll
+    for (int q = 0; q < V; ++q) m = fmaxf(m, v[j][q]);
+  }
+  m = row_reduce<MaxOp, LANES>(m, smem);
+
+  float s = 0.0f;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const size_t c = (size_t)lane + (size_t)j * LANES;
+    const bool in = active && c < colsv;
+#pragma unroll
+    for (int q = 0; q < V; ++q) {
+      float e = in ? expf(v[j][q] - m) : 0.0f;
+      v[j][q] = e;
+      s += e;
+    }
+  }
+  s = row_reduce<SumOp, LANES>(s, smem);
+
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const size_t c = (size_t)lane + (size_t)j * LANES;
+    if (active && c < colsv) {
+      if (VEC) st4(out + row * cols + 4 * c, make_float4(v[j][0] / s, v[j][V > 1 ? 1 : 0] / s, v[j][V > 1 ? 2 : 0] / s,
+                                                        v[j][V > 1 ? 3 : 0] / s));
+      else out[row * cols + c] = v[j][0] / s;
+    }
+  }
+}
+
+template <bool VEC, int LANES, int ITEMS>
+__global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(size_t rows, size_t cols,
+                                                                                float* x_grad,
+                                                                                const float* __restrict__ out,
+                                                                                const float* out_grad, float beta) {
+  __shared__ float smem[16];
+  constexpr int V = VEC ? 4 : 1;
+  constexpr int RPB = LANES <= 64 ? 256 / LANES : 1;
+  const size_t colsv = cols / V;
+  const int lane = threadIdx.x % LANES;
+  const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / LANES;
+  const bool active = row < rows;
+
+  float s[ITEMS][V], g[ITEMS][V];
+  float dot = 0.0f;
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const size_t c = (size_t)lane + (size_t)j * LANES;
+    if (active && c < colsv) {
+      if (VEC) {
+        float4 a = ld4(out + row * cols + 4 * c), b = ld4(out_grad + row * cols + 4 * c);
+        s[j][0] = a.x; s[j][V > 1 ? 1 : 0] = a.y; s[j][V > 1 ? 2 : 0] = a.z; s[j][V > 1 ? 3 : 0] = a.w;
+        g[j][0] = b.x; g[j][V > 1 ? 1 : 0] = b.y; g[j][V > 1 ? 2 : 0] = b.z; g[j][V > 1 ? 3 : 0] = b.w;
+      } else {
+        s[j][0] = out[row * cols + c];
+        g[j][0] = out_grad[row * cols + c];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < V; ++q) { s[j][q] = 0.0f; g[j][q] = 0.0f; }
+    }
+#pragma unroll
+    for (int q = 0; q < V; ++q) dot += s[j][q] * g[j][q];
+  }
+  dot = row_reduce<SumOp, LANES>(dot, smem);
+
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const size_t c = (size_t)lane + (size_t)j * LANES;
+    if (active && c < colsv) {
+      float r[V];
+#pragma unroll
+      for (int q = 0; q < V; ++q) r[q] = s[j][q] * (g[j][q] - dot);
+      float* p = x_grad + row * cols + c * V;
+      if (beta != 0.0f) {
+        if (VEC) {
+          float4 o = ld4(p);
+          r[0] = beta * o.x + r[0]; r[V > 1 ? 1 : 0] = beta * o.y + r[V > 1 ? 1 : 0];
+          r[V > 1 ? 2 : 0] = beta * o.z + r[V > 1 ? 2 : 0]; r[V > 1 ? 3 : 0] = beta * o.w + r[V > 1 ? 3 : 0];
+        } else {
+          r[0] = beta * p[0] + r[0];
+        }
+      }
+      if (VEC) st4(p, make_float4(r[0], r[V > 1 ? 1 : 0], r[V > 1 ? 2 : 0], r[V > 1 ? 3 : 0]));
+      else p[0] = r[0];
+    }
+  }
+}
+
+// Rows too long for registers: one block per row, three sweeps over global memory (the later
+// sweeps hit L2 for rows up to a few MB).
+__global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(size_t cols, const float* __restrict__ x,
+                                                                  float* __restrict__ out) {
+  __shared__ float smem[16];
+  const float* xr = x + (size_t)blockIdx.x * cols;
+  float* o = out + (size_t)blockIdx.x * cols;
+  float m = -__builtin_huge_valf();
+  for (size_t c = threadIdx.x; c < cols; c += 1024) m = fmaxf(m, xr[c]);
+  m = block_reduce<MaxOp>(m, smem);
+  float s = 0.0f;
+  for (size_t c = threadIdx.x; c < cols; c += 1024) s += expf(xr[c] - m);
+  s = block_reduce<SumOp>(s, smem);
+  for (size_t c = threadIdx.x; c < cols; c += 1024) o[c] = expf(xr[c] - m) / s;
+}
+
+__global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, float* x_grad,
+                                                                  const float* __restrict__ out, const float* out_grad,
+                                                                  float beta) {
+  __shared__ float smem[16];
+  const size_t base = (size_t)blockIdx.x * cols;
+  float dot = 0.0f;
+  for (size_t c = threadIdx.x; c < cols; c += 1024) dot += out[base + c] * out_grad[base + c];
+  dot = block_reduce<SumOp>(dot, smem);
+  for (size_t c = threadIdx.x; c < cols; c += 1024) {
+    float r = out[base + c] * (out_grad[base + c] - dot);
+    x_grad[base + c] = beta != 0.0f ? beta * x_grad[base + c] + r : r;
+  }
+}
+
+struct SoftmaxCfg {
+  int lanes;  // 0 = streaming fallback
+  int items;
+};
+
+static SoftmaxCfg pick_cfg(size_t colsv) {
+  if (colsv <= 256) {
+    int lanes = 1;
+    while ((size_t)lanes * 4 < colsv) lanes <<= 1;
+    return {lanes, 4};
+  }
+  if (colsv <= 1024) return {256, 4};
+  if (colsv <= 4096) return {1024, 4};
+  return {0, 0};
+}
+
+template <bool FWD, bool VEC>
+static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, float* x_grad,
+                                const float* s, const float* g, float beta) {
+  const size_t colsv = cols / (VEC ? 4 : 1);
+  SoftmaxCfg cfg = pick_cfg(colsv);
+  if (cfg.lanes == 0) {
+    if (FWD) hipLaunchKernelGGL(softmax_fwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x, out);
+    else hipLaunchKernelGGL(softmax_bwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta);
+    return post_launch();
+  }
+#define SL_SM(L, I)                                                                                                  \
+  case L: {                                                                                                          \
+    constexpr int RPB = L <= 64 ? 256 / L : 1;                                                                       \
+    constexpr int BLOCK = L <= 64 ? 256 : L;                                                                         \
+    if (FWD)                                                                                                         \
+      hipLaunchKernelGGL((softmax_fwd_kernel<VEC, L, I>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream,    \
+                         rows, cols, x, out);                                                                        \
+    else                                                                                                             \
+      hipLaunchKernelGGL((softmax_bwd_kernel<VEC, L, I>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream,    \
+                         rows, cols, x_grad, s, g, beta);                                                            \
+    break;                                                                                                           \
+  }
+  switch (cfg.lanes) {
+    SL_SM(1, 4) SL_SM(2, 4) SL_SM(4, 4) SL_SM(8, 4) SL_SM(16, 4) SL_SM(32, 4) SL_SM(64, 4) SL_SM(256, 4) SL_SM(1024, 4)
+  }
+#undef SL_SM
+  return post_launch();
+}
+
+}  // namespace slhip
+
+using namespace slhip;
+
+SLHIP_API int32_t slhip_softmax(slhip_ctx* ctx, size_t samples, size_t features, const float* x, float* out) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
+  SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
+  const bool vec = (features % 4 == 0) && aligned16(x) && aligned16(out);
+  return vec ? softmax_dispatch<true, true>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f)
+             : softmax_dispatch<true, false>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f);
+}
+
+SLHIP_API int32_t slhip_softmax_grad(slhip_ctx* ctx, size_t samples, size_t features, float* x_grad, const float* out,
+                                     const float* out_grad, float beta) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && x_grad && out && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
+  SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
+  const bool vec = (features % 4 == 0) && aligned16(x_grad) && aligned16(out) && aligned16(out_grad);
+  return vec ? softmax_dispatch<false, true>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta)
+             : softmax_dispatch<false, false>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta);
+}

@@ -1,0 +1,356 @@
+"""numpy-in / numpy-out facade over the C ABI, one function per reference slice function or
+trait method (same names and argument meaning as the CPU oracle's front-end), so that a
+parity test is the same call on both sides.  Every call uploads its operands, runs the HIP
+kernels and downloads the result; nothing is computed on the host.
+"""
+import numpy as np
+
+from .device import Context
+
+ADD, SUB, MUL, DIV = 0, 1, 2, 3
+SQUARE, POW, RELU, EXP, CLIP, NEG_LN, SCALE, NEG_DIV = range(8)
+
+_ctx = None
+
+
+def init(ordinal=0):
+    global _ctx
+    if _ctx is None:
+        _ctx = Context(ordinal)
+    return _ctx
+
+
+def ctx():
+    return init(0)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32).ravel()
+
+
+class _Scope:
+    """Frees every device buffer created inside the with-block."""
+
+    def __init__(self):
+        self.c = ctx()
+        self.bufs = []
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        for b in self.bufs:
+            b.free()
+
+    def up(self, a):
+        if a is None:
+            return None
+        b = self.c.array(_f32(a))
+        self.bufs.append(b)
+        return b
+
+    def zeros(self, n):
+        b = self.c.zeros(n)
+        self.bufs.append(b)
+        return b
+
+    def empty(self, n):
+        b = self.c.empty(n)
+        self.bufs.append(b)
+        return b
+
+
+def _ptr(b):
+    return b.ptr if b is not None else None
+
+
+# ---- reductions -------------------------------------------------------------
+def _reduce(name, rows, cols, x, outlen):
+    with _Scope() as s:
+        dx, do = s.up(x), s.empty(outlen)
+        s.c.call(name, rows, cols, dx.ptr, do.ptr)
+        return do.numpy()
+
+
+def sum_rows(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_sum_rows", x.size // cols, cols, x, cols)
+
+
+def sum_cols(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_sum_cols", x.size // cols, cols, x, x.size // cols)
+
+
+def max_rows(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_max_rows", x.size // cols, cols, x, cols)
+
+
+def max_cols(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_max_cols", x.size // cols, cols, x, x.size // cols)
+
+
+def mean_rows(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_mean_rows", x.size // cols, cols, x, cols)
+
+
+def mean_cols(cols, x):
+    x = _f32(x)
+    return _reduce("slhip_mean_cols", x.size // cols, cols, x, x.size // cols)
+
+
+def _scalar(name, x):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, do = s.up(x), s.empty(1)
+        s.c.call(name, x.size, dx.ptr, do.ptr)
+        return do.numpy()[0]
+
+
+def sum_all(x):
+    return float(_scalar("slhip_sum", x))
+
+
+def max_all(x):
+    return float(_scalar("slhip_max", x))
+
+
+def mean(x):
+    return _scalar("slhip_mean", x)
+
+
+def _bcast_grad(name, cols, x_grad, out_grad):
+    with _Scope() as s:
+        dg, do = s.up(x_grad), s.up(out_grad)
+        s.c.call(name, x_grad.size // cols, cols, dg.ptr, do.ptr)
+        x_grad[:] = dg.numpy()
+    return x_grad
+
+
+def sum_rows_grad(cols, x_grad, out_grad):
+    return _bcast_grad("slhip_sum_rows_grad", cols, x_grad, out_grad)
+
+
+def sum_cols_grad(cols, x_grad, out_grad):
+    return _bcast_grad("slhip_sum_cols_grad", cols, x_grad, out_grad)
+
+
+def mean_rows_grad(cols, x_grad, out_grad):
+    return _bcast_grad("slhip_mean_rows_grad", cols, x_grad, out_grad)
+
+
+def mean_cols_grad(cols, x_grad, out_grad):
+    return _bcast_grad("slhip_mean_cols_grad", cols, x_grad, out_grad)
+
+
+def _max_grad(name, cols, out, x, x_grad, out_grad):
+    x = _f32(x)
+    with _Scope() as s:
+        d_out, dx, dg, dog = s.up(out), s.up(x), s.up(x_grad), s.up(out_grad)
+        s.c.call(name, x.size // cols, cols, d_out.ptr, dx.ptr, dg.ptr, dog.ptr)
+        x_grad[:] = dg.numpy()
+    return x_grad
+
+
+def max_rows_grad(cols, out, x, x_grad, out_grad):
+    return _max_grad("slhip_max_rows_grad", cols, out, x, x_grad, out_grad)
+
+
+def max_cols_grad(cols, out, x, x_grad, out_grad):
+    return _max_grad("slhip_max_cols_grad", cols, out, x, x_grad, out_grad)
+
+
+# ---- row op -------------------------------------------------------------------
+def add_row(rows, cols, lhs, rhs, inplace=False):
+    with _Scope() as s:
+        dl, dr = s.up(lhs), s.up(rhs)
+        do = dl if inplace else s.empty(rows * cols)
+        s.c.call("slhip_add_row", rows, cols, dl.ptr, dr.ptr, do.ptr)
+        return do.numpy()
+
+
+def add_row_grad(rows, cols, lhs_grad, rhs_grad, out_grad):
+    with _Scope() as s:
+        dl, dr, dg = s.up(lhs_grad), s.up(rhs_grad), s.up(out_grad)
+        s.c.call("slhip_add_row_grad", rows, cols, dl.ptr, dr.ptr, dg.ptr)
+        lhs_grad[:] = dl.numpy()
+        rhs_grad[:] = dr.numpy()
+    return lhs_grad, rhs_grad
+
+
+def add_row_mut_grad(rows, cols, rhs_grad, out_grad):
+    with _Scope() as s:
+        dr, dg = s.up(rhs_grad), s.up(out_grad)
+        s.c.call("slhip_add_row_mut_grad", rows, cols, dr.ptr, dg.ptr)
+        rhs_grad[:] = dr.numpy()
+    return rhs_grad
+
+
+# ---- elementwise ------------------------------------------------------------------
+def binary_ew(op, l, r):
+    l = _f32(l)
+    with _Scope() as s:
+        dl, dr, do = s.up(l), s.up(r), s.empty(l.size)
+        s.c.call("slhip_ew_binary", int(op), l.size, dl.ptr, dr.ptr, do.ptr)
+        return do.numpy()
+
+
+def binary_ew_grad(op, l, r, lg, rg, g):
+    l = _f32(l)
+    with _Scope() as s:
+        dl, dr, dlg, drg, dg = s.up(l), s.up(r), s.up(lg), s.up(rg), s.up(g)
+        s.c.call("slhip_ew_binary_grad", int(op), l.size, dl.ptr, dr.ptr, _ptr(dlg), _ptr(drg), dg.ptr)
+        if lg is not None:
+            lg[:] = dlg.numpy()
+        if rg is not None:
+            rg[:] = drg.numpy()
+    return lg, rg
+
+
+def unary(op, x, p=0.0, q=0.0):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, do = s.up(x), s.empty(x.size)
+        s.c.call("slhip_ew_unary", int(op), float(p), float(q), x.size, dx.ptr, do.ptr)
+        return do.numpy()
+
+
+def unary_grad(op, x, x_grad, out_grad, p=0.0):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, dg, dog = s.up(x), s.up(x_grad), s.up(out_grad)
+        s.c.call("slhip_ew_unary_grad", int(op), float(p), x.size, dx.ptr, dg.ptr, dog.ptr)
+        x_grad[:] = dg.numpy()
+    return x_grad
+
+
+def ew_chain(a, b, c, d):
+    a = _f32(a)
+    with _Scope() as s:
+        da, db, dc, dd, do = s.up(a), s.up(b), s.up(c), s.up(d), s.empty(a.size)
+        s.c.call("slhip_ew_chain", a.size, da.ptr, db.ptr, dc.ptr, dd.ptr, do.ptr)
+        return do.numpy()
+
+
+# ---- transpose / gemm -----------------------------------------------------------------
+def transpose(rows, cols, a, out=None, assign=False):
+    a = _f32(a)
+    with _Scope() as s:
+        da = s.up(a)
+        do = s.up(out) if out is not None else s.empty(a.size)
+        s.c.call("slhip_transpose", rows, cols, da.ptr, do.ptr, 1.0 if assign else 0.0)
+        res = do.numpy()
+    if out is not None:
+        out[:] = res
+        return out
+    return res
+
+
+def sgemm(ta, tb, m, n, k, a, b, c=None, beta=0.0):
+    a, b = _f32(a), _f32(b)
+    assert a.size == m * k and b.size == k * n, (a.size, b.size, m, n, k)
+    with _Scope() as s:
+        da, db = s.up(a), s.up(b)
+        dc = s.up(c) if c is not None else s.empty(m * n)
+        s.c.call("slhip_sgemm", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dc.ptr, float(beta))
+        res = dc.numpy()
+    if c is not None:
+        c[:] = res
+        return c
+    return res
+
+
+def gemm(m, n, k, a, b, c=None, beta=0.0):
+    """GenericBlas::gemm(m, n, k, a, b, c)."""
+    return sgemm(0, 0, m, n, k, a, b, c, beta)
+
+
+def gemmT(m, n, k, a, b, c=None, beta=0.0):
+    """GenericBlas::gemmT: c = a·bᵀ, b stored n×k."""
+    return sgemm(0, 1, m, n, k, a, b, c, beta)
+
+
+def Tgemm(m, n, k, a, b, c=None, beta=0.0):
+    """GenericBlas::Tgemm: c = aᵀ·b, a stored k×m."""
+    return sgemm(1, 0, m, n, k, a, b, c, beta)
+
+
+def gemm_grad(m, k, n, lhs, rhs, lhs_grad, rhs_grad, out_grad, beta=0.0):
+    with _Scope() as s:
+        dl, dr, dlg, drg, dg = s.up(lhs), s.up(rhs), s.up(lhs_grad), s.up(rhs_grad), s.up(out_grad)
+        s.c.call("slhip_gemm_grad", m, k, n, dl.ptr, dr.ptr, _ptr(dlg), _ptr(drg), dg.ptr, float(beta))
+        if lhs_grad is not None:
+            lhs_grad[:] = dlg.numpy()
+        if rhs_grad is not None:
+            rhs_grad[:] = drg.numpy()
+    return lhs_grad, rhs_grad
+
+
+def linear_fwd(m, k, n, x, w, bias, relu=False, want_pre_act=False):
+    with _Scope() as s:
+        dx, dw, db, do = s.up(x), s.up(w), s.up(bias), s.empty(m * n)
+        dp = s.empty(m * n) if want_pre_act else None
+        s.c.call("slhip_linear_fwd", m, k, n, dx.ptr, dw.ptr, _ptr(db), int(relu), _ptr(dp), do.ptr)
+        if want_pre_act:
+            return do.numpy(), dp.numpy()
+        return do.numpy()
+
+
+# ---- softmax & co ----------------------------------------------------------------------
+def softmax(samples, features, x):
+    with _Scope() as s:
+        dx, do = s.up(x), s.empty(samples * features)
+        s.c.call("slhip_softmax", samples, features, dx.ptr, do.ptr)
+        return do.numpy()
+
+
+def softmax_grad(samples, features, out, out_grad, x_grad=None, beta=0.0):
+    with _Scope() as s:
+        d_out, dg = s.up(out), s.up(out_grad)
+        dx = s.up(x_grad) if x_grad is not None else s.zeros(samples * features)
+        s.c.call("slhip_softmax_grad", samples, features, dx.ptr, d_out.ptr, dg.ptr, float(beta))
+        res = dx.numpy()
+    if x_grad is not None:
+        x_grad[:] = res
+        return x_grad
+    return res
+
+
+def onehot(highest_class, classes):
+    classes = _f32(classes)
+    with _Scope() as s:
+        dc, do = s.up(classes), s.empty(classes.size * highest_class)
+        s.c.call("slhip_onehot", classes.size, highest_class, dc.ptr, do.ptr)
+        return do.numpy()
+
+
+def cce(rows, cols, preds, targets):
+    with _Scope() as s:
+        dp, dt, do = s.up(preds), s.up(targets), s.empty(rows)
+        s.c.call("slhip_cce", rows, cols, dp.ptr, dt.ptr, do.ptr)
+        return do.numpy()
+
+
+def cce_grad(rows, cols, preds, targets):
+    with _Scope() as s:
+        dp, dt, do = s.up(preds), s.up(targets), s.empty(rows * cols)
+        s.c.call("slhip_cce_grad", rows, cols, dp.ptr, dt.ptr, do.ptr)
+        return do.numpy()
+
+
+def sgd_step(p, g, lr):
+    with _Scope() as s:
+        dp, dg = s.up(p), s.up(g)
+        s.c.call("slhip_sgd_step", p.size, dp.ptr, dg.ptr, float(lr))
+        p[:] = dp.numpy()
+    return p
+
+
+def rand_uniform(n, lo, hi, tag, seed):
+    with _Scope() as s:
+        b = s.c.uniform(n, lo, hi, tag, seed)
+        s.bufs.append(b)
+        return b.numpy()

@@ -1,0 +1,394 @@
+"""HIP path vs the CPU oracle, through the C ABI, on identical seeded inputs.
+
+Bars (stated per test):
+  * transpose, max_rows, max_cols and every op that is a single IEEE operation per element:
+    bit-exact;
+  * sums / means: |gpu - oracle| <= 1e-6 * sum|x| per output (the oracle's sequential f32 sum is
+    itself off the exact sum by more than 1e-6 relative for long rows, so the bound is written on
+    the backward-error scale), and |gpu - exact| <= the same bound;
+  * softmax fwd/bwd, pow/exp/ln: 1e-6 relative per element against the f64 evaluation, and against
+    the oracle with the oracle's own distance to the f64 evaluation added;
+  * GEMM: |gpu - exact| <= 1e-5 * sqrt(K) * (|A|·|B|) elementwise.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import golden_cases as gc
+from sliced_amd import rng
+
+pytestmark = pytest.mark.gpu
+
+SEED = rng.DEFAULT_SEED
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+# --------------------------------------------------------------------------- golden vectors
+CASES = gc.load_cases()
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["name"][:50] for c in CASES])
+def test_hip_matches_reference_vector(hip, case):
+    try:
+        gc.run_case(hip, case)
+    except gc.Unsupported as e:
+        pytest.skip("not part of the device path: %s" % e)
+
+
+# --------------------------------------------------------------------------- generator
+def test_device_generator_is_bit_identical_to_host(hip):
+    for n, lo, hi, tag in [(1, -1, 1, 0), (1000, -10, 10, 3), (1 << 20, 0, 1, 7), (12345, -3.5, 0.25, 9)]:
+        say("rand_uniform", n, lo, hi, tag)
+        d = hip.rand_uniform(n, lo, hi, tag, SEED)
+        h = rng.uniform(n, lo, hi, tag, SEED)
+        assert np.array_equal(d, h)
+
+
+# --------------------------------------------------------------------------- GEMM
+GEMM_SHAPES = [
+    (1, 1, 1), (4, 3, 2), (5, 10, 7), (33, 65, 17), (64, 64, 64), (128, 128, 16), (128, 128, 128),
+    (129, 127, 130), (256, 384, 200), (100, 10, 300), (300, 10, 2048), (1024, 64, 1), (1024, 1, 64),
+    (1, 64, 1024), (64, 1, 1024), (384, 256, 784), (200, 136, 1000), (512, 512, 512),
+]
+
+
+def gemm_operands(ta, tb, m, n, k):
+    a = rng.uniform(m * k, -1, 1, tag=0, seed=SEED + m + 7 * n + 13 * k)
+    b = rng.uniform(k * n, -1, 1, tag=1, seed=SEED + m + 7 * n + 13 * k)
+    return a, b
+
+
+def gemm_bound(ta, tb, m, n, k, a, b):
+    A = a.reshape(k, m).T if ta else a.reshape(m, k)
+    B = b.reshape(n, k).T if tb else b.reshape(k, n)
+    exact = A.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    return exact.ravel(), (1e-5 * np.sqrt(k) * scale + 1e-30).ravel()
+
+
+@pytest.mark.parametrize("shape", GEMM_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("form", ["gemm", "gemmT", "Tgemm"])
+def test_gemm_forms(hip, orc, shape, form):
+    m, n, k = shape
+    ta, tb = form == "Tgemm", form == "gemmT"
+    say("gemm", form, m, n, k)
+    a, b = gemm_operands(ta, tb, m, n, k)
+    exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+    got = getattr(hip, form)(m, n, k, a, b)
+    ref = getattr(orc, form)(m, n, k, a, b)
+    assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+    assert np.all(np.abs(got - ref) <= bound)
+    # beta = 1 accumulates into C (`Assign`)
+    c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+    got1 = getattr(hip, form)(m, n, k, a, b, c=c0.copy(), beta=1.0)
+    assert np.all(np.abs(got1 - (exact + c0)) <= bound + 1e-6 * np.abs(c0))
+
+
+def test_gemm_split_k_and_large_tiles(hip, orc):
+    # shapes whose tile grid is small enough that the K dimension is split
+    for (m, n, k, ta, tb) in [(256, 256, 4096, 0, 0), (200, 136, 5000, 1, 0), (128, 384, 3000, 0, 1),
+                              (784, 512, 2048, 1, 0)]:
+        say("split-k gemm", m, n, k, ta, tb)
+        a, b = gemm_operands(ta, tb, m, n, k)
+        exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+        got = hip.sgemm(ta, tb, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        got1 = hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0)
+        assert np.all(np.abs(got1 - (exact + c0)) <= bound + 1e-6 * np.abs(c0))
+
+
+def test_gemm_grad_matches_oracle(hip, orc):
+    for (m, k, n) in [(4, 2, 3), (70, 33, 19), (256, 128, 64), (1024, 64, 1), (1024, 1, 64)]:
+        say("gemm_grad", m, k, n)
+        lhs = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
+        rhs = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
+        g = rng.normal(m * n, 1.0, tag=2, seed=SEED)
+        lg_h, rg_h = np.zeros(m * k, np.float32), np.zeros(k * n, np.float32)
+        lg_o, rg_o = lg_h.copy(), rg_h.copy()
+        hip.gemm_grad(m, k, n, lhs, rhs, lg_h, rg_h, g)
+        orc.gemm_grad(m, k, n, lhs, rhs, lg_o, rg_o, g)
+        tol_l = 1e-5 * np.sqrt(n) * (np.abs(g.reshape(m, n)) @ np.abs(rhs.reshape(k, n)).T).ravel() + 1e-30
+        tol_r = 1e-5 * np.sqrt(m) * (np.abs(lhs.reshape(m, k)).T @ np.abs(g.reshape(m, n))).ravel() + 1e-30
+        assert np.all(np.abs(lg_h - lg_o) <= tol_l)
+        assert np.all(np.abs(rg_h - rg_o) <= tol_r)
+        # a NULL grad (operand without requires_grad) is skipped, the other side still written
+        rg2 = np.zeros(k * n, np.float32)
+        hip.gemm_grad(m, k, n, lhs, rhs, None, rg2, g)
+        assert np.array_equal(rg2, rg_h)
+
+
+def test_linear_fwd_fused_equals_gemm_bias_relu(hip, orc):
+    for (m, k, n) in [(64, 1, 64), (130, 70, 50), (256, 784, 384), (1024, 64, 1), (300, 4096, 200)]:
+        say("linear_fwd", m, k, n)
+        x = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
+        w = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
+        bias = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+        h = hip.gemm(m, n, k, x, w)
+        pre_ref = orc.add_row(m, n, h, bias)          # same f32 add on the device's own product
+        out_ref = orc.unary(orc.RELU, pre_ref)
+        out, pre = hip.linear_fwd(m, k, n, x, w, bias, relu=True, want_pre_act=True)
+        assert np.array_equal(pre, pre_ref)
+        assert np.array_equal(out, out_ref)
+        out2 = hip.linear_fwd(m, k, n, x, w, bias, relu=False)
+        assert np.array_equal(out2, pre_ref)
+
+
+# --------------------------------------------------------------------------- reductions
+RED_SHAPES = [(1, 1), (1, 5), (5, 1), (3, 4), (7, 13), (64, 64), (33, 1000), (1000, 33), (257, 4096), (4096, 257),
+              (16, 40000), (40000, 16), (2, 300001), (300001, 2), (1, 1 << 20), (1 << 20, 1), (2048, 2048),
+              (100, 10), (8192, 10), (5000, 128), (3, 70000)]
+
+
+def sum_bound(x, rows, cols, axis):
+    return 1e-6 * np.abs(x.reshape(rows, cols)).astype(np.float64).sum(axis=axis) + 1e-30
+
+
+@pytest.mark.parametrize("shape", RED_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_reductions(hip, orc, shape):
+    rows, cols = shape
+    say("reductions", rows, cols)
+    x = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED + rows)
+    x64 = x.reshape(rows, cols).astype(np.float64)
+    # max: bit-exact
+    assert np.array_equal(hip.max_cols(cols, x), orc.max_cols(cols, x))
+    assert np.array_equal(hip.max_rows(cols, x), orc.max_rows(cols, x))
+    # sums
+    got, ref = hip.sum_cols(cols, x), orc.sum_cols(cols, x)
+    b = sum_bound(x, rows, cols, 1)
+    assert np.all(np.abs(got - x64.sum(1)) <= b) and np.all(np.abs(got - ref) <= 2 * b + np.abs(ref - x64.sum(1)))
+    got, ref = hip.sum_rows(cols, x), orc.sum_rows(cols, x)
+    b = sum_bound(x, rows, cols, 0)
+    assert np.all(np.abs(got - x64.sum(0)) <= b) and np.all(np.abs(got - ref) <= 2 * b + np.abs(ref - x64.sum(0)))
+    # means
+    got = hip.mean_cols(cols, x)
+    assert np.all(np.abs(got - x64.mean(1)) <= sum_bound(x, rows, cols, 1) / cols + 1e-7 * np.abs(x64.mean(1)))
+    got = hip.mean_rows(cols, x)
+    assert np.all(np.abs(got - x64.mean(0)) <= sum_bound(x, rows, cols, 0) / rows + 1e-7 * np.abs(x64.mean(0)))
+    # scalars
+    tot = x64.sum()
+    bt = 1e-6 * np.abs(x64).sum() + 1e-30
+    assert abs(hip.sum_all(x) - tot) <= bt
+    assert abs(float(hip.mean(x)) - tot / x.size) <= bt / x.size + 1e-7 * abs(tot / x.size)
+    assert hip.max_all(x) == float(x.max())
+
+
+def test_max_is_bit_exact_with_injected_ties_and_negatives(hip, orc):
+    for rows, cols in [(200, 300), (64, 4096), (4096, 64)]:
+        say("max ties", rows, cols)
+        x = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED)
+        x = rng.inject_row_max_ties(x, rows, cols, 0.01)
+        assert np.array_equal(hip.max_cols(cols, x), orc.max_cols(cols, x))
+        x = rng.inject_col_max_ties(x, rows, cols, 0.01)
+        assert np.array_equal(hip.max_rows(cols, x), orc.max_rows(cols, x))
+        xn = -np.abs(x) - 1.0  # all negative: the result must not be clamped at 0
+        assert np.array_equal(hip.max_rows(cols, xn), orc.max_rows(cols, xn))
+        assert np.array_equal(hip.max_cols(cols, xn), orc.max_cols(cols, xn))
+
+
+def test_max_grads_tie_rules(hip, orc):
+    for rows, cols in [(3, 4), (50, 200), (300, 40), (17, 5000), (2000, 1), (1, 2000)]:
+        say("max grads", rows, cols)
+        x = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED + cols)
+        g_r = rng.normal(rows, 1.0, tag=1, seed=SEED)
+        g_c = rng.normal(cols, 1.0, tag=2, seed=SEED)
+        base = rng.normal(rows * cols, 1.0, tag=3, seed=SEED)
+        # first tie only, along the contiguous axis
+        xt = rng.inject_row_max_ties(x.copy(), rows, cols, 0.05)
+        out = orc.max_cols(cols, xt)
+        a = hip.max_cols_grad(cols, out, xt, base.copy(), g_r)
+        b = orc.max_cols_grad(cols, out, xt, base.copy(), g_r)
+        assert np.array_equal(a, b)
+        # all ties, along the strided axis
+        xt = rng.inject_col_max_ties(x.copy(), rows, cols, 0.05)
+        out = orc.max_rows(cols, xt)
+        a = hip.max_rows_grad(cols, out, xt, base.copy(), g_c)
+        b = orc.max_rows_grad(cols, out, xt, base.copy(), g_c)
+        assert np.array_equal(a, b)
+
+
+def test_broadcast_grads_are_bit_exact(hip, orc):
+    for rows, cols in [(3, 4), (5, 7), (128, 256), (1000, 10), (10, 1000), (513, 1028)]:
+        say("broadcast grads", rows, cols)
+        base = rng.normal(rows * cols, 1.0, tag=0, seed=SEED)
+        g_r = rng.normal(rows, 1.0, tag=1, seed=SEED)
+        g_c = rng.normal(cols, 1.0, tag=2, seed=SEED)
+        for name, g in [("sum_rows_grad", g_c), ("sum_cols_grad", g_r), ("mean_rows_grad", g_c),
+                        ("mean_cols_grad", g_r)]:
+            a = getattr(hip, name)(cols, base.copy(), g)
+            b = getattr(orc, name)(cols, base.copy(), g)
+            assert np.array_equal(a, b), name
+
+
+# --------------------------------------------------------------------------- softmax
+SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (64, 1024), (17, 1000), (9, 4096),
+                  (5, 4100), (3, 16384), (2, 16390), (2, 40000), (1000, 1), (50, 64), (50, 257)]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_softmax_forward_backward(hip, orc, shape):
+    rows, cols = shape
+    say("softmax", rows, cols)
+    x = rng.normal(rows * cols, 3.0, tag=0, seed=SEED + cols)
+    g = rng.normal(rows * cols, 1.0, tag=1, seed=SEED + cols)
+    x64 = x.reshape(rows, cols).astype(np.float64)
+    e = np.exp(x64 - x64.max(1, keepdims=True))
+    exact = (e / e.sum(1, keepdims=True)).ravel()
+    got, ref = hip.softmax(rows, cols, x), orc.softmax(rows, cols, x)
+    rel = np.abs(got - exact) / np.maximum(np.abs(exact), 1e-30)
+    assert rel.max() <= 1e-6, rel.max()
+    ref_off = np.abs(ref - exact)
+    assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(exact) + ref_off + 1e-37)
+    assert np.all(np.abs(got.reshape(rows, cols).astype(np.float64).sum(1) - 1.0) <= 1e-6)
+    # backward on the device's own forward output, SET and accumulate
+    s64 = got.reshape(rows, cols).astype(np.float64)
+    g64 = g.reshape(rows, cols).astype(np.float64)
+    dot = (s64 * g64).sum(1, keepdims=True)
+    exact_b = (s64 * (g64 - dot)).ravel()
+    scale = (np.abs(s64) * (np.abs(g64) + (np.abs(s64) * np.abs(g64)).sum(1, keepdims=True))).ravel()
+    bound = 1e-6 * scale + 1e-37          # cancellation in g - <s,g> is priced on the operands' scale
+    gb = hip.softmax_grad(rows, cols, got, g)
+    ob = orc.softmax_grad(rows, cols, got, g)
+    assert np.all(np.abs(gb - exact_b) <= bound), np.max(np.abs(gb - exact_b) / bound)
+    assert np.all(np.abs(gb - ob) <= bound + np.abs(ob - exact_b))
+    base = rng.normal(rows * cols, 1.0, tag=2, seed=SEED)
+    gacc = hip.softmax_grad(rows, cols, got, g, x_grad=base.copy(), beta=1.0)
+    assert np.all(np.abs(gacc - (base + exact_b)) <= bound + 1e-6 * np.abs(base))
+
+
+def test_softmax_grad_constant_seed_is_zero(hip):
+    rows, cols = 64, 1000
+    x = rng.normal(rows * cols, 3.0, tag=0, seed=SEED)
+    s = hip.softmax(rows, cols, x)
+    gz = hip.softmax_grad(rows, cols, s, np.ones(rows * cols, np.float32))
+    assert np.max(np.abs(gz)) <= 1e-6
+
+
+# --------------------------------------------------------------------------- transpose
+TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300), (257, 129), (1024, 1024),
+             (4, 4096), (4096, 4), (1000, 1000), (1, 1 << 18), (1 << 18, 1)]
+
+
+@pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_transpose_bit_exact(hip, orc, shape):
+    rows, cols = shape
+    say("transpose", rows, cols)
+    x = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED)
+    got = hip.transpose(rows, cols, x)
+    assert np.array_equal(got, orc.transpose(rows, cols, x))
+    assert np.array_equal(got, x.reshape(rows, cols).T.ravel())
+    assert np.array_equal(hip.transpose(cols, rows, got), x)           # involution
+    base = rng.uniform(rows * cols, -1, 1, tag=1, seed=SEED)
+    acc = hip.transpose(rows, cols, x, out=base.copy(), assign=True)   # `Assign` (+=)
+    assert np.array_equal(acc, orc.transpose(rows, cols, x, out=base.copy(), assign=True))
+
+
+# --------------------------------------------------------------------------- elementwise / row op
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, 100003, 1 << 20])
+def test_elementwise_ops(hip, orc, n):
+    say("elementwise", n)
+    a = rng.uniform(n, -10, 10, tag=1, seed=SEED)
+    b = rng.uniform(n, -10, 10, tag=2, seed=SEED)
+    c = rng.uniform(n, -10, 10, tag=3, seed=SEED)
+    d = rng.uniform(n, -10, 10, tag=4, seed=SEED)
+    g = rng.normal(n, 1.0, tag=5, seed=SEED)
+    for op in (orc.ADD, orc.SUB, orc.MUL, orc.DIV):
+        assert np.array_equal(hip.binary_ew(op, a, b), orc.binary_ew(op, a, b)), op
+        lg, rg = rng.normal(n, 1.0, tag=6, seed=SEED), rng.normal(n, 1.0, tag=7, seed=SEED)
+        lh, rh = hip.binary_ew_grad(op, a, b, lg.copy(), rg.copy(), g)
+        lo, ro = orc.binary_ew_grad(op, a, b, lg.copy(), rg.copy(), g)
+        if op == orc.DIV:   # 1/r and l/(r*r): the division may differ in the last place
+            assert np.allclose(lh, lo, rtol=1e-6, atol=0) and np.allclose(rh, ro, rtol=1e-6, atol=1e-30)
+        else:
+            assert np.array_equal(lh, lo) and np.array_equal(rh, ro), op
+        only_l, _ = hip.binary_ew_grad(op, a, b, lg.copy(), None, g)
+        assert np.array_equal(only_l, lh)
+    for op in (orc.SQUARE, orc.RELU):
+        assert np.array_equal(hip.unary(op, a), orc.unary(op, a))
+        xg = rng.normal(n, 1.0, tag=8, seed=SEED)
+        assert np.array_equal(hip.unary_grad(op, a, xg.copy(), g), orc.unary_grad(op, a, xg.copy(), g))
+    assert np.array_equal(hip.unary(orc.CLIP, a, -2.5, 3.0), orc.unary(orc.CLIP, a, -2.5, 3.0))
+    assert np.array_equal(hip.unary(orc.SCALE, a, 0.37), orc.unary(orc.SCALE, a, 0.37))
+    assert np.array_equal(hip.unary(orc.NEG_DIV, a, 8192.0), orc.unary(orc.NEG_DIV, a, 8192.0))
+    # transcendental ops: 1e-6 relative against the f64 value
+    a64 = a.astype(np.float64)
+    for p in (2.0, 3.0, 0.5):
+        base = np.abs(a64) if p == 0.5 else a64
+        x32 = base.astype(np.float32)
+        got = hip.unary(orc.POW, x32, p)
+        assert np.all(np.abs(got - base ** p) <= 1e-6 * np.abs(base ** p) + 1e-37), p
+        gg = hip.unary_grad(orc.POW, x32, np.zeros(n, np.float32), g, p)
+        if p != 0.5:
+            ex = p * base ** (p - 1) * g.astype(np.float64)
+            assert np.all(np.abs(gg - ex) <= 2e-6 * np.abs(ex) + 1e-37), p
+    small = (a * np.float32(0.5)).astype(np.float32)
+    got = hip.unary(orc.EXP, small)
+    assert np.all(np.abs(got - np.exp(small.astype(np.float64))) <= 1e-6 * np.exp(small.astype(np.float64)))
+    pos = (np.abs(a) + np.float32(1e-3)).astype(np.float32)
+    got = hip.unary(orc.NEG_LN, pos)
+    ex = -np.log(pos.astype(np.float64))
+    assert np.all(np.abs(got - ex) <= 1e-6 * np.abs(ex) + 1e-7)
+    # fused chain ((a+b)*c - d) -> pow 2 -> square against the op-by-op oracle
+    t = orc.binary_ew(orc.SUB, orc.binary_ew(orc.MUL, orc.binary_ew(orc.ADD, a, b), c), d)
+    ref = orc.unary(orc.SQUARE, orc.unary(orc.POW, t, 2.0))
+    got = hip.ew_chain(a, b, c, d)
+    assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + 1e-37)
+    # sgd
+    p0 = rng.uniform(n, -1, 1, tag=9, seed=SEED)
+    assert np.array_equal(hip.sgd_step(p0.copy(), g, 0.05), orc.sgd_step(p0.copy(), g, 0.05))
+
+
+def test_negative_base_integer_pow_is_finite(hip):
+    x = np.array([-3.0, -0.5, 0.0, 2.0], np.float32)
+    assert np.array_equal(hip.unary(1, x, 2.0), np.array([9.0, 0.25, 0.0, 4.0], np.float32))
+    g = hip.unary_grad(1, x, np.zeros(4, np.float32), np.ones(4, np.float32), 2.0)
+    assert np.array_equal(g, np.array([-6.0, -1.0, 0.0, 4.0], np.float32))
+
+
+def test_row_op_and_bias_grad(hip, orc):
+    for rows, cols in [(3, 5), (1, 9), (9, 1), (1024, 64), (1000, 10), (8192, 10), (300, 2048), (4097, 130)]:
+        say("row op", rows, cols)
+        lhs = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED)
+        rhs = rng.uniform(cols, -10, 10, tag=1, seed=SEED)
+        ref = orc.add_row(rows, cols, lhs, rhs)
+        assert np.array_equal(hip.add_row(rows, cols, lhs, rhs), ref)
+        assert np.array_equal(hip.add_row(rows, cols, lhs, rhs, inplace=True), ref)     # add_row_mut
+        g = rng.normal(rows * cols, 1.0, tag=2, seed=SEED)
+        rg0 = rng.normal(cols, 1.0, tag=3, seed=SEED)
+        b = 1e-6 * (np.abs(g.reshape(rows, cols)).astype(np.float64).sum(0) + np.abs(rg0)) + 1e-30
+        exact = g.reshape(rows, cols).astype(np.float64).sum(0) + rg0
+        got = hip.add_row_mut_grad(rows, cols, rg0.copy(), g)
+        assert np.all(np.abs(got - exact) <= b)
+        lg, rg = hip.add_row_grad(rows, cols, np.full(rows * cols, 7.0, np.float32), rg0.copy(), g)
+        assert np.array_equal(lg, g)                    # lhs_grad is overwritten, not accumulated
+        assert np.all(np.abs(rg - exact) <= b)
+
+
+def test_cce_and_onehot(hip, orc):
+    rows, cols = 500, 10
+    cls = rng.integers(rows, cols, tag=1, seed=SEED).astype(np.float32)
+    t = hip.onehot(cols, cls)
+    assert np.array_equal(t, orc.onehot(cols, cls))
+    p = hip.softmax(rows, cols, rng.normal(rows * cols, 3.0, tag=0, seed=SEED))
+    a, b = hip.cce(rows, cols, p, t), orc.cce(rows, cols, p, t)
+    assert np.all(np.abs(a - b) <= 1e-6 * np.abs(b) + 1e-7)
+    assert np.array_equal(hip.cce_grad(rows, cols, p, t), orc.cce_grad(rows, cols, p, t))
+
+
+# --------------------------------------------------------------------------- error behaviour
+def test_invalid_arguments_return_status_not_crash(hip):
+    c = hip.ctx()
+    lib = c.lib
+    x = c.zeros(16)
+    assert lib.slhip_sum_rows(c.h, 0, 4, x.ptr, x.ptr) == -1            # zero rows
+    assert lib.slhip_sum_rows(c.h, 1 << 40, 1 << 40, x.ptr, x.ptr) == -1  # rows*cols overflows
+    assert lib.slhip_softmax(c.h, 4, 4, None, x.ptr) == -1              # null operand
+    assert lib.slhip_sgemm(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, x.ptr, 0.0) == -4   # C aliases A
+    assert lib.slhip_transpose(c.h, 4, 4, x.ptr, x.ptr, 0.0) == -4
+    assert lib.slhip_ew_unary(c.h, 99, 0.0, 0.0, 4, x.ptr, x.ptr) == -1
+    x.free()
