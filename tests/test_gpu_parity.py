@@ -236,8 +236,12 @@ def test_softmax_forward_backward(hip, orc, shape):
     say("softmax", rows, cols)
     x = rng.normal(rows * cols, 3.0, tag=0, seed=SEED + cols)
     g = rng.normal(rows * cols, 1.0, tag=1, seed=SEED + cols)
-    x64 = x.reshape(rows, cols).astype(np.float64)
-    e = np.exp(x64 - x64.max(1, keepdims=True))
+    # exact value of the function both sides evaluate: the shifted logit x - max is an f32
+    # subtraction in the reference (sub_cols) and on the device, so it is rounded to f32 here too;
+    # exp, sum and division are then carried out in f64
+    x2 = x.reshape(rows, cols)
+    shifted = (x2 - x2.max(1, keepdims=True)).astype(np.float32).astype(np.float64)
+    e = np.exp(shifted)
     exact = (e / e.sum(1, keepdims=True)).ravel()
     got, ref = hip.softmax(rows, cols, x), orc.softmax(rows, cols, x)
     rel = np.abs(got - exact) / np.maximum(np.abs(exact), 1e-30)
