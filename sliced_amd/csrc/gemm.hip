@@ -9,20 +9,25 @@
 // and k = 4 + t for lanes 32..63.
 //
 // Tiling: 256 threads = 4 waves in a 2x2 grid, 128x128 macro tile, each wave 64x64 = four
-// 32x32 accumulators (64 VGPRs), BK = 16 per LDS stage, two LDS stages with register
-// prefetch of the next stage (one barrier per stage).  Workgroup ids are remapped so that each
-// XCD (its own L2) works on a compact group of tiles.  Small grids are split along K; the
-// partial products go to the context workspace and are combined in a fixed order.
+// 32x32 accumulators (64 VGPRs), BK = 32 per LDS stage, two LDS stages with register
+// prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.  Tiles are numbered so that each XCD (its
+// own L2) works along one tile row at a time.  Small grids are split along K; the partial
+// products go to the context workspace and are combined in a fixed order.
 #include "common.hpp"
 
 namespace slhip {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 16;
-constexpr int KC_PITCH = BK + 4;   // [x][k] layout, k contiguous; pitch keeps float4 alignment
-constexpr int XC_PITCH = 128 + 4;  // [k][x] layout, x contiguous
-constexpr int STAGE_FLOATS = 128 * KC_PITCH > BK * XC_PITCH ? 128 * KC_PITCH : BK * XC_PITCH;
+constexpr int BM = 128, BN = 128;
+constexpr int XC_PITCH = 128 + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
+
+template <int BK>
+struct Cfg {
+  static constexpr int KC_PITCH = BK + 4;  // [x][k] layout, k contiguous
+  static constexpr int STAGE_FLOATS = 128 * KC_PITCH > BK * XC_PITCH ? 128 * KC_PITCH : BK * XC_PITCH;
+  static constexpr int NV = BK * 128 / 4 / 256;  // float4 per thread per operand tile
+};
 
 struct GemmArgs {
   size_t M, N, K;
@@ -41,18 +46,21 @@ struct GemmArgs {
 };
 
 // Operand tile held in registers between the global load and the LDS store.
+template <int BK>
 struct Frag {
-  float4 v[2];
+  float4 v[Cfg<BK>::NV];
 };
 
 // k-contiguous source: element (x, k) at src[x*ld + k]; tile 128 x BK.
-__device__ __forceinline__ void load_kc(Frag& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
-                                        size_t x0, size_t k0, bool fast) {
-  const int kq = threadIdx.x & 3, xr = threadIdx.x >> 2;  // 4 float4 per row, 64 rows per pass
+template <int BK, bool FAST>
+__device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+                                        size_t x0, size_t k0) {
+  constexpr int VPR = BK / 4, RPP = 256 / VPR;  // float4 per row, rows per pass
+  const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const size_t x = x0 + xr + 64 * p, k = k0 + 4 * kq;
-    if (fast) {
+  for (int p = 0; p < Cfg<BK>::NV; ++p) {
+    const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
+    if (FAST) {
       f.v[p] = ld4(src + x * ld + k);
     } else {
       float t[4];
@@ -62,20 +70,23 @@ __device__ __forceinline__ void load_kc(Frag& f, const float* __restrict__ src, 
     }
   }
 }
-__device__ __forceinline__ void store_kc(const Frag& f, float* lds) {
-  const int kq = threadIdx.x & 3, xr = threadIdx.x >> 2;
+template <int BK>
+__device__ __forceinline__ void store_kc(const Frag<BK>& f, float* lds) {
+  constexpr int VPR = BK / 4, RPP = 256 / VPR;
+  const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < 2; ++p) st4(lds + (xr + 64 * p) * KC_PITCH + 4 * kq, f.v[p]);
+  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK>::KC_PITCH + 4 * kq, f.v[p]);
 }
 
 // x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x 128.
-__device__ __forceinline__ void load_xc(Frag& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
-                                        size_t x0, size_t k0, bool fast) {
+template <int BK, bool FAST>
+__device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+                                        size_t x0, size_t k0) {
   const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;  // 32 float4 per k-row, 8 rows per pass
 #pragma unroll
-  for (int p = 0; p < 2; ++p) {
+  for (int p = 0; p < Cfg<BK>::NV; ++p) {
     const size_t k = k0 + kr + 8 * p, x = x0 + 4 * xq;
-    if (fast) {
+    if (FAST) {
       f.v[p] = ld4(src + k * ld + x);
     } else {
       float t[4];
@@ -85,20 +96,21 @@ __device__ __forceinline__ void load_xc(Frag& f, const float* __restrict__ src, 
     }
   }
 }
-__device__ __forceinline__ void store_xc(const Frag& f, float* lds) {
+template <int BK>
+__device__ __forceinline__ void store_xc(const Frag<BK>& f, float* lds) {
   const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;
 #pragma unroll
-  for (int p = 0; p < 2; ++p) st4(lds + (kr + 8 * p) * XC_PITCH + 4 * xq, f.v[p]);
+  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (kr + 8 * p) * XC_PITCH + 4 * xq, f.v[p]);
 }
 
 // MFMA fragments of one 8-wide k group for the two 32-row blocks of this wave's 64 rows.
 // KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's 64 rows/cols.
-template <bool KC>
+template <bool KC, int BK>
 __device__ __forceinline__ void read_frag(float (&out)[2][4], const float* lds, int x_base, int kk8, int r, int h) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     if (KC) {
-      float4 t = ld4(lds + (x_base + 32 * i + r) * KC_PITCH + kk8 * 8 + 4 * h);
+      float4 t = ld4(lds + (x_base + 32 * i + r) * Cfg<BK>::KC_PITCH + kk8 * 8 + 4 * h);
       out[i][0] = t.x; out[i][1] = t.y; out[i][2] = t.z; out[i][3] = t.w;
     } else {
 #pragma unroll
@@ -107,43 +119,107 @@ __device__ __forceinline__ void read_frag(float (&out)[2][4], const float* lds, 
   }
 }
 
-// Linear workgroup id -> tile, so that the workgroups resident on one XCD (ids congruent mod 8)
-// form a contiguous run of tiles, walked in groups of 8 tile rows.
-__device__ __forceinline__ void tile_of_block(unsigned bid, unsigned nblocks, unsigned tiles_m, unsigned tiles_n,
-                                              unsigned& tm, unsigned& tn) {
-  constexpr unsigned NXCD = 8, GROUP_M = 8;
-  const unsigned xcd = bid % NXCD, slot = bid / NXCD;
-  const unsigned base = nblocks / NXCD, rem = nblocks % NXCD;
-  const unsigned pid = xcd * base + (xcd < rem ? xcd : rem) + slot;
+// Linear workgroup id -> tile.  Tiles are walked in groups of 8 tile rows, row index fastest.
+// The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, so with a group
+// height of 8 every XCD (its own L2) keeps working along ONE tile row of the group: its A panel
+// stays put in that L2 while the B panels stream through.  Measured on 4096^3: an explicit
+// remap that instead gave each XCD a compact 8x8 block of tiles was no faster for A*B and
+// At*B and 25 % slower for A*Bt.
+__device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
+                                              unsigned& tn) {
+  constexpr unsigned GROUP_M = 8;
   const unsigned in_group = GROUP_M * tiles_n;
-  const unsigned group = pid / in_group;
+  const unsigned group = bid / in_group;
   const unsigned first_m = group * GROUP_M;
   const unsigned gsize = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
-  const unsigned local = pid % in_group;
+  const unsigned local = bid % in_group;
   tm = first_m + local % gsize;
   tn = local / gsize;
 }
 
-template <bool TA, bool TB>
+// The k loop over tiles [kt_begin, kt_end) of one workgroup.  FAST = every tile in the range is
+// complete and 16-byte loadable, so the global loads are unconditional float4 loads; otherwise
+// every element is bounds-checked and zero-filled.  The two variants are separate loops on
+// purpose: when both kinds of load sat behind a branch in ONE loop body the compiler folded them
+// into the per-element form, which cost 19 % of the kernel's throughput.
+template <bool TA, bool TB, int BK, bool FAST>
+__device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
+                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
+                                           float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
+  constexpr int KSTEPS = BK / 8;
+  if (kt_begin >= kt_end) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r = lane & 31, h = lane >> 5;
+  // A is KC ([m][k], ld = K) unless transposed ([k][m], ld = M); B is XC ([k][n], ld = N)
+  // unless transposed ([n][k], ld = K).
+  const size_t lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
+
+  Frag<BK> fa, fb;
+  auto load_stage = [&](int kt) {
+    const size_t k0 = kbeg + (size_t)kt * BK;
+    if (TA) load_xc<BK, FAST>(fa, g.A, lda, g.M, kend, m0, k0);
+    else load_kc<BK, FAST>(fa, g.A, lda, g.M, kend, m0, k0);
+    if (TB) load_kc<BK, FAST>(fb, g.B, ldb, g.N, kend, n0, k0);
+    else load_xc<BK, FAST>(fb, g.B, ldb, g.N, kend, n0, k0);
+  };
+  auto store_stage = [&](int s) {
+    if (TA) store_xc<BK>(fa, lds_a[s]); else store_kc<BK>(fa, lds_a[s]);
+    if (TB) store_kc<BK>(fb, lds_b[s]); else store_xc<BK>(fb, lds_b[s]);
+  };
+
+  load_stage(kt_begin);
+  store_stage(0);
+  __syncthreads();
+
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int s = (kt - kt_begin) & 1;
+    if (kt + 1 < kt_end) load_stage(kt + 1);  // global loads fly during the MFMA block below
+    // Fragment reads run one k-group ahead of the MFMAs that consume them, so the LDS latency
+    // is covered by 16 MFMAs (1024 cycles) of the same wave.  The scheduling barriers keep the
+    // compiler from sinking the reads back down to their first use.
+    float a[2][2][4], b[2][2][4];
+    read_frag<!TA, BK>(a[0], lds_a[s], wm * 64, 0, r, h);
+    read_frag<TB, BK>(b[0], lds_b[s], wn * 64, 0, r, h);
+#pragma unroll
+    for (int kk8 = 0; kk8 < KSTEPS; ++kk8) {
+      const int cur = kk8 & 1, nxt = cur ^ 1;
+      if (kk8 + 1 < KSTEPS) {
+        read_frag<!TA, BK>(a[nxt], lds_a[s], wm * 64, kk8 + 1, r, h);
+        read_frag<TB, BK>(b[nxt], lds_b[s], wn * 64, kk8 + 1, r, h);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][t], b[cur][j][t], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt + 1 < kt_end) store_stage(s ^ 1);
+    __syncthreads();  // also frees both stages for whoever runs next
+  }
+}
+
+template <bool TA, bool TB, int BK>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
-  __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE_FLOATS];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE_FLOATS];
+  constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
+  __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
 
   unsigned tm, tn;
-  tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tm, tn);
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
   const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
   const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
+  const int kfull = (int)((kend - kbeg) / BK);  // complete tiles
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
   const int r = lane & 31, h = lane >> 5;
-
-  // A is KC ([m][k], ld = K) unless transposed ([k][m], ld = M); B is XC ([k][n], ld = N)
-  // unless transposed ([n][k], ld = K).
-  const size_t lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
-  const bool a_full_x = m0 + BM <= g.M, b_full_x = n0 + BN <= g.N;
 
   floatx16 acc[2][2];
 #pragma unroll
@@ -153,45 +229,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  Frag fa, fb;
-  auto load_stage = [&](int kt) {
-    const size_t k0 = kbeg + (size_t)kt * BK;
-    const bool full_k = k0 + BK <= kend;
-    if (TA) load_xc(fa, g.A, lda, g.M, kend, m0, k0, g.a_vec && a_full_x && full_k);
-    else load_kc(fa, g.A, lda, g.M, kend, m0, k0, g.a_vec && a_full_x && full_k);
-    if (TB) load_kc(fb, g.B, ldb, g.N, kend, n0, k0, g.b_vec && b_full_x && full_k);
-    else load_xc(fb, g.B, ldb, g.N, kend, n0, k0, g.b_vec && b_full_x && full_k);
-  };
-  auto store_stage = [&](int s) {
-    if (TA) store_xc(fa, lds_a[s]); else store_kc(fa, lds_a[s]);
-    if (TB) store_kc(fb, lds_b[s]); else store_xc(fb, lds_b[s]);
-  };
-
-  if (ktiles > 0) {
-    load_stage(0);
-    store_stage(0);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int s = kt & 1;
-    if (kt + 1 < ktiles) load_stage(kt + 1);
-#pragma unroll
-    for (int kk8 = 0; kk8 < BK / 8; ++kk8) {
-      float a[2][4], b[2][4];
-      read_frag<!TA>(a, lds_a[s], wm * 64, kk8, r, h);
-      read_frag<TB>(b, lds_b[s], wn * 64, kk8, r, h);
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][t], b[j][t], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < ktiles) store_stage(s ^ 1);
-    __syncthreads();
-  }
+  // interior workgroups run their complete k tiles through the vector-load loop; edge tiles,
+  // unaligned operands and the k remainder go through the checked loop
+  const bool fast = g.a_vec && g.b_vec && m0 + BM <= g.M && n0 + BN <= g.N;
+  const int nfast = fast ? kfull : 0;
+  gemm_tiles<TA, TB, BK, true>(g, 0, nfast, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, false>(g, nfast, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
@@ -263,6 +306,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
   }
 }
 
+constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form at 2048^3 and above
+
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
                         float* C, float beta, const float* bias, int relu, float* pre_act) {
   GemmArgs g;
@@ -278,19 +323,26 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   g.a_vec = aligned16(A) && lda % 4 == 0;
   g.b_vec = aligned16(B) && ldb % 4 == 0;
 
-  // split K when the tile grid alone leaves most CUs idle
+  // Split K when the tile grid alone leaves CUs idle.  Two workgroups fit a CU, so the chip runs
+  // `slots` workgroups at a time; pick the split count whose last round of workgroups is the
+  // fullest (ties: the smaller count, which writes fewer partial results).
   const size_t tiles = tiles_m * tiles_n;
-  const size_t want = (size_t)ctx->num_cu * 2;
+  const size_t slots = (size_t)ctx->num_cu * 2;
   size_t splits = 1;
-  if (tiles < want && K >= 8 * BK) {
-    splits = (want + tiles - 1) / tiles;
-    const size_t max_by_k = K / (4 * BK);  // every split keeps >= 4 stages
-    if (splits > max_by_k) splits = max_by_k;
-    if (splits > 32) splits = 32;
+  if (tiles < slots && K >= 512) {
+    size_t max_splits = K / 128;  // every split keeps >= 128 of K
+    if (max_splits > 32) max_splits = 32;
     const size_t fit = ctx->workspace_bytes / (M * N * sizeof(float));
-    if (splits > fit) splits = fit;
-    if (splits < 1) splits = 1;
+    if (max_splits > fit) max_splits = fit;
+    double best = 0.0;
+    for (size_t sp = 1; sp <= max_splits; ++sp) {
+      const size_t wgs = tiles * sp;
+      const size_t rounds = (wgs + slots - 1) / slots;
+      const double eff = (double)wgs / (double)(rounds * slots);
+      if (eff > best + 1e-9) { best = eff; splits = sp; }
+    }
   }
+  constexpr int BK = GEMM_BK;
   size_t k_chunk = (K + splits - 1) / splits;
   k_chunk = (k_chunk + BK - 1) / BK * BK;
   if (k_chunk == 0) k_chunk = BK;
@@ -301,10 +353,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   g.partial = (float*)ctx->workspace;
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
-  if (!ta && !tb) hipLaunchKernelGGL((gemm_kernel<false, false>), grid, dim3(256), 0, ctx->stream, g);
-  else if (!ta && tb) hipLaunchKernelGGL((gemm_kernel<false, true>), grid, dim3(256), 0, ctx->stream, g);
-  else if (ta && !tb) hipLaunchKernelGGL((gemm_kernel<true, false>), grid, dim3(256), 0, ctx->stream, g);
-  else hipLaunchKernelGGL((gemm_kernel<true, true>), grid, dim3(256), 0, ctx->stream, g);
+#define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g)
+  if (!ta && !tb) SL_GEMM(false, false);
+  else if (!ta && tb) SL_GEMM(false, true);
+  else if (ta && !tb) SL_GEMM(true, false);
+  else SL_GEMM(true, true);
+#undef SL_GEMM
   int32_t rc = post_launch();
   if (rc || splits == 1) return rc;
 

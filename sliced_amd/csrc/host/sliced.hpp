@@ -1,0 +1,450 @@
+// Host-side device layer above the C ABI: the part of the reference's `custos` device model that
+// its array-op path relies on, re-stated for a HIP device.
+//
+//   HIP            device: one slhip context (one in-order stream), the buffer registry, the
+//                  gradient map, the autograd tape and the call-position cache
+//                  (reference usage: `CPU::<Autograd<Cached<Base>>>::new()`, examples/sine_net.rs:124)
+//   Buffer         {id, device pointer, len, requires_grad}; copies share the allocation
+//   Matrix         {Buffer, rows, cols} with one method per op (reference: src/matrix.rs:21-25,98-378)
+//
+// Semantics taken from how the reference uses custos (the crate itself is not in its tree):
+//   * retrieve(len) hands out a ZEROED buffer (slice_sum_rows2 accumulates into it,
+//     src/ops2/sum/cpu.rs:78-84); in cached mode the same call position of the next
+//     `range` iteration gets the same allocation again (examples/sine_net.rs:135);
+//   * every forward op pushes a closure on the tape (`add_grad_fn`, src/ops.rs:38 ...); the
+//     closure looks gradients up by buffer id: grad() reads, grad_mut() creates zeroed;
+//   * backward() seeds the output gradient with ones (tests/test_add.rs:17-23) and runs the
+//     closures in reverse; backward_with(g) seeds with g (examples/nn.rs:233); the tape is
+//     cleared afterwards;
+//   * every gradient accumulates (`+=`) except gemm_grad, softmax_grad, transpose_grad and the
+//     lhs side of add_row_grad, which overwrite, as the reference's CPU device does
+//     (src/ops2/gemm/grad/cpu_stack.rs:36-39, src/ops2/softmax/grad/cpu.rs:53-60,
+//     src/ops2/transpose/cpu.rs:22-23, src/ops2/row_op/grad/cpu.rs:61).
+//
+// Nothing here computes: every op is one call into libsliced_hip.so.
+#pragma once
+#include <cstdint>
+#include <cstdio>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "sliced_hip.h"
+
+namespace sliced {
+
+struct Error : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+inline void check(int32_t rc, const char* what) {
+  if (rc != 0) throw Error(std::string(what) + " failed (" + std::to_string(rc) + "): " + slhip_last_error_string());
+}
+
+class HIP;
+
+struct Buffer {
+  HIP* dev = nullptr;
+  uint64_t id = 0;
+  float* ptr = nullptr;
+  size_t len = 0;
+  bool requires_grad = true;  // custos buffers take part in autograd unless `no_grad()` was called
+
+  bool valid() const { return ptr != nullptr; }
+  inline std::vector<float> read() const;
+  inline void write(const float* host, size_t n) const;
+  inline Buffer grad() const;  // throws if no gradient was ever written for this buffer
+  inline void backward() const;
+  inline void backward_with(const Buffer& g) const;
+};
+
+// How gemm_grad / softmax_grad / transpose_grad write: 0 = overwrite (the reference's CPU
+// device), 1 = accumulate (its OpenCL device, src/ops2/gemm/grad/opencl.rs:20,33).
+struct GradPolicy {
+  float gemm_beta = 0.0f;
+  float softmax_beta = 0.0f;
+  float transpose_beta = 0.0f;
+};
+
+class HIP {
+ public:
+  GradPolicy policy;
+
+  explicit HIP(int ordinal = 0, bool cached = true) : cached_(cached) { check(slhip_init(ordinal, &ctx_), "slhip_init"); }
+  ~HIP() {
+    for (auto& kv : allocs_) slhip_free(ctx_, kv.second.ptr);
+    slhip_destroy(ctx_);
+  }
+  HIP(const HIP&) = delete;
+  HIP& operator=(const HIP&) = delete;
+
+  slhip_ctx* ctx() const { return ctx_; }
+  void sync() { check(slhip_sync(ctx_), "slhip_sync"); }
+
+  // ---- buffers ---------------------------------------------------------------------------
+  Buffer alloc(size_t len, bool zero = true) {
+    if (len == 0) throw Error("zero-length buffer");
+    Buffer b;
+    b.dev = this;
+    b.id = next_id_++;
+    b.len = len;
+    check(slhip_malloc(ctx_, len * sizeof(float), (void**)&b.ptr), "slhip_malloc");
+    if (zero) check(slhip_memset(ctx_, b.ptr, 0, len * sizeof(float)), "slhip_memset");
+    allocs_[b.id] = b;
+    return b;
+  }
+  Buffer from(const float* host, size_t len) {
+    Buffer b = alloc(len, false);
+    check(slhip_memcpy_h2d(ctx_, b.ptr, host, len * sizeof(float)), "slhip_memcpy_h2d");
+    return b;
+  }
+  Buffer from(const std::vector<float>& v) { return from(v.data(), v.size()); }
+  Buffer lookup(uint64_t id) const {
+    auto it = allocs_.find(id);
+    if (it == allocs_.end()) throw Error("unknown buffer id " + std::to_string(id));
+    return it->second;
+  }
+  void set_requires_grad(uint64_t id, bool v) {
+    auto it = allocs_.find(id);
+    if (it == allocs_.end()) throw Error("unknown buffer id");
+    it->second.requires_grad = v;
+  }
+  void release(uint64_t id) {
+    auto it = allocs_.find(id);
+    if (it == allocs_.end()) return;
+    check(slhip_free(ctx_, it->second.ptr), "slhip_free");
+    allocs_.erase(it);
+    auto g = grads_.find(id);
+    if (g != grads_.end()) {  // the gradient lives and dies with its buffer
+      const uint64_t gid = g->second.id;
+      grads_.erase(g);
+      release(gid);
+    }
+  }
+
+  // Output buffer of an op.  Cached mode: position `cursor_` of this iteration; the buffer is
+  // zeroed only when the op accumulates into it (`zero`), every other op overwrites all of it.
+  Buffer retrieve(size_t len, bool zero = false) {
+    if (!cached_) return alloc(len, zero);
+    if (cursor_ < cache_.size() && cache_[cursor_].len == len) {
+      Buffer b = cache_[cursor_++];
+      if (zero) check(slhip_memset(ctx_, b.ptr, 0, len * sizeof(float)), "slhip_memset");
+      return b;
+    }
+    // first iteration, or the op sequence changed: (re)build the cache from here on
+    for (size_t i = cursor_; i < cache_.size(); ++i) release(cache_[i].id);
+    cache_.resize(cursor_);
+    Buffer b = alloc(len, zero);
+    cache_.push_back(b);
+    ++cursor_;
+    return b;
+  }
+
+  // `for epoch in device.range(0..n)`: every iteration starts at cache position 0.
+  struct Range {
+    HIP* dev;
+    size_t n;
+    struct It {
+      HIP* dev;
+      size_t i;
+      size_t operator*() const { return i; }
+      bool operator!=(const It& o) const { return i != o.i; }
+      It& operator++() { ++i; dev->cursor_ = 0; return *this; }
+    };
+    It begin() { dev->cursor_ = 0; return {dev, 0}; }
+    It end() { return {dev, n}; }
+  };
+  Range range(size_t n) { return Range{this, n}; }
+
+  // ---- autograd --------------------------------------------------------------------------
+  void add_grad_fn(std::function<void()> f) { if (tape_enabled_) tape_.push_back(std::move(f)); }
+  void enable_tape(bool on) { tape_enabled_ = on; }
+  size_t tape_len() const { return tape_.size(); }
+
+  bool has_grad(uint64_t id) const { return grads_.count(id) != 0; }
+  Buffer grad(const Buffer& b) const {
+    auto it = grads_.find(b.id);
+    if (it == grads_.end()) throw Error("buffer " + std::to_string(b.id) + " has no gradient");
+    return it->second;
+  }
+  Buffer grad_mut(const Buffer& b) {
+    auto it = grads_.find(b.id);
+    if (it != grads_.end()) return it->second;
+    Buffer g = alloc(b.len, true);
+    g.requires_grad = false;
+    grads_[b.id] = g;
+    return g;
+  }
+  void zero_grad() {
+    for (auto& kv : grads_) check(slhip_memset(ctx_, kv.second.ptr, 0, kv.second.len * sizeof(float)), "slhip_memset");
+  }
+  void run_tape() {
+    for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
+    tape_.clear();
+  }
+  void backward(const Buffer& out) {
+    Buffer g = grad_mut(out);
+    check(slhip_fill(ctx_, g.len, 1.0f, g.ptr), "slhip_fill");
+    run_tape();
+  }
+  void backward_with(const Buffer& out, const Buffer& seed) {
+    if (seed.len != out.len) throw Error("backward_with: seed length differs");
+    Buffer g = grad_mut(out);
+    check(slhip_memcpy_d2d(ctx_, g.ptr, seed.ptr, g.len * sizeof(float)), "slhip_memcpy_d2d");
+    run_tape();
+  }
+
+  // ---- ops: forward + tape registration (reference: the *MayGrad impls in src/ops.rs) ------
+  // GemmMayGrad::gemm  src/ops.rs:250-289
+  Buffer gemm(size_t m, size_t k, size_t n, const Buffer& lhs, const Buffer& rhs) {
+    expect(lhs, m * k, "gemm lhs"); expect(rhs, k * n, "gemm rhs");
+    Buffer out = retrieve(m * n);
+    check(slhip_gemm(ctx_, m, k, n, lhs.ptr, rhs.ptr, out.ptr), "slhip_gemm");
+    uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
+      float* lg = l.requires_grad ? grad_mut(l).ptr : nullptr;
+      float* rg = r.requires_grad ? grad_mut(r).ptr : nullptr;
+      check(slhip_gemm_grad(ctx_, m, k, n, l.ptr, r.ptr, lg, rg, grad(o).ptr, policy.gemm_beta), "slhip_gemm_grad");
+    });
+    return out;
+  }
+
+  // Linear forward fused into the GEMM epilogue: relu?(x·w + bias) in one kernel.  On the tape
+  // it is the same three closures the unfused sequence gemm -> add_row_mut -> relu leaves
+  // (examples/sine_net.rs:32-40, src/matrix.rs:169-190), merged into one.
+  Buffer linear(size_t m, size_t k, size_t n, const Buffer& x, const Buffer& w, const Buffer& bias, bool relu) {
+    expect(x, m * k, "linear x"); expect(w, k * n, "linear w"); expect(bias, n, "linear bias");
+    Buffer pre = relu ? retrieve(m * n) : Buffer();
+    Buffer out = retrieve(m * n);
+    check(slhip_linear_fwd(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, relu ? 1 : 0, relu ? pre.ptr : nullptr, out.ptr),
+          "slhip_linear_fwd");
+    uint64_t xi = x.id, wi = w.id, bi = bias.id, oi = out.id, pi = relu ? pre.id : 0;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), wb = lookup(wi), bb = lookup(bi), o = lookup(oi);
+      Buffer g = grad(o);
+      if (relu) {  // relu grad: pre.grad += (pre >= 0) * out.grad
+        Buffer p = lookup(pi);
+        Buffer pg = grad_mut(p);
+        check(slhip_ew_unary_grad(ctx_, SLHIP_RELU, 0.0f, p.len, p.ptr, pg.ptr, g.ptr), "relu grad");
+        g = pg;
+      }
+      check(slhip_add_row_mut_grad(ctx_, m, n, grad_mut(bb).ptr, g.ptr), "bias grad");
+      float* xg = xb.requires_grad ? grad_mut(xb).ptr : nullptr;
+      float* wg = wb.requires_grad ? grad_mut(wb).ptr : nullptr;
+      check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
+    });
+    return out;
+  }
+
+  // RowOpMayGrad::add_row  src/ops.rs:323-356
+  Buffer add_row(size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
+    expect(lhs, rows * cols, "add_row lhs"); expect(rhs, cols, "add_row rhs");
+    Buffer out = retrieve(rows * cols);
+    check(slhip_add_row(ctx_, rows, cols, lhs.ptr, rhs.ptr, out.ptr), "slhip_add_row");
+    uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
+      check(slhip_add_row_grad(ctx_, rows, cols, grad_mut(l).ptr, grad_mut(r).ptr, grad(o).ptr), "slhip_add_row_grad");
+    });
+    return out;
+  }
+  // RowOpMayGrad::add_row_mut  src/ops.rs:358-374 — in place; lhs keeps its id and gradient
+  void add_row_mut(size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
+    expect(lhs, rows * cols, "add_row_mut lhs"); expect(rhs, cols, "add_row_mut rhs");
+    check(slhip_add_row(ctx_, rows, cols, lhs.ptr, rhs.ptr, lhs.ptr), "slhip_add_row");
+    uint64_t li = lhs.id, ri = rhs.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), r = lookup(ri);
+      check(slhip_add_row_mut_grad(ctx_, rows, cols, grad_mut(r).ptr, grad(l).ptr), "slhip_add_row_mut_grad");
+    });
+  }
+
+  // BinaryOpsMayGrad::{add,sub,mul}  src/ops.rs:115-171
+  Buffer binary(int op, const Buffer& lhs, const Buffer& rhs) {
+    if (lhs.len != rhs.len) throw Error("binary op: lengths differ");
+    Buffer out = retrieve(lhs.len);
+    check(slhip_ew_binary(ctx_, op, lhs.len, lhs.ptr, rhs.ptr, out.ptr), "slhip_ew_binary");
+    uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
+      // the reference touches both gradients whatever requires_grad says (src/ops.rs:118-128)
+      check(slhip_ew_binary_grad(ctx_, op, l.len, l.ptr, r.ptr, grad_mut(l).ptr, grad_mut(r).ptr, grad(o).ptr),
+            "slhip_ew_binary_grad");
+    });
+    return out;
+  }
+  Buffer add(const Buffer& l, const Buffer& r) { return binary(SLHIP_ADD, l, r); }
+  Buffer sub(const Buffer& l, const Buffer& r) { return binary(SLHIP_SUB, l, r); }
+  Buffer mul(const Buffer& l, const Buffer& r) { return binary(SLHIP_MUL, l, r); }
+
+  // apply_fn + add_unary_grad: square (src/ops.rs:25-45), pow (:64-77), relu (src/matrix.rs:169-190)
+  Buffer unary(int op, const Buffer& x, float p = 0.0f, float q = 0.0f, bool with_grad = true) {
+    Buffer out = retrieve(x.len);
+    check(slhip_ew_unary(ctx_, op, p, q, x.len, x.ptr, out.ptr), "slhip_ew_unary");
+    if (with_grad) {
+      uint64_t xi = x.id, oi = out.id;
+      add_grad_fn([=] {
+        Buffer xb = lookup(xi), o = lookup(oi);
+        check(slhip_ew_unary_grad(ctx_, op, p, xb.len, xb.ptr, grad_mut(xb).ptr, grad(o).ptr), "slhip_ew_unary_grad");
+      });
+    }
+    return out;
+  }
+  Buffer square(const Buffer& x) { return unary(SLHIP_SQUARE, x); }
+  Buffer pow(const Buffer& x, float rhs) { return unary(SLHIP_POW, x, rhs); }
+  Buffer relu(const Buffer& x) { return unary(SLHIP_RELU, x); }
+  Buffer exp(const Buffer& x) { return unary(SLHIP_EXP, x, 0, 0, false); }                        // src/ops.rs:435-440
+  Buffer clip(const Buffer& x, float lo, float hi) { return unary(SLHIP_CLIP, x, lo, hi, false); }  // src/ops.rs:419-425
+
+  // TransposeMayGrad::transpose  src/ops.rs:207-220
+  Buffer transpose(size_t rows, size_t cols, const Buffer& x) {
+    expect(x, rows * cols, "transpose");
+    Buffer out = retrieve(x.len);
+    check(slhip_transpose(ctx_, rows, cols, x.ptr, out.ptr, 0.0f), "slhip_transpose");
+    uint64_t xi = x.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), o = lookup(oi);
+      check(slhip_transpose(ctx_, cols, rows, grad(o).ptr, grad_mut(xb).ptr, policy.transpose_beta), "transpose_grad");
+    });
+    return out;
+  }
+
+  // SoftmaxMayGrad::softmax  src/ops.rs:751-778
+  Buffer softmax(size_t samples, size_t features, const Buffer& x) {
+    expect(x, samples * features, "softmax");
+    Buffer out = retrieve(x.len);
+    check(slhip_softmax(ctx_, samples, features, x.ptr, out.ptr), "slhip_softmax");
+    uint64_t xi = x.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), o = lookup(oi);
+      check(slhip_softmax_grad(ctx_, samples, features, grad_mut(xb).ptr, o.ptr, grad(o).ptr, policy.softmax_beta),
+            "slhip_softmax_grad");
+    });
+    return out;
+  }
+
+  // Reductions with gradients: SumColsMayGrad (src/ops.rs:592-611), SumRows (forward + the slice
+  // gradient; the reference's own wrapper is `unimplemented!()`, src/ops.rs:553-567),
+  // MaxCols/MaxRows (:471-491, :515-534), MeanCols/MeanRows (:635-651, :675-684).
+  enum Red { SUM_ROWS, SUM_COLS, MAX_ROWS, MAX_COLS, MEAN_ROWS, MEAN_COLS };
+  Buffer reduce(Red kind, size_t rows, size_t cols, const Buffer& x) {
+    expect(x, rows * cols, "reduction");
+    const bool over_rows = kind == SUM_ROWS || kind == MAX_ROWS || kind == MEAN_ROWS;
+    Buffer out = retrieve(over_rows ? cols : rows);
+    typedef int32_t (*Fwd)(slhip_ctx*, size_t, size_t, const float*, float*);
+    static const Fwd fwd[] = {slhip_sum_rows, slhip_sum_cols, slhip_max_rows, slhip_max_cols, slhip_mean_rows,
+                              slhip_mean_cols};
+    check(fwd[kind](ctx_, rows, cols, x.ptr, out.ptr), "reduction");
+    uint64_t xi = x.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), o = lookup(oi);
+      float* xg = grad_mut(xb).ptr;
+      const float* og = grad(o).ptr;
+      switch (kind) {
+        case SUM_ROWS: check(slhip_sum_rows_grad(ctx_, rows, cols, xg, og), "sum_rows_grad"); break;
+        case SUM_COLS: check(slhip_sum_cols_grad(ctx_, rows, cols, xg, og), "sum_cols_grad"); break;
+        case MAX_ROWS: check(slhip_max_rows_grad(ctx_, rows, cols, o.ptr, xb.ptr, xg, og), "max_rows_grad"); break;
+        case MAX_COLS: check(slhip_max_cols_grad(ctx_, rows, cols, o.ptr, xb.ptr, xg, og), "max_cols_grad"); break;
+        case MEAN_ROWS: check(slhip_mean_rows_grad(ctx_, rows, cols, xg, og), "mean_rows_grad"); break;
+        case MEAN_COLS: check(slhip_mean_cols_grad(ctx_, rows, cols, xg, og), "mean_cols_grad"); break;
+      }
+    });
+    return out;
+  }
+
+  // Mean::mean  src/ops2/mean/mod.rs:15-17 — a host scalar, not on the tape
+  float mean(const Buffer& x) {
+    Buffer s = scalar_scratch();
+    check(slhip_mean(ctx_, x.len, x.ptr, s.ptr), "slhip_mean");
+    float v;
+    check(slhip_memcpy_d2h(ctx_, &v, s.ptr, sizeof(float)), "slhip_memcpy_d2h");
+    return v;
+  }
+
+  // SGD of the examples (examples/sine_net.rs:105-116): value -= grad * lr, on the device
+  void sgd_step(const Buffer& p, float lr) {
+    check(slhip_sgd_step(ctx_, p.len, p.ptr, grad(p).ptr, lr), "slhip_sgd_step");
+  }
+
+ private:
+  static void expect(const Buffer& b, size_t len, const char* what) {
+    if (!b.valid() || b.len != len)
+      throw Error(std::string(what) + ": buffer length " + std::to_string(b.len) + " != " + std::to_string(len));
+  }
+  Buffer scalar_scratch() {
+    if (!scratch_.valid()) scratch_ = alloc(1, true);
+    return scratch_;
+  }
+
+  slhip_ctx* ctx_ = nullptr;
+  bool cached_;
+  uint64_t next_id_ = 1;
+  std::unordered_map<uint64_t, Buffer> allocs_;
+  std::unordered_map<uint64_t, Buffer> grads_;
+  std::vector<std::function<void()>> tape_;
+  bool tape_enabled_ = true;
+  std::vector<Buffer> cache_;
+  size_t cursor_ = 0;
+  Buffer scratch_;
+};
+
+inline std::vector<float> Buffer::read() const {
+  std::vector<float> v(len);
+  check(slhip_memcpy_d2h(dev->ctx(), v.data(), ptr, len * sizeof(float)), "slhip_memcpy_d2h");
+  return v;
+}
+inline void Buffer::write(const float* host, size_t n) const {
+  if (n != len) throw Error("write: length differs");
+  check(slhip_memcpy_h2d(dev->ctx(), ptr, host, len * sizeof(float)), "slhip_memcpy_h2d");
+}
+inline Buffer Buffer::grad() const { return dev->grad(*this); }
+inline void Buffer::backward() const { dev->backward(*this); }
+inline void Buffer::backward_with(const Buffer& g) const { dev->backward_with(*this, g); }
+
+// ---------------------------------------------------------------------------------------------
+// Matrix: {Buffer, rows, cols} with a method per op (src/matrix.rs).
+// ---------------------------------------------------------------------------------------------
+class Matrix {
+ public:
+  Buffer data;
+  size_t rows = 0, cols = 0;
+
+  Matrix() = default;
+  Matrix(Buffer b, size_t r, size_t c) : data(b), rows(r), cols(c) {
+    if (b.len != r * c) throw Error("Matrix: buffer length != rows*cols");  // src/matrix/impl_from.rs:7-10
+  }
+  Matrix(HIP& dev, size_t r, size_t c) : data(dev.alloc(r * c, true)), rows(r), cols(c) {}
+  Matrix(HIP& dev, size_t r, size_t c, const std::vector<float>& v) : Matrix(dev.from(v), r, c) {}
+
+  HIP& device() const { return *data.dev; }
+  Matrix require_grad() { data.requires_grad = true; data.dev->set_requires_grad(data.id, true); return *this; }
+  Matrix no_grad() { data.requires_grad = false; data.dev->set_requires_grad(data.id, false); return *this; }
+  std::vector<float> read() const { return data.read(); }
+  Matrix grad() const { return Matrix(data.grad(), rows, cols); }
+  void backward() const { data.backward(); }
+  void backward_with(const Matrix& g) const { data.backward_with(g.data); }
+
+  Matrix T() const { return Matrix(device().transpose(rows, cols, data), cols, rows); }                         // :98-107
+  Matrix gemm(const Matrix& rhs) const { return Matrix(device().gemm(rows, cols, rhs.cols, data, rhs.data), rows, rhs.cols); }  // :111-122
+  Matrix add(const Matrix& rhs) const { return Matrix(device().add(data, rhs.data), rows, cols); }              // :127-132
+  Matrix sub(const Matrix& rhs) const { return Matrix(device().sub(data, rhs.data), rows, cols); }              // :409-417
+  Matrix mul(const Matrix& rhs) const { return Matrix(device().mul(data, rhs.data), rows, cols); }              // :137-142
+  Matrix add_row(const Matrix& rhs) const { return Matrix(device().add_row(rows, cols, data, rhs.data), rows, cols); }  // :146-156
+  void add_row_mut(const Matrix& rhs) { device().add_row_mut(rows, cols, data, rhs.data); }                     // :160-165
+  Matrix relu() const { return Matrix(device().relu(data), rows, cols); }                                       // :169-190
+  Matrix squared() const { return Matrix(device().square(data), rows, cols); }                                  // :275-288
+  Matrix pow(float rhs) const { return Matrix(device().pow(data, rhs), rows, cols); }                           // :292-297
+  Matrix softmax() const { return Matrix(device().softmax(rows, cols, data), rows, cols); }                     // :368-378
+  Matrix sum_cols() const { return Matrix(device().reduce(HIP::SUM_COLS, rows, cols, data), rows, 1); }         // :329-334
+  // The reference's Matrix::max_rows / max_cols wrap the reduced buffer as (rows, cols) and trip
+  // its own length assert unless one dimension is 1 (src/matrix.rs:301-325); here the result
+  // carries its true shape.
+  Matrix max_rows() const { return Matrix(device().reduce(HIP::MAX_ROWS, rows, cols, data), 1, cols); }
+  Matrix max_cols() const { return Matrix(device().reduce(HIP::MAX_COLS, rows, cols, data), rows, 1); }
+  Matrix as_dims(size_t r, size_t c) const { return Matrix(data, r, c); }                                       // :383-390
+};
+
+}  // namespace sliced

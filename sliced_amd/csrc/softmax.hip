@@ -32,23 +32,37 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
 
   float v[ITEMS][V];
   float m = NEG_INF;
+  // every lane of the row holds ITEMS full vectors: unconditional loads, all in flight together
+  const bool full = active && (size_t)LANES * ITEMS <= colsv;
+  if (VEC && full) {
+    float4 t[ITEMS];
 #pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    const size_t c = (size_t)lane + (size_t)j * LANES;
-    if (active && c < colsv) {
-      if (VEC) {
-        float4 t = ld4s(x + row * cols + 4 * c);
-        v[j][0] = t.x; v[j][V > 1 ? 1 : 0] = t.y; v[j][V > 1 ? 2 : 0] = t.z; v[j][V > 1 ? 3 : 0] = t.w;
-      } else {
-        v[j][0] = x[row * cols + c];
-      }
-    } else {
+    for (int j = 0; j < ITEMS; ++j) t[j] = ld4s(x + row * cols + 4 * ((size_t)lane + (size_t)j * LANES));
 #pragma unroll
-      for (int q = 0; q < V; ++q) v[j][q] = NEG_INF;
+    for (int j = 0; j < ITEMS; ++j) {
+      v[j][0] = t[j].x; v[j][V > 1 ? 1 : 0] = t[j].y; v[j][V > 1 ? 2 : 0] = t[j].z; v[j][V > 1 ? 3 : 0] = t[j].w;
     }
+  } else {
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const size_t c = (size_t)lane + (size_t)j * LANES;
+      if (active && c < colsv) {
+        if (VEC) {
+          float4 t = ld4s(x + row * cols + 4 * c);
+          v[j][0] = t.x; v[j][V > 1 ? 1 : 0] = t.y; v[j][V > 1 ? 2 : 0] = t.z; v[j][V > 1 ? 3 : 0] = t.w;
+        } else {
+          v[j][0] = x[row * cols + c];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < V; ++q) v[j][q] = NEG_INF;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
     for (int q = 0; q < V; ++q) m = fmaxf(m, v[j][q]);
-  }
   m = row_reduce<MaxOp, LANES>(m, smem);
 
   float s = 0.0f;
@@ -91,25 +105,43 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
 
   float s[ITEMS][V], g[ITEMS][V];
   float dot = 0.0f;
+  const bool full = active && (size_t)LANES * ITEMS <= colsv;
+  if (VEC && full) {
+    float4 a[ITEMS], b[ITEMS];
 #pragma unroll
-  for (int j = 0; j < ITEMS; ++j) {
-    const size_t c = (size_t)lane + (size_t)j * LANES;
-    if (active && c < colsv) {
-      if (VEC) {
-        float4 a = ld4s(out + row * cols + 4 * c), b = ld4s(out_grad + row * cols + 4 * c);
-        s[j][0] = a.x; s[j][V > 1 ? 1 : 0] = a.y; s[j][V > 1 ? 2 : 0] = a.z; s[j][V > 1 ? 3 : 0] = a.w;
-        g[j][0] = b.x; g[j][V > 1 ? 1 : 0] = b.y; g[j][V > 1 ? 2 : 0] = b.z; g[j][V > 1 ? 3 : 0] = b.w;
-      } else {
-        s[j][0] = out[row * cols + c];
-        g[j][0] = out_grad[row * cols + c];
-      }
-    } else {
-#pragma unroll
-      for (int q = 0; q < V; ++q) { s[j][q] = 0.0f; g[j][q] = 0.0f; }
+    for (int j = 0; j < ITEMS; ++j) {
+      const size_t off = row * cols + 4 * ((size_t)lane + (size_t)j * LANES);
+      a[j] = ld4s(out + off);
+      b[j] = ld4s(out_grad + off);
     }
 #pragma unroll
-    for (int q = 0; q < V; ++q) dot += s[j][q] * g[j][q];
+    for (int j = 0; j < ITEMS; ++j) {
+      s[j][0] = a[j].x; s[j][V > 1 ? 1 : 0] = a[j].y; s[j][V > 1 ? 2 : 0] = a[j].z; s[j][V > 1 ? 3 : 0] = a[j].w;
+      g[j][0] = b[j].x; g[j][V > 1 ? 1 : 0] = b[j].y; g[j][V > 1 ? 2 : 0] = b[j].z; g[j][V > 1 ? 3 : 0] = b[j].w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const size_t c = (size_t)lane + (size_t)j * LANES;
+      if (active && c < colsv) {
+        if (VEC) {
+          float4 a = ld4s(out + row * cols + 4 * c), b = ld4s(out_grad + row * cols + 4 * c);
+          s[j][0] = a.x; s[j][V > 1 ? 1 : 0] = a.y; s[j][V > 1 ? 2 : 0] = a.z; s[j][V > 1 ? 3 : 0] = a.w;
+          g[j][0] = b.x; g[j][V > 1 ? 1 : 0] = b.y; g[j][V > 1 ? 2 : 0] = b.z; g[j][V > 1 ? 3 : 0] = b.w;
+        } else {
+          s[j][0] = out[row * cols + c];
+          g[j][0] = out_grad[row * cols + c];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < V; ++q) { s[j][q] = 0.0f; g[j][q] = 0.0f; }
+      }
+    }
   }
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j)
+#pragma unroll
+    for (int q = 0; q < V; ++q) dot += s[j][q] * g[j][q];
   dot = row_reduce<SumOp, LANES>(dot, smem);
 
 #pragma unroll

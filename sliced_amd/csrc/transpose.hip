@@ -25,17 +25,28 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 
   if (VEC_LD) {
     const int lx = t & 15, ly = t >> 4;  // 16 float4 per tile row, 16 rows per pass
-    // fully unrolled: all 16 loads of a thread are in flight together (only two tiles fit a CU)
+    // All 16 loads of a thread are issued before the first LDS store: only two tiles fit a CU,
+    // so the bytes in flight have to come from each thread (64 VGPRs), not from occupancy.
+    float4 v[TR / 16];
+    const bool full = r0 + TR <= rows && c0 + TC <= cols;
+    if (full) {
+#pragma unroll
+      for (int p = 0; p < TR / 16; ++p) v[p] = ld4s(x + (r0 + ly + 16 * p) * cols + c0 + 4 * lx);
+    } else {
+#pragma unroll
+      for (int p = 0; p < TR / 16; ++p) {
+        const size_t r = r0 + ly + 16 * p, c = c0 + 4 * lx;
+        // cols % 4 == 0: a vector is all in or all out
+        v[p] = (r < rows && c < cols) ? ld4s(x + r * cols + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
 #pragma unroll
     for (int p = 0; p < TR / 16; ++p) {
       const int rr = ly + 16 * p;
-      const size_t r = r0 + rr, c = c0 + 4 * lx;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (r < rows && c < cols) v = ld4s(x + r * cols + c);  // cols % 4 == 0: a vector is all in or all out
-      tile[rr][4 * lx + 0] = v.x;
-      tile[rr][4 * lx + 1] = v.y;
-      tile[rr][4 * lx + 2] = v.z;
-      tile[rr][4 * lx + 3] = v.w;
+      tile[rr][4 * lx + 0] = v[p].x;
+      tile[rr][4 * lx + 1] = v[p].y;
+      tile[rr][4 * lx + 2] = v[p].z;
+      tile[rr][4 * lx + 3] = v[p].w;
     }
   } else {
     const int lx = t & 63, ly = t >> 6;  // 64 columns, 4 rows per pass

@@ -1,0 +1,276 @@
+"""The C++ host device layer (tape, gradient map, cache) on the GPU, driven the way the
+reference's integration tests drive its devices: forward op, `backward()`, read `.grad()`.
+Expected values are the reference's own (tests/*.rs); the training loops are compared with the
+CPU oracle's loops step by step."""
+import sys
+
+import numpy as np
+import pytest
+
+from sliced_amd import rng
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture()
+def device():
+    from sliced_amd import host
+    d = host.HIP(0, cached=False)
+    yield d
+    d.close()
+
+
+def eq(buf, expect):
+    assert np.array_equal(buf.read(), np.asarray(expect, np.float32)), (buf.read(), expect)
+
+
+# reference: tests/test_gemm.rs:4-43
+def test_gemm(device):
+    lhs = device.buffer([1, 2, 3, 4, 4, 5, 6, 5])
+    rhs = device.buffer([1, 2, 3, 4, 5, 6])
+    out = device.gemm(4, 2, 3, lhs, rhs)
+    eq(out, [9, 12, 15, 19, 26, 33, 24, 33, 42, 26, 37, 48])
+    out.backward()
+    eq(lhs.grad(), [6, 15, 6, 15, 6, 15, 6, 15])
+    eq(rhs.grad(), [14, 14, 14, 16, 16, 16])
+
+
+def test_gemm_skips_operands_without_requires_grad(device):
+    lhs = device.buffer([1, 2, 3, 4, 4, 5, 6, 5]).no_grad()
+    rhs = device.buffer([1, 2, 3, 4, 5, 6])
+    out = device.gemm(4, 2, 3, lhs, rhs)
+    out.backward()
+    assert not lhs.has_grad()            # src/ops2/gemm/grad/cpu_stack.rs:35
+    eq(rhs.grad(), [14, 14, 14, 16, 16, 16])
+
+
+# reference: tests/test_add.rs, test_sub.rs, test_mul.rs
+def test_add_sub_mul(device):
+    lhs, rhs = device.buffer([1, 2, 3, 4, 5]), device.buffer([6, 7, 8, 9, 10])
+    out = device.add(lhs, rhs)
+    eq(out, [7, 9, 11, 13, 15])
+    out.backward()
+    eq(lhs.grad(), [1] * 5)
+    eq(rhs.grad(), [1] * 5)
+    lhs, rhs = device.buffer([1, 2, 3, 4, 5]), device.buffer([6, 7, 8, 9, 10])
+    out = device.sub(lhs, rhs)
+    eq(out, [-5] * 5)
+    out.backward()
+    eq(lhs.grad(), [1] * 5)
+    eq(rhs.grad(), [-1] * 5)
+    lhs, rhs = device.buffer([1, 2, 3, 4, 5]), device.buffer([6, 7, 8, 9, 10])
+    out = device.mul(lhs, rhs)
+    eq(out, [6, 14, 24, 36, 50])
+    out.backward()
+    eq(lhs.grad(), [6, 7, 8, 9, 10])
+    eq(rhs.grad(), [1, 2, 3, 4, 5])
+
+
+# reference: tests/test_pow.rs, tests/test_square.rs, tests/matrix/relu.rs
+def test_pow_square_relu(device):
+    x = device.buffer([1, 2, 3, 4, 5])
+    out = device.pow(x, 3.0)
+    eq(out, [1, 8, 27, 64, 125])
+    out.backward()
+    eq(x.grad(), [3, 12, 27, 48, 75])
+    x = device.buffer([1, 2, 3, 4, 5])
+    out = device.square(x)
+    eq(out, [1, 4, 9, 16, 25])
+    out.backward()
+    eq(x.grad(), [2, 4, 6, 8, 10])
+    x = device.buffer([-1, -3, 2, 5, -1.3])
+    out = device.relu(x)
+    eq(out, [0, 0, 2, 5, 0])
+    out.backward()
+    eq(x.grad(), [0, 0, 1, 1, 0])
+
+
+# reference: tests/test_row_op.rs:3-77
+def test_row_op_and_row_op_mut(device):
+    data = [-1, -3, 4, 5, 2, 2, 1, 5, -3, 2, 2, 4, 3, 2, -1]
+    expect = [0, -1, 7, 9, 7, 3, 3, 8, 1, 7, 3, 6, 6, 6, 4]
+    buf, row = device.buffer(data), device.buffer([1, 2, 3, 4, 5])
+    out = device.add_row(3, 5, buf, row)
+    eq(out, expect)
+    out.backward()
+    eq(row.grad(), [3] * 5)
+    eq(buf.grad(), [1] * 15)
+    buf, row = device.buffer(data), device.buffer([1, 2, 3, 4, 5])
+    device.add_row_mut(3, 5, buf, row)
+    eq(buf, expect)
+    buf.backward()
+    eq(row.grad(), [3] * 5)
+    eq(buf.grad(), [1] * 15)
+
+
+# reference: tests/test_sum_rows.rs, test_sum_cols.rs, test_max_rows.rs, test_max_cols.rs, test_mean.rs
+def test_reductions_under_a_following_op(device):
+    x = device.buffer([4, 2, 1, 3, 6, 1, 3, 1, 5, 4, 1, 1])
+    rhs = device.buffer([1, 4, 2, 3])
+    out = device.mul(device.sum_rows(4, x), rhs)
+    out.backward()
+    eq(x.grad(), [1, 4, 2, 3] * 3)
+    eq(rhs.grad(), [15, 7, 5, 5])
+
+    x = device.buffer([4, 2, 1, 3, 6, 1, 3, 1, 5, 4, 1, 1])
+    rhs = device.buffer([1, 4, 2])
+    out = device.mul(device.sum_cols(4, x), rhs)
+    out.backward()
+    eq(x.grad(), [1, 1, 1, 1, 4, 4, 4, 4, 2, 2, 2, 2])
+    eq(rhs.grad(), [10, 11, 11])
+
+    data = [-3, 2, 3, 1, 1, 5, -5, 4, -9, -2, -4, -1]
+    x, rhs = device.buffer(data), device.buffer([2, 3, 4, 1])
+    out = device.mul(device.max_rows(4, x), rhs)
+    out.backward()
+    eq(x.grad(), [0, 0, 4, 0, 2, 3, 0, 1, 0, 0, 0, 0])
+    eq(rhs.grad(), [1, 5, 3, 4])
+
+    x, rhs = device.buffer(data), device.buffer([1, 4, 2])
+    mc = device.max_cols(3, 4, x)
+    eq(mc, [3, 5, -1])
+    out = device.add(mc, rhs)
+    out.backward()
+    eq(x.grad(), [0, 0, 1, 0, 0, 1, 0, 0, 0, 0, 0, 1])
+    eq(rhs.grad(), [1, 1, 1])
+
+    lhs = device.buffer([2, 3, 4])
+    x = device.buffer([1, 4, 3, 2, 3, 5, 2, 1, 6, -2, 1, 4])
+    out = device.sub(lhs, device.mean_rows(3, x))
+    out.backward()
+    eq(x.grad(), [-0.25] * 12)
+    eq(lhs.grad(), [1, 1, 1])
+
+
+# reference: tests/matrix/transpose.rs, tests/matrix/softmax.rs, tests/matrix/l2_norm_cols.rs
+def test_transpose_softmax_l2norm(device):
+    x = device.buffer([1, 2, 3, 4, 5, 6])
+    xt = device.transpose(2, 3, x)
+    eq(xt, [1, 4, 2, 5, 3, 6])
+    y = device.buffer([-1, 1, 2, -5, -3, 2])
+    out = device.mul(y, xt)
+    out.backward()
+    eq(x.grad(), [-1, 2, -3, 1, -5, 2])          # transpose(3, 2, y)
+
+    x = device.buffer([1, 2, 3, 4, 5, 6])
+    out = device.softmax(2, 3, x)
+    assert np.max(np.abs(out.read() - np.array([0.09003057, 0.24472847, 0.66524096] * 2, np.float32))) < 1e-7
+    out.backward()
+    assert np.max(np.abs(x.grad().read())) < 1e-6
+
+    x = device.buffer([1, 2, 3, 4, 5, 6, 7, 8])
+    out = device.pow(device.sum_cols(4, device.square(x)), 0.5)
+    out.backward()
+    assert np.max(np.abs(x.grad().read()[:4] - np.array([0.1826, 0.3651, 0.5477, 0.7303], np.float32))) < 1e-2
+
+
+# reference: examples/chained_perf.rs:54-91 — cached device, the same chain every iteration
+def test_cached_range_reuses_buffers_and_values():
+    from sliced_amd import host
+    dev = host.HIP(0, cached=True)
+    n = 12345
+    x, b = dev.buffer(np.full(n, 1.3, np.float32)), dev.buffer(np.full(n, 2.1, np.float32))
+    ids = None
+    for epoch in range(5):
+        dev.begin_iteration()
+        squared = dev.square(x)
+        add = dev.add(b, x)
+        mul_b = dev.mul(add, b)
+        mul = dev.mul(squared, x)
+        out = dev.add(mul, mul_b)
+        assert out.read()[0] == np.float32(9.336999)
+        now = [t.id for t in (squared, add, mul_b, mul, out)]
+        if ids is not None:
+            assert now == ids                       # same call position -> same allocation
+        ids = now
+        out.backward()
+        g = x.grad().read()
+        # d/dx (x^3 + (b+x) b) = 3x^2 + b, accumulated over the epochs (no zero_grad here)
+        assert abs(g[0] / (epoch + 1) - (3 * 1.3 ** 2 + 2.1)) < 1e-4
+    dev.zero_grad()
+    assert np.all(x.grad().read() == 0)
+    dev.close()
+
+
+def test_linear_fused_matches_unfused_tape(device):
+    m, k, n = 96, 40, 24
+    x = rng.uniform(m * k, -1, 1, tag=0)
+    w = rng.uniform(k * n, -1, 1, tag=1)
+    b = rng.uniform(n, -1, 1, tag=2)
+    res = []
+    for fused in (False, True):
+        xb, wb, bb = device.buffer(x), device.buffer(w), device.buffer(b)
+        if fused:
+            out = device.linear(m, k, n, xb, wb, bb, True)
+        else:
+            h = device.gemm(m, k, n, xb, wb)
+            device.add_row_mut(m, n, h, bb)
+            out = device.relu(h)
+        out.backward()
+        res.append([out.read(), xb.grad().read(), wb.grad().read(), bb.grad().read()])
+    for a, c in zip(*res):
+        assert np.array_equal(a, c)
+
+
+def test_errors_surface_as_exceptions(device):
+    from sliced_amd import host
+    a = device.buffer([1, 2, 3])
+    with pytest.raises(host.HostError):
+        device.gemm(2, 2, 2, a, a)              # length != rows*cols
+    with pytest.raises(host.HostError):
+        a.grad()                                 # no gradient was ever written
+
+
+# --------------------------------------------------------------------------- training loops
+def loss_parity(got, ref, tol):
+    rel = np.abs(got - ref) / np.maximum(np.abs(ref), 1e-30)
+    return rel.max()
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["op-by-op", "fused-linear"])
+def test_sine_mlp_loss_curve_matches_oracle(orc, fused):
+    """Config 1: batch 1024, 1-64-64-1, MSE, SGD lr 0.01, 200 steps; per-step loss within 1e-4 rel."""
+    from sliced_amd import host
+    cfg = host.C1
+    say("C1", "fused" if fused else "unfused")
+    x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+    p_ref = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+    p_gpu = [a.copy() for a in p_ref]
+    ref = orc.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_ref, cfg["lr"],
+                        cfg["steps"])
+    got, _ = host.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_gpu, cfg["lr"],
+                            cfg["steps"], 0, fused)
+    assert ref[-1] < ref[0]                       # it trains
+    worst = loss_parity(got, ref, 1e-4)
+    say("C1 worst relative loss deviation", worst, "loss", ref[0], "->", ref[-1])
+    assert worst <= 1e-4
+    for a, b in zip(p_gpu, p_ref):
+        assert np.max(np.abs(a - b)) <= 1e-4 * max(1.0, np.max(np.abs(b)))
+
+
+@pytest.mark.parametrize("fused", [False, True], ids=["op-by-op", "fused-linear"])
+def test_classifier_mlp_loss_curve_matches_oracle(orc, fused):
+    """Config 5: batch 8192, 784-2048-2048-10, softmax cross-entropy, SGD lr 0.05, 50 steps."""
+    from sliced_amd import host
+    cfg = host.C5
+    say("C5", "fused" if fused else "unfused")
+    x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+    p_ref = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+    p_gpu = [a.copy() for a in p_ref]
+    global _C5_REF
+    try:
+        ref = _C5_REF
+    except NameError:
+        ref = _C5_REF = orc.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_ref,
+                                      cfg["lr"], cfg["steps"])
+    got, _ = host.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_gpu, cfg["lr"],
+                            cfg["steps"], 0, fused)
+    worst = loss_parity(got, ref, 1e-4)
+    say("C5 worst relative loss deviation", worst, "loss", ref[0], "->", ref[-1])
+    assert np.all(np.isfinite(got))
+    assert worst <= 1e-4
