@@ -1,0 +1,189 @@
+"""Parity at the full benchmark sizes ([16384 x 16384], 2^28-element vectors, [32768 x 4096]
+softmax, 4096^3 GEMM): direct comparison with the threaded CPU oracle where it finishes in
+seconds, plus size-independent properties (involution of the transpose, max over rows == max over
+the columns of the transpose, softmax rows sum to one, linearity of the GEMM).  Inputs are
+generated on the device by the seeded generator, which the small-size tests show to be
+bit-identical to the host generator."""
+import sys
+
+import numpy as np
+import pytest
+
+from sliced_amd import rng
+
+pytestmark = pytest.mark.gpu
+SEED = rng.DEFAULT_SEED
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def big(hip):
+    """x ~ U(-10,10) on [16384 x 16384] with 1 % row-maximum ties injected on the host copy."""
+    c = hip.ctx()
+    R = C = 16384
+    say("generating [16384 x 16384]")
+    d = c.uniform(R * C, -10, 10, 0, SEED)
+    x = d.numpy()
+    x = rng.inject_row_max_ties(x, R, C, 0.01)
+    d.upload(x)
+    yield c, R, C, d, x
+    d.free()
+
+
+def test_reductions_16384_squared_against_oracle(big, orc):
+    c, R, C, d, x = big
+    out_r, out_c = c.empty(R), c.empty(C)
+    say("max_cols / max_rows 16384^2 (bit-exact, with ties)")
+    c.call("slhip_max_cols", R, C, d.ptr, out_r.ptr)
+    assert np.array_equal(out_r.numpy(), orc.max_cols(C, x))
+    c.call("slhip_max_rows", R, C, d.ptr, out_c.ptr)
+    assert np.array_equal(out_c.numpy(), orc.max_rows(C, x))
+    say("sum_cols / sum_rows 16384^2")
+    X = x.reshape(R, C)
+    abs_r = np.abs(X).sum(1, dtype=np.float64)
+    abs_c = np.abs(X).sum(0, dtype=np.float64)
+    c.call("slhip_sum_cols", R, C, d.ptr, out_r.ptr)
+    exact = X.sum(1, dtype=np.float64)
+    got, ref = out_r.numpy(), orc.sum_cols(C, x)
+    assert np.all(np.abs(got - exact) <= 1e-6 * abs_r)
+    assert np.all(np.abs(got - ref) <= 1e-6 * abs_r + np.abs(ref - exact))
+    c.call("slhip_sum_rows", R, C, d.ptr, out_c.ptr)
+    exact = X.sum(0, dtype=np.float64)
+    got, ref = out_c.numpy(), orc.sum_rows(C, x)
+    assert np.all(np.abs(got - exact) <= 1e-6 * abs_c)
+    assert np.all(np.abs(got - ref) <= 1e-6 * abs_c + np.abs(ref - exact))
+    say("mean over 2^28")
+    one = c.empty(1)
+    c.call("slhip_mean", R * C, d.ptr, one.ptr)
+    tot = X.sum(dtype=np.float64)
+    assert abs(float(one.numpy()[0]) - tot / x.size) <= 1e-6 * abs_r.sum() / x.size + 1e-7 * abs(tot / x.size)
+    # degenerate shapes of the same tensor: [1 x 2^28] and [2^28 x 1]
+    say("degenerate shapes")
+    m = float(x.max())
+    for name, rows, cols in [("slhip_max_cols", 1, R * C), ("slhip_max_rows", R * C, 1)]:
+        c.call(name, rows, cols, d.ptr, one.ptr)
+        assert float(one.numpy()[0]) == m
+    for name, rows, cols in [("slhip_sum_cols", 1, R * C), ("slhip_sum_rows", R * C, 1)]:
+        c.call(name, rows, cols, d.ptr, one.ptr)
+        assert abs(float(one.numpy()[0]) - tot) <= 1e-6 * abs_r.sum()
+    for b in (out_r, out_c, one):
+        b.free()
+
+
+def test_max_cols_grad_first_tie_16384_squared(big, orc):
+    c, R, C, d, x = big
+    say("max_cols_grad 16384^2 with 1 % ties")
+    mx = orc.max_cols(C, x)
+    g = rng.normal(R, 1.0, tag=1, seed=SEED)
+    dm, dg, dxg = c.array(mx), c.array(g), c.zeros(R * C)
+    c.call("slhip_max_cols_grad", R, C, dm.ptr, d.ptr, dxg.ptr, dg.ptr)
+    got = dxg.numpy().reshape(R, C)
+    first = np.argmax(x.reshape(R, C) == mx[:, None], axis=1)
+    want = np.zeros((R, C), np.float32)
+    want[np.arange(R), first] = g
+    assert np.array_equal(got, want)
+    for b in (dm, dg, dxg):
+        b.free()
+
+
+def test_transpose_16384_squared(big):
+    c, R, C, d, x = big
+    say("transpose 16384^2: against numpy, and twice = identity")
+    t, tt = c.empty(R * C), c.empty(R * C)
+    c.call("slhip_transpose", R, C, d.ptr, t.ptr, 0.0)
+    assert np.array_equal(t.numpy().reshape(C, R), x.reshape(R, C).T)
+    c.call("slhip_transpose", C, R, t.ptr, tt.ptr, 0.0)
+    assert np.array_equal(tt.numpy(), x)
+    # max over rows == max over the columns of the transpose, bit for bit
+    a, b = c.empty(C), c.empty(C)
+    c.call("slhip_max_rows", R, C, d.ptr, a.ptr)
+    c.call("slhip_max_cols", C, R, t.ptr, b.ptr)
+    assert np.array_equal(a.numpy(), b.numpy())
+    for z in (t, tt, a, b):
+        z.free()
+
+
+def test_elementwise_chain_2_28_against_oracle(big, orc):
+    c, R, C, d, x = big
+    n = R * C
+    say("fused chain on 2^28 elements")
+    db, dc, dd, out = (c.uniform(n, -10, 10, 2, SEED), c.uniform(n, -10, 10, 3, SEED),
+                       c.uniform(n, -10, 10, 4, SEED), c.empty(n))
+    c.call("slhip_ew_chain", n, d.ptr, db.ptr, dc.ptr, dd.ptr, out.ptr)
+    got = out.numpy()
+    b, cc, dd_h = db.numpy(), dc.numpy(), dd.numpy()
+    t = orc.binary_ew(orc.SUB, orc.binary_ew(orc.MUL, orc.binary_ew(orc.ADD, x, b), cc), dd_h)
+    ref = orc.unary(orc.SQUARE, orc.unary(orc.POW, t, 2.0))
+    assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + 1e-37)
+    for z in (db, dc, dd, out):
+        z.free()
+
+
+@pytest.mark.parametrize("shape", [(32768, 4096), (1 << 20, 128), (1 << 17, 1024), (1 << 13, 16384)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_softmax_full_size(hip, orc, shape):
+    rows, cols = shape
+    n = rows * cols
+    c = hip.ctx()
+    say("softmax", rows, cols)
+    x = rng.normal(n, 3.0, tag=0, seed=SEED)
+    g = rng.normal(n, 1.0, tag=1, seed=SEED)
+    dx, dg, ds, dxg = c.array(x), c.array(g), c.empty(n), c.empty(n)
+    c.call("slhip_softmax", rows, cols, dx.ptr, ds.ptr)
+    s = ds.numpy()
+    ref = orc.softmax(rows, cols, x)
+    x2 = x.reshape(rows, cols)
+    shifted = (x2 - x2.max(1, keepdims=True)).astype(np.float32).astype(np.float64)
+    e = np.exp(shifted)
+    exact = (e / e.sum(1, keepdims=True)).ravel()
+    assert np.max(np.abs(s - exact) / np.maximum(exact, 1e-300)) <= 1e-6
+    assert np.all(np.abs(s - ref) <= 1e-6 * exact + np.abs(ref - exact))
+    assert np.max(np.abs(s.reshape(rows, cols).sum(1, dtype=np.float64) - 1.0)) <= 1e-6
+    c.call("slhip_softmax_grad", rows, cols, dxg.ptr, ds.ptr, dg.ptr, 0.0)
+    got = dxg.numpy()
+    S, G = s.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
+    exact_b = (S * (G - (S * G).sum(1, keepdims=True))).ravel()
+    bound = 1e-6 * (np.abs(S) * (np.abs(G) + (np.abs(S) * np.abs(G)).sum(1, keepdims=True))).ravel() + 1e-37
+    assert np.all(np.abs(got - exact_b) <= bound)
+    ob = orc.softmax_grad(rows, cols, s, g)
+    assert np.all(np.abs(got - ob) <= bound + np.abs(ob - exact_b))
+    # a constant upstream gradient gives zero
+    c.call("slhip_fill", n, 1.0, dg.ptr)
+    c.call("slhip_softmax_grad", rows, cols, dxg.ptr, ds.ptr, dg.ptr, 0.0)
+    assert np.max(np.abs(dxg.numpy())) <= 1e-6
+    for z in (dx, dg, ds, dxg):
+        z.free()
+
+
+@pytest.mark.parametrize("form", ["A*B", "A*Bt", "At*B"])
+def test_gemm_4096_cubed_against_oracle(hip, orc, form):
+    n = 4096
+    c = hip.ctx()
+    ta, tb = form == "At*B", form == "A*Bt"
+    say("gemm 4096^3", form)
+    a = rng.uniform(n * n, -1, 1, tag=0, seed=SEED)
+    b = rng.uniform(n * n, -1, 1, tag=1, seed=SEED)
+    da, db, dc = c.array(a), c.array(b), c.empty(n * n)
+    c.call("slhip_sgemm", int(ta), int(tb), n, n, n, da.ptr, db.ptr, dc.ptr, 0.0)
+    got = dc.numpy()
+    fn = orc.Tgemm if ta else orc.gemmT if tb else orc.gemm
+    ref = fn(n, n, n, a, b)
+    # |a||b| sums to about K/4 per entry; the bar is 1e-5*sqrt(K) of that scale
+    A = a.reshape(n, n).T if ta else a.reshape(n, n)
+    B = b.reshape(n, n).T if tb else b.reshape(n, n)
+    rows = rng.integers(64, n, tag=5, seed=SEED)
+    scale = (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    exact = A[rows].astype(np.float64) @ B.astype(np.float64)
+    tol = 1e-5 * np.sqrt(n) * scale
+    assert np.all(np.abs(got.reshape(n, n)[rows] - exact) <= tol)
+    assert np.all(np.abs(got - ref) <= 1e-5 * np.sqrt(n) * (n / 4.0) * 0.5)
+    # linearity: (2A)·B == 2·(A·B) exactly (scaling by two commutes with every rounding)
+    c.call("slhip_ew_unary", 6, 2.0, 0.0, n * n, da.ptr, da.ptr)
+    c.call("slhip_sgemm", int(ta), int(tb), n, n, n, da.ptr, db.ptr, dc.ptr, 0.0)
+    assert np.array_equal(dc.numpy(), got * np.float32(2.0))
+    for z in (da, db, dc):
+        z.free()
