@@ -32,13 +32,15 @@ extern "C" {
 
 typedef struct slhip_ctx slhip_ctx;
 typedef struct slhip_event slhip_event;
+typedef struct slhip_graph slhip_graph;
 
 enum {
   SLHIP_OK = 0,
   SLHIP_EINVAL = -1,     /* null pointer, zero/overflowing dims, unknown op code */
   SLHIP_ENODEVICE = -2,  /* no HIP device / wrong architecture */
   SLHIP_EWORKSPACE = -3, /* request does not fit the context workspace */
-  SLHIP_EALIAS = -4      /* forbidden overlap of operands */
+  SLHIP_EALIAS = -4,     /* forbidden overlap of operands */
+  SLHIP_ECAPTURE = -5    /* call not allowed while the context records a graph (or none is recording) */
 };
 
 /* BinaryElementWise op codes (reference: src/ops2/binary_ew/mod.rs:55-100). */
@@ -85,6 +87,23 @@ int32_t slhip_event_create(slhip_ctx* ctx, slhip_event** ev);
 int32_t slhip_event_record(slhip_ctx* ctx, slhip_event* ev);
 int32_t slhip_event_elapsed_ms(slhip_event* start, slhip_event* stop, float* ms); /* waits for stop */
 int32_t slhip_event_destroy(slhip_event* ev);
+
+/* Record once, replay many: between slhip_graph_begin and slhip_graph_end every op issued on
+ * the context is recorded into a HIP graph instead of being run; slhip_graph_launch replays
+ * the whole recording as one launch.  This is the device-side form of the reference's lazy
+ * mode (`Autograd<Lazy<Base>>` + `dev.run()`, examples/sine_net.rs:178-220), where ops are
+ * recorded on the first pass and re-run each epoch.  Pointers and sizes are baked into the
+ * recording: every buffer it names must stay allocated until slhip_graph_destroy.  While
+ * recording, the calls that wait or touch the allocator (slhip_malloc, slhip_free,
+ * slhip_memcpy_h2d, slhip_memcpy_d2h, slhip_sync, slhip_event_record, slhip_memset with a
+ * non-zero byte) return SLHIP_ECAPTURE and end nothing; the recording contains kernel nodes
+ * only (device-to-device copies and zero fills are recorded as kernels, never as
+ * memcpy/memset nodes). */
+int32_t slhip_graph_begin(slhip_ctx* ctx);
+int32_t slhip_graph_end(slhip_ctx* ctx, slhip_graph** graph);
+int32_t slhip_graph_launch(slhip_ctx* ctx, slhip_graph* graph);
+int32_t slhip_graph_node_count(slhip_graph* graph, size_t* nodes);
+int32_t slhip_graph_destroy(slhip_graph* graph);
 
 /* Seeded counter-based uniform fill: x[i] = lo + (hi-lo) * u(seed, tag, i), u a 24-bit
  * fraction from splitmix64((seed ^ (tag << 40)) + i).  Replaces RandOp::rand

@@ -35,6 +35,11 @@ PROTOTYPES = {
     "slhip_event_record": [c_vp, c_vp],
     "slhip_event_elapsed_ms": [c_vp, c_vp, C.POINTER(C.c_float)],
     "slhip_event_destroy": [c_vp],
+    "slhip_graph_begin": [c_vp],
+    "slhip_graph_end": [c_vp, C.POINTER(c_vp)],
+    "slhip_graph_launch": [c_vp, c_vp],
+    "slhip_graph_node_count": [c_vp, C.POINTER(c_sz)],
+    "slhip_graph_destroy": [c_vp],
     "slhip_rand_uniform": [c_vp, C.c_uint64, C.c_uint64, C.c_float, C.c_float, c_sz, c_vp],
     "slhip_sgemm": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_gemm": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp],

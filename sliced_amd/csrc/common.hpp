@@ -19,10 +19,17 @@ struct slhip_ctx {
   size_t workspace_bytes = 0;
   int num_cu = 256;
   char name[64] = {0};
+  bool capturing = false;        // between slhip_graph_begin and slhip_graph_end
 };
 
 struct slhip_event {
   hipEvent_t ev;
+};
+
+struct slhip_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  size_t nodes = 0;
 };
 
 namespace slhip {
@@ -37,6 +44,14 @@ int32_t hip_fail(hipError_t e, const char* what);
   do {                                                          \
     hipError_t _e = (expr);                                     \
     if (_e != hipSuccess) return slhip::hip_fail(_e, #expr);    \
+  } while (0)
+
+#define SLHIP_NOT_CAPTURING(ctx)                                                        \
+  do {                                                                                 \
+    if ((ctx)->capturing) {                                                            \
+      slhip::set_error("%s: not allowed while the context records a graph", __func__); \
+      return SLHIP_ECAPTURE;                                                           \
+    }                                                                                  \
   } while (0)
 
 #define SLHIP_REQUIRE(cond, msg)                                \

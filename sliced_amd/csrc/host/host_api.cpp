@@ -157,13 +157,16 @@ SLH_API int slh_sgd_step(void* dev, uint64_t p, float lr) {
 // Three-layer MLP d_in -> d_h -> relu -> d_h -> relu -> d_out on a fresh device object.
 // kind 0 = sine fit (MSE on the tape), 1 = classifier (softmax + cce).  W1..b3 are updated in
 // place.  `warmup` untimed steps run first (they train too); seconds = wall time of `steps`.
+// mode: bit 0 = fused Linear forward, bit 1 = record one step as a graph and replay it.
 SLH_API int slh_mlp_train(int ordinal, int kind, size_t batch, size_t d_in, size_t d_h, size_t d_out, const float* x,
                           const float* target, float* W1, float* b1, float* W2, float* b2, float* W3, float* b3,
-                          float lr, size_t steps, size_t warmup, int fused, float* losses, double* seconds) {
+                          float lr, size_t steps, size_t warmup, int mode, float* losses, double* seconds,
+                          size_t* graph_nodes) {
   return guard([&] {
     HIP dev(ordinal, true);
     float* params[6] = {W1, b1, W2, b2, W3, b3};
-    MlpResult r = mlp_train(dev, kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmup, losses, fused != 0);
+    MlpResult r = mlp_train(dev, kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmup, losses, mode);
     if (seconds) *seconds = r.seconds;
+    if (graph_nodes) *graph_nodes = r.graph_nodes;
   });
 }

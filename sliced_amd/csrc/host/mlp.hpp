@@ -43,14 +43,24 @@ struct SGD {
 
 struct MlpResult {
   double seconds = 0.0;  // wall time of the timed steps, device idle on both sides
+  size_t graph_nodes = 0;  // kernels per recorded step (MLP_GRAPH only)
+};
+
+enum MlpMode {
+  MLP_FUSED = 1,  // Linear (+ReLU) forward as one kernel
+  MLP_GRAPH = 2   // step 0 runs eagerly, step 1 is recorded, every later step replays the recording
 };
 
 // kind 0: MSE on the tape (sub, square, sum_cols, mul by 1/n; seed 1).
 // kind 1: softmax on the tape, cce / cce_grad off the tape, backward_with.
 // `params` are six host arrays W1,b1,W2,b2,W3,b3 and receive the trained values back.
+// Without MLP_GRAPH the host reads the loss back every step, as the examples do; with it the
+// losses collect in a device array and are read once at the end (the lazy example reads
+// `loss.replace()` after `dev.run()`, examples/sine_net.rs:209-212).
 inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t d_h, size_t d_out, const float* x_host,
                            const float* target_host, float* const params[6], float lr, size_t steps, size_t warmup,
-                           float* losses, bool fused) {
+                           float* losses, int mode) {
+  const bool fused = (mode & MLP_FUSED) != 0, graph = (mode & MLP_GRAPH) != 0;
   Linear lin1(dev, d_in, d_h, params[0], params[1]);
   Linear lin2(dev, d_h, d_h, params[2], params[3]);
   Linear lin3(dev, d_h, d_out, params[4], params[5]);
@@ -66,16 +76,11 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
   // loss pieces of kind 1 live outside the cache: they are not tape outputs
   Buffer loss_rows = kind == 1 ? dev.alloc(batch, true) : Buffer();
   Buffer seed = kind == 1 ? dev.alloc(n_out, true) : Buffer();
+  Buffer loss_dev = dev.alloc(1, true);
+  Buffer loss_log = graph ? dev.alloc(warmup + steps, true) : Buffer();
 
-  MlpResult res;
-  std::chrono::steady_clock::time_point t0;
-  size_t it = 0;
-  for (size_t step : dev.range(warmup + steps)) {
-    (void)step;
-    if (it == warmup) {
-      dev.sync();
-      t0 = std::chrono::steady_clock::now();
-    }
+  // One training step.  Leaves the loss in loss_dev; reads it back unless `deferred`.
+  auto train_step = [&](bool deferred) -> float {
     dev.zero_grad();
     Matrix out;
     if (fused) {
@@ -87,29 +92,59 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
       Matrix h2 = lin2.forward(h1).relu();
       out = lin3.forward(h2);
     }
-    float loss_val;
+    float loss_val = 0.0f;
     if (kind == 0) {
       Matrix d = out.sub(y);
       Matrix q = d.squared();
       Matrix s = q.as_dims(1, n_out).sum_cols();  // one row: the sum over every element
       Matrix L = s.mul(c);
-      loss_val = L.read()[0];
+      if (deferred) dev.copy(L.data, 0, loss_dev, 0, 1);
+      else loss_val = L.read()[0];
       L.backward();
     } else {
       Matrix p = out.softmax();
       check(slhip_cce(dev.ctx(), batch, d_out, p.data.ptr, y.data.ptr, loss_rows.ptr), "slhip_cce");
-      loss_val = dev.mean(loss_rows);
+      if (deferred) dev.mean_to(loss_rows, loss_dev);
+      else loss_val = dev.mean(loss_rows);
       check(slhip_cce_grad(dev.ctx(), batch, d_out, p.data.ptr, y.data.ptr, seed.ptr), "slhip_cce_grad");
       p.data.backward_with(seed);
     }
     sgd.step(dev, lin1);
     sgd.step(dev, lin2);
     sgd.step(dev, lin3);
-    if (it >= warmup) losses[it - warmup] = loss_val;
-    ++it;
+    return loss_val;
+  };
+
+  MlpResult res;
+  Graph recorded;
+  std::chrono::steady_clock::time_point t0;
+  for (size_t it : dev.range(warmup + steps)) {
+    if (it == warmup) {
+      dev.sync();
+      t0 = std::chrono::steady_clock::now();
+    }
+    if (!graph) {
+      const float loss_val = train_step(false);
+      if (it >= warmup) losses[it - warmup] = loss_val;
+      continue;
+    }
+    if (it == 0) {
+      train_step(true);  // eagerly: fills the cache and the gradient map
+    } else {
+      if (!recorded.valid()) {
+        recorded = dev.record([&] { train_step(true); });
+        res.graph_nodes = recorded.nodes();
+      }
+      recorded.run();
+    }
+    dev.copy(loss_dev, 0, loss_log, it, 1);
   }
   dev.sync();
   res.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  if (graph) {
+    std::vector<float> log = loss_log.read();
+    for (size_t i = 0; i < steps; ++i) losses[i] = log[warmup + i];
+  }
   // warm-up steps train too: hand back what the timed steps ended with
   const Linear* ls[3] = {&lin1, &lin2, &lin3};
   for (int i = 0; i < 3; ++i) {

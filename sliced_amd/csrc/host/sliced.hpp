@@ -45,6 +45,32 @@ inline void check(int32_t rc, const char* what) {
 
 class HIP;
 
+// A recorded op sequence (see HIP::record): run() replays it as one launch.
+class Graph {
+ public:
+  Graph() = default;
+  Graph(slhip_ctx* ctx, slhip_graph* g) : ctx_(ctx), g_(g) {}
+  Graph(Graph&& o) noexcept : ctx_(o.ctx_), g_(o.g_) { o.g_ = nullptr; }
+  Graph& operator=(Graph&& o) noexcept {
+    if (this != &o) { slhip_graph_destroy(g_); ctx_ = o.ctx_; g_ = o.g_; o.g_ = nullptr; }
+    return *this;
+  }
+  Graph(const Graph&) = delete;
+  Graph& operator=(const Graph&) = delete;
+  ~Graph() { slhip_graph_destroy(g_); }
+  bool valid() const { return g_ != nullptr; }
+  void run() const { check(slhip_graph_launch(ctx_, g_), "slhip_graph_launch"); }
+  size_t nodes() const {
+    size_t n = 0;
+    check(slhip_graph_node_count(g_, &n), "slhip_graph_node_count");
+    return n;
+  }
+
+ private:
+  slhip_ctx* ctx_ = nullptr;
+  slhip_graph* g_ = nullptr;
+};
+
 struct Buffer {
   HIP* dev = nullptr;
   uint64_t id = 0;
@@ -157,6 +183,28 @@ class HIP {
     It end() { return {dev, n}; }
   };
   Range range(size_t n) { return Range{this, n}; }
+
+  // Record once, replay many — the reference's lazy device (`Autograd<Lazy<Base>>`, `dev.run()`,
+  // examples/sine_net.rs:178-220) as a HIP graph.  body() issues ops as usual (forward, backward,
+  // optimiser step); none of them runs, all of them land in the returned Graph.  body() must not
+  // allocate or read back: run the same sequence eagerly once before, so that the cache and the
+  // gradient map already hold every buffer it names, and keep those buffers alive while the
+  // Graph is in use.
+  template <class F>
+  Graph record(F&& body) {
+    check(slhip_graph_begin(ctx_), "slhip_graph_begin");
+    slhip_graph* g = nullptr;
+    try {
+      body();
+    } catch (...) {
+      slhip_graph_end(ctx_, &g);
+      slhip_graph_destroy(g);
+      tape_.clear();
+      throw;
+    }
+    check(slhip_graph_end(ctx_, &g), "slhip_graph_end");
+    return Graph(ctx_, g);
+  }
 
   // ---- autograd --------------------------------------------------------------------------
   void add_grad_fn(std::function<void()> f) { if (tape_enabled_) tape_.push_back(std::move(f)); }
@@ -362,6 +410,16 @@ class HIP {
     float v;
     check(slhip_memcpy_d2h(ctx_, &v, s.ptr, sizeof(float)), "slhip_memcpy_d2h");
     return v;
+  }
+
+  // The same reduction left on the device (for recorded sequences, which cannot read back)
+  void mean_to(const Buffer& x, const Buffer& out) {
+    expect(out, 1, "mean_to out");
+    check(slhip_mean(ctx_, x.len, x.ptr, out.ptr), "slhip_mean");
+  }
+  void copy(const Buffer& src, size_t src_off, const Buffer& dst, size_t dst_off, size_t n) {
+    if (src_off + n > src.len || dst_off + n > dst.len) throw Error("copy: range outside the buffer");
+    check(slhip_memcpy_d2d(ctx_, dst.ptr + dst_off, src.ptr + src_off, n * sizeof(float)), "slhip_memcpy_d2d");
   }
 
   // SGD of the examples (examples/sine_net.rs:105-116): value -= grad * lr, on the device

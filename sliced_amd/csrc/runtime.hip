@@ -33,6 +33,14 @@ __global__ __launch_bounds__(64) void copy4_kernel(size_t n4, const float* __res
   if (i < n4) st4s(dst + 4 * i, ld4s(src + 4 * i));
 }
 
+// Whatever the vector copy cannot take (tails, small or unaligned copies), as words or bytes.
+template <class T>
+__global__ void copy_kernel(size_t n, const T* __restrict__ src, T* __restrict__ dst) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) dst[i] = src[i];
+}
+
 __device__ __forceinline__ uint64_t splitmix64(uint64_t s) {
   uint64_t z = s + 0x9E3779B97F4A7C15ull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -115,6 +123,12 @@ SLHIP_API int32_t slhip_init_on_stream(int32_t ordinal, void* stream, slhip_ctx*
 SLHIP_API int32_t slhip_destroy(slhip_ctx* ctx) {
   if (!ctx) return SLHIP_OK;
   (void)hipSetDevice(ctx->device);
+  if (ctx->capturing) {  // abandon an unfinished recording so that the stream can be waited on
+    hipGraph_t g = nullptr;
+    (void)hipStreamEndCapture(ctx->stream, &g);
+    if (g) (void)hipGraphDestroy(g);
+    (void)hipGetLastError();
+  }
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->workspace) (void)hipFree(ctx->workspace);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
@@ -139,6 +153,7 @@ SLHIP_API size_t slhip_workspace_bytes(slhip_ctx* ctx) { return ctx ? ctx->works
 SLHIP_API int32_t slhip_malloc(slhip_ctx* ctx, size_t bytes, void** dptr) {
   SLHIP_REQUIRE(ctx && dptr, "null argument");
   SLHIP_REQUIRE(bytes > 0, "zero-byte allocation");
+  SLHIP_NOT_CAPTURING(ctx);
   *dptr = nullptr;
   SLHIP_CHECK_HIP(hipMalloc(dptr, bytes));
   return SLHIP_OK;
@@ -147,6 +162,7 @@ SLHIP_API int32_t slhip_malloc(slhip_ctx* ctx, size_t bytes, void** dptr) {
 SLHIP_API int32_t slhip_free(slhip_ctx* ctx, void* dptr) {
   SLHIP_REQUIRE(ctx, "null context");
   if (!dptr) return SLHIP_OK;
+  SLHIP_NOT_CAPTURING(ctx);
   SLHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
   SLHIP_CHECK_HIP(hipFree(dptr));
   return SLHIP_OK;
@@ -155,6 +171,7 @@ SLHIP_API int32_t slhip_free(slhip_ctx* ctx, void* dptr) {
 SLHIP_API int32_t slhip_memcpy_h2d(slhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
   SLHIP_REQUIRE(ctx && dst && src, "null argument");
   if (bytes == 0) return SLHIP_OK;
+  SLHIP_NOT_CAPTURING(ctx);
   SLHIP_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
   // pageable host memory: the source may be reused by the caller as soon as we return
   SLHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
@@ -164,28 +181,40 @@ SLHIP_API int32_t slhip_memcpy_h2d(slhip_ctx* ctx, void* dst, const void* src, s
 SLHIP_API int32_t slhip_memcpy_d2h(slhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
   SLHIP_REQUIRE(ctx && dst && src, "null argument");
   if (bytes == 0) return SLHIP_OK;
+  SLHIP_NOT_CAPTURING(ctx);
   SLHIP_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
   SLHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
   return SLHIP_OK;
 }
 
+// Device-to-device copies are kernels, never runtime copies: faster for large buffers, and a
+// recording (slhip_graph_begin) then holds kernel nodes only.
 SLHIP_API int32_t slhip_memcpy_d2d(slhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
   SLHIP_REQUIRE(ctx && dst && src, "null argument");
   if (bytes == 0 || dst == src) return SLHIP_OK;
-  const size_t n4 = bytes / 16;
-  if (bytes >= (size_t(1) << 20) && aligned16(dst) && aligned16(src) && (n4 + 63) / 64 <= 0x7fffffffu) {
+  size_t done = 0;
+  if (bytes >= 4096 && aligned16(dst) && aligned16(src)) {
+    const size_t n4 = bytes / 16;
+    SLHIP_REQUIRE((n4 + 63) / 64 <= 0x7fffffffu, "copy too large for one launch");
     hipLaunchKernelGGL(copy4_kernel, dim3((unsigned)((n4 + 63) / 64)), dim3(64), 0, ctx->stream, n4,
                        (const float*)src, (float*)dst);
     int32_t rc = post_launch();
     if (rc) return rc;
-    const size_t done = n4 * 16;
+    done = n4 * 16;
     if (done == bytes) return SLHIP_OK;
-    SLHIP_CHECK_HIP(hipMemcpyAsync((char*)dst + done, (const char*)src + done, bytes - done,
-                                   hipMemcpyDeviceToDevice, ctx->stream));
-    return SLHIP_OK;
   }
-  SLHIP_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
-  return SLHIP_OK;
+  const char* s = (const char*)src + done;
+  char* d = (char*)dst + done;
+  const size_t rest = bytes - done;
+  if ((rest & 3) == 0 && (((uintptr_t)s | (uintptr_t)d) & 3) == 0) {
+    const size_t n = rest / 4;
+    unsigned grid = (unsigned)(n / 256 + 1 < 8192 ? n / 256 + 1 : 8192);
+    hipLaunchKernelGGL(copy_kernel<uint32_t>, dim3(grid), dim3(256), 0, ctx->stream, n, (const uint32_t*)s, (uint32_t*)d);
+  } else {
+    unsigned grid = (unsigned)(rest / 256 + 1 < 8192 ? rest / 256 + 1 : 8192);
+    hipLaunchKernelGGL(copy_kernel<uint8_t>, dim3(grid), dim3(256), 0, ctx->stream, rest, (const uint8_t*)s, (uint8_t*)d);
+  }
+  return post_launch();
 }
 
 SLHIP_API int32_t slhip_memset(slhip_ctx* ctx, void* dptr, int32_t value, size_t bytes) {
@@ -198,6 +227,7 @@ SLHIP_API int32_t slhip_memset(slhip_ctx* ctx, void* dptr, int32_t value, size_t
     hipLaunchKernelGGL(fill_kernel, dim3(grid), dim3(256), 0, ctx->stream, n, 0.0f, (float*)dptr);
     return post_launch();
   }
+  SLHIP_NOT_CAPTURING(ctx);  // a memset node: kept out of recordings
   SLHIP_CHECK_HIP(hipMemsetAsync(dptr, value, bytes, ctx->stream));
   return SLHIP_OK;
 }
@@ -212,6 +242,7 @@ SLHIP_API int32_t slhip_fill(slhip_ctx* ctx, size_t n, float value, float* x) {
 
 SLHIP_API int32_t slhip_sync(slhip_ctx* ctx) {
   SLHIP_REQUIRE(ctx, "null context");
+  SLHIP_NOT_CAPTURING(ctx);
   SLHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
   return SLHIP_OK;
 }
@@ -230,6 +261,7 @@ SLHIP_API int32_t slhip_event_create(slhip_ctx* ctx, slhip_event** ev) {
 
 SLHIP_API int32_t slhip_event_record(slhip_ctx* ctx, slhip_event* ev) {
   SLHIP_REQUIRE(ctx && ev, "null argument");
+  SLHIP_NOT_CAPTURING(ctx);
   SLHIP_CHECK_HIP(hipEventRecord(ev->ev, ctx->stream));
   return SLHIP_OK;
 }
@@ -245,6 +277,64 @@ SLHIP_API int32_t slhip_event_destroy(slhip_event* ev) {
   if (!ev) return SLHIP_OK;
   (void)hipEventDestroy(ev->ev);
   delete ev;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_graph_begin(slhip_ctx* ctx) {
+  SLHIP_REQUIRE(ctx, "null context");
+  SLHIP_NOT_CAPTURING(ctx);
+  // relaxed mode: other threads of the process (a framework's allocator, say) stay unrestricted;
+  // this library refuses its own waiting and allocating calls while `capturing` is set
+  SLHIP_CHECK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+  ctx->capturing = true;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_graph_end(slhip_ctx* ctx, slhip_graph** graph) {
+  SLHIP_REQUIRE(ctx && graph, "null argument");
+  *graph = nullptr;
+  if (!ctx->capturing) {
+    set_error("slhip_graph_end: the context is not recording");
+    return SLHIP_ECAPTURE;
+  }
+  ctx->capturing = false;
+  hipGraph_t g = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+  if (e != hipSuccess || !g) {
+    if (g) (void)hipGraphDestroy(g);
+    return hip_fail(e != hipSuccess ? e : hipErrorUnknown, "hipStreamEndCapture");
+  }
+  slhip_graph* out = new slhip_graph();
+  out->graph = g;
+  e = hipGraphGetNodes(g, nullptr, &out->nodes);
+  if (e == hipSuccess) e = hipGraphInstantiate(&out->exec, g, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(g);
+    delete out;
+    return hip_fail(e, "hipGraphInstantiate");
+  }
+  *graph = out;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_graph_launch(slhip_ctx* ctx, slhip_graph* graph) {
+  SLHIP_REQUIRE(ctx && graph && graph->exec, "null argument");
+  SLHIP_NOT_CAPTURING(ctx);
+  SLHIP_CHECK_HIP(hipGraphLaunch(graph->exec, ctx->stream));
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_graph_node_count(slhip_graph* graph, size_t* nodes) {
+  SLHIP_REQUIRE(graph && nodes, "null argument");
+  *nodes = graph->nodes;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_graph_destroy(slhip_graph* graph) {
+  if (!graph) return SLHIP_OK;
+  if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+  if (graph->graph) (void)hipGraphDestroy(graph->graph);
+  delete graph;
   return SLHIP_OK;
 }
 

@@ -10,6 +10,7 @@ Bars (stated per test):
     the oracle with the oracle's own distance to the f64 evaluation added;
   * GEMM: |gpu - exact| <= 1e-5 * sqrt(K) * (|A|·|B|) elementwise.
 """
+import ctypes as C
 import sys
 
 import numpy as np
@@ -118,9 +119,9 @@ def test_gemm_grad_matches_oracle(hip, orc):
         assert np.all(np.abs(lg_h - lg_o) <= tol_l)
         assert np.all(np.abs(rg_h - rg_o) <= tol_r)
         # a NULL grad (operand without requires_grad) is skipped, the other side still written
-        rg2 = np.zeros(k * n, np.float32)
-        hip.gemm_grad(m, k, n, lhs, rhs, None, rg2, g)
-        assert np.array_equal(rg2, rg_h)
+        rg = np.zeros(k * n, np.float32)
+        hip.gemm_grad(m, k, n, lhs, rhs, None, rg, g)
+        assert np.array_equal(rg, rg_h)
 
 
 def test_linear_fwd_fused_equals_gemm_bias_relu(hip, orc):
@@ -396,3 +397,71 @@ def test_invalid_arguments_return_status_not_crash(hip):
     assert lib.slhip_transpose(c.h, 4, 4, x.ptr, x.ptr, 0.0) == -4
     assert lib.slhip_ew_unary(c.h, 99, 0.0, 0.0, 4, x.ptr, x.ptr) == -1
     x.free()
+
+
+# --------------------------------------------------------------------------- recorded sequences
+def test_recorded_sequence_replays_like_eager_calls(hip, orc):
+    """Record gemm (split-K) -> bias row op -> relu -> softmax -> column sums -> scaled copy once,
+    replay it several times with eager work and waits in between, and compare every replay bit for
+    bit with the same calls made eagerly on the same inputs."""
+    c = hip.ctx()
+    lib = c.lib
+    m, k, n = 96, 1024, 40
+    a0 = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
+    w = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
+    bias = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+    da, dw, db = c.array(a0), c.array(w), c.array(bias)
+    y, s, col, keep = c.empty(m * n), c.empty(m * n), c.zeros(n), c.zeros(n)
+
+    def sequence():
+        c.call("slhip_gemm", m, k, n, da.ptr, dw.ptr, y.ptr)
+        c.call("slhip_add_row", m, n, y.ptr, db.ptr, y.ptr)
+        c.call("slhip_ew_unary", 2, 0.0, 0.0, m * n, y.ptr, y.ptr)
+        c.call("slhip_softmax", m, n, y.ptr, s.ptr)
+        c.call("slhip_memset", col.ptr, 0, col.nbytes)
+        c.call("slhip_sum_rows", m, n, s.ptr, col.ptr)
+        c.call("slhip_memcpy_d2d", keep.ptr, col.ptr, col.nbytes)
+        # the input moves on, so that every replay computes something new
+        c.call("slhip_ew_unary", 6, 0.5, 0.0, m * k, da.ptr, da.ptr)
+
+    eager = []
+    for _ in range(4):
+        sequence()
+        eager.append((keep.numpy(), s.numpy()))
+    da.upload(a0)
+
+    c.call("slhip_graph_begin")
+    # waiting or allocating calls are refused while recording, and leave the recording intact
+    p = C.c_void_p()
+    assert lib.slhip_malloc(c.h, 64, C.byref(p)) == -5
+    assert lib.slhip_sync(c.h) == -5
+    assert lib.slhip_memset(c.h, col.ptr, 1, 4) == -5
+    assert lib.slhip_graph_begin(c.h) == -5
+    sequence()
+    g = C.c_void_p()
+    c.call("slhip_graph_end", C.byref(g))
+    nodes = C.c_size_t()
+    assert lib.slhip_graph_node_count(g, C.byref(nodes)) == 0
+    say("recorded nodes:", nodes.value)
+    assert nodes.value >= 8
+    # nothing ran while recording
+    assert np.array_equal(da.numpy(), a0)
+    none = C.c_void_p()
+    assert lib.slhip_graph_end(c.h, C.byref(none)) == -5    # not recording any more
+
+    scratch = c.empty(1 << 16)
+    for i in range(4):
+        c.call("slhip_graph_launch", g)
+        # eager work on other buffers and a wait between the replays
+        c.call("slhip_fill", scratch.n, float(i), scratch.ptr)
+        c.sync()
+        got_keep, got_s = keep.numpy(), s.numpy()
+        assert np.array_equal(got_keep, eager[i][0]), i
+        assert np.array_equal(got_s, eager[i][1]), i
+        assert float(scratch.numpy()[-1]) == float(i)
+    # against the oracle as well (first replay's inputs)
+    ref = orc.softmax(m, n, orc.unary(orc.RELU, orc.add_row(m, n, orc.gemm(m, n, k, a0, w), bias)))
+    assert np.max(np.abs(eager[0][1] - ref)) <= 1e-5
+    assert lib.slhip_graph_destroy(g) == 0
+    for z in (da, dw, db, y, s, col, keep, scratch):
+        z.free()

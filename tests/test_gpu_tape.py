@@ -276,3 +276,31 @@ def test_classifier_mlp_loss_curve_matches_oracle(orc, fused):
     say("C5 worst relative loss deviation", worst, "loss", ref[0], "->", ref[-1])
     assert np.all(np.isfinite(got))
     assert worst <= 1e-4
+
+
+@pytest.mark.parametrize("name,steps", [("C1", 200), ("C5", 12)])
+def test_recorded_step_replays_match_the_eager_loop(orc, name, steps):
+    """One training step recorded as a graph and replayed: the loss curve and the trained
+    parameters are bit-identical to the eager loop (same kernels in the same order), which the
+    tests above hold to the oracle; C1 is compared with the oracle here as well."""
+    from sliced_amd import host
+    cfg = host.C1 if name == "C1" else host.C5
+    say(name, "recorded step,", steps, "steps")
+    x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+    p0 = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+    args = (cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t)
+    p_eager = [a.copy() for a in p0]
+    eager, _ = host.mlp_train(*args, p_eager, cfg["lr"], steps, 0, True)
+    for warmup in (0, 3):     # the recording happens inside / before the timed steps
+        p_graph = [a.copy() for a in p0]
+        info = {}
+        got, _ = host.mlp_train(*args, p_graph, cfg["lr"], steps - warmup, warmup, True, graph=True, info=info)
+        say(name, "kernels per recorded step:", info["graph_nodes"])
+        assert info["graph_nodes"] > 10
+        assert np.array_equal(got, eager[warmup:])
+        for a, b in zip(p_graph, p_eager):
+            assert np.array_equal(a, b)
+    if name == "C1":
+        p_ref = [a.copy() for a in p0]
+        ref = orc.mlp_train(*args, p_ref, cfg["lr"], steps)
+        assert loss_parity(eager, ref, 1e-4) <= 1e-4
