@@ -223,6 +223,11 @@ int32_t slhip_ew_chain(slhip_ctx* ctx, size_t n, const float* a, const float* b,
  *   cce_grad : grad = (−(t/p))/rows                  (examples/nn.rs:140-152)
  *   onehot   : out[r·classes + (size_t)cls[r]] = 1, rest 0 (src/ops2/onehot/cpu.rs:40-44) */
 int32_t slhip_sgd_step(slhip_ctx* ctx, size_t n, float* p, const float* g, float lr);
+/* The same update for `count` parameter tensors in one launch per 8 tensors (the examples call
+ * the step once per layer, examples/sine_net.rs:157-159).  params, grads and lens are HOST
+ * arrays of `count` device pointers / lengths. */
+int32_t slhip_sgd_step_multi(slhip_ctx* ctx, size_t count, float* const* params, const float* const* grads,
+                             const size_t* lens, float lr);
 int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets, float* loss);
 int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
                        float* grad);

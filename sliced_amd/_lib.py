@@ -72,6 +72,7 @@ PROTOTYPES = {
     "slhip_ew_unary_grad": [c_vp, c_i32, C.c_float, c_sz, c_vp, c_vp, c_vp],
     "slhip_ew_chain": [c_vp, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
     "slhip_sgd_step": [c_vp, c_sz, c_vp, c_vp, C.c_float],
+    "slhip_sgd_step_multi": [c_vp, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_onehot": [c_vp, c_sz, c_sz, c_vp, c_vp],

@@ -371,6 +371,59 @@ SLHIP_API int32_t slhip_sgd_step(slhip_ctx* ctx, size_t n, float* p, const float
   return ew_launch(ctx, n, a);
 }
 
+// Up to SGD_MULTI_MAX parameter tensors per launch; blockIdx.y picks the tensor.
+constexpr int SGD_MULTI_MAX = 8;
+struct SgdMultiArgs {
+  float* p[SGD_MULTI_MAX];
+  const float* g[SGD_MULTI_MAX];
+  size_t n[SGD_MULTI_MAX];
+  int vec[SGD_MULTI_MAX];
+};
+
+__global__ __launch_bounds__(256) void sgd_multi_kernel(SgdMultiArgs a, float lr) {
+  const int t = blockIdx.y;
+  float* __restrict__ p = a.p[t];
+  const float* __restrict__ g = a.g[t];
+  const size_t n = a.n[t];
+  const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
+  size_t done = 0;
+  if (a.vec[t]) {
+    const size_t n4 = n / 4;
+    for (size_t i = tid; i < n4; i += stride) {
+      float4 pv = ld4(p + 4 * i);
+      const float4 gv = ld4(g + 4 * i);
+      pv.x -= gv.x * lr; pv.y -= gv.y * lr; pv.z -= gv.z * lr; pv.w -= gv.w * lr;
+      st4(p + 4 * i, pv);
+    }
+    done = n4 * 4;
+  }
+  for (size_t i = done + tid; i < n; i += stride) p[i] -= g[i] * lr;
+}
+
+SLHIP_API int32_t slhip_sgd_step_multi(slhip_ctx* ctx, size_t count, float* const* params, const float* const* grads,
+                                       const size_t* lens, float lr) {
+  SLHIP_REQUIRE(ctx && params && grads && lens, "null argument");
+  SLHIP_REQUIRE(count > 0, "no tensors");
+  for (size_t i = 0; i < count; ++i) SLHIP_REQUIRE(params[i] && grads[i] && lens[i] > 0, "null or empty tensor");
+  for (size_t first = 0; first < count; first += SGD_MULTI_MAX) {
+    const size_t m = count - first < (size_t)SGD_MULTI_MAX ? count - first : (size_t)SGD_MULTI_MAX;
+    SgdMultiArgs a;
+    size_t longest = 0;
+    for (size_t i = 0; i < (size_t)SGD_MULTI_MAX; ++i) {
+      const size_t j = first + (i < m ? i : 0);  // unused slots repeat the first tensor; no block reads them
+      a.p[i] = params[j]; a.g[i] = grads[j]; a.n[i] = lens[j];
+      a.vec[i] = aligned16(params[j]) && aligned16(grads[j]);
+      if (i < m && lens[j] > longest) longest = lens[j];
+    }
+    size_t blocks = (longest / 4 + 255) / 256 + 1;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)blocks, (unsigned)m), dim3(256), 0, ctx->stream, a, lr);
+    int32_t rc = post_launch();
+    if (rc) return rc;
+  }
+  return SLHIP_OK;
+}
+
 SLHIP_API int32_t slhip_add_row(slhip_ctx* ctx, size_t rows, size_t cols, const float* lhs, const float* rhs,
                                 float* out) {
   size_t len;

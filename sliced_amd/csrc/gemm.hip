@@ -13,6 +13,8 @@
 // prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.  Tiles are numbered so that each XCD (its
 // own L2) works along one tile row at a time.  Small grids are split along K; the partial
 // products go to the context workspace and are combined in a fixed order.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace slhip {
@@ -51,8 +53,18 @@ struct Frag {
   float4 v[Cfg<BK>::NV];
 };
 
+// How a k tile is fetched from global memory.
+//   LOAD_FAST   the whole tile is inside the operand and 16-byte loadable: unconditional float4
+//   LOAD_VCLAMP the k range is complete and the operand is 16-byte loadable, but the tile hangs
+//               over the operand's edge in x: float4 loads from clamped rows, zeroed afterwards
+//   LOAD_SCALAR anything else: one load per element from clamped coordinates, zeroed afterwards
+// No variant branches around a load, so all loads of a tile are in flight together (a version
+// with one branch per element took about 15 us per k tile on tiny problems: each load waited for
+// the one before it).
+enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2 };
+
 // k-contiguous source: element (x, k) at src[x*ld + k]; tile 128 x BK.
-template <int BK, bool FAST>
+template <int BK, int MODE>
 __device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
   constexpr int VPR = BK / 4, RPP = 256 / VPR;  // float4 per row, rows per pass
@@ -60,12 +72,22 @@ __device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ s
 #pragma unroll
   for (int p = 0; p < Cfg<BK>::NV; ++p) {
     const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
-    if (FAST) {
+    if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + x * ld + k);
+    } else if (MODE == LOAD_VCLAMP) {
+      const bool in = x < X;
+      const float4 t = ld4(src + (in ? x : X - 1) * ld + k);
+      f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
+      const bool xin = x < X;
+      const float* row = src + (xin ? x : X - 1) * ld;
       float t[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) t[q] = (x < X && k + q < Kend) ? src[x * ld + k + q] : 0.0f;
+      for (int q = 0; q < 4; ++q) {
+        const bool in = xin && k + q < Kend;
+        const float val = row[k + q < Kend ? k + q : Kend - 1];
+        t[q] = in ? val : 0.0f;
+      }
       f.v[p] = make_float4(t[0], t[1], t[2], t[3]);
     }
   }
@@ -78,20 +100,31 @@ __device__ __forceinline__ void store_kc(const Frag<BK>& f, float* lds) {
   for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK>::KC_PITCH + 4 * kq, f.v[p]);
 }
 
-// x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x 128.
-template <int BK, bool FAST>
+// x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x 128.  LOAD_VCLAMP relies on
+// X % 4 == 0 (implied by ld % 4 == 0, ld being X here): a float4 is inside or outside as a whole.
+template <int BK, int MODE>
 __device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
   const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;  // 32 float4 per k-row, 8 rows per pass
 #pragma unroll
   for (int p = 0; p < Cfg<BK>::NV; ++p) {
     const size_t k = k0 + kr + 8 * p, x = x0 + 4 * xq;
-    if (FAST) {
+    if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + k * ld + x);
+    } else if (MODE == LOAD_VCLAMP) {
+      const bool in = x < X;
+      const float4 t = ld4(src + k * ld + (in ? x : X - 4));
+      f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
+      const bool kin = k < Kend;
+      const float* row = src + (kin ? k : Kend - 1) * ld;
       float t[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) t[q] = (k < Kend && x + q < X) ? src[k * ld + x + q] : 0.0f;
+      for (int q = 0; q < 4; ++q) {
+        const bool in = kin && x + q < X;
+        const float val = row[x + q < X ? x + q : X - 1];
+        t[q] = in ? val : 0.0f;
+      }
       f.v[p] = make_float4(t[0], t[1], t[2], t[3]);
     }
   }
@@ -137,12 +170,11 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = local / gsize;
 }
 
-// The k loop over tiles [kt_begin, kt_end) of one workgroup.  FAST = every tile in the range is
-// complete and 16-byte loadable, so the global loads are unconditional float4 loads; otherwise
-// every element is bounds-checked and zero-filled.  The two variants are separate loops on
-// purpose: when both kinds of load sat behind a branch in ONE loop body the compiler folded them
-// into the per-element form, which cost 19 % of the kernel's throughput.
-template <bool TA, bool TB, int BK, bool FAST>
+// The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
+// modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
+// ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
+// kernel's throughput.
+template <bool TA, bool TB, int BK, int MODE>
 __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
                                            size_t m0, size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
                                            float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
@@ -159,10 +191,10 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   Frag<BK> fa, fb;
   auto load_stage = [&](int kt) {
     const size_t k0 = kbeg + (size_t)kt * BK;
-    if (TA) load_xc<BK, FAST>(fa, g.A, lda, g.M, kend, m0, k0);
-    else load_kc<BK, FAST>(fa, g.A, lda, g.M, kend, m0, k0);
-    if (TB) load_kc<BK, FAST>(fb, g.B, ldb, g.N, kend, n0, k0);
-    else load_xc<BK, FAST>(fb, g.B, ldb, g.N, kend, n0, k0);
+    if (TA) load_xc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
+    else load_kc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
+    if (TB) load_kc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
+    else load_xc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
   };
   auto store_stage = [&](int s) {
     if (TA) store_xc<BK>(fa, lds_a[s]); else store_kc<BK>(fa, lds_a[s]);
@@ -241,12 +273,14 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // interior workgroups run their complete k tiles through the vector-load loop; edge tiles,
-  // unaligned operands and the k remainder go through the checked loop
-  const bool fast = g.a_vec && g.b_vec && m0 + BM <= g.M && n0 + BN <= g.N;
-  const int nfast = fast ? kfull : 0;
-  gemm_tiles<TA, TB, BK, true>(g, 0, nfast, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, false>(g, nfast, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  // complete k tiles of 16-byte loadable operands go through a vector-load loop (interior
+  // workgroups the unclamped one); unaligned operands and the k remainder through the scalar one
+  const bool vec = g.a_vec && g.b_vec;
+  const bool inside = m0 + BM <= g.M && n0 + BN <= g.N;
+  const int nvec = vec ? kfull : 0;
+  if (inside) gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  else gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, nvec, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
@@ -274,6 +308,95 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
         dst[idx] = val;
       }
     }
+}
+
+// Small and skinny problems.  One wave owns one 32x32 tile of C and feeds the matrix core straight
+// from global memory: per group of 8 k it loads 4 + 4 scalars per lane (the k permutation of the
+// header comment makes them 4 MFMA operand pairs) and issues 4 MFMAs; up to 16 waves of a
+// workgroup split the k range of one tile and combine their accumulators through LDS in wave
+// order, so the result does not depend on timing.  Next to the tiled kernel it wastes matrix-core
+// cycles on narrow tiles and reads operands uncoalesced, but its code is a few hundred bytes:
+// the tiled kernel spends about 13 us per launch before its first MFMA retires (fetching
+// its long unrolled code cold), which is most of the time of a [1024 x 64] x [64 x 64] product.
+template <bool TA, bool TB>
+__global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
+  extern __shared__ float red[];  // [waves][16][64]
+  const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const size_t tm = blockIdx.x / g.tiles_n, tn = blockIdx.x % g.tiles_n;
+  const size_t m0 = tm * 32, n0 = tn * 32;
+  const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
+  const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
+  const size_t groups = (kend - kbeg + 7) / 8, per = (groups + nw - 1) / nw;
+  const size_t gbeg = wk * per, gend = gbeg + per < groups ? gbeg + per : groups;
+  // rows / columns past the edge are clamped: they compute copies that are never stored
+  const size_t row = m0 + r < g.M ? m0 + r : g.M - 1, col = n0 + r < g.N ? n0 + r : g.N - 1;
+  const float* ap = TA ? g.A + row : g.A + row * g.K;
+  const float* bp = TB ? g.B + col * g.K : g.B + col;
+  const size_t astep = TA ? g.M : 1, bstep = TB ? 1 : g.N;
+
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  // NG groups of 8 k at a time: all 8*NG loads are issued before the first MFMA needs one
+  auto run_groups = [&](size_t gi, auto ng_tag) {
+    constexpr int NG = decltype(ng_tag)::value;
+    float a[NG][4], b[NG][4];
+#pragma unroll
+    for (int u = 0; u < NG; ++u) {
+      const size_t k = kbeg + (gi + u) * 8 + 4 * h;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const bool in = k + t < kend;
+        const size_t kc = in ? k + t : kend - 1;
+        const float av = ap[kc * astep], bv = bp[kc * bstep];
+        a[u][t] = in ? av : 0.0f;
+        b[u][t] = in ? bv : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NG; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
+  };
+  size_t gi = gbeg;
+  for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>());
+  for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>());
+
+  if (nw > 1) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[(wk * 16 + v) * 64 + lane] = acc[v];
+    __syncthreads();
+  }
+  // accumulator register v of lane (r, h): row 8*(v/4) + 4*h + v%4, column r; the waves share
+  // the 16 registers out between them
+  const bool raw = g.splits > 1;
+  float* dst = raw ? g.partial + (size_t)blockIdx.y * g.M * g.N : g.C;
+  const size_t c = n0 + r;
+  if (c >= g.N) return;
+  const float bias = (!raw && g.bias) ? g.bias[c] : 0.0f;
+  auto finish = [&](int v, float val) {
+    const size_t rr = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+    if (rr >= g.M) return;
+    const size_t idx = rr * g.N + c;
+    if (!raw) {
+      if (g.beta != 0.0f) val = g.beta * g.C[idx] + val;
+      if (g.bias) val = val + bias;
+      if (g.pre_act) g.pre_act[idx] = val;
+      if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
+    }
+    dst[idx] = val;
+  };
+  if (nw == 1) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) finish(v, acc[v]);
+  } else {
+    for (int v = wk; v < 16; v += nw) {
+      float val = red[v * 64 + lane];
+      for (int w = 1; w < nw; ++w) val += red[(w * 16 + v) * 64 + lane];
+      finish(v, val);
+    }
+  }
 }
 
 // C = sum_z partial[z] (z ascending) + beta*C, then bias / relu.
@@ -318,6 +441,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
   }
 }
 
+static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) {
+  const size_t mn = g.M * g.N;
+  const int vec = (mn % 4 == 0) && (g.N % 4 == 0) && aligned16(g.C) && (!g.bias || aligned16(g.bias)) &&
+                  (!g.pre_act || aligned16(g.pre_act));
+  size_t blocks = ((vec ? mn / 4 : mn) + 255) / 256;
+  const size_t cap = (size_t)ctx->num_cu * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, mn, g.N, (unsigned)splits,
+                     (const float*)ctx->workspace, g.C, g.beta, g.bias, g.relu, g.pre_act, vec);
+  return post_launch();
+}
+
 constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form at 2048^3 and above
 
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
@@ -325,15 +460,59 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   GemmArgs g;
   g.M = M; g.N = N; g.K = K; g.A = A; g.B = B; g.C = C; g.beta = beta;
   g.bias = bias; g.relu = relu; g.pre_act = pre_act;
+  const size_t lda = ta ? M : K, ldb = tb ? K : N;
+  g.a_vec = aligned16(A) && lda % 4 == 0;
+  g.b_vec = aligned16(B) && ldb % 4 == 0;
+  g.partial = (float*)ctx->workspace;
+  const size_t mn_bytes = M * N * sizeof(float);
+
+  // Small (<= 2^25 flop) and skinny (an output side <= 32, or K <= 16) products: wave-per-tile kernel.
+  if (2.0 * (double)M * (double)N * (double)K <= 33554432.0 || M <= 32 || N <= 32 || K <= 16) {
+    const size_t wt_m = (M + 31) / 32, wt_n = (N + 31) / 32;
+    if (wt_m * wt_n > 0x7fffffffu) {
+      set_error("sgemm: %zu x %zu tiles exceed one launch", wt_m, wt_n);
+      return SLHIP_EINVAL;
+    }
+    g.tiles_m = (unsigned)wt_m; g.tiles_n = (unsigned)wt_n;
+    const size_t tiles = wt_m * wt_n, groups = (K + 7) / 8;
+    // waves per workgroup: each keeps >= 4 groups of k (one unrolled batch of loads); then
+    // whole-grid splits of K until the chip has about 8 waves per CU, each split keeping >= 8
+    // groups per wave
+    unsigned nw = 1;
+    while (nw < 16 && groups >= (size_t)nw * 2 * 4) nw *= 2;
+    size_t splits = 1;
+    const size_t want = (size_t)ctx->num_cu * 8;
+    if (tiles * nw < want) {
+      splits = (want + tiles * nw - 1) / (tiles * nw);
+      const size_t most = groups / ((size_t)nw * 8);
+      if (splits > most) splits = most;
+      if (splits > 64) splits = 64;
+      if (splits > ctx->workspace_bytes / mn_bytes) splits = ctx->workspace_bytes / mn_bytes;
+      if (splits < 1) splits = 1;
+    }
+    size_t k_chunk = ((K + splits - 1) / splits + 7) / 8 * 8;
+    splits = (K + k_chunk - 1) / k_chunk;
+    g.splits = (unsigned)splits;
+    g.k_chunk = k_chunk;
+    dim3 wgrid((unsigned)tiles, (unsigned)splits);
+    const size_t lds = nw > 1 ? (size_t)nw * 16 * 64 * sizeof(float) : 0;
+#define SL_WGEMM(TA_, TB_) hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_>), wgrid, dim3(64 * nw), lds, ctx->stream, g)
+    if (!ta && !tb) SL_WGEMM(false, false);
+    else if (!ta && tb) SL_WGEMM(false, true);
+    else if (ta && !tb) SL_WGEMM(true, false);
+    else SL_WGEMM(true, true);
+#undef SL_WGEMM
+    int32_t rc = post_launch();
+    if (rc || splits == 1) return rc;
+    return splitk_combine(ctx, g, splits);
+  }
+
   const size_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   if (tiles_m * tiles_n > 0x7fffffffu) {
     set_error("sgemm: %zu x %zu tiles exceed one launch", tiles_m, tiles_n);
     return SLHIP_EINVAL;
   }
   g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
-  const size_t lda = ta ? M : K, ldb = tb ? K : N;
-  g.a_vec = aligned16(A) && lda % 4 == 0;
-  g.b_vec = aligned16(B) && ldb % 4 == 0;
 
   // Split K when the tile grid alone leaves CUs idle.  Two workgroups fit a CU, so the chip runs
   // `slots` workgroups at a time; pick the split count whose last round of workgroups is the
@@ -344,7 +523,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   if (tiles < slots && K >= 512) {
     size_t max_splits = K / 128;  // every split keeps >= 128 of K
     if (max_splits > 32) max_splits = 32;
-    const size_t fit = ctx->workspace_bytes / (M * N * sizeof(float));
+    const size_t fit = ctx->workspace_bytes / mn_bytes;
     if (max_splits > fit) max_splits = fit;
     double best = 0.0;
     for (size_t sp = 1; sp <= max_splits; ++sp) {
@@ -362,7 +541,6 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   if (splits < 1) splits = 1;
   g.splits = (unsigned)splits;
   g.k_chunk = k_chunk;
-  g.partial = (float*)ctx->workspace;
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
 #define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g)
@@ -374,15 +552,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   int32_t rc = post_launch();
   if (rc || splits == 1) return rc;
 
-  const size_t mn = M * N;
-  const int vec = (mn % 4 == 0) && (N % 4 == 0) && aligned16(C) && (!bias || aligned16(bias)) &&
-                  (!pre_act || aligned16(pre_act));
-  size_t blocks = ((vec ? mn / 4 : mn) + 255) / 256;
-  const size_t cap = (size_t)ctx->num_cu * 16;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, mn, N, (unsigned)splits,
-                     (const float*)ctx->workspace, C, beta, bias, relu, pre_act, vec);
-  return post_launch();
+  return splitk_combine(ctx, g, splits);
 }
 
 static bool overlaps(const float* a, size_t na, const float* b, size_t nb) {

@@ -39,6 +39,15 @@ struct SGD {
     dev.sgd_step(l.weights.data, lr);
     dev.sgd_step(l.bias.data, lr);
   }
+  // every layer's parameters in one launch
+  void step(HIP& dev, std::initializer_list<Linear*> layers) const {
+    std::vector<Buffer> params;
+    for (Linear* l : layers) {
+      params.push_back(l->weights.data);
+      params.push_back(l->bias.data);
+    }
+    dev.sgd_step(params, lr);
+  }
 };
 
 struct MlpResult {
@@ -109,9 +118,13 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
       check(slhip_cce_grad(dev.ctx(), batch, d_out, p.data.ptr, y.data.ptr, seed.ptr), "slhip_cce_grad");
       p.data.backward_with(seed);
     }
-    sgd.step(dev, lin1);
-    sgd.step(dev, lin2);
-    sgd.step(dev, lin3);
+    if (fused) {
+      sgd.step(dev, {&lin1, &lin2, &lin3});
+    } else {
+      sgd.step(dev, lin1);
+      sgd.step(dev, lin2);
+      sgd.step(dev, lin3);
+    }
     return loss_val;
   };
 

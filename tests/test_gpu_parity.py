@@ -55,6 +55,8 @@ GEMM_SHAPES = [
     (1, 1, 1), (4, 3, 2), (5, 10, 7), (33, 65, 17), (64, 64, 64), (128, 128, 16), (128, 128, 128),
     (129, 127, 130), (256, 384, 200), (100, 10, 300), (300, 10, 2048), (1024, 64, 1), (1024, 1, 64),
     (1, 64, 1024), (64, 1, 1024), (384, 256, 784), (200, 136, 1000), (512, 512, 512),
+    # one wave per 32x32 tile: k split over waves and over the grid, skinny sides, ragged edges
+    (32, 32, 100003), (2000, 10, 1000), (40, 1000, 10), (16, 3000, 500), (31, 33, 4099), (96, 64, 64),
 ]
 
 
@@ -383,6 +385,33 @@ def test_cce_and_onehot(hip, orc):
     a, b = hip.cce(rows, cols, p, t), orc.cce(rows, cols, p, t)
     assert np.all(np.abs(a - b) <= 1e-6 * np.abs(b) + 1e-7)
     assert np.array_equal(hip.cce_grad(rows, cols, p, t), orc.cce_grad(rows, cols, p, t))
+
+
+def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):
+    """Eleven tensors (two launches of up to eight), aligned and not, one of them long."""
+    c = hip.ctx()
+    lens = [1, 3, 64, 65, 1000, 4096, 10, 2048 * 10, 7, 300001, 129]
+    pool_p, pool_g = c.empty(sum(lens) + 16), c.empty(sum(lens) + 16)
+    p_host = rng.uniform(pool_p.n, -1, 1, tag=0, seed=SEED)
+    g_host = rng.uniform(pool_g.n, -1, 1, tag=1, seed=SEED)
+    pool_p.upload(p_host)
+    pool_g.upload(g_host)
+    offs, o = [], 1                                   # start one float in: the first tensors are not 16-byte aligned
+    for n in lens:
+        offs.append(o)
+        o += n
+    P = (C.c_void_p * len(lens))(*[pool_p.ptr + 4 * o for o in offs])
+    G = (C.c_void_p * len(lens))(*[pool_g.ptr + 4 * o for o in offs])
+    N = (C.c_size_t * len(lens))(*lens)
+    c.call("slhip_sgd_step_multi", len(lens), P, G, N, 0.05)
+    got = pool_p.numpy()
+    want = p_host.copy()
+    for o, n in zip(offs, lens):
+        want[o:o + n] = orc.sgd_step(p_host[o:o + n].copy(), g_host[o:o + n], 0.05)
+    assert np.array_equal(got, want)
+    assert c.lib.slhip_sgd_step_multi(c.h, 0, P, G, N, 0.05) == -1
+    pool_p.free()
+    pool_g.free()
 
 
 # --------------------------------------------------------------------------- error behaviour
