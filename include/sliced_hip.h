@@ -57,7 +57,9 @@ enum {
   SLHIP_CLIP = 4,
   SLHIP_NEG_LN = 5,
   SLHIP_SCALE = 6,
-  SLHIP_NEG_DIV = 7
+  SLHIP_NEG_DIV = 7,
+  SLHIP_TANH = 8,   /* src/matrix.rs:206-227: tanh x, gradient 1 - tanh(x)^2 */
+  SLHIP_SIGMOID = 9 /* src/matrix.rs:231-258: 1/(1+exp(-x)), gradient exp(-x)/(1+exp(-x))^2 */
 };
 
 /* ---------------------------------------------------------------- runtime ----------
@@ -199,6 +201,23 @@ int32_t slhip_add_row_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* lhs_
                            const float* out_grad);
 int32_t slhip_add_row_mut_grad(slhip_ctx* ctx, size_t rows, size_t cols, float* rhs_grad, const float* out_grad);
 
+/* RowOp::row_op with a named op (src/ops2/row_op/mod.rs:17-30, slice_row_op
+ * src/ops2/row_op/cpu.rs:67-80): out[r,c] = f(lhs[r,c], rhs[c]), f = SLHIP_ADD..SLHIP_DIV, and
+ * its gradients (slice_row_op_grad_lhs / _rhs, src/ops2/row_op/grad/cpu.rs:66-88):
+ *     lhs_grad[r,c] += df/dlhs * out_grad[r,c]      rhs_grad[c] += sum_r df/drhs * out_grad[r,c]
+ * ColOp::col_op (src/ops2/col_op/mod.rs:20-57, slice_col_op src/ops2/col_op/cpu.rs:40-50) is the
+ * same with the vector indexed by the row: out[r,c] = f(lhs[r,c], rhs[r]); sub_cols = SLHIP_SUB,
+ * div_cols = SLHIP_DIV; gradients as slice_col_op_grad_lhs / _rhs
+ * (src/ops2/col_op/grad/cpu.rs:41-88).  Either gradient pointer may be NULL (skipped). */
+int32_t slhip_row_op(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                     float* out);
+int32_t slhip_row_op_grad(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                          float* lhs_grad, float* rhs_grad, const float* out_grad);
+int32_t slhip_col_op(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                     float* out);
+int32_t slhip_col_op_grad(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                          float* lhs_grad, float* rhs_grad, const float* out_grad);
+
 /* ---------------------------------------------------------------- elementwise ------
  * BinaryElementWise::{add,sub,mul,div} (src/ops2/binary_ew/mod.rs:55-100) and
  * BinaryElementWiseGrad with the closures of BinaryOpsMayGrad (src/ops.rs:115-171;
@@ -232,6 +251,13 @@ int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, 
 int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
                        float* grad);
 int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* out);
+/* onehot_grad (src/ops2/onehot/grad/cpu.rs:3-12): cls_grad[r] += out_grad[r*classes + cls[r]]. */
+int32_t slhip_onehot_grad(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* cls_grad,
+                          const float* out_grad);
+/* diagflat (src/ops2/diagflat/cpu.rs:42-46): out[n×n] = diag(x), every other entry zero;
+ * diagflat_grad (src/ops2/diagflat/grad/cpu.rs:34-38): x_grad[i] += out_grad[i*n + i]. */
+int32_t slhip_diagflat(slhip_ctx* ctx, size_t n, const float* x, float* out);
+int32_t slhip_diagflat_grad(slhip_ctx* ctx, size_t n, float* x_grad, const float* out_grad);
 
 #ifdef __cplusplus
 }

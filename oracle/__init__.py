@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "liboracle.so")
 
 ADD, SUB, MUL, DIV = 0, 1, 2, 3
-SQUARE, POW, RELU, EXP, CLIP, NEG_LN, SCALE, NEG_DIV = range(8)
+SQUARE, POW, RELU, EXP, CLIP, NEG_LN, SCALE, NEG_DIV, TANH, SIGMOID = range(10)
 
 
 def build(force=False):
@@ -182,6 +182,29 @@ def col_op(op, cols, lhs, rhs):
     return out
 
 
+def row_op(op, cols, lhs, rhs):
+    lhs = f32(lhs).ravel()
+    out = np.empty_like(lhs)
+    lib().orc_row_op(int(op), _sz(cols), _sz(lhs.size), _p(lhs), _p(f32(rhs)), _p(out))
+    return out
+
+
+def _bcast_op_grad(by_row_index, op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    lhs = f32(lhs).ravel()
+    lib().orc_bcast_op_grad(by_row_index, int(op), _sz(cols), _sz(lhs.size), _p(lhs), _p(f32(rhs)),
+                            _p(lhs_grad) if lhs_grad is not None else None,
+                            _p(rhs_grad) if rhs_grad is not None else None, _p(f32(out_grad).ravel()))
+    return lhs_grad, rhs_grad
+
+
+def row_op_grad(op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    return _bcast_op_grad(0, op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad)
+
+
+def col_op_grad(op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    return _bcast_op_grad(1, op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad)
+
+
 # ---- elementwise ------------------------------------------------------------
 def binary_ew(op, l, r):
     l, r = f32(l).ravel(), f32(r).ravel()
@@ -294,11 +317,23 @@ def diagflat(x):
     return out
 
 
+def diagflat_grad(x_grad, out_grad):
+    lib().orc_diagflat_grad(_sz(x_grad.size), _p(x_grad), _p(f32(out_grad).ravel()))
+    return x_grad
+
+
 def onehot(highest_class, classes):
     classes = f32(classes).ravel()
     out = np.zeros(classes.size * highest_class, np.float32)
     lib().orc_onehot(_sz(highest_class), _sz(classes.size), _p(classes), _p(out))
     return out
+
+
+def onehot_grad(highest_class, classes, classes_grad, out_grad):
+    classes = f32(classes).ravel()
+    lib().orc_onehot_grad(_sz(highest_class), _sz(classes.size), _p(classes), _p(classes_grad),
+                          _p(f32(out_grad).ravel()))
+    return classes_grad
 
 
 def cce(rows, cols, preds, targets):

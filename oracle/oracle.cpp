@@ -295,6 +295,51 @@ ORC_API void orc_col_op(int op, size_t cols, size_t len, const float* lhs, const
     for (size_t c = 0; c < cols; ++c) out[r * cols + c] = bin(op, lhs[r * cols + c], rhs[r]);
 }
 
+// row_op / col_op gradients with a named op (src/ops2/row_op/grad/cpu.rs:66-88,
+// src/ops2/col_op/grad/cpu.rs:41-88): lhs_grad += dL(lhs, rhs) * out_grad elementwise, the
+// broadcast side accumulates dR(lhs, rhs) * out_grad over the other axis, one `+=` per element in
+// row-major order.  dL / dR as the reference's tests write them: div -> 1/rhs and
+// lhs / -(rhs*rhs) (src/ops2/col_op/grad/cpu.rs:115,146).
+// GOLDEN: src/ops2/col_op/grad/cpu.rs:97-161; src/ops2/row_op/grad/cpu.rs:94-111 (mul).
+static inline float bin_dl(int op, float l, float r) {
+  switch (op) {
+    case 0: case 1: return 1.0f;
+    case 2: return r;
+    default: return 1.0f / r;
+  }
+}
+static inline float bin_dr(int op, float l, float r) {
+  switch (op) {
+    case 0: return 1.0f;
+    case 1: return -1.0f;
+    case 2: return l;
+    default: return l / (-(r * r));
+  }
+}
+// by_row_index = 1: col_op (rhs has one entry per row); 0: row_op (one entry per column).
+ORC_API void orc_bcast_op_grad(int by_row_index, int op, size_t cols, size_t len, const float* lhs, const float* rhs,
+                               float* lhs_grad, float* rhs_grad, const float* out_grad) {
+  size_t rows = len / cols;
+  if (lhs_grad)
+    for (size_t r = 0; r < rows; ++r)
+      for (size_t c = 0; c < cols; ++c) {
+        const size_t i = r * cols + c;
+        lhs_grad[i] += bin_dl(op, lhs[i], rhs[by_row_index ? r : c]) * out_grad[i];
+      }
+  if (rhs_grad)
+    for (size_t r = 0; r < rows; ++r)
+      for (size_t c = 0; c < cols; ++c) {
+        const size_t i = r * cols + c, j = by_row_index ? r : c;
+        rhs_grad[j] += bin_dr(op, lhs[i], rhs[j]) * out_grad[i];
+      }
+}
+// row_op forward with a named op (src/ops2/row_op/cpu.rs:67-80)
+ORC_API void orc_row_op(int op, size_t cols, size_t len, const float* lhs, const float* rhs, float* out) {
+  size_t rows = len / cols;
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t c = 0; c < cols; ++c) out[r * cols + c] = bin(op, lhs[r * cols + c], rhs[c]);
+}
+
 // ---------------------------------------------------------------------------
 // binary_ew  (src/ops2/binary_ew/cpu_stack.rs:42-55, grad/cpu_stack.rs:40-88)
 // ---------------------------------------------------------------------------
@@ -343,7 +388,11 @@ ORC_API void orc_add_ew_grad(size_t len, float* lg, float* rg, const float* g) {
 //   op 5 neg_ln : -(ln x)         (cce, examples/nn.rs:137; no grad)
 //   op 6 scale  : x*p             (helper: -(v)/rows of cce_grad is op 7)
 //   op 7 neg_div: (-x)/p          (examples/nn.rs:151)
-// GOLDEN: tests/test_square.rs:12,19; tests/test_pow.rs:15,20; tests/matrix/relu.rs:12,20.
+//   op 8 tanh   : tanhf(x)        grad 1 - tanh(x)^2             (src/matrix.rs:206-227)
+//   op 9 sigmoid: 1/(1+exp(-x))   grad exp(-x)/(1+exp(-x))^2     (src/matrix.rs:231-258)
+// GOLDEN: tests/test_square.rs:12,19; tests/test_pow.rs:15,20; tests/matrix/relu.rs:12,20;
+// tests/matrix/tanh.rs:12-31.  sigmoid has no vector in the reference: pinned by the closed form
+// against an f64 evaluation and by a finite difference (tests/test_oracle_math.py).
 // ---------------------------------------------------------------------------
 static inline float un(int op, float x, float p, float q) {
   switch (op) {
@@ -354,6 +403,8 @@ static inline float un(int op, float x, float p, float q) {
     case 4: return fminf(fmaxf(x, p), q);
     case 5: return -logf(x);
     case 6: return x * p;
+    case 8: return tanhf(x);
+    case 9: return 1.0f / (1.0f + expf(-x));
     default: return (-x) / p;
   }
 }
@@ -364,6 +415,8 @@ static inline float un_grad(int op, float x, float p) {
     case 2: return x >= 0.0f ? 1.0f : 0.0f;
     case 3: return expf(x);
     case 6: return p;
+    case 8: { const float t = tanhf(x); return 1.0f - t * t; }
+    case 9: { const float e = expf(-x); const float d = 1.0f + e; return e / (d * d); }
     default: return 0.0f;
   }
 }
@@ -556,6 +609,15 @@ ORC_API void orc_softmax_grad(size_t samples, size_t features, float* x_grad, co
 // ---------------------------------------------------------------------------
 ORC_API void orc_onehot(size_t highest_class, size_t n, const float* classes, float* onehot) {
   for (size_t r = 0; r < n; ++r) onehot[r * highest_class + (size_t)classes[r]] = 1.0f;
+}
+// onehot_grad  src/ops2/onehot/grad/cpu.rs:3-12.  GOLDEN: :18-38.
+ORC_API void orc_onehot_grad(size_t highest_class, size_t n, const float* classes, float* classes_grad,
+                             const float* out_grad) {
+  for (size_t r = 0; r < n; ++r) classes_grad[r] += out_grad[r * highest_class + (size_t)classes[r]];
+}
+// diagflat_grad  src/ops2/diagflat/grad/cpu.rs:34-38.  GOLDEN: :44-60.
+ORC_API void orc_diagflat_grad(size_t n, float* x_grad, const float* out_grad) {
+  for (size_t i = 0; i < n; ++i) x_grad[i] += out_grad[n * i + i];
 }
 
 // ---------------------------------------------------------------------------

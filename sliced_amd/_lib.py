@@ -72,6 +72,13 @@ PROTOTYPES = {
     "slhip_ew_unary_grad": [c_vp, c_i32, C.c_float, c_sz, c_vp, c_vp, c_vp],
     "slhip_ew_chain": [c_vp, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
     "slhip_sgd_step": [c_vp, c_sz, c_vp, c_vp, C.c_float],
+    "slhip_row_op": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp],
+    "slhip_row_op_grad": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
+    "slhip_col_op": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp],
+    "slhip_col_op_grad": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
+    "slhip_diagflat": [c_vp, c_sz, c_vp, c_vp],
+    "slhip_diagflat_grad": [c_vp, c_sz, c_vp, c_vp],
+    "slhip_onehot_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_sgd_step_multi": [c_vp, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],

@@ -1,0 +1,244 @@
+// Row / column broadcast ops with an op code, diagflat and the onehot gradient: the part of the
+// reference's op surface beside the training hot path (reference: src/ops2/row_op, src/ops2/col_op,
+// src/ops2/diagflat, src/ops2/onehot).  Plain streaming kernels, one element per thread; the
+// reductions of the broadcast-side gradients go through partial sums in the context workspace
+// and are combined in a fixed order.
+#include "common.hpp"
+
+namespace slhip {
+
+__device__ __forceinline__ float bc_apply(int op, float a, float b) {
+  switch (op) {
+    case SLHIP_ADD: return a + b;
+    case SLHIP_SUB: return a - b;
+    case SLHIP_MUL: return a * b;
+    default: return a / b;
+  }
+}
+// d f(l, r) / d l   and   d f(l, r) / d r, as the reference's tests write them
+// (src/ops2/col_op/grad/cpu.rs:115,146: 1/rhs and lhs / -(rhs*rhs) for div)
+__device__ __forceinline__ float bc_dl(int op, float l, float r) {
+  switch (op) {
+    case SLHIP_ADD: return 1.0f;
+    case SLHIP_SUB: return 1.0f;
+    case SLHIP_MUL: return r;
+    default: return 1.0f / r;
+  }
+}
+__device__ __forceinline__ float bc_dr(int op, float l, float r) {
+  switch (op) {
+    case SLHIP_ADD: return 1.0f;
+    case SLHIP_SUB: return -1.0f;
+    case SLHIP_MUL: return l;
+    default: return l / (-(r * r));
+  }
+}
+
+// BY_ROW_INDEX: the broadcast vector is indexed by the row (col_op), else by the column (row_op).
+template <bool BY_ROW_INDEX>
+__global__ __launch_bounds__(256) void bc_fwd_kernel(int op, size_t len, size_t cols, const float* __restrict__ lhs,
+                                                     const float* __restrict__ v, float* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= len) return;
+  const size_t r = i / cols;
+  out[i] = bc_apply(op, lhs[i], v[BY_ROW_INDEX ? r : i - r * cols]);
+}
+
+template <bool BY_ROW_INDEX>
+__global__ __launch_bounds__(256) void bc_grad_lhs_kernel(int op, size_t len, size_t cols, const float* __restrict__ lhs,
+                                                          const float* __restrict__ v, float* __restrict__ lhs_grad,
+                                                          const float* __restrict__ g) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= len) return;
+  const size_t r = i / cols;
+  lhs_grad[i] += bc_dl(op, lhs[i], v[BY_ROW_INDEX ? r : i - r * cols]) * g[i];
+}
+
+// col_op: v_grad[r] += sum_c dR(lhs[r,c], v[r]) * g[r,c]; one wave per row
+__global__ __launch_bounds__(256) void colop_grad_rhs_kernel(int op, size_t rows, size_t cols,
+                                                             const float* __restrict__ lhs, const float* __restrict__ v,
+                                                             float* __restrict__ v_grad, const float* __restrict__ g) {
+  const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const float vr = v[r];
+  float s = 0.0f;
+  for (size_t c = lane; c < cols; c += 64) s += bc_dr(op, lhs[r * cols + c], vr) * g[r * cols + c];
+  s = wave_reduce<SumOp>(s);
+  if (lane == 0) v_grad[r] += s;
+}
+
+// row_op: v_grad[c] += sum_r dR(lhs[r,c], v[c]) * g[r,c]; G row groups write partials, then one
+// thread per column adds them up in group order
+__global__ __launch_bounds__(256) void rowop_grad_rhs_partial_kernel(int op, size_t rows, size_t cols, size_t G,
+                                                                     const float* __restrict__ lhs,
+                                                                     const float* __restrict__ v,
+                                                                     const float* __restrict__ g, float* __restrict__ part) {
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= cols * G) return;
+  const size_t grp = t / cols, c = t - grp * cols;
+  const float vc = v[c];
+  float s = 0.0f;
+  for (size_t r = grp; r < rows; r += G) s += bc_dr(op, lhs[r * cols + c], vc) * g[r * cols + c];
+  part[grp * cols + c] = s;
+}
+__global__ __launch_bounds__(256) void rowop_grad_rhs_final_kernel(size_t cols, size_t G, const float* __restrict__ part,
+                                                                   float* __restrict__ v_grad) {
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  float s = part[c];
+  for (size_t grp = 1; grp < G; ++grp) s += part[grp * cols + c];
+  v_grad[c] += s;
+}
+
+__global__ __launch_bounds__(256) void diagflat_kernel(size_t n, const float* __restrict__ x, float* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n * n) return;
+  const size_t r = i / n, c = i - r * n;
+  out[i] = r == c ? x[r] : 0.0f;
+}
+__global__ __launch_bounds__(256) void diagflat_grad_kernel(size_t n, float* __restrict__ x_grad,
+                                                            const float* __restrict__ out_grad) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x_grad[i] += out_grad[i * n + i];
+}
+__global__ __launch_bounds__(256) void onehot_grad_kernel(size_t n, size_t classes, const float* __restrict__ cls,
+                                                          float* __restrict__ cls_grad, const float* __restrict__ out_grad) {
+  const size_t r = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  const size_t c = (size_t)cls[r];
+  if (c < classes) cls_grad[r] += out_grad[r * classes + c];
+}
+
+static bool grid_for(size_t threads, unsigned* blocks) {
+  const size_t b = (threads + 255) / 256;
+  if (b == 0 || b > 0x7fffffffu) return false;
+  *blocks = (unsigned)b;
+  return true;
+}
+
+template <bool BY_ROW_INDEX>
+static int32_t bc_forward(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* v,
+                          float* out) {
+  size_t len;
+  unsigned blocks;
+  if (!checked_len(rows, cols, &len) || !grid_for(len, &blocks)) {
+    set_error("broadcast op: bad dims %zu x %zu", rows, cols);
+    return SLHIP_EINVAL;
+  }
+  if (op < SLHIP_ADD || op > SLHIP_DIV) {
+    set_error("broadcast op: unknown op %d", op);
+    return SLHIP_EINVAL;
+  }
+  hipLaunchKernelGGL((bc_fwd_kernel<BY_ROW_INDEX>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out);
+  return post_launch();
+}
+
+template <bool BY_ROW_INDEX>
+static int32_t bc_backward(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* v,
+                           float* lhs_grad, float* v_grad, const float* g) {
+  size_t len;
+  unsigned blocks;
+  if (!checked_len(rows, cols, &len) || !grid_for(len, &blocks)) {
+    set_error("broadcast op grad: bad dims %zu x %zu", rows, cols);
+    return SLHIP_EINVAL;
+  }
+  if (op < SLHIP_ADD || op > SLHIP_DIV) {
+    set_error("broadcast op grad: unknown op %d", op);
+    return SLHIP_EINVAL;
+  }
+  if (lhs_grad) {
+    hipLaunchKernelGGL((bc_grad_lhs_kernel<BY_ROW_INDEX>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v,
+                       lhs_grad, g);
+    int32_t rc = post_launch();
+    if (rc) return rc;
+  }
+  if (!v_grad) return SLHIP_OK;
+  if (BY_ROW_INDEX) {
+    const size_t b = (rows + 3) / 4;
+    if (b > 0x7fffffffu) {
+      set_error("col_op grad: %zu rows exceed one launch", rows);
+      return SLHIP_EINVAL;
+    }
+    hipLaunchKernelGGL(colop_grad_rhs_kernel, dim3((unsigned)b), dim3(256), 0, ctx->stream, op, rows, cols, lhs, v, v_grad, g);
+    return post_launch();
+  }
+  // row groups: enough threads to fill the chip, never more groups than rows or than the workspace holds
+  size_t G = ((size_t)ctx->num_cu * 2048 + cols - 1) / cols;
+  if (G > rows) G = rows;
+  if (G > 1024) G = 1024;
+  const size_t fit = ctx->workspace_bytes / (cols * sizeof(float));
+  if (fit == 0) {
+    set_error("row_op grad: %zu columns exceed the workspace", cols);
+    return SLHIP_EWORKSPACE;
+  }
+  if (G > fit) G = fit;
+  if (G < 1) G = 1;
+  unsigned pb, fb;
+  if (!grid_for(cols * G, &pb) || !grid_for(cols, &fb)) {
+    set_error("row_op grad: %zu columns exceed one launch", cols);
+    return SLHIP_EINVAL;
+  }
+  float* part = (float*)ctx->workspace;
+  hipLaunchKernelGGL(rowop_grad_rhs_partial_kernel, dim3(pb), dim3(256), 0, ctx->stream, op, rows, cols, G, lhs, v, g, part);
+  int32_t rc = post_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(rowop_grad_rhs_final_kernel, dim3(fb), dim3(256), 0, ctx->stream, cols, G, (const float*)part, v_grad);
+  return post_launch();
+}
+
+}  // namespace slhip
+
+using namespace slhip;
+
+SLHIP_API int32_t slhip_row_op(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                               float* out) {
+  SLHIP_REQUIRE(ctx && lhs && rhs && out, "null argument");
+  return bc_forward<false>(ctx, op, rows, cols, lhs, rhs, out);
+}
+
+SLHIP_API int32_t slhip_row_op_grad(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs,
+                                    const float* rhs, float* lhs_grad, float* rhs_grad, const float* out_grad) {
+  SLHIP_REQUIRE(ctx && lhs && rhs && out_grad, "null argument");
+  return bc_backward<false>(ctx, op, rows, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad);
+}
+
+SLHIP_API int32_t slhip_col_op(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs, const float* rhs,
+                               float* out) {
+  SLHIP_REQUIRE(ctx && lhs && rhs && out, "null argument");
+  return bc_forward<true>(ctx, op, rows, cols, lhs, rhs, out);
+}
+
+SLHIP_API int32_t slhip_col_op_grad(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, const float* lhs,
+                                    const float* rhs, float* lhs_grad, float* rhs_grad, const float* out_grad) {
+  SLHIP_REQUIRE(ctx && lhs && rhs && out_grad, "null argument");
+  return bc_backward<true>(ctx, op, rows, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad);
+}
+
+SLHIP_API int32_t slhip_diagflat(slhip_ctx* ctx, size_t n, const float* x, float* out) {
+  SLHIP_REQUIRE(ctx && x && out, "null argument");
+  size_t len;
+  unsigned blocks;
+  SLHIP_REQUIRE(checked_len(n, n, &len) && grid_for(len, &blocks), "bad length");
+  hipLaunchKernelGGL(diagflat_kernel, dim3(blocks), dim3(256), 0, ctx->stream, n, x, out);
+  return post_launch();
+}
+
+SLHIP_API int32_t slhip_diagflat_grad(slhip_ctx* ctx, size_t n, float* x_grad, const float* out_grad) {
+  SLHIP_REQUIRE(ctx && x_grad && out_grad, "null argument");
+  size_t len;
+  unsigned blocks;
+  SLHIP_REQUIRE(checked_len(n, n, &len) && grid_for(n, &blocks), "bad length");
+  hipLaunchKernelGGL(diagflat_grad_kernel, dim3(blocks), dim3(256), 0, ctx->stream, n, x_grad, out_grad);
+  return post_launch();
+}
+
+SLHIP_API int32_t slhip_onehot_grad(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* cls_grad,
+                                    const float* out_grad) {
+  SLHIP_REQUIRE(ctx && cls && cls_grad && out_grad, "null argument");
+  size_t len;
+  unsigned blocks;
+  SLHIP_REQUIRE(checked_len(n, classes, &len) && grid_for(n, &blocks), "bad dims");
+  hipLaunchKernelGGL(onehot_grad_kernel, dim3(blocks), dim3(256), 0, ctx->stream, n, classes, cls, cls_grad, out_grad);
+  return post_launch();
+}

@@ -136,6 +136,8 @@ struct UnF {
       case SLHIP_CLIP: o[0] = fminf(fmaxf(x, p), q); break;
       case SLHIP_NEG_LN: o[0] = -logf(x); break;
       case SLHIP_SCALE: o[0] = x * p; break;
+      case SLHIP_TANH: o[0] = tanhf(x); break;
+      case SLHIP_SIGMOID: o[0] = 1.0f / (1.0f + expf(-x)); break;
       default: o[0] = (-x) / p; break;
     }
   }
@@ -153,6 +155,8 @@ struct UnGradF {
       case SLHIP_POW: d = pow_ref(x, p - 1.0f) * p; break;
       case SLHIP_RELU: d = x >= 0.0f ? 1.0f : 0.0f; break;
       case SLHIP_EXP: d = expf(x); break;
+      case SLHIP_TANH: { const float t = tanhf(x); d = 1.0f - t * t; break; }
+      case SLHIP_SIGMOID: { const float e = expf(-x); const float s = 1.0f + e; d = e / (s * s); break; }
       default: d = p; break;  // SLHIP_SCALE
     }
     o[0] += d * g;
@@ -330,7 +334,7 @@ SLHIP_API int32_t slhip_ew_unary(slhip_ctx* ctx, int32_t op, float p, float q, s
   }
   switch (op) {
     SL_UN(SLHIP_SQUARE) SL_UN(SLHIP_POW) SL_UN(SLHIP_RELU) SL_UN(SLHIP_EXP) SL_UN(SLHIP_CLIP)
-    SL_UN(SLHIP_NEG_LN) SL_UN(SLHIP_SCALE) SL_UN(SLHIP_NEG_DIV)
+    SL_UN(SLHIP_NEG_LN) SL_UN(SLHIP_SCALE) SL_UN(SLHIP_NEG_DIV) SL_UN(SLHIP_TANH) SL_UN(SLHIP_SIGMOID)
     default: break;
   }
 #undef SL_UN
@@ -349,6 +353,7 @@ SLHIP_API int32_t slhip_ew_unary_grad(slhip_ctx* ctx, int32_t op, float p, size_
   }
   switch (op) {
     SL_UNG(SLHIP_SQUARE) SL_UNG(SLHIP_POW) SL_UNG(SLHIP_RELU) SL_UNG(SLHIP_EXP) SL_UNG(SLHIP_SCALE)
+    SL_UNG(SLHIP_TANH) SL_UNG(SLHIP_SIGMOID)
     default: break;
   }
 #undef SL_UNG

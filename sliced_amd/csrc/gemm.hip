@@ -514,26 +514,33 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   }
   g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
 
-  // Split K when the tile grid alone leaves CUs idle.  Two workgroups fit a CU, so the chip runs
-  // `slots` workgroups at a time; pick the split count whose last round of workgroups is the
-  // fullest (ties: the smaller count, which writes fewer partial results).
+  // Split K when the tile grid alone leaves CUs idle.  The split count minimises a cost model
+  // fitted to MI355X timings of this kernel (512^3 ... 2048x2048x8192, 1..32 splits, within
+  // about 10 %): two workgroups share a CU, a k tile takes 4.35 us when they do and 2.43 us when
+  // a workgroup has the CU to itself (at most one workgroup per CU in flight); workgroups run in
+  // rounds of `slots`; every round costs 6 us on top (first loads, epilogue); combining the
+  // partial products costs 4 us plus their bytes, written and read once, at 5 TB/s.
+  constexpr int BK = GEMM_BK;
   const size_t tiles = tiles_m * tiles_n;
   const size_t slots = (size_t)ctx->num_cu * 2;
   size_t splits = 1;
-  if (tiles < slots && K >= 512) {
-    size_t max_splits = K / 128;  // every split keeps >= 128 of K
+  const size_t kt_total = (K + BK - 1) / BK;
+  if (tiles < slots && kt_total >= 4) {
+    size_t max_splits = kt_total / 2;  // every split keeps at least two k tiles
     if (max_splits > 32) max_splits = 32;
     const size_t fit = ctx->workspace_bytes / mn_bytes;
     if (max_splits > fit) max_splits = fit;
-    double best = 0.0;
+    double best = 1e300;
     for (size_t sp = 1; sp <= max_splits; ++sp) {
+      const size_t kt = (kt_total + sp - 1) / sp;
       const size_t wgs = tiles * sp;
-      const size_t rounds = (wgs + slots - 1) / slots;
-      const double eff = (double)wgs / (double)(rounds * slots);
-      if (eff > best + 1e-9) { best = eff; splits = sp; }
+      const size_t full_rounds = wgs / slots, rest = wgs % slots;
+      double t = (double)full_rounds * (kt * 4.35 + 6.0);
+      if (rest) t += kt * ((full_rounds == 0 ? rest <= slots / 2 : rest <= slots / 4) ? 2.43 : 4.35) + 6.0;
+      if (sp > 1) t += 4.0 + 2.0 * (double)sp * (double)mn_bytes / 5.0e6;
+      if (t < best) { best = t; splits = sp; }
     }
   }
-  constexpr int BK = GEMM_BK;
   size_t k_chunk = (K + splits - 1) / splits;
   k_chunk = (k_chunk + BK - 1) / BK * BK;
   if (k_chunk == 0) k_chunk = BK;

@@ -120,6 +120,26 @@ SLH_API int slh_unary(void* dev, int op, float p, float q, uint64_t x, int with_
     *out = d->unary(op, d->lookup(x), p, q, with_grad != 0).id;
   });
 }
+// by_row_index 0: row_op (rhs has one entry per column), 1: col_op (one per row); op = SLHIP_ADD..DIV
+SLH_API int slh_bcast_op(void* dev, int by_row_index, int op, size_t rows, size_t cols, uint64_t lhs, uint64_t rhs,
+                         uint64_t* out) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    *out = d->bcast_op(by_row_index != 0, op, rows, cols, d->lookup(lhs), d->lookup(rhs)).id;
+  });
+}
+SLH_API int slh_diagflat(void* dev, uint64_t x, uint64_t* out) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    *out = d->diagflat(d->lookup(x)).id;
+  });
+}
+SLH_API int slh_onehot(void* dev, size_t classes, uint64_t cls, uint64_t* out) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    *out = d->onehot(classes, d->lookup(cls)).id;
+  });
+}
 SLH_API int slh_transpose(void* dev, size_t rows, size_t cols, uint64_t x, uint64_t* out) {
   return guard([&] {
     HIP* d = (HIP*)dev;

@@ -315,6 +315,51 @@ class HIP {
     });
   }
 
+  // RowOp::row_op / ColOp::col_op with a named op (src/ops2/row_op/mod.rs:17-30,
+  // src/ops2/col_op/mod.rs:20-57) and their gradients (RowOpGrad / ColOpGrad::row_op_grad,
+  // src/ops2/row_op/grad.rs:12-41, src/ops2/col_op/grad.rs:12-27): both sides accumulate.
+  Buffer bcast_op(bool by_row_index, int op, size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
+    expect(lhs, rows * cols, "row/col op lhs"); expect(rhs, by_row_index ? rows : cols, "row/col op rhs");
+    Buffer out = retrieve(rows * cols);
+    check((by_row_index ? slhip_col_op : slhip_row_op)(ctx_, op, rows, cols, lhs.ptr, rhs.ptr, out.ptr), "row/col op");
+    uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
+      check((by_row_index ? slhip_col_op_grad : slhip_row_op_grad)(ctx_, op, rows, cols, l.ptr, r.ptr, grad_mut(l).ptr,
+                                                                   grad_mut(r).ptr, grad(o).ptr),
+            "row/col op grad");
+    });
+    return out;
+  }
+  Buffer row_op(int op, size_t rows, size_t cols, const Buffer& l, const Buffer& r) { return bcast_op(false, op, rows, cols, l, r); }
+  Buffer col_op(int op, size_t rows, size_t cols, const Buffer& l, const Buffer& r) { return bcast_op(true, op, rows, cols, l, r); }
+  Buffer sub_cols(size_t rows, size_t cols, const Buffer& l, const Buffer& r) { return col_op(SLHIP_SUB, rows, cols, l, r); }
+  Buffer div_cols(size_t rows, size_t cols, const Buffer& l, const Buffer& r) { return col_op(SLHIP_DIV, rows, cols, l, r); }
+
+  // Diagflat::diagflat + DiagflatGrad (src/ops2/diagflat/mod.rs, grad/cpu.rs:34-38)
+  Buffer diagflat(const Buffer& x) {
+    Buffer out = retrieve(x.len * x.len);
+    check(slhip_diagflat(ctx_, x.len, x.ptr, out.ptr), "slhip_diagflat");
+    uint64_t xi = x.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), o = lookup(oi);
+      check(slhip_diagflat_grad(ctx_, xb.len, grad_mut(xb).ptr, grad(o).ptr), "slhip_diagflat_grad");
+    });
+    return out;
+  }
+
+  // Onehot::onehot + onehot_grad (src/ops2/onehot/cpu.rs:40-44, grad/cpu.rs:3-12)
+  Buffer onehot(size_t classes, const Buffer& cls) {
+    Buffer out = retrieve(cls.len * classes);
+    check(slhip_onehot(ctx_, cls.len, classes, cls.ptr, out.ptr), "slhip_onehot");
+    uint64_t ci = cls.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer c = lookup(ci), o = lookup(oi);
+      check(slhip_onehot_grad(ctx_, c.len, classes, c.ptr, grad_mut(c).ptr, grad(o).ptr), "slhip_onehot_grad");
+    });
+    return out;
+  }
+
   // BinaryOpsMayGrad::{add,sub,mul}  src/ops.rs:115-171
   Buffer binary(int op, const Buffer& lhs, const Buffer& rhs) {
     if (lhs.len != rhs.len) throw Error("binary op: lengths differ");
@@ -349,6 +394,8 @@ class HIP {
   Buffer square(const Buffer& x) { return unary(SLHIP_SQUARE, x); }
   Buffer pow(const Buffer& x, float rhs) { return unary(SLHIP_POW, x, rhs); }
   Buffer relu(const Buffer& x) { return unary(SLHIP_RELU, x); }
+  Buffer tanh(const Buffer& x) { return unary(SLHIP_TANH, x); }        // src/matrix.rs:206-227
+  Buffer sigmoid(const Buffer& x) { return unary(SLHIP_SIGMOID, x); }  // src/matrix.rs:231-258
   Buffer exp(const Buffer& x) { return unary(SLHIP_EXP, x, 0, 0, false); }                        // src/ops.rs:435-440
   Buffer clip(const Buffer& x, float lo, float hi) { return unary(SLHIP_CLIP, x, lo, hi, false); }  // src/ops.rs:419-425
 
@@ -544,6 +591,10 @@ class Matrix {
   Matrix squared() const { return Matrix(device().square(data), rows, cols); }                                  // :275-288
   Matrix pow(float rhs) const { return Matrix(device().pow(data, rhs), rows, cols); }                           // :292-297
   Matrix softmax() const { return Matrix(device().softmax(rows, cols, data), rows, cols); }                     // :368-378
+  Matrix tanh() const { return Matrix(device().tanh(data), rows, cols); }                                       // :206-227
+  Matrix sigmoid() const { return Matrix(device().sigmoid(data), rows, cols); }                                 // :231-258
+  Matrix l2_norm_cols() const { return squared().sum_cols().pow(0.5f); }                                        // :337-355
+  Matrix diagflat() const { return Matrix(device().diagflat(data), data.len, data.len); }                       // :359-364
   Matrix sum_cols() const { return Matrix(device().reduce(HIP::SUM_COLS, rows, cols, data), rows, 1); }         // :329-334
   // The reference's Matrix::max_rows / max_cols wrap the reduced buffer as (rows, cols) and trip
   // its own length assert unless one dimension is 1 (src/matrix.rs:301-325); here the result

@@ -22,7 +22,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libsliced_host.so")
 
 ADD, SUB, MUL, DIV = 0, 1, 2, 3
-SQUARE, POW, RELU, EXP, CLIP, NEG_LN, SCALE, NEG_DIV = range(8)
+SQUARE, POW, RELU, EXP, CLIP, NEG_LN, SCALE, NEG_DIV, TANH, SIGMOID = range(10)
 SUM_ROWS, SUM_COLS, MAX_ROWS, MAX_COLS, MEAN_ROWS, MEAN_COLS = range(6)
 
 _h = None
@@ -168,11 +168,39 @@ class HIP:
     def relu(self, x):
         return self._un(RELU, x)
 
+    def tanh(self, x):
+        return self._un(TANH, x)
+
+    def sigmoid(self, x):
+        return self._un(SIGMOID, x)
+
     def exp(self, x):
         return self._un(EXP, x, with_grad=False)
 
     def clip(self, x, lo, hi):
         return self._un(CLIP, x, lo, hi, with_grad=False)
+
+    def row_op(self, op, rows, cols, lhs, rhs):
+        return self._out(lib().slh_bcast_op, 0, int(op), _sz(rows), _sz(cols), _u64(lhs.id), _u64(rhs.id))
+
+    def col_op(self, op, rows, cols, lhs, rhs):
+        return self._out(lib().slh_bcast_op, 1, int(op), _sz(rows), _sz(cols), _u64(lhs.id), _u64(rhs.id))
+
+    def sub_cols(self, rows, cols, lhs, rhs):
+        return self.col_op(SUB, rows, cols, lhs, rhs)
+
+    def div_cols(self, rows, cols, lhs, rhs):
+        return self.col_op(DIV, rows, cols, lhs, rhs)
+
+    def diagflat(self, x):
+        return self._out(lib().slh_diagflat, _u64(x.id))
+
+    def onehot(self, classes, cls):
+        return self._out(lib().slh_onehot, _sz(classes), _u64(cls.id))
+
+    def l2_norm_cols(self, rows, cols, x):
+        """Matrix::l2_norm_cols (src/matrix.rs:337-355): squared().sum_cols().pow(1/2)."""
+        return self.pow(self._red(SUM_COLS, cols, self.square(x), rows), 0.5)
 
     def transpose(self, rows, cols, x):
         return self._out(lib().slh_transpose, _sz(rows), _sz(cols), _u64(x.id))

@@ -319,6 +319,73 @@ def softmax_grad(samples, features, out, out_grad, x_grad=None, beta=0.0):
     return res
 
 
+def _bcast_op(name, op, cols, lhs, rhs):
+    lhs = _f32(lhs)
+    with _Scope() as s:
+        dl, dr, do = s.up(lhs), s.up(rhs), s.empty(lhs.size)
+        s.c.call(name, int(op), lhs.size // cols, cols, dl.ptr, dr.ptr, do.ptr)
+        return do.numpy()
+
+
+def row_op(op, cols, lhs, rhs):
+    return _bcast_op("slhip_row_op", op, cols, lhs, rhs)
+
+
+def col_op(op, cols, lhs, rhs):
+    return _bcast_op("slhip_col_op", op, cols, lhs, rhs)
+
+
+def _bcast_op_grad(name, op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    lhs = _f32(lhs)
+    with _Scope() as s:
+        dl, dr, dg = s.up(lhs), s.up(rhs), s.up(out_grad)
+        dlg, drg = s.up(lhs_grad), s.up(rhs_grad)
+        s.c.call(name, int(op), lhs.size // cols, cols, dl.ptr, dr.ptr, dlg.ptr if dlg else None,
+                 drg.ptr if drg else None, dg.ptr)
+        if lhs_grad is not None:
+            lhs_grad[:] = dlg.numpy()
+        if rhs_grad is not None:
+            rhs_grad[:] = drg.numpy()
+    return lhs_grad, rhs_grad
+
+
+def row_op_grad(op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    return _bcast_op_grad("slhip_row_op_grad", op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad)
+
+
+def col_op_grad(op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    return _bcast_op_grad("slhip_col_op_grad", op, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad)
+
+
+def mul_row_grad(cols, lhs, rhs, lhs_grad, rhs_grad, out_grad):
+    return row_op_grad(2, cols, lhs, rhs, lhs_grad, rhs_grad, out_grad)
+
+
+def diagflat(x):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, do = s.up(x), s.empty(x.size * x.size)
+        s.c.call("slhip_diagflat", x.size, dx.ptr, do.ptr)
+        return do.numpy()
+
+
+def diagflat_grad(x_grad, out_grad):
+    with _Scope() as s:
+        dx, dg = s.up(x_grad), s.up(out_grad)
+        s.c.call("slhip_diagflat_grad", x_grad.size, dx.ptr, dg.ptr)
+        x_grad[:] = dx.numpy()
+    return x_grad
+
+
+def onehot_grad(highest_class, classes, classes_grad, out_grad):
+    classes = _f32(classes)
+    with _Scope() as s:
+        dc, dcg, dg = s.up(classes), s.up(classes_grad), s.up(out_grad)
+        s.c.call("slhip_onehot_grad", classes.size, highest_class, dc.ptr, dcg.ptr, dg.ptr)
+        classes_grad[:] = dcg.numpy()
+    return classes_grad
+
+
 def onehot(highest_class, classes):
     classes = _f32(classes)
     with _Scope() as s:

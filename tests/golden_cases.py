@@ -11,7 +11,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
-UN = {"square": 0, "pow": 1, "relu": 2, "exp": 3}
+UN = {"square": 0, "pow": 1, "relu": 2, "exp": 3, "tanh": 8, "sigmoid": 9}
 
 
 def load_cases():
@@ -70,6 +70,20 @@ def run_case(be, c):
         check(rg, c["expect_rhs"], tol, c["name"])
     elif fn == "col_op":
         check(need(fn)(OPS[c["op"]], c["cols"], f32(c["lhs"]), f32(c["rhs"])), c["expect"], tol, c["name"])
+    elif fn == "col_op_grad":
+        lhs = f32(c["lhs"])
+        lg, rg = np.zeros(lhs.size, np.float32), np.zeros(lhs.size // c["cols"], np.float32)
+        lg, rg = need(fn)(OPS[c["op"]], c["cols"], lhs, f32(c["rhs"]), lg, rg, f32(c["out_grad"]))
+        if "expect_lhs" in c:
+            check(lg, c["expect_lhs"], tol, c["name"])
+        if "expect_rhs" in c:
+            check(rg, c["expect_rhs"], tol, c["name"])
+    elif fn == "diagflat_grad":
+        check(need(fn)(np.zeros(c["n"], np.float32), f32(c["out_grad"])), c["expect"], tol, c["name"])
+    elif fn == "onehot_grad":
+        cls = f32(c["classes"])
+        check(need(fn)(c["highest_class"], cls, np.zeros(cls.size, np.float32), f32(c["out_grad"])), c["expect"], tol,
+              c["name"])
     elif fn == "binary_ew":
         check(need(fn)(OPS[c["op"]], f32(c["lhs"]), f32(c["rhs"])), c["expect"], tol, c["name"])
     elif fn == "binary_ew_with_grad":

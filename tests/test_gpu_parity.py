@@ -387,6 +387,66 @@ def test_cce_and_onehot(hip, orc):
     assert np.array_equal(hip.cce_grad(rows, cols, p, t), orc.cce_grad(rows, cols, p, t))
 
 
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 10), (257, 129), (4096, 33), (5, 70000), (2000, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("kind", ["row_op", "col_op"])
+def test_broadcast_ops_with_op_code(hip, orc, shape, kind):
+    """row_op / col_op: forward and the elementwise gradient are one IEEE operation (two for the
+    gradient) per element: bit-exact; the broadcast-side gradient is a sum: 1e-6 of sum|terms|."""
+    rows, cols = shape
+    n = rows * cols
+    lhs = rng.uniform(n, 0.5, 2.0, tag=0, seed=SEED)
+    v = rng.uniform(rows if kind == "col_op" else cols, 0.5, 2.0, tag=1, seed=SEED)
+    g = rng.normal(n, 1.0, tag=2, seed=SEED)
+    for op in (orc.ADD, orc.SUB, orc.MUL, orc.DIV):
+        say(kind, rows, cols, "op", op)
+        assert np.array_equal(getattr(hip, kind)(op, cols, lhs, v), getattr(orc, kind)(op, cols, lhs, v))
+        lg0 = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+        vg0 = rng.uniform(v.size, -1, 1, tag=4, seed=SEED)
+        lg_h, vg_h = getattr(hip, kind + "_grad")(op, cols, lhs, v, lg0.copy(), vg0.copy(), g)
+        lg_o, vg_o = getattr(orc, kind + "_grad")(op, cols, lhs, v, lg0.copy(), vg0.copy(), g)
+        assert np.array_equal(lg_h, lg_o)
+        # terms of the broadcast-side sum, in f64, for the bound
+        L, G = lhs.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
+        V = v.astype(np.float64)[:, None] if kind == "col_op" else v.astype(np.float64)[None, :]
+        dr = {orc.ADD: np.ones_like(L), orc.SUB: -np.ones_like(L), orc.MUL: L, orc.DIV: -L / (V * V)}[op] * G
+        axis = 1 if kind == "col_op" else 0
+        bound = 1e-6 * (np.abs(dr).sum(axis) + np.abs(vg0)) + 1e-30
+        exact = vg0 + dr.sum(axis)
+        assert np.all(np.abs(vg_h - exact) <= bound + 1e-6 * np.abs(exact))
+        assert np.all(np.abs(vg_h - vg_o) <= bound + np.abs(vg_o - exact))
+        # one side only
+        lg1, _ = getattr(hip, kind + "_grad")(op, cols, lhs, v, lg0.copy(), None, g)
+        assert np.array_equal(lg1, lg_o)
+
+
+def test_tanh_sigmoid_diagflat_onehot_grad(hip, orc):
+    x = rng.normal(100003, 2.0, tag=0, seed=SEED)
+    g = rng.normal(x.size, 1.0, tag=1, seed=SEED)
+    x64 = x.astype(np.float64)
+    for op, f, df in [(orc.TANH, np.tanh, lambda v: 1 - np.tanh(v) ** 2),
+                      (orc.SIGMOID, lambda v: 1 / (1 + np.exp(-v)), lambda v: np.exp(-v) / (1 + np.exp(-v)) ** 2)]:
+        got, ref = hip.unary(op, x), orc.unary(op, x)
+        assert np.all(np.abs(got - f(x64)) <= 1e-6 * np.abs(f(x64)) + 1e-37)
+        assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + np.abs(ref - f(x64)) + 1e-37)
+        xg0 = rng.uniform(x.size, -1, 1, tag=2, seed=SEED)
+        gg, gr = hip.unary_grad(op, x, xg0.copy(), g), orc.unary_grad(op, x, xg0.copy(), g)
+        exact = xg0 + df(x64) * g
+        # 1 - tanh(x)^2 cancels near |tanh| = 1: the reference's own formula carries an absolute
+        # error of a few ulp(1) there, whoever evaluates it
+        bound = (3e-7 + 2e-6 * np.abs(df(x64))) * np.abs(g) + 2e-6 * np.abs(xg0) + 1e-37
+        assert np.all(np.abs(gg - exact) <= bound)
+        assert np.all(np.abs(gg - gr) <= bound + np.abs(gr - exact))
+    v = rng.uniform(300, -1, 1, tag=3, seed=SEED)
+    assert np.array_equal(hip.diagflat(v), orc.diagflat(v))
+    og = rng.normal(300 * 300, 1.0, tag=4, seed=SEED)
+    assert np.array_equal(hip.diagflat_grad(np.ones(300, np.float32), og), orc.diagflat_grad(np.ones(300, np.float32), og))
+    cls = rng.integers(5000, 10, tag=5, seed=SEED).astype(np.float32)
+    og = rng.normal(5000 * 10, 1.0, tag=6, seed=SEED)
+    assert np.array_equal(hip.onehot_grad(10, cls, np.ones(5000, np.float32), og),
+                          orc.onehot_grad(10, cls, np.ones(5000, np.float32), og))
+
+
 def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):
     """Eleven tensors (two launches of up to eight), aligned and not, one of them long."""
     c = hip.ctx()

@@ -169,6 +169,84 @@ def test_transpose_softmax_l2norm(device):
     assert np.max(np.abs(x.grad().read()[:4] - np.array([0.1826, 0.3651, 0.5477, 0.7303], np.float32))) < 1e-2
 
 
+# reference: tests/matrix/tanh.rs:12-31; sigmoid (src/matrix.rs:231-258) has no reference vector:
+# closed form in f64
+def test_tanh_sigmoid_on_the_tape(device):
+    x = device.buffer([-1, -3, 2, 5, -1.3, 0])
+    out = device.tanh(x)
+    assert np.max(np.abs(out.read() - np.array([-0.7615942, -0.9950548, 0.9640276, 0.9999092, -0.8617231, 0.]))) < 1e-6
+    out.backward()
+    want = np.array([0.41997433, 0.009865999, 0.070650816, 0.00018155575, 0.25743324, 1.0])
+    assert np.max(np.abs(x.grad().read() - want)) < 1e-6
+    v = np.array([-2.0, -0.5, 0.0, 0.25, 3.0])
+    x = device.buffer(v)
+    out = device.sigmoid(x)
+    s = 1 / (1 + np.exp(-v))
+    assert np.max(np.abs(out.read() - s)) < 1e-6
+    out.backward()
+    assert np.max(np.abs(x.grad().read() - s * (1 - s))) < 1e-6
+
+
+# reference: src/ops2/col_op/cpu.rs:56-72 (forward), src/ops2/col_op/grad/cpu.rs:97-161 (div grads),
+# src/ops2/row_op/grad/cpu.rs:94-111 (mul grads), src/ops2/diagflat/grad/cpu.rs:44-60,
+# src/ops2/onehot/grad/cpu.rs:18-38, tests/matrix/l2_norm_cols.rs
+def test_col_op_row_op_diagflat_onehot_on_the_tape(device):
+    from sliced_amd import host
+    lhs = device.buffer([1, -1, 3, 4, 2, 2, 3, 4, 1, 1, 2, 0, 3, 3, -2])
+    rhs = device.buffer([3, 2, 1])
+    out = device.col_op(host.ADD, 3, 5, lhs, rhs)
+    eq(out, [4, 2, 6, 7, 5, 4, 5, 6, 3, 3, 3, 1, 4, 4, -1])
+    out.backward()                                  # runs (and clears) the tape
+    eq(lhs.grad(), [1] * 15)
+    eq(rhs.grad(), [5, 5, 5])
+
+    lhs = device.buffer([1, 2, 3, 4, 5, 6])
+    rhs = device.buffer([-3, 2])
+    out = device.div_cols(2, 3, lhs, rhs)
+    seed = device.buffer([1.4, 2.5, 3.3, 4, 5, 6])
+    out.backward_with(seed)
+    assert np.max(np.abs(lhs.grad().read() - np.array([1.4 / -3, 2.5 / -3, 3.3 / -3, 2, 2.5, 3]))) < 1e-6
+    gf = lambda l, r: l / -(r * r)
+    want = [gf(1, -3) * 1.4 + gf(2, -3) * 2.5 + gf(3, -3) * 3.3, gf(4, 2) * 4 + gf(5, 2) * 5 + gf(6, 2) * 6]
+    assert np.max(np.abs(rhs.grad().read() - np.array(want))) < 1e-5
+
+    # sub_cols: d/dlhs = 1, d/drhs = -1 summed over the row
+    lhs = device.buffer([1, 2, 3, 4, 5, 6])
+    rhs = device.buffer([0.5, -1])
+    out = device.sub_cols(2, 3, lhs, rhs)
+    eq(out, [0.5, 1.5, 2.5, 5, 6, 7])
+    out.backward()
+    eq(lhs.grad(), [1] * 6)
+    eq(rhs.grad(), [-3, -3])
+
+    # row_op multiply: lhs.grad = rhs[c] * g, rhs.grad[c] = sum_r lhs[r,c] * g[r,c]
+    lhs = device.buffer([1, 2, 3, 4, 5, 6])
+    rhs = device.buffer([2, -1, 0.5])
+    out = device.row_op(host.MUL, 2, 3, lhs, rhs)
+    eq(out, [2, -2, 1.5, 8, -5, 3])
+    out.backward()
+    eq(lhs.grad(), [2, -1, 0.5, 2, -1, 0.5])
+    eq(rhs.grad(), [5, 7, 9])
+
+    x = device.buffer([4, 5, 3, -3])
+    d = device.diagflat(x)
+    eq(d, [4, 0, 0, 0, 0, 5, 0, 0, 0, 0, 3, 0, 0, 0, 0, -3])
+    d.backward_with(device.buffer([4, 1, 3, -3, 2, 5, 3, 1, 2, 6, 3, -3, 2, 7, 3, -3]))
+    eq(x.grad(), [4, 5, 3, -3])
+
+    cls = device.buffer([0, 1, 4, 3])
+    oh = device.onehot(5, cls)
+    eq(oh, [1, 0, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 1, 0])
+    oh.backward_with(device.buffer([2, -1, 3, 7, -2, 1, 3, 2, 4, 3, 3, -2, 3, -2, 1, 5, 6, -1, 4, 5]))
+    eq(cls.grad(), [2, 3, 1, 4])
+
+    x = device.buffer([1, 2, 3, 4, 5, 6, 7, 8])
+    out = device.l2_norm_cols(2, 4, x)
+    assert np.max(np.abs(out.read() - np.sqrt([30.0, 174.0]))) < 1e-5
+    out.backward()
+    assert np.max(np.abs(x.grad().read()[:4] - np.array([0.1826, 0.3651, 0.5477, 0.7303]))) < 1e-4
+
+
 # reference: examples/chained_perf.rs:54-91 — cached device, the same chain every iteration
 def test_cached_range_reuses_buffers_and_values():
     from sliced_amd import host

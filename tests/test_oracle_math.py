@@ -150,7 +150,8 @@ def test_unary_and_binary_grads_by_finite_differences(orc):
     x = np.array([-2.5, -0.5, 0.75, 1.5, 3.0], np.float32)
     one = np.ones_like(x)
     for op, p, f in [(orc.SQUARE, 0.0, lambda v: v * v), (orc.POW, 3.0, lambda v: v ** 3), (orc.EXP, 0.0, np.exp),
-                     (orc.SCALE, 0.37, lambda v: 0.37 * v)]:
+                     (orc.SCALE, 0.37, lambda v: 0.37 * v), (orc.TANH, 0.0, np.tanh),
+                     (orc.SIGMOID, 0.0, lambda v: 1.0 / (1.0 + np.exp(-v)))]:
         g = orc.unary_grad(op, x, np.zeros_like(x), one, p)
         x64 = x.astype(np.float64)
         fd = (f(x64 + 1e-6) - f(x64 - 1e-6)) / 2e-6
@@ -190,6 +191,56 @@ def test_row_op_and_loss_helpers(orc):
     pp = rng.uniform(20, -1, 1, tag=5)
     gg = rng.normal(20, 1.0, tag=6)
     assert np.array_equal(orc.sgd_step(pp.copy(), gg, 0.05), (pp - (gg * np.float32(0.05)).astype(np.float32)))
+
+
+@pytest.mark.parametrize("by_row_index", [False, True], ids=["row_op", "col_op"])
+def test_broadcast_op_grads_against_f64_and_finite_differences(orc, by_row_index):
+    """row_op / col_op with a named op: forward against numpy broadcasting; gradients against the
+    f64 chain rule and, for the broadcast side, a finite difference of sum(out * g)."""
+    rows, cols = 6, 4
+    lhs = rng.uniform(rows * cols, 0.5, 2.0, tag=0)
+    v = rng.uniform(rows if by_row_index else cols, 0.5, 2.0, tag=1)
+    g = rng.normal(rows * cols, 1.0, tag=2)
+    L, G = lhs.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
+    bc = (lambda vec: vec.astype(np.float64)[:, None]) if by_row_index else (lambda vec: vec.astype(np.float64)[None, :])
+    axis = 1 if by_row_index else 0
+    fwd = orc.col_op if by_row_index else orc.row_op
+    bwd = orc.col_op_grad if by_row_index else orc.row_op_grad
+    fs = {orc.ADD: lambda a, b: a + b, orc.SUB: lambda a, b: a - b, orc.MUL: lambda a, b: a * b,
+          orc.DIV: lambda a, b: a / b}
+    for op, f in fs.items():
+        assert np.allclose(fwd(op, cols, lhs, v).reshape(rows, cols), f(L, bc(v)), rtol=1e-6), op
+        lg0, vg0 = rng.uniform(rows * cols, -1, 1, tag=3), rng.uniform(v.size, -1, 1, tag=4)
+        lg, vg = bwd(op, cols, lhs, v, lg0.copy(), vg0.copy(), g)
+        eps = 1e-6
+        d_l = (f(L + eps, bc(v)) - f(L - eps, bc(v))) / (2 * eps)
+        assert np.allclose(lg.reshape(rows, cols), lg0.reshape(rows, cols) + d_l * G, rtol=1e-4, atol=1e-5), op
+        fd = np.zeros(v.size)
+        for j in range(v.size):
+            vp, vm = v.astype(np.float64).copy(), v.astype(np.float64).copy()
+            vp[j] += eps; vm[j] -= eps
+            fd[j] = (np.sum(f(L, bc(vp)) * G) - np.sum(f(L, bc(vm)) * G)) / (2 * eps)
+        assert np.allclose(vg, vg0 + fd, rtol=1e-4, atol=1e-4), op
+        # a NULL side is skipped
+        lg2, _ = bwd(op, cols, lhs, v, lg0.copy(), None, g)
+        assert np.array_equal(lg2, lg)
+    if not by_row_index:   # the multiply-only restatement of the reference's own test agrees
+        a = orc.mul_row_grad(cols, lhs, v, np.zeros(rows * cols, np.float32), np.zeros(cols, np.float32), g)
+        b = orc.row_op_grad(orc.MUL, cols, lhs, v, np.zeros(rows * cols, np.float32), np.zeros(cols, np.float32), g)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_diagflat_and_onehot_gradients_pick_the_stored_entries(orc):
+    n = 5
+    x = rng.uniform(n, -1, 1, tag=0)
+    d = orc.diagflat(x).reshape(n, n)
+    assert np.array_equal(np.diag(d), x) and np.count_nonzero(d - np.diag(np.diag(d))) == 0
+    og = rng.normal(n * n, 1.0, tag=1)
+    assert np.array_equal(orc.diagflat_grad(np.ones(n, np.float32), og), 1 + np.diag(og.reshape(n, n)))
+    cls = rng.integers(7, 4, tag=2).astype(np.float32)
+    og = rng.normal(7 * 4, 1.0, tag=3)
+    got = orc.onehot_grad(4, cls, np.zeros(7, np.float32), og)
+    assert np.array_equal(got, og.reshape(7, 4)[np.arange(7), cls.astype(int)])
 
 
 def _mlp_numpy_f64(kind, batch, d_in, d_h, d_out, x, t, params, lr, steps):
