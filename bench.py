@@ -28,9 +28,9 @@ sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # HBM-side bytes of one 4096^3 A*B launch, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
-# this program (profiles/gemm_4096_hbm_traffic.md): (557240.8 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
+# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (723572.7 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.
-GEMM_4096_TRAFFIC_BYTES = int((557240.8 * 2.0 + 65536.0) * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((723572.7 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 
@@ -73,17 +73,56 @@ def spin_up(ctx, seconds=0.4):
         x.free()
 
 
-def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0):
+def timed_cold(ctx, fn, steps, scratch):
+    """HIP-event ms per launch with the caches (L2 and the 256 MiB memory-side cache) swept between
+    launches by a fill of a 1 GiB scratch buffer; the sweep is outside the event pair."""
+    e0, e1 = ctx.event(), ctx.event()
+    total = 0.0
+    for _ in range(steps):
+        ctx.call("slhip_fill", scratch.n, 1.0, scratch.ptr)
+        ctx.record(e0)
+        fn()
+        ctx.record(e1)
+        total += ctx.elapsed_ms(e0, e1)
+    ctx.lib.slhip_event_destroy(e0)
+    ctx.lib.slhip_event_destroy(e1)
+    return total / steps
+
+
+def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, cold_scratch=None):
     a = ctx.uniform(m * k, -1, 1, 0, SEED)
     b = ctx.uniform(k * n, -1, 1, 1, SEED)
     c = ctx.zeros(m * n)
     fn = lambda: ctx.call("slhip_sgemm", ta, tb, m, n, k, a.ptr, b.ptr, c.ptr, beta)
     wall, ev = timed(ctx, fn, steps, warmup)
+    flop = 2.0 * m * n * k
+    res = {"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
+           "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS}
+    if cold_scratch is not None:
+        cold = timed_cold(ctx, fn, max(5, steps // 2), cold_scratch)
+        res["ms_kernel_caches_swept"] = cold
+        res["tflops_kernel_caches_swept"] = flop / cold / 1e9
     for x in (a, b, c):
         x.free()
-    flop = 2.0 * m * n * k
-    return {"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
-            "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS}
+    return res
+
+
+def shader_clock_mhz():
+    """Best effort: the current shader clock from sysfs (the level marked '*' in pp_dpm_sclk); None
+    where it cannot be read.  Reads files only: no other program is started from this process."""
+    import glob
+    import re
+    best = None
+    for path in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+        try:
+            with open(path) as f:
+                for line in f:
+                    m = re.search(r"(\d+)\s*Mhz\s*\*", line, re.I)
+                    if m:
+                        best = max(best or 0, int(m.group(1)))
+        except OSError:
+            pass
+    return best
 
 
 def bw_entry(name, algo_bytes, wall, ev):
@@ -170,7 +209,37 @@ def cpu_baseline(m, n, k):
     oracle.gemm(ms, ms, ms, a[:ms * ms], b[:ms * ms])
     dt1 = time.perf_counter() - t0
     res["single_thread_TFLOPs_at_1024"] = 2.0 * ms ** 3 / dt1 / 1e12
+    res["ops"] = cpu_streaming_ops(oracle, cores)
     return res
+
+
+def cpu_streaming_ops(oracle, cores):
+    """The bandwidth-bound ops on the host: GB/s of the same algorithmic bytes on a bounded sample
+    ([8192 x 4096] = 128 MiB per tensor), once on one thread (the reference's loops are
+    single-threaded) and once on every core."""
+    rows, cols = 8192, 4096
+    n = rows * cols
+    rs = np.random.RandomState(2)
+    x = rs.uniform(-10, 10, n).astype(np.float32)
+    g = rs.standard_normal(n).astype(np.float32)
+    s = oracle.softmax(rows, cols, x)
+    cases = [("sum_rows", 4 * n, lambda: oracle.sum_rows(cols, x)), ("sum_cols", 4 * n, lambda: oracle.sum_cols(cols, x)),
+             ("max_rows", 4 * n, lambda: oracle.max_rows(cols, x)), ("max_cols", 4 * n, lambda: oracle.max_cols(cols, x)),
+             ("transpose", 8 * n, lambda: oracle.transpose(rows, cols, x)),
+             ("softmax fwd", 8 * n, lambda: oracle.softmax(rows, cols, x)),
+             ("softmax bwd", 12 * n, lambda: oracle.softmax_grad(rows, cols, s, g)),
+             ("square (one elementwise op)", 8 * n, lambda: oracle.unary(oracle.SQUARE, x))]
+    out = {"sample": "[%d x %d] f32 per tensor" % (rows, cols)}
+    for name, nbytes, fn in cases:
+        row = {}
+        for label, th in (("GBps_1_thread", 1), ("GBps_%d_threads" % cores, cores)):
+            oracle.set_threads(th)
+            t0 = time.perf_counter()
+            fn()
+            row[label] = nbytes / (time.perf_counter() - t0) / 1e9
+        out[name] = row
+    oracle.set_threads(1)
+    return out
 
 
 def main():
@@ -197,13 +266,25 @@ def main():
     head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup)
     log("gemm NN", head)
     suite = {}
+    # the clock while the matrix cores are busy: queue 0.3 s of launches, sample, then wait
+    a, b, c = ctx.uniform(M * K, -1, 1, 0, SEED), ctx.uniform(K * N, -1, 1, 1, SEED), ctx.zeros(M * N)
+    for _ in range(min(200, int(300 / max(head["ms_kernel"], 0.01)) + 1)):
+        ctx.call("slhip_sgemm", 0, 0, M, N, K, a.ptr, b.ptr, c.ptr, 0.0)
+    time.sleep(0.15)
+    suite["shader_clock_mhz_under_gemm_load"] = shader_clock_mhz()
+    ctx.sync()
+    for x in (a, b, c):
+        x.free()
+    log("sclk under load:", suite["shader_clock_mhz_under_gemm_load"])
     parts = set(args.only.split(",")) if args.only else {"gemm", "sweep", "bandwidth", "mlp"}
     if args.no_suite:
         parts = set()
     if "gemm" in parts:
-        suite["gemm_4096"] = {"A*B": head,
-                              "A*Bt": bench_gemm(ctx, M, N, K, 0, 1, args.steps, args.warmup),
-                              "At*B": bench_gemm(ctx, M, N, K, 1, 0, args.steps, args.warmup)}
+        scratch = ctx.empty(1 << 28)
+        suite["gemm_4096"] = {"A*B": bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup, cold_scratch=scratch),
+                              "A*Bt": bench_gemm(ctx, M, N, K, 0, 1, args.steps, args.warmup, cold_scratch=scratch),
+                              "At*B": bench_gemm(ctx, M, N, K, 1, 0, args.steps, args.warmup, cold_scratch=scratch)}
+        scratch.free()
         log(suite["gemm_4096"])
     if "sweep" in parts:
         sweep = {}
@@ -239,7 +320,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
-                   "kernel": "gemm_kernel<false,false> 128x128x16 tiles, v_mfma_f32_32x32x2_f32"},
+                   "kernel": "gemm_kernel<false,false,32>: 128x128 tiles, BK=32, v_mfma_f32_32x32x2_f32"},
         "roofline": {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": head["frac_of_peak"],
                      "traffic": GEMM_4096_TRAFFIC_BYTES if M == 4096 else None},
