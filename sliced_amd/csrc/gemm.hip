@@ -234,6 +234,9 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
         if (kt + 2 < kt_end) load_stage(kt + 2);
       }
       __builtin_amdgcn_sched_barrier(0);
+      // the wave that is in its MFMA block wins the issue arbitration against the wave of the other
+      // workgroup on the same SIMD, which is fetching or waiting (measured: +2 % on A*B, +1 % on At*B)
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -241,6 +244,7 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 #pragma unroll
           for (int j = 0; j < 2; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][t], b[cur][j][t], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();  // stage s^1 is complete, stage s is free; also leaves LDS free for whoever runs next
