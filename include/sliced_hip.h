@@ -251,6 +251,24 @@ int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, 
 int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* preds, const float* targets,
                        float* grad);
 int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* out);
+
+/* Fused losses of the two example loops; every reference op they stand for stays available.
+ * slhip_mse: loss_dev[0] = (sum_i (x_i - y_i)^2) * (1/n) — the chain sub, squared, sum_cols over one
+ *   row, mul by the constant 1/n (loss tape of examples/sine_net.rs:150-156 summed on the device).
+ * slhip_mse_grad: x_grad_i += ((x_i - y_i) * 2) * ((1/n) * upstream_dev[0]) — what the chain's
+ *   gradient functions (src/ops.rs:118-128, :595-611, :38-41, :137-147) produce for x.
+ * slhip_softmax_cce: probs = softmax(logits) (may be NULL), loss_rows[r] = -ln sum_c
+ *   clip(p, 1e-7, 1-1e-7) * t — Matrix::softmax (src/matrix.rs:368-378) + cce (examples/nn.rs:124-143).
+ * slhip_softmax_cce_grad: logits_grad = beta*logits_grad + (p * sum_c t - t) * (upstream_dev[0] / rows):
+ *   cce_grad (examples/nn.rs:145-152) pushed through softmax_grad (src/ops2/softmax/grad/cpu.rs:8-62)
+ *   in closed form, for the loss mean_r loss_rows[r]. */
+int32_t slhip_mse(slhip_ctx* ctx, size_t n, const float* x, const float* y, float* loss_dev /*1*/);
+int32_t slhip_mse_grad(slhip_ctx* ctx, size_t n, const float* x, const float* y, float* x_grad,
+                       const float* upstream_dev /*1*/);
+int32_t slhip_softmax_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float* logits, const float* targets,
+                          float* probs, float* loss_rows /*rows*/);
+int32_t slhip_softmax_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* probs, const float* targets,
+                               float* logits_grad, float beta, const float* upstream_dev /*1*/);
 /* onehot_grad (src/ops2/onehot/grad/cpu.rs:3-12): cls_grad[r] += out_grad[r*classes + cls[r]]. */
 int32_t slhip_onehot_grad(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* cls_grad,
                           const float* out_grad);

@@ -79,6 +79,10 @@ PROTOTYPES = {
     "slhip_diagflat": [c_vp, c_sz, c_vp, c_vp],
     "slhip_diagflat_grad": [c_vp, c_sz, c_vp, c_vp],
     "slhip_onehot_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
+    "slhip_mse": [c_vp, c_sz, c_vp, c_vp, c_vp],
+    "slhip_mse_grad": [c_vp, c_sz, c_vp, c_vp, c_vp, c_vp],
+    "slhip_softmax_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp],
+    "slhip_softmax_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp, C.c_float, c_vp],
     "slhip_sgd_step_multi": [c_vp, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],

@@ -322,7 +322,10 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 // cycles on narrow tiles and reads operands uncoalesced, but its code is a few hundred bytes:
 // the tiled kernel spends about 13 us per launch before its first MFMA retires (fetching
 // its long unrolled code cold), which is most of the time of a [1024 x 64] x [64 x 64] product.
-template <bool TA, bool TB>
+// NG = groups of 8 k whose loads are issued together: 8 for small problems (latency is all that
+// matters: [1024x64]x[64x64] 7.2 -> 5.9 us), 1 for large skinny ones, which have waves enough to
+// hide latency and measured 15-20 % slower with 2, 4 or 8 (8192x10x2048: 41 us against 48).
+template <bool TA, bool TB, int NG>
 __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
   extern __shared__ float red[];  // [waves][16][64]
   const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -344,10 +347,10 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
   // NG groups of 8 k at a time: all 8*NG loads are issued before the first MFMA needs one
   auto run_groups = [&](size_t gi, auto ng_tag) {
-    constexpr int NG = decltype(ng_tag)::value;
-    float a[NG][4], b[NG][4];
+    constexpr int N = decltype(ng_tag)::value;
+    float a[N][4], b[N][4];
 #pragma unroll
-    for (int u = 0; u < NG; ++u) {
+    for (int u = 0; u < N; ++u) {
       const size_t k = kbeg + (gi + u) * 8 + 4 * h;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -359,12 +362,14 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < NG; ++u)
+    for (int u = 0; u < N; ++u)
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
   };
   size_t gi = gbeg;
-  for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>());
+  for (; gi + NG <= gend; gi += NG) run_groups(gi, std::integral_constant<int, NG>());
+  if (NG > 4)
+    for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>());
   for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>());
 
   if (nw > 1) {
@@ -479,11 +484,13 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     }
     g.tiles_m = (unsigned)wt_m; g.tiles_n = (unsigned)wt_n;
     const size_t tiles = wt_m * wt_n, groups = (K + 7) / 8;
-    // waves per workgroup: each keeps >= 4 groups of k (one unrolled batch of loads); then
+    // waves per workgroup (at most 8 for small problems, where 16 measured 10-15 % slower, at
+    // most 16 for large skinny ones, where 8 did): each keeps >= 4 groups of k; then
     // whole-grid splits of K until the chip has about 8 waves per CU, each split keeping >= 8
     // groups per wave
     unsigned nw = 1;
-    while (nw < 16 && groups >= (size_t)nw * 2 * 4) nw *= 2;
+    const bool small = 2.0 * (double)M * (double)N * (double)K <= 33554432.0;
+    while (nw < (small ? 8u : 16u) && groups >= (size_t)nw * 2 * 4) nw *= 2;
     size_t splits = 1;
     const size_t want = (size_t)ctx->num_cu * 8;
     if (tiles * nw < want) {
@@ -500,7 +507,11 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     g.k_chunk = k_chunk;
     dim3 wgrid((unsigned)tiles, (unsigned)splits);
     const size_t lds = nw > 1 ? (size_t)nw * 16 * 64 * sizeof(float) : 0;
-#define SL_WGEMM(TA_, TB_) hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_>), wgrid, dim3(64 * nw), lds, ctx->stream, g)
+#define SL_WGEMM(TA_, TB_)                                                                                        \
+  do {                                                                                                            \
+    if (small) hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_, 8>), wgrid, dim3(64 * nw), lds, ctx->stream, g);    \
+    else hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_, 1>), wgrid, dim3(64 * nw), lds, ctx->stream, g);          \
+  } while (0)
     if (!ta && !tb) SL_WGEMM(false, false);
     else if (!ta && tb) SL_WGEMM(false, true);
     else if (ta && !tb) SL_WGEMM(true, false);

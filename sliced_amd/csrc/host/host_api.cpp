@@ -140,6 +140,18 @@ SLH_API int slh_onehot(void* dev, size_t classes, uint64_t cls, uint64_t* out) {
     *out = d->onehot(classes, d->lookup(cls)).id;
   });
 }
+SLH_API int slh_mse_loss(void* dev, uint64_t x, uint64_t y, uint64_t* out) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    *out = d->mse_loss(d->lookup(x), d->lookup(y)).id;
+  });
+}
+SLH_API int slh_softmax_cce_loss(void* dev, size_t rows, size_t cols, uint64_t logits, uint64_t targets, uint64_t* out) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    *out = d->softmax_cce_loss(rows, cols, d->lookup(logits), d->lookup(targets)).id;
+  });
+}
 SLH_API int slh_transpose(void* dev, size_t rows, size_t cols, uint64_t x, uint64_t* out) {
   return guard([&] {
     HIP* d = (HIP*)dev;
@@ -177,7 +189,8 @@ SLH_API int slh_sgd_step(void* dev, uint64_t p, float lr) {
 // Three-layer MLP d_in -> d_h -> relu -> d_h -> relu -> d_out on a fresh device object.
 // kind 0 = sine fit (MSE on the tape), 1 = classifier (softmax + cce).  W1..b3 are updated in
 // place.  `warmup` untimed steps run first (they train too); seconds = wall time of `steps`.
-// mode: bit 0 = fused Linear forward, bit 1 = record one step as a graph and replay it.
+// mode: bit 0 = fused Linear forward, bit 1 = record one step as a graph and replay it,
+// bit 2 = fused loss kernels.
 SLH_API int slh_mlp_train(int ordinal, int kind, size_t batch, size_t d_in, size_t d_h, size_t d_out, const float* x,
                           const float* target, float* W1, float* b1, float* W2, float* b2, float* W3, float* b3,
                           float lr, size_t steps, size_t warmup, int mode, float* losses, double* seconds,

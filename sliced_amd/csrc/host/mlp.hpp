@@ -57,7 +57,8 @@ struct MlpResult {
 
 enum MlpMode {
   MLP_FUSED = 1,  // Linear (+ReLU) forward as one kernel
-  MLP_GRAPH = 2   // step 0 runs eagerly, step 1 is recorded, every later step replays the recording
+  MLP_GRAPH = 2,  // step 0 runs eagerly, step 1 is recorded, every later step replays the recording
+  MLP_FUSED_LOSS = 4  // the loss chain (MSE, or softmax + cross-entropy) as one forward and one backward kernel
 };
 
 // kind 0: MSE on the tape (sub, square, sum_cols, mul by 1/n; seed 1).
@@ -69,7 +70,7 @@ enum MlpMode {
 inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t d_h, size_t d_out, const float* x_host,
                            const float* target_host, float* const params[6], float lr, size_t steps, size_t warmup,
                            float* losses, int mode) {
-  const bool fused = (mode & MLP_FUSED) != 0, graph = (mode & MLP_GRAPH) != 0;
+  const bool fused = (mode & MLP_FUSED) != 0, graph = (mode & MLP_GRAPH) != 0, fused_loss = (mode & MLP_FUSED_LOSS) != 0;
   Linear lin1(dev, d_in, d_h, params[0], params[1]);
   Linear lin2(dev, d_h, d_h, params[2], params[3]);
   Linear lin3(dev, d_h, d_out, params[4], params[5]);
@@ -102,7 +103,12 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
       out = lin3.forward(h2);
     }
     float loss_val = 0.0f;
-    if (kind == 0) {
+    if (fused_loss) {
+      Buffer L = kind == 0 ? dev.mse_loss(out.data, y.data) : dev.softmax_cce_loss(batch, d_out, out.data, y.data);
+      if (deferred) dev.copy(L, 0, loss_dev, 0, 1);
+      else loss_val = L.read()[0];
+      L.backward();
+    } else if (kind == 0) {
       Matrix d = out.sub(y);
       Matrix q = d.squared();
       Matrix s = q.as_dims(1, n_out).sum_cols();  // one row: the sum over every element

@@ -455,6 +455,38 @@ class HIP {
     return out;
   }
 
+  // Fused losses (one forward and one backward kernel each instead of an op chain); the result is
+  // a one-element buffer on the tape, so `loss.backward()` works as for any other op.
+  // mean squared error == sub, squared, sum_cols over one row, mul by 1/n
+  Buffer mse_loss(const Buffer& x, const Buffer& y) {
+    if (x.len != y.len) throw Error("mse_loss: lengths differ");
+    Buffer out = retrieve(1);
+    check(slhip_mse(ctx_, x.len, x.ptr, y.ptr, out.ptr), "slhip_mse");
+    uint64_t xi = x.id, yi = y.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer xb = lookup(xi), yb = lookup(yi), o = lookup(oi);
+      check(slhip_mse_grad(ctx_, xb.len, xb.ptr, yb.ptr, grad_mut(xb).ptr, grad(o).ptr), "slhip_mse_grad");
+    });
+    return out;
+  }
+  // mean over the rows of the cross-entropy of softmax(logits) against `targets`
+  // == softmax on the tape + cce / cce_grad + backward_with of examples/nn.rs:124-152,229-233
+  Buffer softmax_cce_loss(size_t rows, size_t cols, const Buffer& logits, const Buffer& targets) {
+    expect(logits, rows * cols, "softmax_cce logits"); expect(targets, rows * cols, "softmax_cce targets");
+    Buffer probs = retrieve(rows * cols);
+    Buffer per_row = retrieve(rows);
+    Buffer out = retrieve(1);
+    check(slhip_softmax_cce(ctx_, rows, cols, logits.ptr, targets.ptr, probs.ptr, per_row.ptr), "slhip_softmax_cce");
+    check(slhip_mean(ctx_, rows, per_row.ptr, out.ptr), "slhip_mean");
+    uint64_t li = logits.id, ti = targets.id, pi = probs.id, oi = out.id;
+    add_grad_fn([=] {
+      Buffer l = lookup(li), t = lookup(ti), p = lookup(pi), o = lookup(oi);
+      check(slhip_softmax_cce_grad(ctx_, rows, cols, p.ptr, t.ptr, grad_mut(l).ptr, policy.softmax_beta, grad(o).ptr),
+            "slhip_softmax_cce_grad");
+    });
+    return out;
+  }
+
   // Mean::mean  src/ops2/mean/mod.rs:15-17 — a host scalar, not on the tape
   float mean(const Buffer& x) {
     Buffer s = scalar_scratch();

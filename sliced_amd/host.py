@@ -202,6 +202,12 @@ class HIP:
         """Matrix::l2_norm_cols (src/matrix.rs:337-355): squared().sum_cols().pow(1/2)."""
         return self.pow(self._red(SUM_COLS, cols, self.square(x), rows), 0.5)
 
+    def mse_loss(self, x, y):
+        return self._out(lib().slh_mse_loss, _u64(x.id), _u64(y.id))
+
+    def softmax_cce_loss(self, rows, cols, logits, targets):
+        return self._out(lib().slh_softmax_cce_loss, _sz(rows), _sz(cols), _u64(logits.id), _u64(targets.id))
+
     def transpose(self, rows, cols, x):
         return self._out(lib().slh_transpose, _sz(rows), _sz(cols), _u64(x.id))
 
@@ -264,7 +270,7 @@ def mlp_data(kind, batch, d_in, d_out, seed=rng.DEFAULT_SEED):
 
 
 def mlp_train(kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmup=0, fused=False, ordinal=0,
-              graph=False, info=None):
+              graph=False, info=None, fused_loss=False):
     """Runs the C++ training loop on the GPU.  params (six float32 arrays) are updated in place.
     graph=True records one step as a HIP graph and replays it (losses are read once at the end).
     Returns (losses[steps], seconds for the timed steps); info, a dict, receives graph_nodes."""
@@ -275,7 +281,7 @@ def mlp_train(kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmu
     x = np.ascontiguousarray(x, np.float32)
     target = np.ascontiguousarray(target, np.float32)
     _ck(lib().slh_mlp_train(ordinal, int(kind), _sz(batch), _sz(d_in), _sz(d_h), _sz(d_out), p(x), p(target),
-                            *[p(a) for a in params], _f(lr), _sz(steps), _sz(warmup), int(bool(fused)) | (2 if graph else 0),
+                            *[p(a) for a in params], _f(lr), _sz(steps), _sz(warmup), int(bool(fused)) | (2 if graph else 0) | (4 if fused_loss else 0),
                             p(losses), C.byref(secs), C.byref(nodes)))
     if info is not None:
         info["graph_nodes"] = nodes.value
@@ -286,12 +292,12 @@ C1 = dict(kind=0, batch=1024, d_in=1, d_h=64, d_out=1, lr=0.01, steps=200)
 C5 = dict(kind=1, batch=8192, d_in=784, d_h=2048, d_out=10, lr=0.05, steps=50)
 
 
-def run_config(cfg, fused, warmup=0, steps=None, graph=False, info=None):
+def run_config(cfg, fused, warmup=0, steps=None, graph=False, info=None, fused_loss=False):
     steps = steps or cfg["steps"]
     x, t = mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
     params = mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
     losses, secs = mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, params,
-                             cfg["lr"], steps, warmup, fused, graph=graph, info=info)
+                             cfg["lr"], steps, warmup, fused, graph=graph, info=info, fused_loss=fused_loss)
     return losses, secs, params
 
 
@@ -299,10 +305,11 @@ def bench_mlp(steps_c5=50, steps_c1=200):
     out = {}
     for name, cfg, steps in (("C5 classifier 784-2048-2048-10 batch 8192", C5, steps_c5),
                              ("C1 sine fit 1-64-64-1 batch 1024", C1, steps_c1)):
-        for fused, graph, label in ((False, False, "op by op"), (True, False, "fused linear"),
-                                    (True, True, "fused linear, recorded step replayed")):
+        for fused, graph, floss, label in ((False, False, False, "op by op"), (True, False, False, "fused linear"),
+                                           (True, True, False, "fused linear, recorded step replayed"),
+                                           (True, True, True, "fused linear and loss, recorded step replayed")):
             info = {}
-            losses, secs, _ = run_config(cfg, fused, warmup=5, steps=steps, graph=graph, info=info)
+            losses, secs, _ = run_config(cfg, fused, warmup=5, steps=steps, graph=graph, info=info, fused_loss=floss)
             out["%s (%s)" % (name, label)] = {
                 "steps_per_s": steps / secs, "ms_per_step": 1e3 * secs / steps,
                 "first_loss": float(losses[0]), "last_loss": float(losses[-1])}

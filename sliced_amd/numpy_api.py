@@ -377,6 +377,39 @@ def diagflat_grad(x_grad, out_grad):
     return x_grad
 
 
+def mse(x, y):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, dy, do = s.up(x), s.up(y), s.empty(1)
+        s.c.call("slhip_mse", x.size, dx.ptr, dy.ptr, do.ptr)
+        return do.numpy()[0]
+
+
+def mse_grad(x, y, x_grad, upstream=1.0):
+    x = _f32(x)
+    with _Scope() as s:
+        dx, dy, dg, du = s.up(x), s.up(y), s.up(x_grad), s.up(np.array([upstream], np.float32))
+        s.c.call("slhip_mse_grad", x.size, dx.ptr, dy.ptr, dg.ptr, du.ptr)
+        x_grad[:] = dg.numpy()
+    return x_grad
+
+
+def softmax_cce(rows, cols, logits, targets):
+    """(probs, loss per row)"""
+    with _Scope() as s:
+        dl, dt, dp, do = s.up(logits), s.up(targets), s.empty(rows * cols), s.empty(rows)
+        s.c.call("slhip_softmax_cce", rows, cols, dl.ptr, dt.ptr, dp.ptr, do.ptr)
+        return dp.numpy(), do.numpy()
+
+
+def softmax_cce_grad(rows, cols, probs, targets, logits_grad, beta=0.0, upstream=1.0):
+    with _Scope() as s:
+        dp, dt, dg, du = s.up(probs), s.up(targets), s.up(logits_grad), s.up(np.array([upstream], np.float32))
+        s.c.call("slhip_softmax_cce_grad", rows, cols, dp.ptr, dt.ptr, dg.ptr, float(beta), du.ptr)
+        logits_grad[:] = dg.numpy()
+    return logits_grad
+
+
 def onehot_grad(highest_class, classes, classes_grad, out_grad):
     classes = _f32(classes)
     with _Scope() as s:

@@ -447,6 +447,66 @@ def test_tanh_sigmoid_diagflat_onehot_grad(hip, orc):
                           orc.onehot_grad(10, cls, np.ones(5000, np.float32), og))
 
 
+@pytest.mark.parametrize("n", [1, 5, 1024, 4099, 1 << 20, 3000001])
+def test_fused_mse_against_the_op_chain(hip, orc, n):
+    """slhip_mse == sub, squared, sum over one row, mul by 1/n of the oracle; its gradient is the
+    chain's own product ((x-y)*2)*((1/n)*1), bit for bit."""
+    x = rng.uniform(n, -2, 2, tag=0, seed=SEED)
+    y = rng.uniform(n, -2, 2, tag=1, seed=SEED)
+    c = np.array([1.0 / n], np.float32)
+    d = orc.binary_ew(orc.SUB, x, y)
+    q = orc.unary(orc.SQUARE, d)
+    ref = orc.binary_ew(orc.MUL, orc.sum_cols(n, q), c)[0]
+    exact = np.sum(d.astype(np.float64) ** 2) / n
+    got = hip.mse(x, y)
+    assert abs(got - exact) <= 1e-6 * exact + 1e-37
+    assert abs(got - ref) <= 1e-6 * exact + abs(ref - exact)
+    xg0 = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+    for up in (1.0, -0.25):
+        gs, _ = orc.binary_ew_grad(orc.MUL, np.zeros(1, np.float32), c, np.zeros(1, np.float32), np.zeros(1, np.float32),
+                                   np.array([up], np.float32))                       # s.grad = c * upstream
+        qg = orc.sum_cols_grad(n, np.zeros(n, np.float32), gs)
+        dg = orc.unary_grad(orc.SQUARE, d, np.zeros(n, np.float32), qg)
+        want, _ = orc.binary_ew_grad(orc.SUB, x, y, xg0.copy(), np.zeros(n, np.float32), dg)
+        assert np.array_equal(hip.mse_grad(x, y, xg0.copy(), up), want)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (7, 3), (8192, 10), (300, 1000), (5, 70001)], ids=lambda s: "x".join(map(str, s)))
+def test_fused_softmax_cross_entropy_against_the_op_chain(hip, orc, shape):
+    rows, cols = shape
+    n = rows * cols
+    x = rng.normal(n, 3.0, tag=0, seed=SEED)
+    cls = rng.integers(rows, cols, tag=1, seed=SEED)
+    t = np.zeros((rows, cols), np.float32)
+    t[np.arange(rows), cls] = 1.0
+    t = t.ravel()
+    p_ref = orc.softmax(rows, cols, x)
+    loss_ref = orc.cce(rows, cols, p_ref, t)
+    p, loss = hip.softmax_cce(rows, cols, x, t)
+    X = x.reshape(rows, cols).astype(np.float64)
+    sh = (x.reshape(rows, cols) - x.reshape(rows, cols).max(1, keepdims=True)).astype(np.float32).astype(np.float64)
+    P = np.exp(sh) / np.exp(sh).sum(1, keepdims=True)
+    assert np.all(np.abs(p.reshape(rows, cols) - P) <= 1e-6 * P + 1e-37)
+    L = -np.log(np.sum(np.clip(P, 1e-7, 1 - 1e-7) * t.reshape(rows, cols), 1))
+    assert np.all(np.abs(loss - L) <= 2e-6 * np.maximum(np.abs(L), 1.0))
+    assert np.all(np.abs(loss - loss_ref) <= 2e-6 * np.maximum(np.abs(L), 1.0) + np.abs(loss_ref - L))
+    # gradient of mean_r loss_r wrt the logits: (p - t)/rows; the reference's chain is cce_grad
+    # (unclipped p) pushed through softmax_grad
+    for beta, up in ((0.0, 1.0), (1.0, 0.5)):
+        lg0 = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+        got = hip.softmax_cce_grad(rows, cols, p, t, lg0.copy(), beta, up)
+        exact = beta * lg0 + up * (p.astype(np.float64) - t) / rows
+        bound = 2e-6 * (np.abs(p) + np.abs(t)) * abs(up) / rows + 1e-7 * np.abs(beta * lg0) + 1e-37
+        assert np.all(np.abs(got - exact) <= bound)
+    seed = orc.cce_grad(rows, cols, p_ref, t)
+    if np.all(np.isfinite(seed)):                       # the chain divides by p: inf once a probability underflows
+        chain = orc.softmax_grad(rows, cols, p_ref, seed)
+        got = hip.softmax_cce_grad(rows, cols, p, t, np.zeros(n, np.float32))
+        exact = (P - t.reshape(rows, cols)).ravel() / rows
+        scale = (np.abs(P) + 1.0).ravel() / rows
+        assert np.all(np.abs(got - chain) <= 4e-6 * scale + np.abs(chain - exact))
+
+
 def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):
     """Eleven tensors (two launches of up to eight), aligned and not, one of them long."""
     c = hip.ctx()

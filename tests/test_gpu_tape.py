@@ -382,3 +382,34 @@ def test_recorded_step_replays_match_the_eager_loop(orc, name, steps):
         p_ref = [a.copy() for a in p0]
         ref = orc.mlp_train(*args, p_ref, cfg["lr"], steps)
         assert loss_parity(eager, ref, 1e-4) <= 1e-4
+
+
+@pytest.mark.parametrize("name,steps", [("C1", 200), ("C5", 50)])
+def test_fused_loss_training_matches_oracle_and_its_own_replay(orc, name, steps):
+    """Fused Linear + fused loss kernels: per-step loss within 1e-4 of the oracle's op-by-op loop;
+    the replayed recording bit-identical to the eager run of the same kernels."""
+    from sliced_amd import host
+    cfg = host.C1 if name == "C1" else host.C5
+    say(name, "fused loss,", steps, "steps")
+    x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+    p0 = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+    args = (cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t)
+    global _C5_REF
+    if name == "C5" and "_C5_REF" in globals():
+        ref = _C5_REF
+    else:
+        ref = orc.mlp_train(*args, [a.copy() for a in p0], cfg["lr"], steps)
+        if name == "C5":
+            _C5_REF = ref
+    p_eager = [a.copy() for a in p0]
+    eager, _ = host.mlp_train(*args, p_eager, cfg["lr"], steps, 0, True, fused_loss=True)
+    worst = loss_parity(eager, ref, 1e-4)
+    say(name, "fused loss: worst relative loss deviation", worst)
+    assert np.all(np.isfinite(eager)) and worst <= 1e-4
+    p_graph = [a.copy() for a in p0]
+    info = {}
+    got, _ = host.mlp_train(*args, p_graph, cfg["lr"], steps, 0, True, graph=True, info=info, fused_loss=True)
+    say(name, "kernels per recorded step:", info["graph_nodes"])
+    assert np.array_equal(got, eager)
+    for a, b in zip(p_graph, p_eager):
+        assert np.array_equal(a, b)
