@@ -534,6 +534,37 @@ def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):
     pool_g.free()
 
 
+# --------------------------------------------------------------------------- runtime
+def test_context_on_a_callers_stream(hip, orc):
+    """slhip_init_on_stream: ops run on a stream the caller created and still owns afterwards."""
+    from sliced_amd import _lib
+    rt = C.CDLL("libamdhip64.so")
+    stream = C.c_void_p()
+    assert rt.hipStreamCreate(C.byref(stream)) == 0
+    lib = _lib.load()
+    h = C.c_void_p()
+    assert lib.slhip_init_on_stream(0, stream, C.byref(h)) == 0
+    got = C.c_void_p()
+    assert lib.slhip_stream(h, C.byref(got)) == 0 and got.value == stream.value
+    assert lib.slhip_workspace_bytes(h) >= (64 << 20)
+    name = C.create_string_buffer(64)
+    assert lib.slhip_device_name(h, name, 64) == 0 and b"gfx950" in name.value
+    n = 1000
+    x = rng.uniform(n, -1, 1, tag=0, seed=SEED)
+    dx, dy = C.c_void_p(), C.c_void_p()
+    assert lib.slhip_malloc(h, 4 * n, C.byref(dx)) == 0 and lib.slhip_malloc(h, 4 * n, C.byref(dy)) == 0
+    assert lib.slhip_memcpy_h2d(h, dx, x.ctypes.data, 4 * n) == 0
+    assert lib.slhip_ew_unary(h, 0, 0.0, 0.0, n, dx, dy) == 0           # square, on the caller's stream
+    assert rt.hipStreamSynchronize(stream) == 0                          # the caller waits on its own stream
+    out = np.empty(n, np.float32)
+    assert lib.slhip_memcpy_d2h(h, out.ctypes.data, dy, 4 * n) == 0
+    assert np.array_equal(out, orc.unary(orc.SQUARE, x))
+    assert lib.slhip_free(h, dx) == 0 and lib.slhip_free(h, dy) == 0
+    assert lib.slhip_destroy(h) == 0
+    assert rt.hipStreamQuery(stream) == 0                                # still a valid, idle stream
+    assert rt.hipStreamDestroy(stream) == 0
+
+
 # --------------------------------------------------------------------------- error behaviour
 def test_invalid_arguments_return_status_not_crash(hip):
     c = hip.ctx()
