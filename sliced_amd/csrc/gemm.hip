@@ -325,7 +325,9 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 // NG = groups of 8 k whose loads are issued together: 8 for small problems (latency is all that
 // matters: [1024x64]x[64x64] 7.2 -> 5.9 us), 1 for large skinny ones, which have waves enough to
 // hide latency and measured 15-20 % slower with 2, 4 or 8 (8192x10x2048: 41 us against 48).
-template <bool TA, bool TB, int NG>
+// FULL = every k range is a whole number of groups and the k-contiguous operands are 16-byte
+// loadable: no bounds checks, and a k-contiguous operand comes in as one float4 per group.
+template <bool TA, bool TB, int NG, bool FULL>
 __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
   extern __shared__ float red[];  // [waves][16][64]
   const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6, nw = blockDim.x >> 6;
@@ -352,13 +354,30 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
 #pragma unroll
     for (int u = 0; u < N; ++u) {
       const size_t k = kbeg + (gi + u) * 8 + 4 * h;
+      if (FULL) {
+        if (!TA) {
+          const float4 v = ld4(ap + k);
+          a[u][0] = v.x; a[u][1] = v.y; a[u][2] = v.z; a[u][3] = v.w;
+        } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const bool in = k + t < kend;
-        const size_t kc = in ? k + t : kend - 1;
-        const float av = ap[kc * astep], bv = bp[kc * bstep];
-        a[u][t] = in ? av : 0.0f;
-        b[u][t] = in ? bv : 0.0f;
+          for (int t = 0; t < 4; ++t) a[u][t] = ap[(k + t) * astep];
+        }
+        if (TB) {
+          const float4 v = ld4(bp + k);
+          b[u][0] = v.x; b[u][1] = v.y; b[u][2] = v.z; b[u][3] = v.w;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) b[u][t] = bp[(k + t) * bstep];
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const bool in = k + t < kend;
+          const size_t kc = in ? k + t : kend - 1;
+          const float av = ap[kc * astep], bv = bp[kc * bstep];
+          a[u][t] = in ? av : 0.0f;
+          b[u][t] = in ? bv : 0.0f;
+        }
       }
     }
 #pragma unroll
@@ -475,8 +494,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   g.partial = (float*)ctx->workspace;
   const size_t mn_bytes = M * N * sizeof(float);
 
-  // Small (<= 2^25 flop) and skinny (an output side <= 32, or K <= 16) products: wave-per-tile kernel.
-  if (2.0 * (double)M * (double)N * (double)K <= 33554432.0 || M <= 32 || N <= 32 || K <= 16) {
+  // Small and skinny (an output side <= 32, or K <= 16) products: wave-per-tile kernel.  "Small" is
+  // <= 6e8 flop when the kernel can use its unchecked vector-load form (it then beats the tiled
+  // kernel up to about 700^3: 512^3 takes 7.2 us against 17.4), <= 2^25 flop otherwise.
+  const double flop = 2.0 * (double)M * (double)N * (double)K;
+  const bool wave_full = K % 8 == 0 && (ta || g.a_vec) && (!tb || g.b_vec);
+  if (flop <= (wave_full ? 6.0e8 : 33554432.0) || M <= 32 || N <= 32 || K <= 16) {
     const size_t wt_m = (M + 31) / 32, wt_n = (N + 31) / 32;
     if (wt_m * wt_n > 0x7fffffffu) {
       set_error("sgemm: %zu x %zu tiles exceed one launch", wt_m, wt_n);
@@ -489,7 +512,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     // whole-grid splits of K until the chip has about 8 waves per CU, each split keeping >= 8
     // groups per wave
     unsigned nw = 1;
-    const bool small = 2.0 * (double)M * (double)N * (double)K <= 33554432.0;
+    const bool small = flop <= 33554432.0;
     while (nw < (small ? 8u : 16u) && groups >= (size_t)nw * 2 * 4) nw *= 2;
     size_t splits = 1;
     const size_t want = (size_t)ctx->num_cu * 8;
@@ -507,16 +530,23 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     g.k_chunk = k_chunk;
     dim3 wgrid((unsigned)tiles, (unsigned)splits);
     const size_t lds = nw > 1 ? (size_t)nw * 16 * 64 * sizeof(float) : 0;
-#define SL_WGEMM(TA_, TB_)                                                                                        \
-  do {                                                                                                            \
-    if (small) hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_, 8>), wgrid, dim3(64 * nw), lds, ctx->stream, g);    \
-    else hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_, 1>), wgrid, dim3(64 * nw), lds, ctx->stream, g);          \
+    // whole groups of 8 k everywhere (k_chunk is a multiple of 8) and float4-loadable k-contiguous operands
+    const bool full = wave_full;
+#define SL_WGEMM2(TA_, TB_, NG_, FULL_) \
+  hipLaunchKernelGGL((gemm_wave_kernel<TA_, TB_, NG_, FULL_>), wgrid, dim3(64 * nw), lds, ctx->stream, g)
+#define SL_WGEMM(TA_, TB_)                                   \
+  do {                                                       \
+    if (small && full) SL_WGEMM2(TA_, TB_, 8, true);         \
+    else if (small) SL_WGEMM2(TA_, TB_, 8, false);           \
+    else if (full) SL_WGEMM2(TA_, TB_, 1, true);             \
+    else SL_WGEMM2(TA_, TB_, 1, false);                      \
   } while (0)
     if (!ta && !tb) SL_WGEMM(false, false);
     else if (!ta && tb) SL_WGEMM(false, true);
     else if (ta && !tb) SL_WGEMM(true, false);
     else SL_WGEMM(true, true);
 #undef SL_WGEMM
+#undef SL_WGEMM2
     int32_t rc = post_launch();
     if (rc || splits == 1) return rc;
     return splitk_combine(ctx, g, splits);
