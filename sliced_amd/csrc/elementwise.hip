@@ -68,9 +68,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_kernel(size_t n, EwArgs<NIN, NOUT
 template <int NIN, int NOUT, class F>
 int32_t ew_launch(slhip_ctx* ctx, size_t n, EwArgs<NIN, NOUT, F> a) {
   if (n == 0) return SLHIP_OK;
-  bool vec = true;
-  for (int j = 0; j < NIN; ++j) vec = vec && aligned16(a.in[j]);
-  for (int j = 0; j < NOUT; ++j) vec = vec && aligned16(a.out[j]);
+  const bool vec = true;  // dword-aligned vector accesses: any float* qualifies
   const size_t threads = vec ? ((n >> 2) > 3 ? (n >> 2) : 4) : n;
   const size_t blocks = (threads + EW_BLOCK - 1) / EW_BLOCK;
   if (blocks > 0x7fffffffu) {
@@ -209,8 +207,8 @@ __global__ __launch_bounds__(EW_BLOCK) void bcast_kernel(size_t rows, size_t col
     if (MODE == 0 || MODE == 3) { t = ld4s(a + off); av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w; }
     if (MODE != 0) { t = ld4s(out + off); o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w; }
     if (MODE == 2) { vv[0] = vv[1] = vv[2] = vv[3] = DIVCOLS ? v[r] / s : v[r]; }
-    else { t = ld4(v + c); vv[0] = t.x; vv[1] = t.y; vv[2] = t.z; vv[3] = t.w; }
-    if (MODE == 3) { t = ld4(g + c); gv[0] = t.x; gv[1] = t.y; gv[2] = t.z; gv[3] = t.w; }
+    else { t = ld4g(v + c); vv[0] = t.x; vv[1] = t.y; vv[2] = t.z; vv[3] = t.w; }
+    if (MODE == 3) { t = ld4g(g + c); gv[0] = t.x; gv[1] = t.y; gv[2] = t.z; gv[3] = t.w; }
   } else {
     if (MODE == 0 || MODE == 3) av[0] = a[off];
     if (MODE != 0) o[0] = out[off];
@@ -231,8 +229,7 @@ __global__ __launch_bounds__(EW_BLOCK) void bcast_kernel(size_t rows, size_t col
 template <int MODE, bool DIVCOLS = false>
 int32_t bcast_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* a, const float* v, const float* g,
                      float* out, float s) {
-  bool vec = (cols % 4 == 0) && aligned16(out) && (MODE == 2 || aligned16(v)) &&
-             ((MODE != 0 && MODE != 3) || aligned16(a)) && (MODE != 3 || aligned16(g));
+  bool vec = cols % 4 == 0;  // a thread's vector must lie inside one row; alignment does not matter
   const size_t total = rows * (vec ? cols / 4 : cols);
   const size_t blocks = (total + EW_BLOCK - 1) / EW_BLOCK;
   if (blocks > 0x7fffffffu) {
@@ -395,10 +392,10 @@ __global__ __launch_bounds__(256) void sgd_multi_kernel(SgdMultiArgs a, float lr
   if (a.vec[t]) {
     const size_t n4 = n / 4;
     for (size_t i = tid; i < n4; i += stride) {
-      float4 pv = ld4(p + 4 * i);
-      const float4 gv = ld4(g + 4 * i);
+      float4 pv = ld4g(p + 4 * i);
+      const float4 gv = ld4g(g + 4 * i);
       pv.x -= gv.x * lr; pv.y -= gv.y * lr; pv.z -= gv.z * lr; pv.w -= gv.w * lr;
-      st4(p + 4 * i, pv);
+      st4g(p + 4 * i, pv);
     }
     done = n4 * 4;
   }
@@ -417,7 +414,7 @@ SLHIP_API int32_t slhip_sgd_step_multi(slhip_ctx* ctx, size_t count, float* cons
     for (size_t i = 0; i < (size_t)SGD_MULTI_MAX; ++i) {
       const size_t j = first + (i < m ? i : 0);  // unused slots repeat the first tensor; no block reads them
       a.p[i] = params[j]; a.g[i] = grads[j]; a.n[i] = lens[j];
-      a.vec[i] = aligned16(params[j]) && aligned16(grads[j]);
+      a.vec[i] = 1;
       if (i < m && lens[j] > longest) longest = lens[j];
     }
     size_t blocks = (longest / 4 + 255) / 256 + 1;

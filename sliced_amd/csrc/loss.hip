@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void mse_partial_kernel(size_t n, const float*
   float s = 0.0f;
   if (vec) {  // chunk is a multiple of 4 (always) and both pointers are 16-byte aligned
     for (size_t i = beg + 4 * (size_t)threadIdx.x; i + 3 < end; i += 1024) {
-      const float4 a = ld4(x + i), b = ld4(y + i);
+      const float4 a = ld4g(x + i), b = ld4g(y + i);
       const float d0 = a.x - b.x, d1 = a.y - b.y, d2 = a.z - b.z, d3 = a.w - b.w;
       s += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
     }
@@ -123,7 +123,7 @@ SLHIP_API int32_t slhip_mse(slhip_ctx* ctx, size_t n, const float* x, const floa
   }
   const size_t chunk = ((n + blocks - 1) / blocks + 3) / 4 * 4;
   blocks = (n + chunk - 1) / chunk;
-  const int vec = aligned16(x) && aligned16(y);
+  const int vec = 1;
   float* part = (float*)ctx->workspace;
   hipLaunchKernelGGL(mse_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, y, part, chunk, vec);
   int32_t rc = post_launch();

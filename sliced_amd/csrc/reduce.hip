@@ -115,7 +115,7 @@ template <class Op>
 static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
   // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
   if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, rows * sizeof(float));
-  const bool vec = (cols % 4 == 0) && aligned16(x);
+  const bool vec = cols % 4 == 0;
   const size_t colsv = cols / (vec ? 4 : 1);
   // few long rows: split every row so the whole chip is busy
   unsigned nseg = 1;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void colreduce_kernel(size_t rows, size_t cols
     }
     SL_ACC(a0, a1) SL_ACC(a2, a3) SL_ACC(a0, a2)
 #undef SL_ACC
-    st4(part + g * cols + cv * 4, a0);
+    st4g(part + g * cols + cv * 4, a0);
   } else {
     float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
     for (; r + 3 * G < rows; r += 4 * G, p += 4 * step) {
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(1024) void fullreduce_final_kernel(size_t n, const 
 
 template <class Op>
 static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin) {
-  const bool vec = aligned16(x);
+  const bool vec = true;
   size_t items = vec ? (n >> 2) + 1 : n;
   size_t blocks = (items + 256 * 16 - 1) / (256 * 16);
   size_t cap = (size_t)ctx->num_cu * 8;
@@ -305,7 +305,7 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
   if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin);
   // one row: the reduction over rows is that row itself
   if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, cols * sizeof(float));
-  const bool vec = (cols % 4 == 0) && aligned16(x);
+  const bool vec = cols % 4 == 0;
   const size_t colsv = cols / (vec ? 4 : 1);
   // number of row groups: about 512 threads per CU (measured optimum: 7.0 TB/s at 131072
   // threads on [16384 x 16384]; 5.4 TB/s at four times as many), at least 16 rows per thread

@@ -193,7 +193,7 @@ SLHIP_API int32_t slhip_memcpy_d2d(slhip_ctx* ctx, void* dst, const void* src, s
   SLHIP_REQUIRE(ctx && dst && src, "null argument");
   if (bytes == 0 || dst == src) return SLHIP_OK;
   size_t done = 0;
-  if (bytes >= 4096 && aligned16(dst) && aligned16(src)) {
+  if (bytes >= 4096 && (((uintptr_t)dst | (uintptr_t)src) & 3) == 0) {
     const size_t n4 = bytes / 16;
     SLHIP_REQUIRE((n4 + 63) / 64 <= 0x7fffffffu, "copy too large for one launch");
     hipLaunchKernelGGL(copy4_kernel, dim3((unsigned)((n4 + 63) / 64)), dim3(64), 0, ctx->stream, n4,

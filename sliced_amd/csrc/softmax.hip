@@ -251,7 +251,7 @@ SLHIP_API int32_t slhip_softmax(slhip_ctx* ctx, size_t samples, size_t features,
   SLHIP_REQUIRE(ctx && x && out, "null argument");
   SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
   SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
-  const bool vec = (features % 4 == 0) && aligned16(x) && aligned16(out);
+  const bool vec = features % 4 == 0;
   return vec ? softmax_dispatch<true, true>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f)
              : softmax_dispatch<true, false>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f);
 }
@@ -262,7 +262,7 @@ SLHIP_API int32_t slhip_softmax_grad(slhip_ctx* ctx, size_t samples, size_t feat
   SLHIP_REQUIRE(ctx && x_grad && out && out_grad, "null argument");
   SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
   SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
-  const bool vec = (features % 4 == 0) && aligned16(x_grad) && aligned16(out) && aligned16(out_grad);
+  const bool vec = features % 4 == 0;
   return vec ? softmax_dispatch<false, true>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta)
              : softmax_dispatch<false, false>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta);
 }

@@ -534,6 +534,67 @@ def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):
     pool_g.free()
 
 
+# --------------------------------------------------------------------------- views at odd offsets
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_operands_that_are_only_float_aligned(hip, orc, off):
+    """Every operand sits `off` floats into its allocation (and outputs at a different offset): the
+    vector paths must not assume 16-byte alignment.  Same bars as for aligned operands."""
+    c = hip.ctx()
+    rows, cols = 300, 1024
+    n = rows * cols
+    x = rng.uniform(n, -3, 3, tag=0, seed=SEED)
+    g = rng.normal(n, 1.0, tag=1, seed=SEED)
+    pool_x, pool_g = c.empty(n + 8), c.empty(n + 8)
+    pool_o, pool_v = c.zeros(n + 8), c.zeros(max(rows, cols) + 8)
+    dx, dg = pool_x.view(off, n), pool_g.view(off, n)
+    oo = (off + 1) % 4
+    do = pool_o.view(oo, n)
+    dx.upload(x); dg.upload(g)
+    vr, vc = pool_v.view(off, rows), pool_v.view(off, cols)
+    say("offset", off)
+    # reductions
+    c.call("slhip_max_cols", rows, cols, dx.ptr, vr.ptr); assert np.array_equal(vr.numpy(), orc.max_cols(cols, x))
+    c.call("slhip_max_rows", rows, cols, dx.ptr, vc.ptr); assert np.array_equal(vc.numpy(), orc.max_rows(cols, x))
+    c.call("slhip_sum_cols", rows, cols, dx.ptr, vr.ptr)
+    assert np.all(np.abs(vr.numpy() - x.reshape(rows, cols).sum(1, dtype=np.float64)) <= sum_bound(x, rows, cols, 1))
+    c.call("slhip_sum_rows", rows, cols, dx.ptr, vc.ptr)
+    assert np.all(np.abs(vc.numpy() - x.reshape(rows, cols).sum(0, dtype=np.float64)) <= sum_bound(x, rows, cols, 0))
+    one = pool_v.view(off, 1)
+    c.call("slhip_sum", n, dx.ptr, one.ptr)
+    assert abs(float(one.numpy()[0]) - x.sum(dtype=np.float64)) <= 1e-6 * np.abs(x).sum(dtype=np.float64)
+    # transpose, elementwise, bias row op: bit-exact
+    c.call("slhip_transpose", rows, cols, dx.ptr, do.ptr, 0.0); assert np.array_equal(do.numpy(), orc.transpose(rows, cols, x))
+    c.call("slhip_ew_binary", orc.MUL, n, dx.ptr, dg.ptr, do.ptr); assert np.array_equal(do.numpy(), orc.binary_ew(orc.MUL, x, g))
+    c.call("slhip_ew_unary", orc.RELU, 0.0, 0.0, n, dx.ptr, do.ptr); assert np.array_equal(do.numpy(), orc.unary(orc.RELU, x))
+    bias = x[:cols].copy()
+    vc.upload(bias)
+    c.call("slhip_add_row", rows, cols, dx.ptr, vc.ptr, do.ptr); assert np.array_equal(do.numpy(), orc.add_row(rows, cols, x, bias))
+    c.call("slhip_memcpy_d2d", do.ptr, dx.ptr, 4 * n); assert np.array_equal(do.numpy(), x)
+    # softmax forward / backward
+    c.call("slhip_softmax", rows, cols, dx.ptr, do.ptr)
+    s = do.numpy()
+    ref = orc.softmax(rows, cols, x)
+    assert np.all(np.abs(s - ref) <= 2e-6 * ref + 1e-37)
+    c.call("slhip_softmax_grad", rows, cols, pool_x.view(oo, n).ptr, do.ptr, dg.ptr, 0.0)   # x's pool is free to overwrite now
+    got = pool_x.view(oo, n).numpy()
+    ob = orc.softmax_grad(rows, cols, s, g)
+    S, G = s.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
+    bound = 2e-6 * (np.abs(S) * (np.abs(G) + (np.abs(S) * np.abs(G)).sum(1, keepdims=True))).ravel() + 1e-37
+    assert np.all(np.abs(got - ob) <= bound)
+    # GEMM, all forms, tiled and wave-per-tile sizes
+    for (m, nn, k) in [(300, 256, 512), (96, 40, 64)]:
+        a = rng.uniform(m * k, -1, 1, tag=3, seed=SEED)
+        b = rng.uniform(k * nn, -1, 1, tag=4, seed=SEED)
+        da, db, dc = pool_x.view(off, m * k), pool_g.view(off, k * nn), pool_o.view(oo, m * nn)
+        da.upload(a); db.upload(b)
+        for ta, tb in ((0, 0), (0, 1), (1, 0)):
+            c.call("slhip_sgemm", ta, tb, m, nn, k, da.ptr, db.ptr, dc.ptr, 0.0)
+            exact, bound = gemm_bound(ta, tb, m, nn, k, a, b)
+            assert np.all(np.abs(dc.numpy() - exact) <= bound), (m, nn, k, ta, tb)
+    for z in (pool_x, pool_g, pool_o, pool_v):
+        z.free()
+
+
 # --------------------------------------------------------------------------- runtime
 def test_context_on_a_callers_stream(hip, orc):
     """slhip_init_on_stream: ops run on a stream the caller created and still owns afterwards."""
