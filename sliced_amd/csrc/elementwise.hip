@@ -226,23 +226,68 @@ __global__ __launch_bounds__(EW_BLOCK) void bcast_kernel(size_t rows, size_t col
   else out[off] = o[0];
 }
 
+// Rows of odd length: the matrix is walked as one flat run of vectors, each element finds its
+// own row and column (one division per thread, then increments).
+template <int MODE, bool DIVCOLS, class IDX>
+__global__ __launch_bounds__(EW_BLOCK) void bcast_flat_kernel(size_t len, size_t cols, const float* a,
+                                                              const float* __restrict__ v, const float* __restrict__ g,
+                                                              float* out, float s) {
+  const size_t i = (size_t)blockIdx.x * EW_BLOCK + threadIdx.x;
+  const size_t e0 = 4 * i;
+  if (e0 >= len) return;
+  IDX r = (IDX)e0 / (IDX)cols;
+  IDX c = (IDX)e0 - r * (IDX)cols;
+  const bool whole = e0 + 3 < len;
+  float av[4] = {0.f, 0.f, 0.f, 0.f}, o[4] = {0.f, 0.f, 0.f, 0.f};
+  if (whole) {
+    float4 t;
+    if (MODE == 0 || MODE == 3) { t = ld4s(a + e0); av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w; }
+    if (MODE != 0) { t = ld4s(out + e0); o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w; }
+  } else {
+    for (size_t q = 0; e0 + q < len; ++q) {
+      if (MODE == 0 || MODE == 3) av[q] = a[e0 + q];
+      if (MODE != 0) o[q] = out[e0 + q];
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (e0 + q < len) {
+      if (MODE == 0) o[q] = av[q] + v[c];
+      else if (MODE == 1) o[q] += s * v[c];
+      else if (MODE == 2) o[q] += DIVCOLS ? v[r] / s : v[r];
+      else if (av[q] == v[c]) o[q] += g[c];
+    }
+    if (++c == (IDX)cols) { c = 0; ++r; }
+  }
+  if (whole) st4s(out + e0, make_float4(o[0], o[1], o[2], o[3]));
+  else
+    for (size_t q = 0; e0 + q < len; ++q) out[e0 + q] = o[q];
+}
+
 template <int MODE, bool DIVCOLS = false>
 int32_t bcast_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* a, const float* v, const float* g,
                      float* out, float s) {
-  bool vec = cols % 4 == 0;  // a thread's vector must lie inside one row; alignment does not matter
-  const size_t total = rows * (vec ? cols / 4 : cols);
+  const bool vec = cols % 4 == 0;  // a thread's vector lies inside one row; alignment does not matter
+  const size_t total = vec ? rows * (cols / 4) : (rows * cols + 3) / 4;
   const size_t blocks = (total + EW_BLOCK - 1) / EW_BLOCK;
   if (blocks > 0x7fffffffu) {
     set_error("broadcast op: %zu x %zu exceeds one launch", rows, cols);
     return SLHIP_EINVAL;
   }
-  const bool small = total <= 0xffffffffu;
-#define SL_BC(VECF, IDXT)                                                                                        \
-  hipLaunchKernelGGL((bcast_kernel<MODE, VECF, DIVCOLS, IDXT>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, ctx->stream, \
+  const bool small = rows * cols <= 0xffffffffu;  // 32-bit index arithmetic whenever the matrix allows it
+  if (vec) {
+#define SL_BC(IDXT)                                                                                                  \
+  hipLaunchKernelGGL((bcast_kernel<MODE, true, DIVCOLS, IDXT>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, ctx->stream, \
                      rows, cols, a, v, g, out, s)
-  if (vec) { if (small) SL_BC(true, uint32_t); else SL_BC(true, size_t); }
-  else { if (small) SL_BC(false, uint32_t); else SL_BC(false, size_t); }
+    if (small) SL_BC(uint32_t); else SL_BC(size_t);
 #undef SL_BC
+  } else {
+#define SL_BF(IDXT)                                                                                                      \
+  hipLaunchKernelGGL((bcast_flat_kernel<MODE, DIVCOLS, IDXT>), dim3((unsigned)blocks), dim3(EW_BLOCK), 0, ctx->stream, \
+                     rows * cols, cols, a, v, g, out, s)
+    if (small) SL_BF(uint32_t); else SL_BF(size_t);
+#undef SL_BF
+  }
   return post_launch();
 }
 

@@ -17,7 +17,10 @@ __device__ __forceinline__ float row_reduce(float v, float* smem) {
   return block_reduce<Op>(v, smem);
 }
 
-template <bool VEC, int LANES, int ITEMS>
+// TAIL: the row length is not a multiple of 4 (VEC only): lane 0 also takes the up to 3 floats
+// beyond the last whole vector.  A template parameter because even an untaken tail costs the
+// whole-vector rows 10-15 % of their bandwidth.
+template <bool VEC, int LANES, int ITEMS, bool TAIL>
 __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(size_t rows, size_t cols,
                                                                                 const float* __restrict__ x,
                                                                                 float* __restrict__ out) {
@@ -59,10 +62,17 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
       }
     }
   }
+  // a row of odd length ends in up to 3 floats beyond its last whole vector: lane 0 takes them
+  const int rem = TAIL ? (int)(cols & 3) : 0;
+  const bool tail = TAIL && rem != 0 && active && lane == 0;
+  float tv[3] = {NEG_INF, NEG_INF, NEG_INF};
+  if (tail)
+    for (int q = 0; q < rem; ++q) tv[q] = x[row * cols + 4 * colsv + q];
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
     for (int q = 0; q < V; ++q) m = fmaxf(m, v[j][q]);
+  if (TAIL) m = fmaxf(m, fmaxf(tv[0], fmaxf(tv[1], tv[2])));
   m = row_reduce<MaxOp, LANES>(m, smem);
 
   float s = 0.0f;
@@ -77,7 +87,14 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
       s += e;
     }
   }
+  if (tail)
+    for (int q = 0; q < rem; ++q) {
+      tv[q] = expf(tv[q] - m);
+      s += tv[q];
+    }
   s = row_reduce<SumOp, LANES>(s, smem);
+  if (tail)
+    for (int q = 0; q < rem; ++q) out[row * cols + 4 * colsv + q] = tv[q] / s;
 
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
@@ -90,7 +107,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
   }
 }
 
-template <bool VEC, int LANES, int ITEMS>
+template <bool VEC, int LANES, int ITEMS, bool TAIL>
 __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(size_t rows, size_t cols,
                                                                                 float* x_grad,
                                                                                 const float* __restrict__ out,
@@ -142,7 +159,23 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
   for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
     for (int q = 0; q < V; ++q) dot += s[j][q] * g[j][q];
+  // the up to 3 floats beyond the last whole vector of a row of odd length: lane 0 takes them
+  const int rem = TAIL ? (int)(cols & 3) : 0;
+  const bool tail = TAIL && rem != 0 && active && lane == 0;
+  float ts[3] = {0.f, 0.f, 0.f}, tg[3] = {0.f, 0.f, 0.f};
+  if (tail)
+    for (int q = 0; q < rem; ++q) {
+      ts[q] = out[row * cols + 4 * colsv + q];
+      tg[q] = out_grad[row * cols + 4 * colsv + q];
+      dot += ts[q] * tg[q];
+    }
   dot = row_reduce<SumOp, LANES>(dot, smem);
+  if (tail)
+    for (int q = 0; q < rem; ++q) {
+      float* p = x_grad + row * cols + 4 * colsv + q;
+      const float r = ts[q] * (tg[q] - dot);
+      *p = beta != 0.0f ? beta * *p + r : r;
+    }
 
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
@@ -167,20 +200,43 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
   }
 }
 
-// Rows too long for registers: one block per row, three sweeps over global memory (the later
-// sweeps hit L2 for rows up to a few MB).
+// Rows too long for registers: one block per row and two sweeps over global memory, float4 at
+// a time with a scalar tail.  The first sweep keeps a running maximum and a sum of exponentials
+// relative to it per thread (rescaled whenever the maximum moves); the block then combines the
+// per-thread pairs, and the second sweep (which finds the row in L2 or the memory-side cache)
+// writes exp(x - max) / sum.
+__device__ __forceinline__ void online_add(float& m, float& s, float v) {
+  if (v > m) {
+    s = s * expf(m - v);  // m = -inf on the first element: s is 0 and stays 0
+    m = v;
+  }
+  s += expf(v - m);
+}
 __global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(size_t cols, const float* __restrict__ x,
                                                                   float* __restrict__ out) {
   __shared__ float smem[16];
   const float* xr = x + (size_t)blockIdx.x * cols;
   float* o = out + (size_t)blockIdx.x * cols;
-  float m = -__builtin_huge_valf();
-  for (size_t c = threadIdx.x; c < cols; c += 1024) m = fmaxf(m, xr[c]);
-  m = block_reduce<MaxOp>(m, smem);
-  float s = 0.0f;
-  for (size_t c = threadIdx.x; c < cols; c += 1024) s += expf(xr[c] - m);
-  s = block_reduce<SumOp>(s, smem);
-  for (size_t c = threadIdx.x; c < cols; c += 1024) o[c] = expf(xr[c] - m) / s;
+  const size_t nv = cols >> 2;
+  float m = -__builtin_huge_valf(), s = 0.0f;
+  for (size_t c = threadIdx.x; c < nv; c += 1024) {
+    const float4 t = ld4g(xr + 4 * c);
+    const float m4 = fmaxf(fmaxf(t.x, t.y), fmaxf(t.z, t.w));
+    if (m4 > m) {
+      s = s * expf(m - m4);
+      m = m4;
+    }
+    s += (expf(t.x - m) + expf(t.y - m)) + (expf(t.z - m) + expf(t.w - m));
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) online_add(m, s, xr[c]);
+  const float M = block_reduce<MaxOp>(m, smem);
+  // threads that saw no element hold (m, s) = (-inf, 0): their term is 0, not exp(-inf + inf)
+  const float S = block_reduce<SumOp>(s > 0.0f ? s * expf(m - M) : 0.0f, smem);
+  for (size_t c = threadIdx.x; c < nv; c += 1024) {
+    const float4 t = ld4g(xr + 4 * c);
+    st4s(o + 4 * c, make_float4(expf(t.x - M) / S, expf(t.y - M) / S, expf(t.z - M) / S, expf(t.w - M) / S));
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) o[c] = expf(xr[c] - M) / S;
 }
 
 __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, float* x_grad,
@@ -188,12 +244,29 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
                                                                   float beta) {
   __shared__ float smem[16];
   const size_t base = (size_t)blockIdx.x * cols;
+  const float* sr = out + base;
+  const float* gr = out_grad + base;
+  float* xr = x_grad + base;
+  const size_t nv = cols >> 2;
   float dot = 0.0f;
-  for (size_t c = threadIdx.x; c < cols; c += 1024) dot += out[base + c] * out_grad[base + c];
+  for (size_t c = threadIdx.x; c < nv; c += 1024) {
+    const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
+    dot += (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) dot += sr[c] * gr[c];
   dot = block_reduce<SumOp>(dot, smem);
-  for (size_t c = threadIdx.x; c < cols; c += 1024) {
-    float r = out[base + c] * (out_grad[base + c] - dot);
-    x_grad[base + c] = beta != 0.0f ? beta * x_grad[base + c] + r : r;
+  for (size_t c = threadIdx.x; c < nv; c += 1024) {
+    const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
+    float4 r = make_float4(a.x * (b.x - dot), a.y * (b.y - dot), a.z * (b.z - dot), a.w * (b.w - dot));
+    if (beta != 0.0f) {
+      const float4 p = ld4g(xr + 4 * c);
+      r = make_float4(beta * p.x + r.x, beta * p.y + r.y, beta * p.z + r.z, beta * p.w + r.w);
+    }
+    st4s(xr + 4 * c, r);
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) {
+    const float r = sr[c] * (gr[c] - dot);
+    xr[c] = beta != 0.0f ? beta * xr[c] + r : r;
   }
 }
 
@@ -223,22 +296,27 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
     else hipLaunchKernelGGL(softmax_bwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta);
     return post_launch();
   }
-#define SL_SM(L, I)                                                                                                  \
-  case L: {                                                                                                          \
+#define SL_SM2(L, I, T)                                                                                              \
+  do {                                                                                                               \
     constexpr int RPB = L <= 64 ? 256 / L : 1;                                                                       \
     constexpr int BLOCK = L <= 64 ? 256 : L;                                                                         \
     if (FWD)                                                                                                         \
-      hipLaunchKernelGGL((softmax_fwd_kernel<VEC, L, I>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream,    \
+      hipLaunchKernelGGL((softmax_fwd_kernel<VEC, L, I, T>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
                          rows, cols, x, out);                                                                        \
     else                                                                                                             \
-      hipLaunchKernelGGL((softmax_bwd_kernel<VEC, L, I>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream,    \
+      hipLaunchKernelGGL((softmax_bwd_kernel<VEC, L, I, T>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
                          rows, cols, x_grad, s, g, beta);                                                            \
-    break;                                                                                                           \
-  }
+  } while (0)
+#define SL_SM(L, I)                                  \
+  case L:                                            \
+    if (VEC && (cols & 3)) SL_SM2(L, I, true);       \
+    else SL_SM2(L, I, false);                        \
+    break;
   switch (cfg.lanes) {
     SL_SM(1, 4) SL_SM(2, 4) SL_SM(4, 4) SL_SM(8, 4) SL_SM(16, 4) SL_SM(32, 4) SL_SM(64, 4) SL_SM(256, 4) SL_SM(1024, 4)
   }
 #undef SL_SM
+#undef SL_SM2
   return post_launch();
 }
 
@@ -251,7 +329,7 @@ SLHIP_API int32_t slhip_softmax(slhip_ctx* ctx, size_t samples, size_t features,
   SLHIP_REQUIRE(ctx && x && out, "null argument");
   SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
   SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
-  const bool vec = features % 4 == 0;
+  const bool vec = features >= 4;  // any row length: dword-aligned float4 accesses plus a scalar tail
   return vec ? softmax_dispatch<true, true>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f)
              : softmax_dispatch<true, false>(ctx, samples, features, x, out, nullptr, nullptr, nullptr, 0.0f);
 }
@@ -262,7 +340,7 @@ SLHIP_API int32_t slhip_softmax_grad(slhip_ctx* ctx, size_t samples, size_t feat
   SLHIP_REQUIRE(ctx && x_grad && out && out_grad, "null argument");
   SLHIP_REQUIRE(checked_len(samples, features, &len), "bad dims");
   SLHIP_REQUIRE(samples <= 0x7fffffffu, "too many rows for one launch");
-  const bool vec = features % 4 == 0;
+  const bool vec = features >= 4;  // any row length: dword-aligned float4 accesses plus a scalar tail
   return vec ? softmax_dispatch<false, true>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta)
              : softmax_dispatch<false, false>(ctx, samples, features, nullptr, nullptr, x_grad, out, out_grad, beta);
 }

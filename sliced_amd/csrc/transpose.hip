@@ -36,8 +36,14 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 #pragma unroll
       for (int p = 0; p < TR / 16; ++p) {
         const size_t r = r0 + ly + 16 * p, c = c0 + 4 * lx;
-        // cols % 4 == 0: a vector is all in or all out
-        v[p] = (r < rows && c < cols) ? ld4s(x + r * cols + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r >= rows || c >= cols) {
+          v[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else if (c + 3 < cols) {
+          v[p] = ld4s(x + r * cols + c);
+        } else {  // the vector that straddles the end of a row of odd length
+          const float* xr = x + r * cols;
+          v[p] = make_float4(xr[c], c + 1 < cols ? xr[c + 1] : 0.f, c + 2 < cols ? xr[c + 2] : 0.f, 0.f);
+        }
       }
     }
 #pragma unroll
@@ -64,14 +70,20 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
     for (int p = 0; p < TC / 4; ++p) {
       const int cc = ly + 4 * p;  // input column = output row
       const size_t oc = c0 + cc, orow0 = r0 + 4 * lx;
-      if (oc < cols && orow0 < rows) {  // rows % 4 == 0
+      if (oc < cols && orow0 < rows) {
         float4 v = make_float4(tile[4 * lx + 0][cc], tile[4 * lx + 1][cc], tile[4 * lx + 2][cc], tile[4 * lx + 3][cc]);
         float* p_out = out + oc * rows + orow0;
-        if (ACC) {
-          float4 o = ld4s(p_out);
-          v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+        if (orow0 + 3 < rows) {
+          if (ACC) {
+            float4 o = ld4s(p_out);
+            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+          }
+          st4s(p_out, v);
+        } else {  // the vector that straddles the end of an output row of odd length
+          const float e[3] = {v.x, v.y, v.z};
+          for (int q = 0; q < 3; ++q)
+            if (orow0 + q < rows) p_out[q] = ACC ? p_out[q] + e[q] : e[q];
         }
-        st4s(p_out, v);
       }
     }
   } else {
@@ -85,6 +97,32 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
         *p_out = v;
       }
     }
+  }
+}
+
+// Matrices with at most 32 columns (or rows): the tile above would be mostly empty.  One thread
+// per long-axis index walks the short axis; the strided side of every access pattern stays inside
+// a few cache lines that the neighbouring iterations reuse.
+template <bool ACC>
+__global__ __launch_bounds__(256) void transpose_few_cols_kernel(size_t rows, size_t cols, const float* __restrict__ x,
+                                                                 float* out) {
+  const size_t r = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  for (size_t c = 0; c < cols; ++c) {
+    const float v = x[r * cols + c];
+    float* p = out + c * rows + r;  // coalesced over r
+    *p = ACC ? *p + v : v;
+  }
+}
+template <bool ACC>
+__global__ __launch_bounds__(256) void transpose_few_rows_kernel(size_t rows, size_t cols, const float* __restrict__ x,
+                                                                 float* out) {
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  for (size_t r = 0; r < rows; ++r) {
+    const float v = x[r * cols + c];  // coalesced over c
+    float* p = out + c * rows + r;
+    *p = ACC ? *p + v : v;
   }
 }
 
@@ -113,11 +151,26 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     hipLaunchKernelGGL(axpy_copy_kernel, dim3((unsigned)((len + 63) / 64)), dim3(64), 0, ctx->stream, len, x, out);
     return post_launch();
   }
+  if (cols <= 32 || rows <= 32) {
+    const size_t longer = cols <= 32 ? rows : cols;
+    SLHIP_REQUIRE((longer + 255) / 256 <= 0x7fffffffu, "matrix too large for one launch");
+    const dim3 g((unsigned)((longer + 255) / 256));
+    if (cols <= 32) {
+      if (acc) hipLaunchKernelGGL(transpose_few_cols_kernel<true>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
+      else hipLaunchKernelGGL(transpose_few_cols_kernel<false>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
+    } else {
+      if (acc) hipLaunchKernelGGL(transpose_few_rows_kernel<true>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
+      else hipLaunchKernelGGL(transpose_few_rows_kernel<false>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
+    }
+    return post_launch();
+  }
   const size_t tiles_r = (rows + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;
   SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
   const unsigned grid = (unsigned)(tiles_r * tiles_c);
-  const bool vld = cols % 4 == 0;
-  const bool vst = rows % 4 == 0;
+  // rows and columns of any length take the vector paths (dword-aligned float4); the scalar
+  // variants remain for matrices narrower than one vector
+  const bool vld = cols >= 4;
+  const bool vst = rows >= 4;
 #define SL_TR(L, S, A) \
   hipLaunchKernelGGL((transpose_kernel<L, S, A>), dim3(grid), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r)
   if (vld && vst) { if (acc) SL_TR(true, true, true); else SL_TR(true, true, false); }

@@ -216,7 +216,8 @@ def test_max_grads_tie_rules(hip, orc):
 
 
 def test_broadcast_grads_are_bit_exact(hip, orc):
-    for rows, cols in [(3, 4), (5, 7), (128, 256), (1000, 10), (10, 1000), (513, 1028)]:
+    for rows, cols in [(3, 4), (5, 7), (128, 256), (1000, 10), (10, 1000), (513, 1028), (1234, 679), (3, 100003),
+                       (100003, 3), (1, 1)]:
         say("broadcast grads", rows, cols)
         base = rng.normal(rows * cols, 1.0, tag=0, seed=SEED)
         g_r = rng.normal(rows, 1.0, tag=1, seed=SEED)
@@ -230,7 +231,9 @@ def test_broadcast_grads_are_bit_exact(hip, orc):
 
 # --------------------------------------------------------------------------- softmax
 SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (64, 1024), (17, 1000), (9, 4096),
-                  (5, 4100), (3, 16384), (2, 16390), (2, 40000), (1000, 1), (50, 64), (50, 257)]
+                  (5, 4100), (3, 16384), (2, 16390), (2, 40000), (1000, 1), (50, 64), (50, 257),
+                  # odd row lengths: the scalar tail of the vector paths, register-resident and streaming
+                  (6, 7), (5, 5), (300, 1001), (3, 4099), (3, 16387), (2, 40003), (4, 100001), (700, 6789)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -278,7 +281,10 @@ def test_softmax_grad_constant_seed_is_zero(hip):
 
 # --------------------------------------------------------------------------- transpose
 TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300), (257, 129), (1024, 1024),
-             (4, 4096), (4096, 4), (1000, 1000), (1, 1 << 18), (1 << 18, 1)]
+             (4, 4096), (4096, 4), (1000, 1000), (1, 1 << 18), (1 << 18, 1),
+             # rows / columns of odd length on the vector paths, and the few-rows / few-columns kernels
+             (4097, 4097), (1234, 679), (300, 1001), (1001, 300), (100000, 7), (7, 100000), (33, 1000), (1000, 33),
+             (2, 5), (32, 70000), (259, 66)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -358,7 +364,8 @@ def test_negative_base_integer_pow_is_finite(hip):
 
 
 def test_row_op_and_bias_grad(hip, orc):
-    for rows, cols in [(3, 5), (1, 9), (9, 1), (1024, 64), (1000, 10), (8192, 10), (300, 2048), (4097, 130)]:
+    for rows, cols in [(3, 5), (1, 9), (9, 1), (1024, 64), (1000, 10), (8192, 10), (300, 2048), (4097, 130),
+                       (1234, 679), (7, 100003), (100003, 3), (2, 2)]:
         say("row op", rows, cols)
         lhs = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED)
         rhs = rng.uniform(cols, -10, 10, tag=1, seed=SEED)
