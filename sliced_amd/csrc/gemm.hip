@@ -45,7 +45,7 @@ struct GemmArgs {
   size_t k_chunk;     // multiple of BK
   float* partial;
   int a_vec, b_vec;   // the operand's leading dimension is a multiple of 4: rows split into whole float4 loads
-  int aligned;        // both operand bases are 16-byte aligned as well
+  size_t m_fast;      // M when both operand bases are 16-byte aligned as well, else 0: no tile counts as interior
 };
 
 // Operand tile held in registers between the global load and the LDS store.
@@ -284,9 +284,9 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
   // complete k tiles of float4-loadable operands go through a vector-load loop (interior
   // workgroups the unclamped one); unaligned operands and the k remainder through the scalar one
   const bool vec = g.a_vec && g.b_vec;
-  const bool inside = m0 + BM <= g.M && n0 + BN <= g.N;
+  const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
   const int nvec = vec ? kfull : 0;
-  if (inside && g.aligned) gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  if (inside) gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
   else gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
   gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, nvec, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
@@ -494,7 +494,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   const size_t lda = ta ? M : K, ldb = tb ? K : N;
   g.a_vec = lda % 4 == 0;  // dword-aligned vector loads: the leading dimension decides, not the base
   g.b_vec = ldb % 4 == 0;
-  g.aligned = aligned16(A) && aligned16(B);
+  g.m_fast = (aligned16(A) && aligned16(B)) ? M : 0;
   g.partial = (float*)ctx->workspace;
   const size_t mn_bytes = M * N * sizeof(float);
 
