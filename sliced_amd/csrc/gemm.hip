@@ -292,30 +292,49 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
+  // No load may sit between two stores: C, pre_act and dst can be the same memory as far as the
+  // compiler knows, so a `beta * C[idx]` read after a store waits for that store, 64 times in a
+  // row (measured: 7.5 us per workgroup, more than a 128x128x128 product itself).  Hence: first
+  // every read (C for beta), then only stores; and the common plain case is its own loop.
   const bool raw = g.splits > 1;
   float* dst = raw ? g.partial + (size_t)blockIdx.y * g.M * g.N : g.C;
+  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
+  auto for_each = [&](auto&& fn) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const size_t col = n0 + wn * 64 + 32 * j + r;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const size_t row = m0 + wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
+          if (interior || (row < g.M && col < g.N)) fn(i, j, v, row * g.N + col, col);
+        }
+      }
+  };
+  if (raw || (g.beta == 0.0f && !g.bias && !g.pre_act && !g.relu)) {
+    for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
+    return;
+  }
+  if (g.beta != 0.0f)
+    for_each([&](int i, int j, int v, size_t idx, size_t) { acc[i][j][v] = g.beta * g.C[idx] + acc[i][j][v]; });
+  if (g.bias) {
+    float bv[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const size_t col = n0 + wn * 64 + 32 * j + r;
-      if (col >= g.N) continue;
-      const float bv = (!raw && g.bias) ? g.bias[col] : 0.0f;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const size_t row = m0 + wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
-        if (row >= g.M) continue;
-        const size_t idx = row * g.N + col;
-        float val = acc[i][j][v];
-        if (!raw) {
-          if (g.beta != 0.0f) val = g.beta * g.C[idx] + val;
-          if (g.bias) val = val + bv;
-          if (g.pre_act) g.pre_act[idx] = val;
-          if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
-        }
-        dst[idx] = val;
-      }
+      bv[j] = col < g.N ? g.bias[col] : 0.0f;
     }
+    for_each([&](int i, int j, int v, size_t, size_t) { acc[i][j][v] = acc[i][j][v] + bv[j]; });
+  }
+  if (g.pre_act) for_each([&](int i, int j, int v, size_t idx, size_t) { g.pre_act[idx] = acc[i][j][v]; });
+  if (g.relu)
+    for_each([&](int i, int j, int v, size_t idx, size_t) {
+      const float val = acc[i][j][v];
+      dst[idx] = (val >= 0.0f ? 1.0f : 0.0f) * val;
+    });
+  else
+    for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
 }
 
 // Small and skinny problems.  One wave owns one 32x32 tile of C and feeds the matrix core straight
@@ -407,28 +426,45 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
   const size_t c = n0 + r;
   if (c >= g.N) return;
   const float bias = (!raw && g.bias) ? g.bias[c] : 0.0f;
-  auto finish = [&](int v, float val) {
-    const size_t rr = m0 + 8 * (v / 4) + 4 * h + (v % 4);
-    if (rr >= g.M) return;
-    const size_t idx = rr * g.N + c;
-    if (!raw) {
-      if (g.beta != 0.0f) val = g.beta * g.C[idx] + val;
-      if (g.bias) val = val + bias;
-      if (g.pre_act) g.pre_act[idx] = val;
-      if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
-    }
-    dst[idx] = val;
-  };
-  if (nw == 1) {
+  // Register v goes to the wave with v % nw == wk (nw is a power of two).  As in the tiled kernel's
+  // epilogue, every read (LDS partials, C for beta) comes before the first store.
+  float val[16];
+  bool mine[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) finish(v, acc[v]);
-  } else {
-    for (int v = wk; v < 16; v += nw) {
-      float val = red[v * 64 + lane];
-      for (int w = 1; w < nw; ++w) val += red[(w * 16 + v) * 64 + lane];
-      finish(v, val);
+  for (int v = 0; v < 16; ++v) {
+    const size_t rr = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+    mine[v] = (v & (nw - 1)) == wk && rr < g.M;
+    val[v] = acc[v];
+    if (nw > 1 && mine[v]) {
+      float t = red[v * 64 + lane];
+      for (int w = 1; w < nw; ++w) t += red[(w * 16 + v) * 64 + lane];
+      val[v] = t;
     }
   }
+  auto idx_of = [&](int v) { return (m0 + 8 * (v / 4) + 4 * h + (v % 4)) * g.N + c; };
+  if (!raw) {
+    if (g.beta != 0.0f) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (mine[v]) val[v] = g.beta * g.C[idx_of(v)] + val[v];
+    }
+    if (g.bias) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) val[v] = val[v] + bias;
+    }
+    if (g.pre_act) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (mine[v]) g.pre_act[idx_of(v)] = val[v];
+    }
+    if (g.relu) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) val[v] = (val[v] >= 0.0f ? 1.0f : 0.0f) * val[v];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v)
+    if (mine[v]) dst[idx_of(v)] = val[v];
 }
 
 // C = sum_z partial[z] (z ascending) + beta*C, then bias / relu.
