@@ -66,23 +66,31 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
   __syncthreads();
   if (VEC_ST) {
     const int lx = t & 63, ly = t >> 6;  // 64 float4 per output row, 4 output rows per pass
+    const size_t orow0 = r0 + 4 * lx;
+    // `+=`: all reads of the old output before the first store (a read after a store to what may be
+    // the same memory waits for that store)
+    float4 old[TC / 4];
+    if (ACC) {
+#pragma unroll
+      for (int p = 0; p < TC / 4; ++p) {
+        const size_t oc = c0 + ly + 4 * p;
+        old[p] = (oc < cols && orow0 + 3 < rows) ? ld4s(out + oc * rows + orow0) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
 #pragma unroll
     for (int p = 0; p < TC / 4; ++p) {
       const int cc = ly + 4 * p;  // input column = output row
-      const size_t oc = c0 + cc, orow0 = r0 + 4 * lx;
+      const size_t oc = c0 + cc;
       if (oc < cols && orow0 < rows) {
         float4 v = make_float4(tile[4 * lx + 0][cc], tile[4 * lx + 1][cc], tile[4 * lx + 2][cc], tile[4 * lx + 3][cc]);
         float* p_out = out + oc * rows + orow0;
         if (orow0 + 3 < rows) {
-          if (ACC) {
-            float4 o = ld4s(p_out);
-            v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
-          }
+          if (ACC) { v.x += old[p].x; v.y += old[p].y; v.z += old[p].z; v.w += old[p].w; }
           st4s(p_out, v);
         } else {  // the vector that straddles the end of an output row of odd length
-          const float e[3] = {v.x, v.y, v.z};
-          for (int q = 0; q < 3; ++q)
-            if (orow0 + q < rows) p_out[q] = ACC ? p_out[q] + e[q] : e[q];
+          if (orow0 < rows) p_out[0] = ACC ? p_out[0] + v.x : v.x;
+          if (orow0 + 1 < rows) p_out[1] = ACC ? p_out[1] + v.y : v.y;
+          if (orow0 + 2 < rows) p_out[2] = ACC ? p_out[2] + v.z : v.z;
         }
       }
     }
