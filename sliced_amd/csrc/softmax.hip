@@ -11,10 +11,20 @@
 namespace slhip {
 
 // Reduce over the LANES threads that share a row (LANES <= 64: shuffles; else: whole block).
+// Across waves: one barrier per reduction.  Every wave leaves its partial in its own slot of
+// `smem` (a different 16-float slot group per call site, so no barrier is needed before the
+// slots are written again) and every thread folds all the partials itself.
 template <class Op, int LANES>
 __device__ __forceinline__ float row_reduce(float v, float* smem) {
   if (LANES <= 64) return wave_reduce<Op, (LANES <= 64 ? LANES : 64)>(v);
-  return block_reduce<Op>(v, smem);
+  constexpr int NW = LANES / 64;
+  v = wave_reduce<Op>(v);
+  if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = smem[0];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) r = Op::apply(r, smem[w]);
+  return r;
 }
 
 // TAIL: the row length is not a multiple of 4 (VEC only): lane 0 also takes the up to 3 floats
@@ -24,7 +34,7 @@ template <bool VEC, int LANES, int ITEMS, bool TAIL>
 __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(size_t rows, size_t cols,
                                                                                 const float* __restrict__ x,
                                                                                 float* __restrict__ out) {
-  __shared__ float smem[16];
+  __shared__ float smem[32];
   constexpr int V = VEC ? 4 : 1;
   constexpr int RPB = LANES <= 64 ? 256 / LANES : 1;
   const size_t colsv = cols / V;
@@ -92,7 +102,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
       tv[q] = expf(tv[q] - m);
       s += tv[q];
     }
-  s = row_reduce<SumOp, LANES>(s, smem);
+  s = row_reduce<SumOp, LANES>(s, smem + 16);
   // Long rows (a block per row) are close to ALU-bound on exp and the division: they multiply by
   // the reciprocal of the sum (at most 1.5 ulp from the quotient, +3 % bandwidth on rows of
   // 16384); short rows divide, as the reference does.
