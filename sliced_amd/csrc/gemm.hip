@@ -58,9 +58,9 @@ struct Frag {
 //   LOAD_FAST   the whole tile is inside the operand, float4-loadable and 16-byte aligned:
 //               unconditional aligned float4 (the aligned type measures 2 % faster on A*B than the
 //               dword-aligned one, although both become global_load_dwordx4)
-//   LOAD_VCLAMP the k range is complete and the operand is float4-loadable, but the tile hangs
-//               over the operand's edge in x or a base is only dword-aligned: dword-aligned float4
-//               loads from clamped rows, zeroed afterwards
+//   LOAD_VCLAMP the operand is float4-loadable, but the tile hangs over the operand's edge in x
+//               or k, or a base is only dword-aligned: dword-aligned float4 loads from clamped
+//               coordinates, zeroed afterwards
 //   LOAD_SCALAR anything else: one load per element from clamped coordinates, zeroed afterwards
 // No variant branches around a load, so all loads of a tile are in flight together (a version
 // with one branch per element took about 15 us per k tile on tiny problems: each load waited for
@@ -79,8 +79,9 @@ __device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ s
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + x * ld + k);
     } else if (MODE == LOAD_VCLAMP) {
-      const bool in = x < X;
-      const float4 t = ld4g(src + (in ? x : X - 1) * ld + k);
+      // ld = K is a multiple of 4 here and so are k and Kend - Kbegin: a vector is inside or outside as a whole
+      const bool in = x < X && k < Kend;
+      const float4 t = ld4g(src + (x < X ? x : X - 1) * ld + (k < Kend ? k : Kend - 4));
       f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
       const bool xin = x < X;
@@ -116,8 +117,8 @@ __device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ s
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + k * ld + x);
     } else if (MODE == LOAD_VCLAMP) {
-      const bool in = x < X;
-      const float4 t = ld4g(src + k * ld + (in ? x : X - 4));
+      const bool in = x < X && k < Kend;
+      const float4 t = ld4g(src + (k < Kend ? k : Kend - 1) * ld + (x < X ? x : X - 4));
       f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
       const bool kin = k < Kend;
@@ -281,14 +282,18 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // complete k tiles of float4-loadable operands go through a vector-load loop (interior
-  // workgroups the unclamped one); unaligned operands and the k remainder through the scalar one
+  // float4-loadable operands go through the vector-load loops: interior workgroups run their
+  // complete k tiles unclamped and the k remainder clamped, edge workgroups everything clamped;
+  // operands whose rows do not split into float4 take the scalar loop
   const bool vec = g.a_vec && g.b_vec;
   const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
-  const int nvec = vec ? kfull : 0;
-  if (inside) gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  else gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, 0, nvec, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, nvec, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  if (vec) {
+    const int nfast = inside ? kfull : 0;
+    gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nfast, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+    gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, nfast, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  } else {
+    gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  }
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
