@@ -9,13 +9,15 @@
  *     slhip_last_error_string() describes the last failure on the calling thread;
  *   - all matrices are f32, row-major, contiguous (len = rows * cols), as in the reference;
  *   - data pointers are DEVICE pointers; a context owns one in-order HIP stream and every op
- *     is asynchronous on it.  Only slhip_memcpy_d2h, slhip_sync and slhip_event_elapsed_ms
- *     wait;
+ *     is asynchronous on it.  Only slhip_memcpy_h2d, slhip_memcpy_d2h, slhip_free, slhip_sync and
+ *     slhip_event_elapsed_ms wait;
  *   - a context is used from one host thread at a time (the reference's devices are
  *     single-threaded, RefCell-style);
  *   - the library never allocates inside an op call: partial results of the two-stage
  *     reductions and of split-K GEMM live in a workspace that slhip_init allocates once;
- *   - no aliasing between inputs and outputs unless a comment allows it.
+ *   - no aliasing between inputs and outputs unless a comment allows it;
+ *   - pointers need only the 4-byte alignment of a float: views at odd offsets into an
+ *     allocation and rows of odd length stay on the vector paths.
  *
  * Naming trap kept from the reference: *_rows reduces OVER the rows (output length = cols),
  * *_cols reduces OVER the columns (output length = rows).
