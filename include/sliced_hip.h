@@ -126,6 +126,14 @@ int32_t slhip_rand_uniform(slhip_ctx* ctx, uint64_t seed, uint64_t tag, float lo
  * C must not overlap A or B. */
 int32_t slhip_sgemm(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
                     const float* a, const float* b, float* c, float beta);
+/* How the tiled kernel treats a tile grid that does not fill the chip's last round of
+ * workgroups.  SLHIP_TAIL_AUTO (the default) lets a cost model choose between running it as it
+ * is, splitting K for every tile, and spreading the k range of the last round's tiles evenly over
+ * one more round of workgroups; SLHIP_TAIL_WHOLE never spreads, SLHIP_TAIL_SPREAD spreads
+ * whenever the shape allows it.  All three give the same result up to summation order, and each
+ * is deterministic.  A tuning and testing knob: no counterpart in the reference. */
+enum { SLHIP_TAIL_AUTO = 0, SLHIP_TAIL_WHOLE = 1, SLHIP_TAIL_SPREAD = 2 };
+int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy);
 
 /* Gemm::gemm (src/ops2/gemm/mod.rs:21-32), trait argument order (m, k, n). */
 int32_t slhip_gemm(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,

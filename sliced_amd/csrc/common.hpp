@@ -20,6 +20,7 @@ struct slhip_ctx {
   int num_cu = 256;
   char name[64] = {0};
   bool capturing = false;        // between slhip_graph_begin and slhip_graph_end
+  int gemm_tail = 0;             // SLHIP_TAIL_*: how the tiled GEMM treats a partly filled last round
 };
 
 struct slhip_event {

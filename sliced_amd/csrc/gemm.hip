@@ -13,333 +13,16 @@
 // prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.  Tiles are numbered so that each XCD (its
 // own L2) works along one tile row at a time.  Small grids are split along K; the partial
 // products go to the context workspace and are combined in a fixed order.
-#include <type_traits>
-
-#include "common.hpp"
+#include "gemm_tile.hpp"
 
 namespace slhip {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-constexpr int BM = 128, BN = 128;
-constexpr int XC_PITCH = 128 + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
-
-template <int BK>
-struct Cfg {
-  static constexpr int KC_PITCH = BK + 4;  // [x][k] layout, k contiguous
-  static constexpr int STAGE_FLOATS = 128 * KC_PITCH > BK * XC_PITCH ? 128 * KC_PITCH : BK * XC_PITCH;
-  static constexpr int NV = BK * 128 / 4 / 256;  // float4 per thread per operand tile
-};
-
-struct GemmArgs {
-  size_t M, N, K;
-  const float* A;
-  const float* B;
-  float* C;
-  float beta;
-  const float* bias;  // may be null
-  int relu;
-  float* pre_act;     // may be null
-  unsigned tiles_m, tiles_n;
-  unsigned splits;    // > 1: write raw partial sums to `partial[z][M*N]`
-  size_t k_chunk;     // multiple of BK
-  float* partial;
-  int a_vec, b_vec;   // the operand's leading dimension is a multiple of 4: rows split into whole float4 loads
-  size_t m_fast;      // M when both operand bases are 16-byte aligned as well, else 0: no tile counts as interior
-};
-
-// Operand tile held in registers between the global load and the LDS store.
-template <int BK>
-struct Frag {
-  float4 v[Cfg<BK>::NV];
-};
-
-// How a k tile is fetched from global memory.
-//   LOAD_FAST   the whole tile is inside the operand, float4-loadable and 16-byte aligned:
-//               unconditional aligned float4 (the aligned type measures 2 % faster on A*B than the
-//               dword-aligned one, although both become global_load_dwordx4)
-//   LOAD_VCLAMP the operand is float4-loadable, but the tile hangs over the operand's edge in x
-//               or k, or a base is only dword-aligned: dword-aligned float4 loads from clamped
-//               coordinates, zeroed afterwards
-//   LOAD_SCALAR anything else: one load per element from clamped coordinates, zeroed afterwards
-// No variant branches around a load, so all loads of a tile are in flight together (a version
-// with one branch per element took about 15 us per k tile on tiny problems: each load waited for
-// the one before it).
-enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2 };
-
-// k-contiguous source: element (x, k) at src[x*ld + k]; tile 128 x BK.
-template <int BK, int MODE>
-__device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
-                                        size_t x0, size_t k0) {
-  constexpr int VPR = BK / 4, RPP = 256 / VPR;  // float4 per row, rows per pass
-  const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
-#pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) {
-    const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
-    if (MODE == LOAD_FAST) {
-      f.v[p] = ld4(src + x * ld + k);
-    } else if (MODE == LOAD_VCLAMP) {
-      // ld = K is a multiple of 4 here and so are k and Kend - Kbegin: a vector is inside or outside as a whole
-      const bool in = x < X && k < Kend;
-      const float4 t = ld4g(src + (x < X ? x : X - 1) * ld + (k < Kend ? k : Kend - 4));
-      f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
-    } else {
-      const bool xin = x < X;
-      const float* row = src + (xin ? x : X - 1) * ld;
-      float t[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const bool in = xin && k + q < Kend;
-        const float val = row[k + q < Kend ? k + q : Kend - 1];
-        t[q] = in ? val : 0.0f;
-      }
-      f.v[p] = make_float4(t[0], t[1], t[2], t[3]);
-    }
-  }
-}
-template <int BK>
-__device__ __forceinline__ void store_kc(const Frag<BK>& f, float* lds) {
-  constexpr int VPR = BK / 4, RPP = 256 / VPR;
-  const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
-#pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK>::KC_PITCH + 4 * kq, f.v[p]);
-}
-
-// x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x 128.  LOAD_VCLAMP relies on
-// X % 4 == 0 (implied by ld % 4 == 0, ld being X here): a float4 is inside or outside as a whole.
-template <int BK, int MODE>
-__device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
-                                        size_t x0, size_t k0) {
-  const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;  // 32 float4 per k-row, 8 rows per pass
-#pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) {
-    const size_t k = k0 + kr + 8 * p, x = x0 + 4 * xq;
-    if (MODE == LOAD_FAST) {
-      f.v[p] = ld4(src + k * ld + x);
-    } else if (MODE == LOAD_VCLAMP) {
-      const bool in = x < X && k < Kend;
-      const float4 t = ld4g(src + (k < Kend ? k : Kend - 1) * ld + (x < X ? x : X - 4));
-      f.v[p] = in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
-    } else {
-      const bool kin = k < Kend;
-      const float* row = src + (kin ? k : Kend - 1) * ld;
-      float t[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const bool in = kin && x + q < X;
-        const float val = row[x + q < X ? x + q : X - 1];
-        t[q] = in ? val : 0.0f;
-      }
-      f.v[p] = make_float4(t[0], t[1], t[2], t[3]);
-    }
-  }
-}
-template <int BK>
-__device__ __forceinline__ void store_xc(const Frag<BK>& f, float* lds) {
-  const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;
-#pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (kr + 8 * p) * XC_PITCH + 4 * xq, f.v[p]);
-}
-
-// MFMA fragments of one 8-wide k group for the two 32-row blocks of this wave's 64 rows.
-// KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's 64 rows/cols.
-template <bool KC, int BK>
-__device__ __forceinline__ void read_frag(float (&out)[2][4], const float* lds, int x_base, int kk8, int r, int h) {
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    if (KC) {
-      float4 t = ld4(lds + (x_base + 32 * i + r) * Cfg<BK>::KC_PITCH + kk8 * 8 + 4 * h);
-      out[i][0] = t.x; out[i][1] = t.y; out[i][2] = t.z; out[i][3] = t.w;
-    } else {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) out[i][t] = lds[(kk8 * 8 + 4 * h + t) * XC_PITCH + x_base + 32 * i + r];
-    }
-  }
-}
-
-// Linear workgroup id -> tile.  Tiles are walked in groups of 8 tile rows, row index fastest.
-// The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, so with a group
-// height of 8 every XCD (its own L2) keeps working along ONE tile row of the group: its A panel
-// stays put in that L2 while the B panels stream through.  Measured on 4096^3: an explicit
-// remap that instead gave each XCD a compact 8x8 block of tiles was no faster for A*B and
-// At*B and 25 % slower for A*Bt.
-__device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
-                                              unsigned& tn) {
-  constexpr unsigned GROUP_M = 8;
-  const unsigned in_group = GROUP_M * tiles_n;
-  const unsigned group = bid / in_group;
-  const unsigned first_m = group * GROUP_M;
-  const unsigned gsize = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
-  const unsigned local = bid % in_group;
-  tm = first_m + local % gsize;
-  tn = local / gsize;
-}
-
-// The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
-// modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
-// ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
-// kernel's throughput.
-template <bool TA, bool TB, int BK, int MODE>
-__device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
-                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
-                                           float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
-  constexpr int KSTEPS = BK / 8;
-  constexpr int REFILL_AT = (TA && !TB) ? KSTEPS - 1 : (KSTEPS > 1 ? 1 : 0);
-  if (kt_begin >= kt_end) return;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int r = lane & 31, h = lane >> 5;
-  // A is KC ([m][k], ld = K) unless transposed ([k][m], ld = M); B is XC ([k][n], ld = N)
-  // unless transposed ([n][k], ld = K).
-  const size_t lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
-
-  Frag<BK> fa, fb;
-  auto load_stage = [&](int kt) {
-    const size_t k0 = kbeg + (size_t)kt * BK;
-    if (TA) load_xc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    else load_kc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    if (TB) load_kc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
-    else load_xc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
-  };
-  auto store_stage = [&](int s) {
-    if (TA) store_xc<BK>(fa, lds_a[s]); else store_kc<BK>(fa, lds_a[s]);
-    if (TB) store_kc<BK>(fb, lds_b[s]); else store_xc<BK>(fb, lds_b[s]);
-  };
-
-  // Software pipeline over the k tiles.  While tile kt is multiplied out of LDS stage s:
-  //   * the registers hold tile kt+1 (its global loads were issued one iteration ago);
-  //   * before k-group REFILL_AT of tile kt those registers are stored to stage s^1 and the global
-  //     loads of tile kt+2 are issued, so that both the LDS stores and the load issue hide behind
-  //     the remaining MFMA groups (16 MFMAs = 1024 cycles each) instead of sitting between the
-  //     MFMA block and the barrier.  Where in the block the refill goes was measured per form on
-  //     4096^3 (TFLOP/s at group 1 / at the last group): A*B 128.9 / 125.0, A*Bt 135.7 / 135.6,
-  //     At*B 122.7 / 125.3;
-  //   * MFMA fragments are read from LDS one k-group ahead of the MFMAs that consume them.
-  // The scheduling barriers keep the compiler from sinking the reads and stores back down.
-  load_stage(kt_begin);
-  store_stage(0);
-  if (kt_begin + 1 < kt_end) load_stage(kt_begin + 1);
-  __syncthreads();
-
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const int s = (kt - kt_begin) & 1;
-    float a[2][2][4], b[2][2][4];
-    read_frag<!TA, BK>(a[0], lds_a[s], wm * 64, 0, r, h);
-    read_frag<TB, BK>(b[0], lds_b[s], wn * 64, 0, r, h);
-#pragma unroll
-    for (int kk8 = 0; kk8 < KSTEPS; ++kk8) {
-      const int cur = kk8 & 1, nxt = cur ^ 1;
-      if (kk8 + 1 < KSTEPS) {
-        read_frag<!TA, BK>(a[nxt], lds_a[s], wm * 64, kk8 + 1, r, h);
-        read_frag<TB, BK>(b[nxt], lds_b[s], wn * 64, kk8 + 1, r, h);
-      }
-      if (kk8 == REFILL_AT) {
-        // stage s^1 was last read in the previous iteration, which ended with a barrier
-        if (kt + 1 < kt_end) store_stage(s ^ 1);
-        if (kt + 2 < kt_end) load_stage(kt + 2);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // the wave that is in its MFMA block wins the issue arbitration against the wave of the other
-      // workgroup on the same SIMD, which is fetching or waiting (measured: +2 % on A*B, +1 % on At*B)
-      __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][t], b[cur][j][t], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_s_setprio(0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();  // stage s^1 is complete, stage s is free; also leaves LDS free for whoever runs next
-  }
-}
 
 template <bool TA, bool TB, int BK>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
   constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
   __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
   __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
-
-  unsigned tm, tn;
-  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
-  const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
-  const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
-  const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
-  const int kfull = (int)((kend - kbeg) / BK);  // complete tiles
-
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int r = lane & 31, h = lane >> 5;
-
-  floatx16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  // float4-loadable operands go through the vector-load loops: interior workgroups run their
-  // complete k tiles unclamped and the k remainder clamped, edge workgroups everything clamped;
-  // operands whose rows do not split into float4 take the scalar loop
-  const bool vec = g.a_vec && g.b_vec;
-  const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
-  if (vec) {
-    const int nfast = inside ? kfull : 0;
-    gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nfast, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-    gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, nfast, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  } else {
-    gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  }
-
-  // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
-  //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
-  // No load may sit between two stores: C, pre_act and dst can be the same memory as far as the
-  // compiler knows, so a `beta * C[idx]` read after a store waits for that store, 64 times in a
-  // row (measured: 7.5 us per workgroup, more than a 128x128x128 product itself).  Hence: first
-  // every read (C for beta), then only stores; and the common plain case is its own loop.
-  const bool raw = g.splits > 1;
-  float* dst = raw ? g.partial + (size_t)blockIdx.y * g.M * g.N : g.C;
-  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
-  auto for_each = [&](auto&& fn) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const size_t col = n0 + wn * 64 + 32 * j + r;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const size_t row = m0 + wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
-          if (interior || (row < g.M && col < g.N)) fn(i, j, v, row * g.N + col, col);
-        }
-      }
-  };
-  if (raw || (g.beta == 0.0f && !g.bias && !g.pre_act && !g.relu)) {
-    for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
-    return;
-  }
-  if (g.beta != 0.0f)
-    for_each([&](int i, int j, int v, size_t idx, size_t) { acc[i][j][v] = g.beta * g.C[idx] + acc[i][j][v]; });
-  if (g.bias) {
-    float bv[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + wn * 64 + 32 * j + r;
-      bv[j] = col < g.N ? g.bias[col] : 0.0f;
-    }
-    for_each([&](int i, int j, int v, size_t, size_t) { acc[i][j][v] = acc[i][j][v] + bv[j]; });
-  }
-  if (g.pre_act) for_each([&](int i, int j, int v, size_t idx, size_t) { g.pre_act[idx] = acc[i][j][v]; });
-  if (g.relu)
-    for_each([&](int i, int j, int v, size_t idx, size_t) {
-      const float val = acc[i][j][v];
-      dst[idx] = (val >= 0.0f ? 1.0f : 0.0f) * val;
-    });
-  else
-    for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
+  gemm_whole_tile<TA, TB, BK>(g, lds_a, lds_b);
 }
 
 // Small and skinny problems.  One wave owns one 32x32 tile of C and feeds the matrix core straight
@@ -525,8 +208,6 @@ static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) 
   return post_launch();
 }
 
-constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form at 2048^3 and above
-
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
                         float* C, float beta, const float* bias, int relu, float* pre_act) {
   GemmArgs g;
@@ -617,12 +298,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   const size_t slots = (size_t)ctx->num_cu * 2;
   size_t splits = 1;
   const size_t kt_total = (K + BK - 1) / BK;
+  double best = 1e300;  // modelled time of the plan chosen so far, in us
   if (tiles < 4 * slots && kt_total >= 4) {
     size_t max_splits = kt_total / 2;  // every split keeps at least two k tiles
     if (max_splits > 32) max_splits = 32;
     const size_t fit = ctx->workspace_bytes / mn_bytes;
     if (max_splits > fit) max_splits = fit;
-    double best = 1e300;
     for (size_t sp = 1; sp <= max_splits; ++sp) {
       const size_t kt = (kt_total + sp - 1) / sp;
       const size_t wgs = tiles * sp;
@@ -640,6 +321,36 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       if (t < best) { best = t; splits = sp; }
     }
   }
+  // The other remedy for a partly filled last round: the spread tail.  The whole rounds run as
+  // whole tiles; the k tiles of the remaining tiles, taken as one sequence, are dealt out evenly to
+  // one more round of workgroups in the same launch, which start as the whole-tile workgroups
+  // retire; their partial tiles are summed in a fixed order by a second kernel.
+  SpreadArgs sp;
+  sp.first = sp.units = sp.total = 0;
+  sp.kt_total = (unsigned)kt_total;
+  size_t spread_workers = 0;
+  if (tiles % slots != 0 && tiles < 16 * slots && kt_total >= 8 && kt_total < (1u << 20) && ctx->gemm_tail != SLHIP_TAIL_WHOLE) {
+    const size_t full = tiles / slots * slots, tail = tiles - full;
+    const size_t total = tail * kt_total;
+    size_t units = (total + slots - 1) / slots;
+    if (units < 4) units = 4;
+    if (units > kt_total) units = kt_total;  // a workgroup's k tiles then touch at most two tiles of C
+    const size_t workers = (total + units - 1) / units;
+    const size_t runs = tail + workers;  // upper bound of partial tiles written
+    if (2 * workers * SPREAD_SLOT * sizeof(float) <= ctx->workspace_bytes && total < (1u << 31)) {
+      const double per_kt = (full == 0 && workers <= slots / 2) ? 2.43 : 4.35;
+      const double t = (double)(full / slots) * ((double)kt_total * 4.35 + 6.0) + (double)units * per_kt + 6.0 + 4.0 +
+                       2.0 * (double)runs * (double)(SPREAD_SLOT * sizeof(float)) / 5.0e6;
+      if (t < best || ctx->gemm_tail == SLHIP_TAIL_SPREAD) {
+        splits = 1;
+        sp.first = (unsigned)full;
+        sp.units = (unsigned)units;
+        sp.total = (unsigned)total;
+        spread_workers = workers;
+      }
+    }
+  }
+
   size_t k_chunk = (K + splits - 1) / splits;
   k_chunk = (k_chunk + BK - 1) / BK * BK;
   if (k_chunk == 0) k_chunk = BK;
@@ -647,6 +358,8 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   if (splits < 1) splits = 1;
   g.splits = (unsigned)splits;
   g.k_chunk = k_chunk;
+
+  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, g, sp, spread_workers, tiles - sp.first);
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
 #define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g)
@@ -679,6 +392,13 @@ SLHIP_API int32_t slhip_sgemm(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, 
     return SLHIP_EALIAS;
   }
   return gemm_run(ctx, trans_a != 0, trans_b != 0, m, n, k, a, b, c, beta, nullptr, 0, nullptr);
+}
+
+SLHIP_API int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy) {
+  SLHIP_REQUIRE(ctx, "null argument");
+  SLHIP_REQUIRE(policy == SLHIP_TAIL_AUTO || policy == SLHIP_TAIL_WHOLE || policy == SLHIP_TAIL_SPREAD, "unknown policy");
+  ctx->gemm_tail = policy;
+  return SLHIP_OK;
 }
 
 SLHIP_API int32_t slhip_gemm(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,

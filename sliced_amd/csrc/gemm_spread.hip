@@ -1,0 +1,155 @@
+// The spread tail of the tiled f32 GEMM: a launch whose tile count is not a multiple of the
+// chip's workgroup slots would leave most CUs idle during its last round.  Here the whole rounds
+// run as whole tiles, and the k tiles of the remaining tiles - taken as one long sequence - are
+// dealt out evenly to one more round of workgroups in the same launch (they start as the
+// whole-tile workgroups retire).  Such a workgroup writes raw partial tiles to the context
+// workspace; a second kernel sums them per tile in ascending k order, so the result does not
+// depend on timing, and applies beta / bias / relu.
+#include "gemm_tile.hpp"
+
+namespace slhip {
+
+// A workgroup of the spread tail: up to two runs of k tiles, each inside one tile of C, each
+// written as a raw partial tile (row-major 128 x 128) to workspace slot 2*w + run.
+template <bool TA, bool TB, int BK>
+__device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
+                                                   float (*lds_b)[Cfg<BK>::STAGE_FLOATS]) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r = lane & 31, h = lane >> 5;
+  const unsigned w = blockIdx.x - sp.first;
+  unsigned u = w * sp.units;
+  const unsigned u_end = u + sp.units < sp.total ? u + sp.units : sp.total;
+  const int kfull = (int)(g.K / BK);  // complete k tiles of the whole product
+  const bool vec = g.a_vec && g.b_vec;
+  for (int run = 0; run < 2 && u < u_end; ++run) {
+    const unsigned ti = u / sp.kt_total;
+    const int ka = (int)(u % sp.kt_total);
+    const int kb = (u_end - u) < (sp.kt_total - (unsigned)ka) ? ka + (int)(u_end - u) : (int)sp.kt_total;
+    u += (unsigned)(kb - ka);
+    unsigned tm, tn;
+    tile_of_block(sp.first + ti, g.tiles_m, g.tiles_n, tm, tn);
+    const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    if (vec) {
+      const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
+      int fast_end = inside ? (kb < kfull ? kb : kfull) : ka;
+      if (fast_end < ka) fast_end = ka;
+      gemm_tiles<TA, TB, BK, LOAD_FAST>(g, ka, fast_end, 0, g.K, m0, n0, lds_a, lds_b, acc);
+      gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, fast_end, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
+    } else {
+      gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
+    }
+
+    float* slot = g.partial + ((size_t)2 * w + run) * SPREAD_SLOT;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          slot[(wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4)) * BN + wn * 64 + 32 * j + r] = acc[i][j][v];
+  }
+}
+
+template <bool TA, bool TB, int BK>
+__global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadArgs sp) {
+  constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
+  __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
+  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK>(g, sp, lds_a, lds_b);
+  else gemm_whole_tile<TA, TB, BK>(g, lds_a, lds_b);
+}
+
+// The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup
+// order), then beta / bias / relu as in the kernel's own epilogue.  Four workgroups per tile, 32
+// rows each.  Workgroup spread_first + w holds k tiles [w*U, (w+1)*U) of the tail's sequence, so
+// tile ti is covered by workgroups (ti*KT)/U .. ((ti+1)*KT - 1)/U, and it is the workgroup's run
+// number ti - (w*U)/KT (0 or 1, since U <= KT).
+__global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArgs sp) {
+  const unsigned ti = blockIdx.x >> 2, quarter = blockIdx.x & 3;
+  unsigned tm, tn;
+  tile_of_block(sp.first + ti, g.tiles_m, g.tiles_n, tm, tn);
+  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const unsigned KT = sp.kt_total, U = sp.units;
+  const unsigned w_first = (ti * KT) / U, w_last = ((ti + 1) * KT - 1) / U;
+  constexpr int PER = 32 * (BN / 4) / 256;  // float4 per thread
+  float4 s[PER], c[PER];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int f = threadIdx.x + 256 * e;
+    const int row_l = quarter * 32 + f / (BN / 4), c4 = f % (BN / 4);
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (unsigned w = w_first; w <= w_last; ++w) {
+      const unsigned run = ti - (w * U) / KT;
+      const float4 p = ld4(g.partial + ((size_t)2 * w + run) * SPREAD_SLOT + row_l * BN + 4 * c4);
+      if (w == w_first) sum = p;
+      else { sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w; }
+    }
+    s[e] = sum;
+    const size_t row = m0 + row_l, col = n0 + 4 * c4;
+    c[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (g.beta != 0.0f && row < g.M) {  // every read of C before the first store
+      const float* cp = g.C + row * g.N + col;
+      if (col + 3 < g.N) c[e] = ld4g(cp);
+      else c[e] = make_float4(col < g.N ? cp[0] : 0.f, col + 1 < g.N ? cp[1] : 0.f, col + 2 < g.N ? cp[2] : 0.f, 0.f);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int f = threadIdx.x + 256 * e;
+    const int row_l = quarter * 32 + f / (BN / 4), c4 = f % (BN / 4);
+    const size_t row = m0 + row_l, col = n0 + 4 * c4;
+    if (row >= g.M || col >= g.N) continue;
+    float v[4] = {s[e].x, s[e].y, s[e].z, s[e].w};
+    const float cv[4] = {c[e].x, c[e].y, c[e].z, c[e].w};
+    const int n_in = col + 3 < g.N ? 4 : (int)(g.N - col);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (g.beta != 0.0f) v[q] = g.beta * cv[q] + v[q];
+      if (g.bias) v[q] = v[q] + (q < n_in ? g.bias[col + q] : 0.0f);
+    }
+    const size_t idx = row * g.N + col;
+    if (n_in == 4) {
+      if (g.pre_act) st4g(g.pre_act + idx, make_float4(v[0], v[1], v[2], v[3]));
+      if (g.relu) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = (v[q] >= 0.0f ? 1.0f : 0.0f) * v[q];
+      }
+      st4g(g.C + idx, make_float4(v[0], v[1], v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int q = 0; q < 3; ++q) {
+        if (q < n_in) {
+          if (g.pre_act) g.pre_act[idx + q] = v[q];
+          g.C[idx + q] = g.relu ? (v[q] >= 0.0f ? 1.0f : 0.0f) * v[q] : v[q];
+        }
+      }
+    }
+  }
+}
+
+int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const SpreadArgs& sp, size_t workers,
+                           size_t tail_tiles) {
+  const dim3 grid((unsigned)(sp.first + workers));
+#define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g, sp)
+  if (!ta && !tb) SL_GEMM(false, false);
+  else if (!ta && tb) SL_GEMM(false, true);
+  else if (ta && !tb) SL_GEMM(true, false);
+  else SL_GEMM(true, true);
+#undef SL_GEMM
+  int32_t rc = post_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(spread_fixup_kernel, dim3((unsigned)(4 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
+  return post_launch();
+}
+
+}  // namespace slhip

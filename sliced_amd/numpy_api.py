@@ -263,6 +263,14 @@ def sgemm(ta, tb, m, n, k, a, b, c=None, beta=0.0):
     return res
 
 
+TAIL_AUTO, TAIL_WHOLE, TAIL_SPREAD = 0, 1, 2
+
+
+def gemm_tail_policy(policy):
+    """How the tiled GEMM treats a partly filled last round of workgroups (a tuning knob)."""
+    ctx().call("slhip_gemm_tail_policy", int(policy))
+
+
 def gemm(m, n, k, a, b, c=None, beta=0.0):
     """GenericBlas::gemm(m, n, k, a, b, c)."""
     return sgemm(0, 0, m, n, k, a, b, c, beta)

@@ -106,6 +106,47 @@ def test_gemm_split_k_and_large_tiles(hip, orc):
         assert np.all(np.abs(got1 - (exact + c0)) <= bound + 1e-6 * np.abs(c0))
 
 
+def test_gemm_spread_tail(hip, orc):
+    # tile grids that do not fill the last round of workgroups: the k range of the last round's
+    # tiles is spread over one more round, partial tiles are summed in a fixed order.  Forced here,
+    # so that small shapes (a tail of 64 tiles, nothing but tail; edge tiles; k remainders; odd
+    # leading dimensions) take the path, and compared with the whole-tile path as well.
+    shapes = [(1000, 1000, 512, 0, 0), (1024, 1024, 1000, 1, 0), (640, 640, 4096, 0, 1), (999, 1001, 515, 0, 0),
+              (129, 257, 4099, 1, 0), (2945, 3001, 290, 0, 1), (3000, 3000, 256, 0, 0), (3100, 2900, 321, 1, 0)]
+    try:
+        for (m, n, k, ta, tb) in shapes:
+            say("spread gemm", m, n, k, ta, tb)
+            a, b = gemm_operands(ta, tb, m, n, k)
+            exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+            hip.gemm_tail_policy(hip.TAIL_SPREAD)
+            got = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+            assert np.array_equal(got, hip.sgemm(ta, tb, m, n, k, a, b))  # same bits on every run
+            c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+            got1 = hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0)
+            assert np.array_equal(got1, got + c0)
+            hip.gemm_tail_policy(hip.TAIL_WHOLE)
+            whole = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - whole) <= 2 * bound)
+            if not ta and not tb:  # the fused Linear epilogue on the spread path
+                bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+                hip.gemm_tail_policy(hip.TAIL_SPREAD)
+                out, pre = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+                pre_ref = orc.add_row(m, n, got, bias)
+                assert np.array_equal(pre, pre_ref)
+                assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+        # the default policy on a grid of 576 tiles with a long k
+        hip.gemm_tail_policy(hip.TAIL_AUTO)
+        m, n, k = 2945, 3001, 1024
+        say("spread gemm, default policy", m, n, k)
+        a, b = gemm_operands(0, 0, m, n, k)
+        exact, bound = gemm_bound(0, 0, m, n, k, a, b)
+        got = hip.sgemm(0, 0, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+    finally:
+        hip.gemm_tail_policy(hip.TAIL_AUTO)
+
+
 def test_gemm_grad_matches_oracle(hip, orc):
     for (m, k, n) in [(4, 2, 3), (70, 33, 19), (256, 128, 64), (1024, 64, 1), (1024, 1, 64)]:
         say("gemm_grad", m, k, n)
