@@ -28,10 +28,10 @@ sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # HBM-side bytes of one 4096^3 A*B launch, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
-# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (768003.5 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
+# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (629346.4 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
-GEMM_4096_TRAFFIC_BYTES = int((768003.5 * 2.0 + 65536.0) * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((629346.4 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 
@@ -289,7 +289,8 @@ def main():
         log(suite["gemm_4096"])
     if "sweep" in parts:
         sweep = {}
-        for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (8192,) * 3, (8192, 2048, 784), (784, 2048, 8192)]:
+        for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (3584,) * 3, (4608,) * 3, (8192,) * 3, (8192, 2048, 784),
+                          (784, 2048, 8192)]:
             st = max(3, args.steps // 4) if m >= 8192 and k >= 8192 else args.steps
             for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
                 r = bench_gemm(ctx, m, n, k, ta, tb, st, 2)
