@@ -17,12 +17,12 @@
 
 namespace slhip {
 
-template <bool TA, bool TB, int BK>
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
   constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
   __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
   __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
-  gemm_whole_tile<TA, TB, BK>(g, lds_a, lds_b);
+  gemm_whole_tile<TA, TB, BK, ONLY_FAST>(g, lds_a, lds_b);
 }
 
 // Small and skinny problems.  One wave owns one 32x32 tile of C and feeds the matrix core straight
@@ -359,10 +359,17 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   g.splits = (unsigned)splits;
   g.k_chunk = k_chunk;
 
-  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, g, sp, spread_workers, tiles - sp.first);
+  // every k tile of every workgroup complete, inside and 16-byte aligned: the kernel without the
+  // clamped loops (k_chunk is a multiple of BK, so only the end of K can leave a partial tile)
+  const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % BM == 0 && N % BN == 0 && K % BK == 0;
+  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, g, sp, spread_workers, tiles - sp.first);
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
-#define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g)
+#define SL_GEMM(TA_, TB_)                                                                                     \
+  do {                                                                                                        \
+    if (only_fast) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, true>), grid, dim3(256), 0, ctx->stream, g); \
+    else hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, false>), grid, dim3(256), 0, ctx->stream, g);     \
+  } while (0)
   if (!ta && !tb) SL_GEMM(false, false);
   else if (!ta && tb) SL_GEMM(false, true);
   else if (ta && !tb) SL_GEMM(true, false);

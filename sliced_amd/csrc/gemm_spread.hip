@@ -11,7 +11,7 @@ namespace slhip {
 
 // A workgroup of the spread tail: up to two runs of k tiles, each inside one tile of C, each
 // written as a raw partial tile (row-major 128 x 128) to workspace slot 2*w + run.
-template <bool TA, bool TB, int BK>
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
 __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
                                                    float (*lds_b)[Cfg<BK>::STAGE_FLOATS]) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -20,8 +20,6 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
   const unsigned w = blockIdx.x - sp.first;
   unsigned u = w * sp.units;
   const unsigned u_end = u + sp.units < sp.total ? u + sp.units : sp.total;
-  const int kfull = (int)(g.K / BK);  // complete k tiles of the whole product
-  const bool vec = g.a_vec && g.b_vec;
   for (int run = 0; run < 2 && u < u_end; ++run) {
     const unsigned ti = u / sp.kt_total;
     const int ka = (int)(u % sp.kt_total);
@@ -39,15 +37,7 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    if (vec) {
-      const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
-      int fast_end = inside ? (kb < kfull ? kb : kfull) : ka;
-      if (fast_end < ka) fast_end = ka;
-      gemm_tiles<TA, TB, BK, LOAD_FAST>(g, ka, fast_end, 0, g.K, m0, n0, lds_a, lds_b, acc);
-      gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, fast_end, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
-    } else {
-      gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
-    }
+    gemm_k_range<TA, TB, BK, ONLY_FAST>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
 
     float* slot = g.partial + ((size_t)2 * w + run) * SPREAD_SLOT;
 #pragma unroll
@@ -60,13 +50,13 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
   }
 }
 
-template <bool TA, bool TB, int BK>
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
 __global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadArgs sp) {
   constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
   __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
   __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
-  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK>(g, sp, lds_a, lds_b);
-  else gemm_whole_tile<TA, TB, BK>(g, lds_a, lds_b);
+  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST>(g, sp, lds_a, lds_b);
+  else gemm_whole_tile<TA, TB, BK, ONLY_FAST>(g, lds_a, lds_b);
 }
 
 // The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup
@@ -137,10 +127,16 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
   }
 }
 
-int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const SpreadArgs& sp, size_t workers,
-                           size_t tail_tiles) {
+int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g, const SpreadArgs& sp,
+                           size_t workers, size_t tail_tiles) {
   const dim3 grid((unsigned)(sp.first + workers));
-#define SL_GEMM(TA_, TB_) hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK>), grid, dim3(256), 0, ctx->stream, g, sp)
+#define SL_GEMM(TA_, TB_)                                                                                              \
+  do {                                                                                                                 \
+    if (only_fast)                                                                                                     \
+      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, true>), grid, dim3(256), 0, ctx->stream, g, sp);       \
+    else                                                                                                               \
+      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, false>), grid, dim3(256), 0, ctx->stream, g, sp);      \
+  } while (0)
   if (!ta && !tb) SL_GEMM(false, false);
   else if (!ta && tb) SL_GEMM(false, true);
   else if (ta && !tb) SL_GEMM(true, false);

@@ -60,14 +60,20 @@ struct Frag {
 //   LOAD_FAST   the whole tile is inside the operand, float4-loadable and 16-byte aligned:
 //               unconditional aligned float4 (the aligned type measures 2 % faster on A*B than the
 //               dword-aligned one, although both become global_load_dwordx4)
-//   LOAD_VCLAMP the operand is float4-loadable, but the tile hangs over the operand's edge in x
-//               or k, or a base is only dword-aligned: dword-aligned float4 loads from clamped
-//               coordinates, zeroed afterwards
-//   LOAD_SCALAR anything else: one load per element from clamped coordinates, zeroed afterwards
+//   LOAD_XCLAMP any operand, any alignment, but only k tiles that end before the operand's last k
+//               index: dword-aligned float4 loads whose x coordinate is clamped into the operand and
+//               nothing else.  Rows and columns outside the operand receive whatever the clamped
+//               load returns - they only reach rows and columns of C that are never stored.  A
+//               vector that straddles the end of a row of odd length reads on into the next row,
+//               which exists because the tile stops short of the last k index.
+//   LOAD_VCLAMP the operand is float4-loadable; any k tile (the k remainder in particular):
+//               dword-aligned float4 loads from coordinates clamped in x and k, zeroed afterwards
+//   LOAD_SCALAR anything else (the last k tiles of operands whose rows do not split into float4):
+//               one load per element from clamped coordinates, zeroed afterwards
 // No variant branches around a load, so all loads of a tile are in flight together (a version
 // with one branch per element took about 15 us per k tile on tiny problems: each load waited for
 // the one before it).
-enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2 };
+enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2, LOAD_XCLAMP = 3 };
 
 // k-contiguous source: element (x, k) at src[x*ld + k]; tile 128 x BK.
 template <int BK, int MODE>
@@ -80,6 +86,8 @@ __device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ s
     const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + x * ld + k);
+    } else if (MODE == LOAD_XCLAMP) {
+      f.v[p] = ld4g(src + (x < X ? x : X - 1) * ld + k);
     } else if (MODE == LOAD_VCLAMP) {
       // ld = K is a multiple of 4 here and so are k and Kend - Kbegin: a vector is inside or outside as a whole
       const bool in = x < X && k < Kend;
@@ -118,6 +126,8 @@ __device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ s
     const size_t k = k0 + kr + 8 * p, x = x0 + 4 * xq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + k * ld + x);
+    } else if (MODE == LOAD_XCLAMP) {
+      f.v[p] = ld4g(src + k * ld + (x < X ? x : X - 4));  // X > 32 on this path
     } else if (MODE == LOAD_VCLAMP) {
       const bool in = x < X && k < Kend;
       const float4 t = ld4g(src + (k < Kend ? k : Kend - 1) * ld + (x < X ? x : X - 4));
@@ -177,11 +187,31 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = local / gsize;
 }
 
+// Where the k loop's code starts relative to a 32-byte boundary is worth up to 4 % of the kernel's
+// speed, repeatably: measured on 4096^3 with the start 0 / 8 / 16 / 24 bytes past a boundary
+// (TFLOP/s): A*B 132.3 / 134.9 / 134.2 / 131.1, A*Bt 139.9 / 139.0 / 141.1 / 139.8, At*B 134.1 /
+// 128.8 / 130.4 / 129.8; odd multiples of 4 bytes were never best, 64-byte alignment adds nothing.
+// Left to chance the start moves whenever code earlier in the file changes, so it is pinned,
+// per form, for the two loops that large products spend their time in.  The best offset is a
+// property of the loop's code: after a change to the loop or to what precedes it in gemm_tiles,
+// measure the four offsets again.  P = offset in units of 8 bytes.
+template <int P>
+__device__ __forceinline__ void pin_loop_start() {
+  static_assert(P >= 0 && P < 4, "offset is 0, 8, 16 or 24 bytes");
+  if (P == 0) asm volatile(".p2align 5");
+  if (P == 1) asm volatile(".p2align 5\n s_nop 0\n s_nop 0");
+  if (P == 2) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
+  if (P == 3) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
+}
+constexpr int PIN_ONLY_FAST[2][2] = {{1, 2}, {0, 1}};  // [TA][TB]; the kernel that holds no other loop
+constexpr int PIN_FAST[2][2] = {{1, 1}, {0, 1}};       // the same loop in the kernel that holds all four
+constexpr int PIN_XCLAMP[2][2] = {{1, 2}, {1, 1}};
+
 // The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
 // ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
 // kernel's throughput.
-template <bool TA, bool TB, int BK, int MODE>
+template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST>
 __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
                                            size_t m0, size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
                                            float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
@@ -223,17 +253,8 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   if (kt_begin + 1 < kt_end) load_stage(kt_begin + 1);
   __syncthreads();
 
-  // Where the loop's code starts relative to a 32-byte boundary is worth up to 4 % of the
-  // kernel's speed, repeatably: measured on 4096^3 with the start 0 / 8 / 16 / 24 bytes past
-  // the boundary (TFLOP/s): A*B 132.3 / 134.9 / 134.2 / 131.1, A*Bt 139.9 / 139.0 / 141.1 / 139.8,
-  // At*B 134.1 / 128.8 / 130.4 / 129.8; odd multiples of 4 bytes were never best.  Left to chance
-  // the start moves whenever code earlier in the file changes, so it is pinned here, per form,
-  // for the loop that interior workgroups spend their time in.
-  if (MODE == LOAD_FAST) {
-    if (TA && !TB) asm volatile(".p2align 5");
-    else if (!TA && TB) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
-    else asm volatile(".p2align 5\n s_nop 0\n s_nop 0");
-  }
+  if (MODE == LOAD_FAST) pin_loop_start<ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
+  if (MODE == LOAD_XCLAMP) pin_loop_start<PIN_XCLAMP[TA][TB]>();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int s = (kt - kt_begin) & 1;
     float a[2][2][4], b[2][2][4];
@@ -269,9 +290,45 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   }
 }
 
+// k tiles [ka, kb) (counted from kbeg; the chunk ends at kend) of the tile at (m0, n0), each
+// stretch with the cheapest load mode that is valid for it:
+//   interior tile of float4-loadable, 16-byte aligned operands: LOAD_FAST for the complete k
+//   tiles, LOAD_VCLAMP for the k remainder;
+//   otherwise (edge tile, base only float-aligned, rows of odd length): LOAD_XCLAMP for the k
+//   tiles that end before the operand's last k index, then LOAD_VCLAMP or, for rows of odd length,
+//   LOAD_SCALAR for the rest (one tile, or the k remainder).
+// ONLY_FAST: the host has checked that every k tile of every tile qualifies for LOAD_FAST (M and N
+// multiples of 128, every k chunk a multiple of BK, operands float4-loadable and 16-byte aligned);
+// the kernel then contains that one loop and nothing else.
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
+__device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, size_t kbeg, size_t kend, size_t m0,
+                                             size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
+                                             float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
+  if (ONLY_FAST) {
+    gemm_tiles<TA, TB, BK, LOAD_FAST, true>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+    return;
+  }
+  const bool vec = g.a_vec && g.b_vec;
+  const bool fast = vec && m0 + BM <= g.m_fast && n0 + BN <= g.N;
+  const int kfull = (int)((kend - kbeg) / BK);             // complete k tiles of the chunk
+  const int before_last = (int)((g.K - 1 - kbeg) / BK);    // k tiles that end before index K - 1
+  int e1 = fast ? (kb < kfull ? kb : kfull) : ka;
+  if (e1 < ka) e1 = ka;
+  int e2 = e1;
+  if (!fast) {
+    e2 = kb < before_last ? kb : before_last;
+    if (e2 < e1) e2 = e1;
+  }
+  const int e3 = vec ? kb : e2;
+  gemm_tiles<TA, TB, BK, LOAD_FAST, false>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+}
+
 // A workgroup that computes one whole tile of C (or, with g.splits > 1, one k chunk of it as a raw
 // partial product): blockIdx.x = tile, blockIdx.y = k chunk.
-template <bool TA, bool TB, int BK>
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
 __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
                                                 float (*lds_b)[Cfg<BK>::STAGE_FLOATS]) {
   unsigned tm, tn;
@@ -280,7 +337,6 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
   const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
   const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
-  const int kfull = (int)((kend - kbeg) / BK);  // complete tiles
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
@@ -294,18 +350,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  // float4-loadable operands go through the vector-load loops: interior workgroups run their
-  // complete k tiles unclamped and the k remainder clamped, edge workgroups everything clamped;
-  // operands whose rows do not split into float4 take the scalar loop
-  const bool vec = g.a_vec && g.b_vec;
-  const bool inside = m0 + BM <= g.m_fast && n0 + BN <= g.N;
-  if (vec) {
-    const int nfast = inside ? kfull : 0;
-    gemm_tiles<TA, TB, BK, LOAD_FAST>(g, 0, nfast, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-    gemm_tiles<TA, TB, BK, LOAD_VCLAMP>(g, nfast, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  } else {
-    gemm_tiles<TA, TB, BK, LOAD_SCALAR>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  }
+  gemm_k_range<TA, TB, BK, ONLY_FAST>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
@@ -355,7 +400,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 }
 
 // Launches the spread-tail kernel and its fix-up (gemm_spread.hip).
-int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const SpreadArgs& sp, size_t workers,
-                           size_t tail_tiles);
+int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g, const SpreadArgs& sp,
+                           size_t workers, size_t tail_tiles);
 
 }  // namespace slhip

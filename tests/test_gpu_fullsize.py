@@ -187,3 +187,34 @@ def test_gemm_4096_cubed_against_oracle(hip, orc, form):
     assert np.array_equal(dc.numpy(), got * np.float32(2.0))
     for z in (da, db, dc):
         z.free()
+
+
+@pytest.mark.parametrize("shape", [(4608, 4608, 1024), (3585, 3457, 1031), (2944, 3072, 2056)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("form", ["A*B", "A*Bt", "At*B"])
+def test_gemm_grids_with_a_partly_filled_last_round(hip, form, shape):
+    """Tile grids that are not a multiple of the chip's workgroup slots (the spread tail under the
+    default policy), with rows of odd length and a k remainder among them: sampled rows against an
+    f64 product, run-to-run bit equality, exact linearity."""
+    m, n, k = shape
+    c = hip.ctx()
+    ta, tb = form == "At*B", form == "A*Bt"
+    say("gemm, partly filled last round", form, m, n, k)
+    a = rng.uniform(m * k, -1, 1, tag=0, seed=SEED + 3)
+    b = rng.uniform(k * n, -1, 1, tag=1, seed=SEED + 3)
+    da, db, dc = c.array(a), c.array(b), c.empty(m * n)
+    c.call("slhip_sgemm", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dc.ptr, 0.0)
+    got = dc.numpy()
+    A = a.reshape(k, m).T if ta else a.reshape(m, k)
+    B = b.reshape(n, k).T if tb else b.reshape(k, n)
+    rows = np.unique(np.concatenate([rng.integers(96, m, tag=5, seed=SEED), [0, m - 1, m - 2, 127, 128]]))
+    exact = A[rows].astype(np.float64) @ B.astype(np.float64)
+    tol = 1e-5 * np.sqrt(k) * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert np.all(np.abs(got.reshape(m, n)[rows] - exact) <= tol)
+    c.call("slhip_sgemm", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dc.ptr, 0.0)
+    assert np.array_equal(dc.numpy(), got)
+    c.call("slhip_ew_unary", 6, 2.0, 0.0, m * k, da.ptr, da.ptr)
+    c.call("slhip_sgemm", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dc.ptr, 0.0)
+    assert np.array_equal(dc.numpy(), got * np.float32(2.0))
+    for z in (da, db, dc):
+        z.free()
