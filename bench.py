@@ -211,7 +211,33 @@ def cpu_baseline(m, n, k):
     dt1 = time.perf_counter() - t0
     res["single_thread_TFLOPs_at_1024"] = 2.0 * ms ** 3 / dt1 / 1e12
     res["ops"] = cpu_streaming_ops(oracle, cores)
+    res["mlp"] = cpu_mlp_steps(oracle, cores)
     return res
+
+
+def cpu_mlp_steps(oracle, cores):
+    """Steps per second of the oracle's training loop (the reference's op sequence on the host) on the
+    two MLP configurations: all 200 steps of the sine fit, a bounded sample of 2 steps of the
+    classifier (260 GFLOP each), on one thread (the reference is single-threaded) and on every core."""
+    try:
+        from sliced_amd import host
+    except Exception as e:  # configurations and seeded data live beside the host layer's bindings
+        return {"skipped": "host layer not built: %s" % e}
+    out = {}
+    for name, cfg, steps_by_threads in (("C1 sine fit 1-64-64-1 batch 1024", host.C1, {1: 200, cores: 200}),
+                                        ("C5 classifier 784-2048-2048-10 batch 8192", host.C5, {1: 1, cores: 2})):
+        x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+        row = {}
+        for th, steps in steps_by_threads.items():
+            params = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+            oracle.set_threads(th)
+            t0 = time.perf_counter()
+            oracle.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, params, cfg["lr"], steps)
+            row["steps_per_s_%d_thread%s" % (th, "" if th == 1 else "s")] = steps / (time.perf_counter() - t0)
+            row["sample_steps_%d_thread%s" % (th, "" if th == 1 else "s")] = steps
+        out[name] = row
+    oracle.set_threads(1)
+    return out
 
 
 def cpu_streaming_ops(oracle, cores):

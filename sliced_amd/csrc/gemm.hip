@@ -8,11 +8,16 @@
 // k permutation inside every group of 8: instruction t (0..3) multiplies k = t for lanes 0..31
 // and k = 4 + t for lanes 32..63.
 //
-// Tiling: 256 threads = 4 waves in a 2x2 grid, 128x128 macro tile, each wave 64x64 = four
-// 32x32 accumulators (64 VGPRs), BK = 32 per LDS stage, two LDS stages with register
-// prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.  Tiles are numbered so that each XCD (its
-// own L2) works along one tile row at a time.  Small grids are split along K; the partial
-// products go to the context workspace and are combined in a fixed order.
+// Tiling (gemm_tile.hpp): 256 threads = 4 waves in a 2x2 grid, 128x128 macro tile, each wave
+// 64x64 = four 32x32 accumulators (64 VGPRs), BK = 32 per LDS stage, two LDS stages with register
+// prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.
+// Tiles are numbered so that each XCD (its own L2) works along one tile row at a time.
+//
+// This file: the plain kernel (one workgroup per tile and k chunk), the wave-per-tile kernel for
+// small and skinny products, the split-K combine, and the host-side plan - which kernel, how
+// many k splits, or the spread tail (gemm_spread.hip) for tile grids that do not fill the chip's
+// last round of workgroups.  Partial products go to the context workspace and are combined in a
+// fixed order, so every plan is deterministic.
 #include "gemm_tile.hpp"
 
 namespace slhip {
