@@ -240,8 +240,10 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     const size_t tiles = wt_m * wt_n, groups = (K + 7) / 8;
     // waves per workgroup (at most 8 for small problems, where 16 measured 10-15 % slower, at
     // most 16 for large skinny ones, where 8 did): each keeps >= 4 groups of k; then
-    // whole-grid splits of K until the chip has about 8 waves per CU, each split keeping >= 8
-    // groups per wave
+    // whole-grid splits of K until the chip has about 8 waves per CU.  A split of a large problem
+    // keeps >= 8 groups per wave.  A split of a small one keeps >= 32: up to there the extra
+    // groups of an unsplit wave (about 1.2 us per 8) cost less than the combine kernel that a
+    // split brings (3-4 us, and one more node in a recorded step)
     unsigned nw = 1;
     const bool small = flop <= 33554432.0;
     while (nw < (small ? 8u : 16u) && groups >= (size_t)nw * 2 * 4) nw *= 2;
@@ -249,7 +251,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     const size_t want = (size_t)ctx->num_cu * 8;
     if (tiles * nw < want) {
       splits = (want + tiles * nw - 1) / (tiles * nw);
-      const size_t most = groups / ((size_t)nw * 8);
+      const size_t most = groups / ((size_t)nw * (small ? 32 : 8));
       if (splits > most) splits = most;
       if (splits > 64) splits = 64;
       if (splits > ctx->workspace_bytes / mn_bytes) splits = ctx->workspace_bytes / mn_bytes;

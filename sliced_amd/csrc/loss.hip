@@ -19,7 +19,7 @@ namespace slhip {
 // ---------------------------------------------------------------- mean squared error
 __global__ __launch_bounds__(256) void mse_partial_kernel(size_t n, const float* __restrict__ x,
                                                           const float* __restrict__ y, float* __restrict__ part,
-                                                          size_t chunk, int vec) {
+                                                          size_t chunk, int vec, float inv_n, float* __restrict__ out) {
   __shared__ float smem[4];
   const size_t beg = (size_t)blockIdx.x * chunk, end = beg + chunk < n ? beg + chunk : n;
   float s = 0.0f;
@@ -41,7 +41,10 @@ __global__ __launch_bounds__(256) void mse_partial_kernel(size_t n, const float*
     }
   }
   s = block_reduce<SumOp>(s, smem);
-  if (threadIdx.x == 0) part[blockIdx.x] = s;
+  if (threadIdx.x == 0) {
+    if (gridDim.x == 1) out[0] = s * inv_n;  // a single block is its own final stage
+    else part[blockIdx.x] = s;
+  }
 }
 
 __global__ __launch_bounds__(64) void mse_final_kernel(unsigned nparts, const float* __restrict__ part, float inv_n,
@@ -125,9 +128,10 @@ SLHIP_API int32_t slhip_mse(slhip_ctx* ctx, size_t n, const float* x, const floa
   blocks = (n + chunk - 1) / chunk;
   const int vec = 1;
   float* part = (float*)ctx->workspace;
-  hipLaunchKernelGGL(mse_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, y, part, chunk, vec);
+  hipLaunchKernelGGL(mse_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, y, part, chunk, vec,
+                     1.0f / (float)n, loss_dev);
   int32_t rc = post_launch();
-  if (rc) return rc;
+  if (rc || blocks == 1) return rc;
   hipLaunchKernelGGL(mse_final_kernel, dim3(1), dim3(64), 0, ctx->stream, (unsigned)blocks, (const float*)part,
                      1.0f / (float)n, loss_dev);
   return post_launch();

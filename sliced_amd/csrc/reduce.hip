@@ -196,15 +196,19 @@ __global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_
   __shared__ float sm[256];
   const int cx = threadIdx.x % CW, ry = threadIdx.x / CW;
   const size_t c = (size_t)blockIdx.x * CW + cx;
-  float a0 = Op::identity(), a1 = a0;
+  float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
   if (c < cols) {
     size_t r = ry;
-    for (; r + RL < rows; r += 2 * RL) {
+    for (; r + 3 * RL < rows; r += 4 * RL) {  // four loads in flight per lane
       a0 = Op::apply(a0, x[r * cols + c]);
       a1 = Op::apply(a1, x[(r + RL) * cols + c]);
+      a2 = Op::apply(a2, x[(r + 2 * RL) * cols + c]);
+      a3 = Op::apply(a3, x[(r + 3 * RL) * cols + c]);
     }
     for (; r < rows; r += RL) a0 = Op::apply(a0, x[r * cols + c]);
   }
+  a0 = Op::apply(a0, a2);
+  a1 = Op::apply(a1, a3);
   sm[threadIdx.x] = Op::apply(a0, a1);
   __syncthreads();
 #pragma unroll
@@ -218,19 +222,20 @@ __global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_
 template <class Op>
 static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out,
                                       Finalize fin) {
-  if (cols >= 64 && rows <= 64) {
-    hipLaunchKernelGGL((colreduce_final_kernel<Op, 64>), dim3(ceil_div(cols, 64)), dim3(256), 0, ctx->stream, rows,
-                       cols, x, out, fin);
-  } else if (cols >= 16) {
-    hipLaunchKernelGGL((colreduce_final_kernel<Op, 16>), dim3(ceil_div(cols, 16)), dim3(256), 0, ctx->stream, rows,
-                       cols, x, out, fin);
-  } else if (cols >= 4) {
-    hipLaunchKernelGGL((colreduce_final_kernel<Op, 4>), dim3(ceil_div(cols, 4)), dim3(256), 0, ctx->stream, rows,
-                       cols, x, out, fin);
-  } else {
-    hipLaunchKernelGGL((colreduce_final_kernel<Op, 1>), dim3(ceil_div(cols, 1)), dim3(256), 0, ctx->stream, rows,
-                       cols, x, out, fin);
-  }
+  // the widest column strip that still leaves every row-lane at most 16 rows
+  int cw = 1;
+  if (cols >= 64 && rows * 64 <= 4096) cw = 64;
+  else if (cols >= 16 && rows * 16 <= 4096) cw = 16;
+  else if (cols >= 4 && rows * 4 <= 4096) cw = 4;
+  else if (rows > 4096) cw = cols >= 16 ? 16 : cols >= 4 ? 4 : 1;  // long inputs: coalescing matters more
+#define SL_CF(CW_)                                                                                                    \
+  hipLaunchKernelGGL((colreduce_final_kernel<Op, CW_>), dim3(ceil_div(cols, CW_)), dim3(256), 0, ctx->stream, rows, cols, \
+                     x, out, fin)
+  if (cw == 64) SL_CF(64);
+  else if (cw == 16) SL_CF(16);
+  else if (cw == 4) SL_CF(4);
+  else SL_CF(1);
+#undef SL_CF
   return post_launch();
 }
 
@@ -291,6 +296,10 @@ static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, 
   size_t cap = (size_t)ctx->num_cu * 8;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
+  if (n <= 16384) {  // short buffers: the one-block kernel reads x itself
+    hipLaunchKernelGGL((fullreduce_final_kernel<Op>), dim3(1), dim3(1024), 0, ctx->stream, n, x, out, fin);
+    return post_launch();
+  }
   float* part = (float*)ctx->workspace;
   if (vec)
     hipLaunchKernelGGL((fullreduce_kernel<Op, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
@@ -320,7 +329,8 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
   if (G > rows / 16) G = rows / 16;
   const size_t ws_floats = ctx->workspace_bytes / sizeof(float);
   if (G > 1 && G * cols > ws_floats) G = ws_floats / cols;
-  if (G <= 1) return colreduce_final_launch<Op>(ctx, rows, cols, x, out, fin);
+  // small matrices: one kernel (a second stage would cost more than it saves, 3-4 us a launch)
+  if (G <= 1 || (rows * cols <= (1u << 18) && rows <= 4096)) return colreduce_final_launch<Op>(ctx, rows, cols, x, out, fin);
   float* part = (float*)ctx->workspace;
   const size_t threads = colsv * G;
   if (vec)
