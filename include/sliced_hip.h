@@ -126,6 +126,13 @@ int32_t slhip_rand_uniform(slhip_ctx* ctx, uint64_t seed, uint64_t tag, float lo
  * C must not overlap A or B. */
 int32_t slhip_sgemm(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
                     const float* a, const float* b, float* c, float beta);
+/* C = beta·C + (op(A)·op(B)) ⊙ (pre >= 0), pre shaped like C: the input gradient of a Linear layer
+ * and the ReLU gradient of the layer before it in one kernel, for tapes that chain them -
+ * GemmGrad's lhs_grad (src/ops2/gemm/grad/cpu_stack.rs:36) followed by relu's grad closure
+ * `x.grad += (x >= 0) * out.grad` (src/matrix.rs:169-190).  With beta = 1 and C the zeroed gradient
+ * of `pre` the result has the bits of the two-op sequence.  C must not overlap A, B or pre. */
+int32_t slhip_sgemm_relu_mask(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
+                              const float* a, const float* b, const float* pre, float* c, float beta);
 /* How the tiled kernel treats a tile grid that does not fill the chip's last round of
  * workgroups.  SLHIP_TAIL_AUTO (the default) lets a cost model choose between running it as it
  * is, splitting K for every tile, and spreading the k range of the last round's tiles evenly over

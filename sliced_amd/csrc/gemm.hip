@@ -136,6 +136,11 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
   }
   auto idx_of = [&](int v) { return (m0 + 8 * (v / 4) + 4 * h + (v % 4)) * g.N + c; };
   if (!raw) {
+    if (g.mask) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (mine[v]) val[v] = (g.mask[idx_of(v)] >= 0.0f ? 1.0f : 0.0f) * val[v];
+    }
     if (g.beta != 0.0f) {
 #pragma unroll
       for (int v = 0; v < 16; ++v)
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N, unsigned splits,
                                                             const float* __restrict__ partial, float* C, float beta,
                                                             const float* __restrict__ bias, int relu, float* pre_act,
-                                                            int vec) {
+                                                            const float* __restrict__ mask, int vec) {
   const size_t stride = (size_t)gridDim.x * 256;
   const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (vec) {
@@ -173,6 +178,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
       for (unsigned z = 1; z < splits; ++z) {
         float4 p = ld4g(partial + (size_t)z * mn + 4 * i);
         s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+      }
+      if (mask) {
+        float4 m = ld4g(mask + 4 * i);
+        s.x *= (m.x >= 0.f ? 1.f : 0.f); s.y *= (m.y >= 0.f ? 1.f : 0.f);
+        s.z *= (m.z >= 0.f ? 1.f : 0.f); s.w *= (m.w >= 0.f ? 1.f : 0.f);
       }
       if (beta != 0.0f) {
         float4 c = ld4g(C + 4 * i);
@@ -193,6 +203,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
     for (size_t i = tid; i < mn; i += stride) {
       float s = partial[i];
       for (unsigned z = 1; z < splits; ++z) s += partial[(size_t)z * mn + i];
+      if (mask) s *= (mask[i] >= 0.f ? 1.f : 0.f);
       if (beta != 0.0f) s = beta * C[i] + s;
       if (bias) s += bias[i % N];
       if (pre_act) pre_act[i] = s;
@@ -209,15 +220,15 @@ static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) 
   const size_t cap = (size_t)ctx->num_cu * 16;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, mn, g.N, (unsigned)splits,
-                     (const float*)ctx->workspace, g.C, g.beta, g.bias, g.relu, g.pre_act, vec);
+                     (const float*)ctx->workspace, g.C, g.beta, g.bias, g.relu, g.pre_act, g.mask, vec);
   return post_launch();
 }
 
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
-                        float* C, float beta, const float* bias, int relu, float* pre_act) {
+                        float* C, float beta, const float* bias, int relu, float* pre_act, const float* mask) {
   GemmArgs g;
   g.M = M; g.N = N; g.K = K; g.A = A; g.B = B; g.C = C; g.beta = beta;
-  g.bias = bias; g.relu = relu; g.pre_act = pre_act;
+  g.bias = bias; g.relu = relu; g.pre_act = pre_act; g.mask = mask;
   const size_t lda = ta ? M : K, ldb = tb ? K : N;
   g.a_vec = lda % 4 == 0;  // dword-aligned vector loads: the leading dimension decides, not the base
   g.b_vec = ldb % 4 == 0;
@@ -405,7 +416,19 @@ SLHIP_API int32_t slhip_sgemm(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, 
     set_error("slhip_sgemm: C overlaps an input");
     return SLHIP_EALIAS;
   }
-  return gemm_run(ctx, trans_a != 0, trans_b != 0, m, n, k, a, b, c, beta, nullptr, 0, nullptr);
+  return gemm_run(ctx, trans_a != 0, trans_b != 0, m, n, k, a, b, c, beta, nullptr, 0, nullptr, nullptr);
+}
+
+SLHIP_API int32_t slhip_sgemm_relu_mask(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
+                                        const float* a, const float* b, const float* pre, float* c, float beta) {
+  size_t mk, kn, mn;
+  SLHIP_REQUIRE(ctx && a && b && c && pre, "null argument");
+  SLHIP_REQUIRE(checked_len(m, k, &mk) && checked_len(k, n, &kn) && checked_len(m, n, &mn), "bad dims");
+  if (overlaps(c, mn, a, mk) || overlaps(c, mn, b, kn) || overlaps(c, mn, pre, mn)) {
+    set_error("slhip_sgemm_relu_mask: C overlaps an input");
+    return SLHIP_EALIAS;
+  }
+  return gemm_run(ctx, trans_a != 0, trans_b != 0, m, n, k, a, b, c, beta, nullptr, 0, nullptr, pre);
 }
 
 SLHIP_API int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy) {
@@ -445,5 +468,5 @@ SLHIP_API int32_t slhip_linear_fwd(slhip_ctx* ctx, size_t m, size_t k, size_t n,
     set_error("slhip_linear_fwd: out overlaps an input");
     return SLHIP_EALIAS;
   }
-  return gemm_run(ctx, false, false, m, n, k, x, w, out, 0.0f, bias, relu != 0, pre_act);
+  return gemm_run(ctx, false, false, m, n, k, x, w, out, 0.0f, bias, relu != 0, pre_act, nullptr);
 }

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
   const unsigned KT = sp.kt_total, U = sp.units;
   const unsigned w_first = (ti * KT) / U, w_last = ((ti + 1) * KT - 1) / U;
   constexpr int PER = 32 * (BN / 4) / 256;  // float4 per thread
-  float4 s[PER], c[PER];
+  float4 s[PER], c[PER], mk[PER];
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int f = threadIdx.x + 256 * e;
@@ -87,10 +87,15 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
     s[e] = sum;
     const size_t row = m0 + row_l, col = n0 + 4 * c4;
     c[e] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (g.beta != 0.0f && row < g.M) {  // every read of C before the first store
-      const float* cp = g.C + row * g.N + col;
-      if (col + 3 < g.N) c[e] = ld4g(cp);
-      else c[e] = make_float4(col < g.N ? cp[0] : 0.f, col + 1 < g.N ? cp[1] : 0.f, col + 2 < g.N ? cp[2] : 0.f, 0.f);
+    mk[e] = c[e];
+    auto read4 = [&](const float* base) {  // a float4 of a row of C's shape, clipped at the row's end
+      const float* cp = base + row * g.N + col;
+      if (col + 3 < g.N) return ld4g(cp);
+      return make_float4(col < g.N ? cp[0] : 0.f, col + 1 < g.N ? cp[1] : 0.f, col + 2 < g.N ? cp[2] : 0.f, 0.f);
+    };
+    if (row < g.M) {  // every read of C and of the mask source before the first store
+      if (g.beta != 0.0f) c[e] = read4(g.C);
+      if (g.mask) mk[e] = read4(g.mask);
     }
   }
 #pragma unroll
@@ -101,9 +106,11 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
     if (row >= g.M || col >= g.N) continue;
     float v[4] = {s[e].x, s[e].y, s[e].z, s[e].w};
     const float cv[4] = {c[e].x, c[e].y, c[e].z, c[e].w};
+    const float mv[4] = {mk[e].x, mk[e].y, mk[e].z, mk[e].w};
     const int n_in = col + 3 < g.N ? 4 : (int)(g.N - col);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
+      if (g.mask) v[q] = (mv[q] >= 0.0f ? 1.0f : 0.0f) * v[q];
       if (g.beta != 0.0f) v[q] = g.beta * cv[q] + v[q];
       if (g.bias) v[q] = v[q] + (q < n_in ? g.bias[col + q] : 0.0f);
     }

@@ -32,6 +32,7 @@ struct GemmArgs {
   const float* bias;  // may be null
   int relu;
   float* pre_act;     // may be null
+  const float* mask;  // may be null; else the product is multiplied by (mask[idx] >= 0) before beta*C is added
   unsigned tiles_m, tiles_n;
   unsigned splits;    // > 1: write raw partial sums to `partial[z][M*N]`
   size_t k_chunk;     // multiple of BK
@@ -374,10 +375,14 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
         }
       }
   };
-  if (raw || (g.beta == 0.0f && !g.bias && !g.pre_act && !g.relu)) {
+  if (raw || (g.beta == 0.0f && !g.bias && !g.pre_act && !g.relu && !g.mask)) {
     for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
     return;
   }
+  if (g.mask)
+    for_each([&](int i, int j, int v, size_t idx, size_t) {
+      acc[i][j][v] = (g.mask[idx] >= 0.0f ? 1.0f : 0.0f) * acc[i][j][v];
+    });
   if (g.beta != 0.0f)
     for_each([&](int i, int j, int v, size_t idx, size_t) { acc[i][j][v] = g.beta * g.C[idx] + acc[i][j][v]; });
   if (g.bias) {

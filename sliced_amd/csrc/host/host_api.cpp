@@ -32,7 +32,13 @@ SLH_API int slh_device_free(void* dev) {
   return guard([&] { delete (HIP*)dev; });
 }
 SLH_API int slh_set_grad_policy(void* dev, float gemm_beta, float softmax_beta, float transpose_beta) {
-  return guard([&] { ((HIP*)dev)->policy = GradPolicy{gemm_beta, softmax_beta, transpose_beta}; });
+  return guard([&] {
+    GradPolicy& p = ((HIP*)dev)->policy;
+    p.gemm_beta = gemm_beta; p.softmax_beta = softmax_beta; p.transpose_beta = transpose_beta;
+  });
+}
+SLH_API int slh_set_fuse_relu_grad(void* dev, int on) {
+  return guard([&] { ((HIP*)dev)->policy.fuse_relu_grad = on != 0; });
 }
 SLH_API int slh_buffer_from(void* dev, const float* host, size_t len, uint64_t* id) {
   return guard([&] { *id = ((HIP*)dev)->from(host, len).id; });

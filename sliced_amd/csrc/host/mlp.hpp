@@ -56,7 +56,7 @@ struct MlpResult {
 };
 
 enum MlpMode {
-  MLP_FUSED = 1,  // Linear (+ReLU) forward as one kernel
+  MLP_FUSED = 1,  // Linear (+ReLU) forward as one kernel, ReLU gradient inside the next layer's input-gradient GEMM
   MLP_GRAPH = 2,  // step 0 runs eagerly, step 1 is recorded, every later step replays the recording
   MLP_FUSED_LOSS = 4  // the loss chain (MSE, or softmax + cross-entropy) as one forward and one backward kernel
 };
@@ -88,6 +88,9 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
   Buffer seed = kind == 1 ? dev.alloc(n_out, true) : Buffer();
   Buffer loss_dev = dev.alloc(1, true);
   Buffer loss_log = graph ? dev.alloc(warmup + steps, true) : Buffer();
+
+  // with the fused Linear the ReLU gradients ride in the next layer's input-gradient GEMM
+  dev.policy.fuse_relu_grad = fused;
 
   // One training step.  Leaves the loss in loss_dev; reads it back unless `deferred`.
   auto train_step = [&](bool deferred) -> float {

@@ -29,6 +29,7 @@
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "sliced_hip.h"
@@ -93,6 +94,11 @@ struct GradPolicy {
   float gemm_beta = 0.0f;
   float softmax_beta = 0.0f;
   float transpose_beta = 0.0f;
+  // A fused Linear whose input is the ReLU output of another fused Linear writes its input gradient
+  // already multiplied by that ReLU's gradient, (g·Wᵀ) ⊙ (pre >= 0), straight into pre's gradient:
+  // one kernel instead of GEMM + elementwise pass, equal values (a zero may change its sign).  Off by
+  // default: it is only the sequence the tape would run when that ReLU output feeds nothing else.
+  bool fuse_relu_grad = false;
 };
 
 class HIP {
@@ -236,6 +242,8 @@ class HIP {
   void run_tape() {
     for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
     tape_.clear();
+    relu_pre_.clear();
+    relu_grad_done_.clear();
   }
   void backward(const Buffer& out) {
     Buffer g = grad_mut(out);
@@ -275,18 +283,34 @@ class HIP {
     check(slhip_linear_fwd(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, relu ? 1 : 0, relu ? pre.ptr : nullptr, out.ptr),
           "slhip_linear_fwd");
     uint64_t xi = x.id, wi = w.id, bi = bias.id, oi = out.id, pi = relu ? pre.id : 0;
+    if (relu) relu_pre_[oi] = pi;
     add_grad_fn([=] {
       Buffer xb = lookup(xi), wb = lookup(wi), bb = lookup(bi), o = lookup(oi);
-      Buffer g = grad(o);
+      Buffer g;
       if (relu) {  // relu grad: pre.grad += (pre >= 0) * out.grad
         Buffer p = lookup(pi);
         Buffer pg = grad_mut(p);
-        check(slhip_ew_unary_grad(ctx_, SLHIP_RELU, 0.0f, p.len, p.ptr, pg.ptr, g.ptr), "relu grad");
+        relu_pre_.erase(oi);
+        if (!relu_grad_done_.erase(oi))  // else the consumer's backward has written pre.grad already
+          check(slhip_ew_unary_grad(ctx_, SLHIP_RELU, 0.0f, p.len, p.ptr, pg.ptr, grad(o).ptr), "relu grad");
         g = pg;
+      } else {
+        g = grad(o);
       }
       check(slhip_add_row_mut_grad(ctx_, m, n, grad_mut(bb).ptr, g.ptr), "bias grad");
       float* xg = xb.requires_grad ? grad_mut(xb).ptr : nullptr;
       float* wg = wb.requires_grad ? grad_mut(wb).ptr : nullptr;
+      auto producer = relu_pre_.find(xi);
+      if (policy.fuse_relu_grad && xg && producer != relu_pre_.end()) {
+        // x is the ReLU output of a fused Linear that is still on the tape
+        Buffer xp = lookup(producer->second);
+        // written the way gemm_grad writes x.grad (policy.gemm_beta; SET by default): pre.grad is
+        // zero at this point, and `0 + v` differs from `v` only in the sign of a zero
+        check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_mut(xp).ptr, policy.gemm_beta),
+              "slhip_sgemm_relu_mask");
+        relu_grad_done_.insert(xi);
+        xg = nullptr;
+      }
       check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
     });
     return out;
@@ -570,6 +594,8 @@ class HIP {
   std::unordered_map<uint64_t, Buffer> grads_;
   std::vector<Slab> slabs_;
   std::vector<std::function<void()>> tape_;
+  std::unordered_map<uint64_t, uint64_t> relu_pre_;   // ReLU output of a fused Linear on the tape -> its pre-activation
+  std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
   bool tape_enabled_ = true;
   std::vector<Buffer> cache_;
   size_t cursor_ = 0;

@@ -263,6 +263,17 @@ def sgemm(ta, tb, m, n, k, a, b, c=None, beta=0.0):
     return res
 
 
+def sgemm_relu_mask(ta, tb, m, n, k, a, b, pre, c=None, beta=0.0):
+    """c = beta*c + (op(a)·op(b)) * (pre >= 0)."""
+    a, b, pre = _f32(a), _f32(b), _f32(pre)
+    assert a.size == m * k and b.size == k * n and pre.size == m * n
+    with _Scope() as s:
+        da, db, dp = s.up(a), s.up(b), s.up(pre)
+        dc = s.up(c) if c is not None else s.empty(m * n)
+        s.c.call("slhip_sgemm_relu_mask", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dp.ptr, dc.ptr, float(beta))
+        return dc.numpy()
+
+
 TAIL_AUTO, TAIL_WHOLE, TAIL_SPREAD = 0, 1, 2
 
 

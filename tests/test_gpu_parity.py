@@ -147,6 +147,30 @@ def test_gemm_spread_tail(hip, orc):
         hip.gemm_tail_policy(hip.TAIL_AUTO)
 
 
+def test_sgemm_relu_mask_equals_gemm_then_relu_grad(hip, orc):
+    # every kernel that has the epilogue: wave per tile, tiled, split K, spread tail
+    shapes = [(64, 64, 64, 0, 1), (1024, 64, 64, 0, 1), (100, 37, 19, 0, 0), (256, 256, 4096, 0, 1), (640, 384, 300, 0, 1),
+              (1000, 1000, 512, 1, 0), (515, 259, 1001, 0, 1)]
+    try:
+        for policy in (hip.TAIL_AUTO, hip.TAIL_SPREAD):
+            hip.gemm_tail_policy(policy)
+            for (m, n, k, ta, tb) in shapes:
+                say("sgemm_relu_mask", policy, m, n, k, ta, tb)
+                a, b = gemm_operands(ta, tb, m, n, k)
+                pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+                pre[::7] = 0.0          # (0 >= 0) passes the gradient, like the reference's relu grad
+                pre[3::11] = -0.0
+                c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+                prod = hip.sgemm(ta, tb, m, n, k, a, b)
+                masked = orc.unary_grad(orc.RELU, pre, np.zeros(m * n, np.float32), prod)   # 0 + (pre >= 0) * prod
+                got = hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre)
+                assert np.array_equal(got, masked)
+                got1 = hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre, c=c0.copy(), beta=1.0)
+                assert np.array_equal(got1, c0 + masked)
+    finally:
+        hip.gemm_tail_policy(hip.TAIL_AUTO)
+
+
 def test_gemm_grad_matches_oracle(hip, orc):
     for (m, k, n) in [(4, 2, 3), (70, 33, 19), (256, 128, 64), (1024, 64, 1), (1024, 1, 64)]:
         say("gemm_grad", m, k, n)

@@ -297,6 +297,32 @@ def test_linear_fused_matches_unfused_tape(device):
         assert np.array_equal(a, c)
 
 
+def test_relu_grad_fused_into_the_next_layers_input_gradient(device):
+    # two fused Linear+ReLU layers and a plain one: with the ReLU gradients riding in the next
+    # layer's input-gradient GEMM every gradient keeps its bits
+    m, d0, d1, d2, d3 = 192, 40, 96, 72, 10
+    x = rng.uniform(m * d0, -1, 1, tag=0)
+    ws = [rng.uniform(a * b, -0.5, 0.5, tag=10 + i) for i, (a, b) in enumerate([(d0, d1), (d1, d2), (d2, d3)])]
+    bs = [rng.uniform(b, -0.5, 0.5, tag=20 + i) for i, b in enumerate([d1, d2, d3])]
+    res = []
+    try:
+        for fuse in (False, True):
+            device.set_fuse_relu_grad(fuse)
+            xb = device.buffer(x)
+            wb = [device.buffer(w) for w in ws]
+            bb = [device.buffer(b) for b in bs]
+            h1 = device.linear(m, d0, d1, xb, wb[0], bb[0], True)
+            h2 = device.linear(m, d1, d2, h1, wb[1], bb[1], True)
+            out = device.linear(m, d2, d3, h2, wb[2], bb[2], False)
+            out.backward()
+            res.append([out.read(), xb.grad().read()] + [w.grad().read() for w in wb] + [b.grad().read() for b in bb])
+    finally:
+        device.set_fuse_relu_grad(False)
+    assert np.abs(res[0][1]).max() > 0
+    for a, c in zip(*res):
+        assert np.array_equal(a, c)
+
+
 def test_errors_surface_as_exceptions(device):
     from sliced_amd import host
     a = device.buffer([1, 2, 3])
