@@ -141,6 +141,13 @@ int32_t slhip_sgemm_relu_mask(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, 
  * is deterministic.  A tuning and testing knob: no counterpart in the reference. */
 enum { SLHIP_TAIL_AUTO = 0, SLHIP_TAIL_WHOLE = 1, SLHIP_TAIL_SPREAD = 2 };
 int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy);
+/* The tile of C that one workgroup of the tiled kernel computes.  SLHIP_TILE_AUTO (the default)
+ * chooses by a cost model (64 x 64, unsplit, for products of a few hundred such tiles and a
+ * moderate K; 128 x 128 otherwise); the others force a tile for every product that takes the tiled
+ * kernel.  Same results up to the summation order of k splits; a tuning and testing knob with no
+ * counterpart in the reference. */
+enum { SLHIP_TILE_AUTO = 0, SLHIP_TILE_128X128 = 1, SLHIP_TILE_64X64 = 3 };
+int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy);
 
 /* Gemm::gemm (src/ops2/gemm/mod.rs:21-32), trait argument order (m, k, n). */
 int32_t slhip_gemm(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,

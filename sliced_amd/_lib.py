@@ -43,6 +43,7 @@ PROTOTYPES = {
     "slhip_rand_uniform": [c_vp, C.c_uint64, C.c_uint64, C.c_float, C.c_float, c_sz, c_vp],
     "slhip_sgemm": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_gemm_tail_policy": [c_vp, c_i32],
+    "slhip_gemm_tile_policy": [c_vp, c_i32],
     "slhip_sgemm_relu_mask": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_gemm": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_gemm_grad": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp, C.c_float],

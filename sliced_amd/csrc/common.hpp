@@ -21,6 +21,7 @@ struct slhip_ctx {
   char name[64] = {0};
   bool capturing = false;        // between slhip_graph_begin and slhip_graph_end
   int gemm_tail = 0;             // SLHIP_TAIL_*: how the tiled GEMM treats a partly filled last round
+  int gemm_tile = 0;             // SLHIP_TILE_*: tile of C per workgroup of the tiled GEMM
 };
 
 struct slhip_event {

@@ -22,12 +22,11 @@
 
 namespace slhip {
 
-template <bool TA, bool TB, int BK, bool ONLY_FAST>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
-  constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
-  __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
-  gemm_whole_tile<TA, TB, BK, ONLY_FAST>(g, lds_a, lds_b);
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<BK, 64 * WM>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 64 * WN>::STAGE_FLOATS];
+  gemm_whole_tile<TA, TB, BK, ONLY_FAST, WM, WN>(g, lds_a, lds_b);
 }
 
 // Small and skinny problems.  One wave owns one 32x32 tile of C and feeds the matrix core straight
@@ -296,9 +295,9 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     return splitk_combine(ctx, g, splits);
   }
 
-  const size_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  if (tiles_m * tiles_n > 0x7fffffffu) {
-    set_error("sgemm: %zu x %zu tiles exceed one launch", tiles_m, tiles_n);
+  size_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  if ((M + 63) / 64 * ((N + 63) / 64) > 0x7fffffffu) {
+    set_error("sgemm: %zu x %zu tiles exceed one launch", (M + 63) / 64, (N + 63) / 64);
     return SLHIP_EINVAL;
   }
   g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
@@ -312,7 +311,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // up to four rounds are considered too: 576 tiles (3072^3) unsplit run one full round and one
   // that is an eighth full, 75 TFLOP/s against 106 with four splits.
   constexpr int BK = GEMM_BK;
-  const size_t tiles = tiles_m * tiles_n;
+  size_t tiles = tiles_m * tiles_n;
   const size_t slots = (size_t)ctx->num_cu * 2;
   size_t splits = 1;
   const size_t kt_total = (K + BK - 1) / BK;
@@ -360,6 +359,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       const double t = (double)(full / slots) * ((double)kt_total * 4.35 + 6.0) + (double)units * per_kt + 6.0 + 4.0 +
                        2.0 * (double)runs * (double)(SPREAD_SLOT * sizeof(float)) / 5.0e6;
       if (t < best || ctx->gemm_tail == SLHIP_TAIL_SPREAD) {
+        best = t;
         splits = 1;
         sp.first = (unsigned)full;
         sp.units = (unsigned)units;
@@ -368,6 +368,34 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       }
     }
   }
+
+  // 64 x 64 tiles, one workgroup per tile and no k split, for products of a few hundred such tiles
+  // and a moderate K, where the plans above spend a third of their time combining partial
+  // products: 1024^3 takes 33 us as 64 tiles x 4 k splits + combine and 28 us as 256 small tiles
+  // (896^3 +12 %, 704^3 +25 %, 2048x512x1024 +18 %).  A small tile's k tile measures 0.75 us with
+  // the CU to itself, 1.25 / 1.8 / 2.3 us when two / three / four workgroups share the CU (4096^3
+  // would run at 116 TFLOP/s that way), plus 5 us per launch; it has to beat the modelled time of
+  // the best 128 x 128 plan by 8 %, the models being good to about that.
+  bool small_tile = false;
+  if (!(ta && tb)) {  // the doubly transposed form is not instantiated for the small tile
+    const size_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+    if (ctx->gemm_tile == SLHIP_TILE_64X64) {
+      small_tile = true;
+    } else if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && best < 1e299 &&
+               tiles64 <= 4 * (size_t)ctx->num_cu) {
+      static const double per_kt[5] = {0.0, 0.75, 1.25, 1.8, 2.3};
+      const size_t share = (tiles64 + ctx->num_cu - 1) / ctx->num_cu;
+      small_tile = (double)kt_total * per_kt[share] + 5.0 < 0.92 * best;
+    }
+    if (small_tile) {
+      tiles_m = (M + 63) / 64; tiles_n = (N + 63) / 64;
+      tiles = tiles64;
+      g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
+      splits = 1;
+      spread_workers = 0;
+    }
+  }
+  const size_t tile_m = small_tile ? 64 : BM, tile_n = small_tile ? 64 : BN;
 
   size_t k_chunk = (K + splits - 1) / splits;
   k_chunk = (k_chunk + BK - 1) / BK * BK;
@@ -379,19 +407,25 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
 
   // every k tile of every workgroup complete, inside and 16-byte aligned: the kernel without the
   // clamped loops (k_chunk is a multiple of BK, so only the end of K can leave a partial tile)
-  const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % BM == 0 && N % BN == 0 && K % BK == 0;
+  const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % tile_m == 0 && N % tile_n == 0 && K % BK == 0;
   if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, g, sp, spread_workers, tiles - sp.first);
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
-#define SL_GEMM(TA_, TB_)                                                                                     \
-  do {                                                                                                        \
-    if (only_fast) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, true>), grid, dim3(256), 0, ctx->stream, g); \
-    else hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, false>), grid, dim3(256), 0, ctx->stream, g);     \
+#define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                  \
+  do {                                                                                                                \
+    if (only_fast) hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, true, WM_, WN_>), grid, dim3(256), 0, ctx->stream, g); \
+    else hipLaunchKernelGGL((gemm_kernel<TA_, TB_, GEMM_BK, false, WM_, WN_>), grid, dim3(256), 0, ctx->stream, g);  \
+  } while (0)
+#define SL_GEMM(TA_, TB_)                       \
+  do {                                          \
+    if (small_tile) SL_GEMM3(TA_, TB_, 1, 1);   \
+    else SL_GEMM3(TA_, TB_, 2, 2);              \
   } while (0)
   if (!ta && !tb) SL_GEMM(false, false);
   else if (!ta && tb) SL_GEMM(false, true);
   else if (ta && !tb) SL_GEMM(true, false);
-  else SL_GEMM(true, true);
+  else SL_GEMM3(true, true, 2, 2);
+#undef SL_GEMM3
 #undef SL_GEMM
   int32_t rc = post_launch();
   if (rc || splits == 1) return rc;
@@ -435,6 +469,13 @@ SLHIP_API int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy) {
   SLHIP_REQUIRE(ctx, "null argument");
   SLHIP_REQUIRE(policy == SLHIP_TAIL_AUTO || policy == SLHIP_TAIL_WHOLE || policy == SLHIP_TAIL_SPREAD, "unknown policy");
   ctx->gemm_tail = policy;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy) {
+  SLHIP_REQUIRE(ctx, "null argument");
+  SLHIP_REQUIRE(policy == SLHIP_TILE_AUTO || policy == SLHIP_TILE_128X128 || policy == SLHIP_TILE_64X64, "unknown policy");
+  ctx->gemm_tile = policy;
   return SLHIP_OK;
 }
 

@@ -12,8 +12,8 @@ namespace slhip {
 // A workgroup of the spread tail: up to two runs of k tiles, each inside one tile of C, each
 // written as a raw partial tile (row-major 128 x 128) to workspace slot 2*w + run.
 template <bool TA, bool TB, int BK, bool ONLY_FAST>
-__device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
-                                                   float (*lds_b)[Cfg<BK>::STAGE_FLOATS]) {
+__device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp, float (*lds_a)[Cfg<BK, 128>::STAGE_FLOATS],
+                                                   float (*lds_b)[Cfg<BK, 128>::STAGE_FLOATS]) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
   const int r = lane & 31, h = lane >> 5;
@@ -37,7 +37,7 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    gemm_k_range<TA, TB, BK, ONLY_FAST>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
+    gemm_k_range<TA, TB, BK, ONLY_FAST, 2, 2>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
 
     float* slot = g.partial + ((size_t)2 * w + run) * SPREAD_SLOT;
 #pragma unroll
@@ -52,11 +52,11 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
 
 template <bool TA, bool TB, int BK, bool ONLY_FAST>
 __global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadArgs sp) {
-  constexpr int STAGE = Cfg<BK>::STAGE_FLOATS;
+  constexpr int STAGE = Cfg<BK, 128>::STAGE_FLOATS;
   __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
   __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
   if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST>(g, sp, lds_a, lds_b);
-  else gemm_whole_tile<TA, TB, BK, ONLY_FAST>(g, lds_a, lds_b);
+  else gemm_whole_tile<TA, TB, BK, ONLY_FAST, 2, 2>(g, lds_a, lds_b);
 }
 
 // The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup

@@ -1,8 +1,12 @@
-// The 128 x 128 tile machinery of the f32 GEMM: argument block, global -> LDS staging, MFMA
-// fragment reads, the software-pipelined k loop and the whole-tile workgroup body.  Shared by the
-// plain kernel (gemm.hip) and the spread-tail kernel (gemm_spread.hip), which are separate
-// translation units on purpose: the plain kernel's k loop gains or loses about 1.5 % with the
-// code the compiler happens to place around it, and a kernel added to its file moved it.
+// The tile machinery of the f32 GEMM: argument block, global -> LDS staging, MFMA fragment reads,
+// the software-pipelined k loop and the whole-tile workgroup body.  Shared by the plain kernel
+// (gemm.hip) and the spread-tail kernel (gemm_spread.hip), which are separate translation units
+// on purpose: the plain kernel's k loop gains or loses about 1.5 % with the code the compiler
+// happens to place around it, and a kernel added to its file moved it.
+//
+// A workgroup is 4 waves in a 2 x 2 grid; every wave owns WM x WN accumulators of 32 x 32, so the
+// workgroup's tile of C is (64*WM) x (64*WN): 128 x 128 for large products, 128 x 64 and 64 x 64
+// for products whose 128 x 128 grid would leave most of the chip idle.
 #pragma once
 #include <type_traits>
 
@@ -14,13 +18,14 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 128, BN = 128;
 constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form at 2048^3 and above
-constexpr int XC_PITCH = 128 + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
 
-template <int BK>
+// One operand tile: XT rows or columns of the operand (64 or 128) by BK of k.
+template <int BK, int XT>
 struct Cfg {
   static constexpr int KC_PITCH = BK + 4;  // [x][k] layout, k contiguous
-  static constexpr int STAGE_FLOATS = 128 * KC_PITCH > BK * XC_PITCH ? 128 * KC_PITCH : BK * XC_PITCH;
-  static constexpr int NV = BK * 128 / 4 / 256;  // float4 per thread per operand tile
+  static constexpr int XC_PITCH = XT + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
+  static constexpr int STAGE_FLOATS = XT * KC_PITCH > BK * XC_PITCH ? XT * KC_PITCH : BK * XC_PITCH;
+  static constexpr int NV = BK * XT / 4 / 256;  // float4 per thread per operand tile
 };
 
 struct GemmArgs {
@@ -41,7 +46,7 @@ struct GemmArgs {
   size_t m_fast;      // M when both operand bases are 16-byte aligned as well, else 0: no tile counts as interior
 };
 
-// Spread tail (gemm_kernel<..., SPREAD = true>): workgroups below `first` compute whole tiles;
+// Spread tail (gemm_spread_kernel): workgroups below `first` compute whole tiles;
 // workgroup first + w computes k tiles [w*units, (w+1)*units) of the sequence "tile `first`, all
 // its kt_total k tiles; tile first + 1, ..." (`total` long).  Kept out of GemmArgs: the plain
 // kernel's code, and with it its speed, depends on the layout of its argument block.
@@ -52,9 +57,9 @@ struct SpreadArgs {
 constexpr size_t SPREAD_SLOT = (size_t)BM * BN;  // floats of one partial tile in the workspace
 
 // Operand tile held in registers between the global load and the LDS store.
-template <int BK>
+template <int BK, int XT>
 struct Frag {
-  float4 v[Cfg<BK>::NV];
+  float4 v[Cfg<BK, XT>::NV];
 };
 
 // How a k tile is fetched from global memory.
@@ -76,14 +81,14 @@ struct Frag {
 // the one before it).
 enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2, LOAD_XCLAMP = 3 };
 
-// k-contiguous source: element (x, k) at src[x*ld + k]; tile 128 x BK.
-template <int BK, int MODE>
-__device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+// k-contiguous source: element (x, k) at src[x*ld + k]; tile XT x BK.
+template <int BK, int XT, int MODE>
+__device__ __forceinline__ void load_kc(Frag<BK, XT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
   constexpr int VPR = BK / 4, RPP = 256 / VPR;  // float4 per row, rows per pass
   const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) {
+  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) {
     const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + x * ld + k);
@@ -108,23 +113,24 @@ __device__ __forceinline__ void load_kc(Frag<BK>& f, const float* __restrict__ s
     }
   }
 }
-template <int BK>
-__device__ __forceinline__ void store_kc(const Frag<BK>& f, float* lds) {
+template <int BK, int XT>
+__device__ __forceinline__ void store_kc(const Frag<BK, XT>& f, float* lds) {
   constexpr int VPR = BK / 4, RPP = 256 / VPR;
   const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK>::KC_PITCH + 4 * kq, f.v[p]);
+  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK, XT>::KC_PITCH + 4 * kq, f.v[p]);
 }
 
-// x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x 128.  LOAD_VCLAMP relies on
+// x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x XT.  LOAD_VCLAMP relies on
 // X % 4 == 0 (implied by ld % 4 == 0, ld being X here): a float4 is inside or outside as a whole.
-template <int BK, int MODE>
-__device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+template <int BK, int XT, int MODE>
+__device__ __forceinline__ void load_xc(Frag<BK, XT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
-  const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;  // 32 float4 per k-row, 8 rows per pass
+  constexpr int XQ = XT / 4, KR = 256 / XQ;  // float4 per k-row (32 or 16), k-rows per pass (8 or 16)
+  const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) {
-    const size_t k = k0 + kr + 8 * p, x = x0 + 4 * xq;
+  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) {
+    const size_t k = k0 + kr + KR * p, x = x0 + 4 * xq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + k * ld + x);
     } else if (MODE == LOAD_XCLAMP) {
@@ -147,25 +153,26 @@ __device__ __forceinline__ void load_xc(Frag<BK>& f, const float* __restrict__ s
     }
   }
 }
-template <int BK>
-__device__ __forceinline__ void store_xc(const Frag<BK>& f, float* lds) {
-  const int xq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+template <int BK, int XT>
+__device__ __forceinline__ void store_xc(const Frag<BK, XT>& f, float* lds) {
+  constexpr int XQ = XT / 4, KR = 256 / XQ;
+  const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK>::NV; ++p) st4(lds + (kr + 8 * p) * XC_PITCH + 4 * xq, f.v[p]);
+  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
 }
 
-// MFMA fragments of one 8-wide k group for the two 32-row blocks of this wave's 64 rows.
-// KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's 64 rows/cols.
-template <bool KC, int BK>
-__device__ __forceinline__ void read_frag(float (&out)[2][4], const float* lds, int x_base, int kk8, int r, int h) {
+// MFMA fragments of one 8-wide k group for the NI 32-row blocks of this wave's rows (or columns).
+// KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's rows/cols in the tile.
+template <bool KC, int BK, int XT, int NI>
+__device__ __forceinline__ void read_frag(float (&out)[NI][4], const float* lds, int x_base, int kk8, int r, int h) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < NI; ++i) {
     if (KC) {
-      float4 t = ld4(lds + (x_base + 32 * i + r) * Cfg<BK>::KC_PITCH + kk8 * 8 + 4 * h);
+      float4 t = ld4(lds + (x_base + 32 * i + r) * Cfg<BK, XT>::KC_PITCH + kk8 * 8 + 4 * h);
       out[i][0] = t.x; out[i][1] = t.y; out[i][2] = t.z; out[i][3] = t.w;
     } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) out[i][t] = lds[(kk8 * 8 + 4 * h + t) * XC_PITCH + x_base + 32 * i + r];
+      for (int t = 0; t < 4; ++t) out[i][t] = lds[(kk8 * 8 + 4 * h + t) * Cfg<BK, XT>::XC_PITCH + x_base + 32 * i + r];
     }
   }
 }
@@ -212,10 +219,11 @@ constexpr int PIN_XCLAMP[2][2] = {{1, 2}, {1, 1}};
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
 // ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
 // kernel's throughput.
-template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST>
+template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST, int WM, int WN>
 __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
-                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
-                                           float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
+                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
+                                           float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;  // the workgroup's tile of C
   constexpr int KSTEPS = BK / 8;
   constexpr int REFILL_AT = (TA && !TB) ? KSTEPS - 1 : (KSTEPS > 1 ? 1 : 0);
   if (kt_begin >= kt_end) return;
@@ -226,17 +234,18 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   // unless transposed ([n][k], ld = K).
   const size_t lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
 
-  Frag<BK> fa, fb;
+  Frag<BK, TM> fa;
+  Frag<BK, TN> fb;
   auto load_stage = [&](int kt) {
     const size_t k0 = kbeg + (size_t)kt * BK;
-    if (TA) load_xc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    else load_kc<BK, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    if (TB) load_kc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
-    else load_xc<BK, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
+    if (TA) load_xc<BK, TM, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
+    else load_kc<BK, TM, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
+    if (TB) load_kc<BK, TN, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
+    else load_xc<BK, TN, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
   };
   auto store_stage = [&](int s) {
-    if (TA) store_xc<BK>(fa, lds_a[s]); else store_kc<BK>(fa, lds_a[s]);
-    if (TB) store_kc<BK>(fb, lds_b[s]); else store_xc<BK>(fb, lds_b[s]);
+    if (TA) store_xc<BK, TM>(fa, lds_a[s]); else store_kc<BK, TM>(fa, lds_a[s]);
+    if (TB) store_kc<BK, TN>(fb, lds_b[s]); else store_xc<BK, TN>(fb, lds_b[s]);
   };
 
   // Software pipeline over the k tiles.  While tile kt is multiplied out of LDS stage s:
@@ -254,19 +263,20 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   if (kt_begin + 1 < kt_end) load_stage(kt_begin + 1);
   __syncthreads();
 
-  if (MODE == LOAD_FAST) pin_loop_start<ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
-  if (MODE == LOAD_XCLAMP) pin_loop_start<PIN_XCLAMP[TA][TB]>();
+  constexpr bool BIG = WM == 2 && WN == 2;  // the offsets were measured for the 128 x 128 tile
+  if (MODE == LOAD_FAST) pin_loop_start<!BIG ? 0 : ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
+  if (MODE == LOAD_XCLAMP) pin_loop_start<BIG ? PIN_XCLAMP[TA][TB] : 0>();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int s = (kt - kt_begin) & 1;
-    float a[2][2][4], b[2][2][4];
-    read_frag<!TA, BK>(a[0], lds_a[s], wm * 64, 0, r, h);
-    read_frag<TB, BK>(b[0], lds_b[s], wn * 64, 0, r, h);
+    float a[2][WM][4], b[2][WN][4];
+    read_frag<!TA, BK, TM, WM>(a[0], lds_a[s], wm * 32 * WM, 0, r, h);
+    read_frag<TB, BK, TN, WN>(b[0], lds_b[s], wn * 32 * WN, 0, r, h);
 #pragma unroll
     for (int kk8 = 0; kk8 < KSTEPS; ++kk8) {
       const int cur = kk8 & 1, nxt = cur ^ 1;
       if (kk8 + 1 < KSTEPS) {
-        read_frag<!TA, BK>(a[nxt], lds_a[s], wm * 64, kk8 + 1, r, h);
-        read_frag<TB, BK>(b[nxt], lds_b[s], wn * 64, kk8 + 1, r, h);
+        read_frag<!TA, BK, TM, WM>(a[nxt], lds_a[s], wm * 32 * WM, kk8 + 1, r, h);
+        read_frag<TB, BK, TN, WN>(b[nxt], lds_b[s], wn * 32 * WN, kk8 + 1, r, h);
       }
       if (kk8 == REFILL_AT) {
         // stage s^1 was last read in the previous iteration, which ended with a barrier
@@ -280,9 +290,9 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < WM; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < WN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][t], b[cur][j][t], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
@@ -301,16 +311,16 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 // ONLY_FAST: the host has checked that every k tile of every tile qualifies for LOAD_FAST (M and N
 // multiples of 128, every k chunk a multiple of BK, operands float4-loadable and 16-byte aligned);
 // the kernel then contains that one loop and nothing else.
-template <bool TA, bool TB, int BK, bool ONLY_FAST>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
 __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, size_t kbeg, size_t kend, size_t m0,
-                                             size_t n0, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
-                                             float (*lds_b)[Cfg<BK>::STAGE_FLOATS], floatx16 (&acc)[2][2]) {
+                                             size_t n0, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
+                                             float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
   if (ONLY_FAST) {
-    gemm_tiles<TA, TB, BK, LOAD_FAST, true>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+    gemm_tiles<TA, TB, BK, LOAD_FAST, true, WM, WN>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
     return;
   }
   const bool vec = g.a_vec && g.b_vec;
-  const bool fast = vec && m0 + BM <= g.m_fast && n0 + BN <= g.N;
+  const bool fast = vec && m0 + 64 * WM <= g.m_fast && n0 + 64 * WN <= g.N;
   const int kfull = (int)((kend - kbeg) / BK);             // complete k tiles of the chunk
   const int before_last = (int)((g.K - 1 - kbeg) / BK);    // k tiles that end before index K - 1
   int e1 = fast ? (kb < kfull ? kb : kfull) : ka;
@@ -321,20 +331,21 @@ __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, 
     if (e2 < e1) e2 = e1;
   }
   const int e3 = vec ? kb : e2;
-  gemm_tiles<TA, TB, BK, LOAD_FAST, false>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_FAST, false, WM, WN>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false, WM, WN>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false, WM, WN>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false, WM, WN>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 }
 
 // A workgroup that computes one whole tile of C (or, with g.splits > 1, one k chunk of it as a raw
 // partial product): blockIdx.x = tile, blockIdx.y = k chunk.
-template <bool TA, bool TB, int BK, bool ONLY_FAST>
-__device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK>::STAGE_FLOATS],
-                                                float (*lds_b)[Cfg<BK>::STAGE_FLOATS]) {
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
+__device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
+                                                float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS]) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
   unsigned tm, tn;
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
   const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
   const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
   const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
@@ -343,34 +354,34 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   const int wm = wave >> 1, wn = wave & 1;
   const int r = lane & 31, h = lane >> 5;
 
-  floatx16 acc[2][2];
+  floatx16 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  gemm_k_range<TA, TB, BK, ONLY_FAST>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
-  //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's 64x64 tile.
+  //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's (32*WM) x (32*WN) tile.
   // No load may sit between two stores: C, pre_act and dst can be the same memory as far as the
   // compiler knows, so a `beta * C[idx]` read after a store waits for that store, 64 times in a
   // row (measured: 7.5 us per workgroup, more than a 128x128x128 product itself).  Hence: first
   // every read (C for beta), then only stores; and the common plain case is its own loop.
   const bool raw = g.splits > 1;
   float* dst = raw ? g.partial + (size_t)blockIdx.y * g.M * g.N : g.C;
-  const bool interior = m0 + BM <= g.M && n0 + BN <= g.N;
+  const bool interior = m0 + TM <= g.M && n0 + TN <= g.N;
   auto for_each = [&](auto&& fn) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const size_t col = n0 + wn * 64 + 32 * j + r;
+      for (int j = 0; j < WN; ++j) {
+        const size_t col = n0 + wn * 32 * WN + 32 * j + r;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const size_t row = m0 + wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
+          const size_t row = m0 + wm * 32 * WM + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
           if (interior || (row < g.M && col < g.N)) fn(i, j, v, row * g.N + col, col);
         }
       }
@@ -386,10 +397,10 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   if (g.beta != 0.0f)
     for_each([&](int i, int j, int v, size_t idx, size_t) { acc[i][j][v] = g.beta * g.C[idx] + acc[i][j][v]; });
   if (g.bias) {
-    float bv[2];
+    float bv[WN];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + wn * 64 + 32 * j + r;
+    for (int j = 0; j < WN; ++j) {
+      const size_t col = n0 + wn * 32 * WN + 32 * j + r;
       bv[j] = col < g.N ? g.bias[col] : 0.0f;
     }
     for_each([&](int i, int j, int v, size_t, size_t) { acc[i][j][v] = acc[i][j][v] + bv[j]; });

@@ -282,6 +282,14 @@ def gemm_tail_policy(policy):
     ctx().call("slhip_gemm_tail_policy", int(policy))
 
 
+TILE_AUTO, TILE_128X128, TILE_64X64 = 0, 1, 3
+
+
+def gemm_tile_policy(policy):
+    """The tile of C per workgroup of the tiled GEMM (a tuning knob)."""
+    ctx().call("slhip_gemm_tile_policy", int(policy))
+
+
 def gemm(m, n, k, a, b, c=None, beta=0.0):
     """GenericBlas::gemm(m, n, k, a, b, c)."""
     return sgemm(0, 0, m, n, k, a, b, c, beta)

@@ -147,6 +147,36 @@ def test_gemm_spread_tail(hip, orc):
         hip.gemm_tail_policy(hip.TAIL_AUTO)
 
 
+def test_gemm_small_tile(hip, orc):
+    # 64 x 64 tiles (chosen by the cost model for products of a few hundred such tiles), forced here
+    # so that edge tiles, rows of odd length, k remainders and the fused epilogues all run on them
+    shapes = [(1000, 1000, 512, 0, 0), (1024, 1024, 1024, 0, 1), (999, 1001, 515, 1, 0), (640, 384, 300, 0, 0),
+              (129, 257, 4099, 0, 1), (2048, 64, 777, 1, 0), (65, 2000, 333, 0, 0)]
+    try:
+        for (m, n, k, ta, tb) in shapes:
+            say("small-tile gemm", m, n, k, ta, tb)
+            a, b = gemm_operands(ta, tb, m, n, k)
+            exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+            hip.gemm_tile_policy(hip.TILE_64X64)
+            got = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+            c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+            assert np.array_equal(hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+            pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+            assert np.array_equal(hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+            if not ta and not tb:
+                bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+                out, pre_act = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+                pre_ref = orc.add_row(m, n, got, bias)
+                assert np.array_equal(pre_act, pre_ref)
+                assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+            hip.gemm_tile_policy(hip.TILE_128X128)
+            big = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - big) <= 2 * bound)
+    finally:
+        hip.gemm_tile_policy(hip.TILE_AUTO)
+
+
 def test_sgemm_relu_mask_equals_gemm_then_relu_grad(hip, orc):
     # every kernel that has the epilogue: wave per tile, tiled, split K, spread tail
     shapes = [(64, 64, 64, 0, 1), (1024, 64, 64, 0, 1), (100, 37, 19, 0, 0), (256, 256, 4096, 0, 1), (640, 384, 300, 0, 1),
