@@ -348,7 +348,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
-                   "kernel": "gemm_kernel<false,false,32,true>: 128x128 tiles, BK=32, v_mfma_f32_32x32x2_f32"},
+                   "kernel": "gemm_kernel<false,false,32,true,2,2>: 128x128 tiles, BK=32, v_mfma_f32_32x32x2_f32"},
         "roofline": {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": head["frac_of_peak"],
                      "traffic": GEMM_4096_TRAFFIC_BYTES if M == 4096 else None},

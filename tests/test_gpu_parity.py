@@ -328,7 +328,9 @@ def test_broadcast_grads_are_bit_exact(hip, orc):
 SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (64, 1024), (17, 1000), (9, 4096),
                   (5, 4100), (3, 16384), (2, 16390), (2, 40000), (1000, 1), (50, 64), (50, 257),
                   # odd row lengths: the scalar tail of the vector paths, register-resident and streaming
-                  (6, 7), (5, 5), (300, 1001), (3, 4099), (3, 16387), (2, 40003), (4, 100001), (700, 6789)]
+                  (6, 7), (5, 5), (300, 1001), (3, 4099), (3, 16387), (2, 40003), (4, 100001), (700, 6789),
+                  # 1025..2048 vectors per row: the forward pass runs 512 lanes there, the backward pass 1024
+                  (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=lambda s: "x".join(map(str, s)))
