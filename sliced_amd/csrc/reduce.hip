@@ -87,6 +87,45 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
   }
 }
 
+// Contiguous-axis reduction of SHORT rows whose length is not a power of two (2, 3, 10, 100 ...):
+// with a few lanes per row every lane would start its loads at a different dword phase and the
+// wave's loads would scatter (measured 2.1-3.2 TB/s).  Here a workgroup streams a contiguous
+// chunk of whole rows into LDS with full-width vector loads, then one thread per row sums its
+// row out of LDS.  The LDS index is skewed by one word per 32 so that threads striding by an even
+// row length do not pile onto the same banks.
+constexpr int RS_CHUNK = 4096;  // floats per workgroup
+__device__ __forceinline__ int rs_skew(int i) { return i + (i >> 5); }
+template <class Op>
+__global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_t cols, size_t rows_per_block,
+                                                              const float* __restrict__ x, float* __restrict__ out,
+                                                              Finalize fin) {
+  __shared__ float buf[RS_CHUNK + RS_CHUNK / 32 + 4];
+  const size_t r0 = (size_t)blockIdx.x * rows_per_block;
+  const size_t nr = r0 + rows_per_block <= rows ? rows_per_block : rows - r0;
+  const int len = (int)(nr * cols);  // <= RS_CHUNK
+  const float* src = x + r0 * cols;
+  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
+    if (i + 3 < len) {
+      const float4 v = ld4s(src + i);
+      buf[rs_skew(i)] = v.x; buf[rs_skew(i + 1)] = v.y; buf[rs_skew(i + 2)] = v.z; buf[rs_skew(i + 3)] = v.w;
+    } else {
+      for (int e = i; e < len; ++e) buf[rs_skew(e)] = src[e];
+    }
+  }
+  __syncthreads();
+  for (size_t r = threadIdx.x; r < nr; r += 256) {
+    const int base = (int)(r * cols);
+    float a0 = Op::identity(), a1 = a0;
+    int c = 0;
+    for (; c + 1 < (int)cols; c += 2) {
+      a0 = Op::apply(a0, buf[rs_skew(base + c)]);
+      a1 = Op::apply(a1, buf[rs_skew(base + c + 1)]);
+    }
+    if (c < (int)cols) a0 = Op::apply(a0, buf[rs_skew(base + c)]);
+    finalize_store(out + r0 + r, Op::apply(a0, a1), fin);
+  }
+}
+
 template <class Op, bool VEC>
 static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, unsigned nseg,
                                 Finalize fin) {
@@ -118,6 +157,13 @@ template <class Op>
 static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
   // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
   if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, rows * sizeof(float));
+  if (cols <= 128 && (cols & (cols - 1)) != 0 && rows >= 1024) {  // many short rows, not a power of two long
+    const size_t rpb = RS_CHUNK / cols;
+    const size_t blocks = (rows + rpb - 1) / rpb;
+    SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
+    hipLaunchKernelGGL((rowreduce_short_kernel<Op>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, rpb, x, out, fin);
+    return post_launch();
+  }
   const bool vec = cols >= 4;  // any row length: dword-aligned float4 loads plus a scalar tail
   const size_t colsv = cols / (vec ? 4 : 1);
   // few long rows: split every row so the whole chip is busy
@@ -144,47 +190,48 @@ static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float
 }
 
 // ---------------------------------------------------------------------------------------
-// Strided-axis reduction, stage 1.  The matrix is viewed as rows x colsv vectors; thread t owns
-// column vector (t % colsv) and the rows g, g+G, g+2G, ... with g = t / colsv, so that one sweep
-// of the whole grid reads one contiguous span of G rows.  Result: partial[g, :] (G x cols).
+// Strided-axis reduction, the streaming stages.  The matrix is read as ONE flat stream of float4,
+// whatever the row length: T threads, 4T a multiple of cols; thread t reads the vectors t, t + T,
+// t + 2T, ...  Component q of every vector it reads lies in the same column, (4t + q) mod cols, so
+// the thread keeps four running values and writes them to partial[4t + q].  `partial` is then a
+// (4T / cols) x cols matrix with the same column structure: the next stage reduces it the same
+// way, until what is left is small enough for colreduce_final_kernel.  Rows of odd length, which a
+// one-column-per-thread kernel with scalar loads reduced at 3.1-3.5 TB/s, stream at the same rate
+// as rows that are a multiple of 4 long; one sweep of the grid reads one contiguous span of 16T bytes.
 // ---------------------------------------------------------------------------------------
-template <class Op, bool VEC>
-__global__ __launch_bounds__(256) void colreduce_kernel(size_t rows, size_t cols, size_t G,
-                                                        const float* __restrict__ x, float* __restrict__ part) {
-  constexpr int V = VEC ? 4 : 1;
-  const size_t colsv = cols / V;
+template <class Op>
+__global__ __launch_bounds__(256) void colreduce_flat_kernel(size_t n, size_t T, const float* __restrict__ x,
+                                                             float* __restrict__ part) {
   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= colsv * G) return;
-  const size_t g = t / colsv, cv = t - g * colsv;
-  const size_t step = G * cols;  // elements between two rows of this thread
-  const float* p = x + g * cols + cv * V;
-  size_t r = g;
-  if (VEC) {
-    float4 a0 = make_float4(Op::identity(), Op::identity(), Op::identity(), Op::identity());
-    float4 a1 = a0, a2 = a0, a3 = a0;
+  if (t >= T) return;
+  const size_t nv = n >> 2;  // whole vectors of the stream
+  const float id = Op::identity();
+  float4 a0 = make_float4(id, id, id, id), a1 = a0, a2 = a0, a3 = a0;
 #define SL_ACC(A, Q) A.x = Op::apply(A.x, Q.x); A.y = Op::apply(A.y, Q.y); A.z = Op::apply(A.z, Q.z); A.w = Op::apply(A.w, Q.w);
-    for (; r + 3 * G < rows; r += 4 * G, p += 4 * step) {
-      float4 v0 = ld4s(p), v1 = ld4s(p + step), v2 = ld4s(p + 2 * step), v3 = ld4s(p + 3 * step);
-      SL_ACC(a0, v0) SL_ACC(a1, v1) SL_ACC(a2, v2) SL_ACC(a3, v3)
-    }
-    for (; r < rows; r += G, p += step) {
-      float4 v0 = ld4s(p);
-      SL_ACC(a0, v0)
-    }
-    SL_ACC(a0, a1) SL_ACC(a2, a3) SL_ACC(a0, a2)
-#undef SL_ACC
-    st4g(part + g * cols + cv * 4, a0);
-  } else {
-    float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
-    for (; r + 3 * G < rows; r += 4 * G, p += 4 * step) {
-      a0 = Op::apply(a0, ld1s(p));
-      a1 = Op::apply(a1, ld1s(p + step));
-      a2 = Op::apply(a2, ld1s(p + 2 * step));
-      a3 = Op::apply(a3, ld1s(p + 3 * step));
-    }
-    for (; r < rows; r += G, p += step) a0 = Op::apply(a0, ld1s(p));
-    part[g * cols + cv] = Op::apply(Op::apply(a0, a1), Op::apply(a2, a3));
+  size_t i = t;
+  for (; i + 3 * T < nv; i += 4 * T) {
+    float4 v0 = ld4s(x + 4 * i), v1 = ld4s(x + 4 * (i + T)), v2 = ld4s(x + 4 * (i + 2 * T)), v3 = ld4s(x + 4 * (i + 3 * T));
+    SL_ACC(a0, v0) SL_ACC(a1, v1) SL_ACC(a2, v2) SL_ACC(a3, v3)
   }
+  for (; i < nv; i += T) {
+    float4 v0 = ld4s(x + 4 * i);
+    SL_ACC(a0, v0)
+  }
+  SL_ACC(a0, a1) SL_ACC(a2, a3) SL_ACC(a0, a2)
+#undef SL_ACC
+  // the up to three floats behind the last whole vector belong to whoever owns their position
+  for (size_t e = nv << 2; e < n; ++e) {
+    const size_t pos = e % (4 * T);
+    if (pos >> 2 == t) {
+      const float v = x[e];
+      const int q = (int)(pos & 3);
+      if (q == 0) a0.x = Op::apply(a0.x, v);
+      else if (q == 1) a0.y = Op::apply(a0.y, v);
+      else if (q == 2) a0.z = Op::apply(a0.z, v);
+      else a0.w = Op::apply(a0.w, v);
+    }
+  }
+  st4g(part + 4 * t, a0);
 }
 
 // Stage 2 (also the only stage for short matrices): a block owns CW adjacent columns, its
@@ -317,31 +364,32 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
   if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin);
   // one row: the reduction over rows is that row itself
   if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, cols * sizeof(float));
-  // Rows of odd length stay on the one-column-per-thread form: its loads are fully coalesced
-  // across the wave, and float4 loads that start at a different dword phase in every row measured
-  // no faster (3.2-3.8 TB/s against 3.1-4.7).
-  const bool vec = cols % 4 == 0;
-  const size_t colsv = cols / (vec ? 4 : 1);
-  // number of row groups: about 512 threads per CU (measured optimum: 7.0 TB/s at 131072
-  // threads on [16384 x 16384]; 5.4 TB/s at four times as many), at least 16 rows per thread
-  const size_t target_threads = (size_t)ctx->num_cu * 512;
-  size_t G = (target_threads + colsv - 1) / colsv;
-  if (G > rows / 16) G = rows / 16;
-  const size_t ws_floats = ctx->workspace_bytes / sizeof(float);
-  if (G > 1 && G * cols > ws_floats) G = ws_floats / cols;
-  // small matrices: one kernel (a second stage would cost more than it saves, 3-4 us a launch)
-  if (G <= 1 || (rows * cols <= (1u << 18) && rows <= 4096)) return colreduce_final_launch<Op>(ctx, rows, cols, x, out, fin);
-  float* part = (float*)ctx->workspace;
-  const size_t threads = colsv * G;
-  if (vec)
-    hipLaunchKernelGGL((colreduce_kernel<Op, true>), dim3(ceil_div(threads, 256)), dim3(256), 0, ctx->stream, rows,
-                       cols, G, x, part);
-  else
-    hipLaunchKernelGGL((colreduce_kernel<Op, false>), dim3(ceil_div(threads, 256)), dim3(256), 0, ctx->stream, rows,
-                       cols, G, x, part);
-  int32_t rc = post_launch();
-  if (rc) return rc;
-  return colreduce_final_launch<Op>(ctx, G, cols, part, out, fin);
+  // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
+  // about 512 per CU (measured optimum: 7.0 TB/s at 131072 threads on [16384 x 16384]; 5.4 TB/s at
+  // four times as many), at least 16 vectors each, and a multiple of cols / gcd(cols, 4) so that
+  // 4T is a multiple of cols.
+  const size_t unit = cols / (cols % 4 == 0 ? 4 : cols % 2 == 0 ? 2 : 1);
+  const float* cur = x;
+  size_t cur_rows = rows;
+  float* ws = (float*)ctx->workspace;
+  size_t ws_left = ctx->workspace_bytes / sizeof(float);
+  while (cur_rows >= 8 && !(cur_rows * cols <= (1u << 18) && cur_rows <= 4096)) {
+    const size_t n = cur_rows * cols, nv = n >> 2;
+    size_t T = (size_t)ctx->num_cu * 512;
+    if (T > nv / 16) T = nv / 16;
+    T = T / unit * unit;
+    if (T < unit) T = unit;
+    if (4 * T > ws_left || 8 * T > n) break;  // no room, or nothing gained: the last stage takes it as it is
+    SLHIP_REQUIRE((T + 255) / 256 <= 0x7fffffffu, "matrix too wide for one launch");
+    hipLaunchKernelGGL((colreduce_flat_kernel<Op>), dim3((unsigned)((T + 255) / 256)), dim3(256), 0, ctx->stream, n, T, cur, ws);
+    int32_t rc = post_launch();
+    if (rc) return rc;
+    cur = ws;
+    cur_rows = 4 * T / cols;
+    ws += 4 * T;
+    ws_left -= 4 * T;
+  }
+  return colreduce_final_launch<Op>(ctx, cur_rows, cols, cur, out, fin);
 }
 
 // ---------------------------------------------------------------------------------------

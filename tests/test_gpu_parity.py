@@ -240,7 +240,11 @@ def test_linear_fwd_fused_equals_gemm_bias_relu(hip, orc):
 # --------------------------------------------------------------------------- reductions
 RED_SHAPES = [(1, 1), (1, 5), (5, 1), (3, 4), (7, 13), (64, 64), (33, 1000), (1000, 33), (257, 4096), (4096, 257),
               (16, 40000), (40000, 16), (2, 300001), (300001, 2), (1, 1 << 20), (1 << 20, 1), (2048, 2048),
-              (100, 10), (8192, 10), (5000, 128), (3, 70000)]
+              (100, 10), (8192, 10), (5000, 128), (3, 70000),
+              # many short rows whose length is not a power of two (LDS-staged contiguous-axis kernel),
+              # odd and even row lengths through the flat strided-axis stages, few rows of great length
+              (5000, 3), (4099, 10), (2000, 100), (1025, 127), (70000, 2), (30011, 7), (9001, 33), (20000, 258),
+              (13, 300001), (9, 100002), (1500, 1001)]
 
 
 def sum_bound(x, rows, cols, axis):
