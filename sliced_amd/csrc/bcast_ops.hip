@@ -1,6 +1,6 @@
 // Row / column broadcast ops with an op code, diagflat and the onehot gradient: the part of the
 // reference's op surface beside the training hot path (reference: src/ops2/row_op, src/ops2/col_op,
-// src/ops2/diagflat, src/ops2/onehot).  Plain streaming kernels, one element per thread; the
+// src/ops2/diagflat, src/ops2/onehot).  Plain streaming kernels; the
 // reductions of the broadcast-side gradients go through partial sums in the context workspace
 // and are combined in a fixed order.
 #include "common.hpp"
@@ -34,24 +34,55 @@ __device__ __forceinline__ float bc_dr(int op, float l, float r) {
   }
 }
 
-// BY_ROW_INDEX: the broadcast vector is indexed by the row (col_op), else by the column (row_op).
-template <bool BY_ROW_INDEX>
-__global__ __launch_bounds__(256) void bc_fwd_kernel(int op, size_t len, size_t cols, const float* __restrict__ lhs,
-                                                     const float* __restrict__ v, float* __restrict__ out) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= len) return;
-  const size_t r = i / cols;
-  out[i] = bc_apply(op, lhs[i], v[BY_ROW_INDEX ? r : i - r * cols]);
+// Forward and lhs gradient.  The matrix is walked as one flat run of float4 (dword-aligned, so any
+// row length and base address): a thread finds the row and column of its first element with one
+// division and steps from there.  BY_ROW_INDEX: the broadcast vector is indexed by the row
+// (col_op), else by the column (row_op).  GRAD: lhs_grad += dL(lhs, v) * g instead of out = f(lhs, v).
+// IDX: 32-bit index arithmetic whenever the matrix allows it.
+template <bool BY_ROW_INDEX, bool GRAD, class IDX>
+__global__ __launch_bounds__(256) void bc_flat_kernel(int op, size_t len, size_t cols, const float* __restrict__ lhs,
+                                                      const float* __restrict__ v, float* out,
+                                                      const float* __restrict__ g) {
+  const size_t e0 = 4 * ((size_t)blockIdx.x * 256 + threadIdx.x);
+  if (e0 >= len) return;
+  IDX r = (IDX)e0 / (IDX)cols;
+  IDX c = (IDX)e0 - r * (IDX)cols;
+  const bool whole = e0 + 3 < len;
+  float l[4] = {0.f, 0.f, 0.f, 0.f}, gv[4] = {0.f, 0.f, 0.f, 0.f}, o[4] = {0.f, 0.f, 0.f, 0.f};
+  if (whole) {
+    float4 t = ld4s(lhs + e0);
+    l[0] = t.x; l[1] = t.y; l[2] = t.z; l[3] = t.w;
+    if (GRAD) {
+      t = ld4s(g + e0); gv[0] = t.x; gv[1] = t.y; gv[2] = t.z; gv[3] = t.w;
+      t = ld4g(out + e0); o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+    }
+  } else {
+    for (size_t q = 0; e0 + q < len; ++q) {
+      l[q] = lhs[e0 + q];
+      if (GRAD) { gv[q] = g[e0 + q]; o[q] = out[e0 + q]; }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (e0 + q < len) {
+      const float vv = v[BY_ROW_INDEX ? r : c];
+      o[q] = GRAD ? o[q] + bc_dl(op, l[q], vv) * gv[q] : bc_apply(op, l[q], vv);
+    }
+    if (++c == (IDX)cols) { c = 0; ++r; }
+  }
+  if (whole) st4g(out + e0, make_float4(o[0], o[1], o[2], o[3]));
+  else
+    for (size_t q = 0; e0 + q < len; ++q) out[e0 + q] = o[q];
 }
 
-template <bool BY_ROW_INDEX>
-__global__ __launch_bounds__(256) void bc_grad_lhs_kernel(int op, size_t len, size_t cols, const float* __restrict__ lhs,
-                                                          const float* __restrict__ v, float* __restrict__ lhs_grad,
-                                                          const float* __restrict__ g) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= len) return;
-  const size_t r = i / cols;
-  lhs_grad[i] += bc_dl(op, lhs[i], v[BY_ROW_INDEX ? r : i - r * cols]) * g[i];
+template <bool BY_ROW_INDEX, bool GRAD>
+static void bc_flat_launch(slhip_ctx* ctx, int op, size_t len, size_t cols, const float* lhs, const float* v, float* out,
+                           const float* g) {
+  const unsigned blocks = (unsigned)(((len + 3) / 4 + 255) / 256);
+  if (len <= 0xffffffffu)
+    hipLaunchKernelGGL((bc_flat_kernel<BY_ROW_INDEX, GRAD, uint32_t>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out, g);
+  else
+    hipLaunchKernelGGL((bc_flat_kernel<BY_ROW_INDEX, GRAD, size_t>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out, g);
 }
 
 // col_op: v_grad[r] += sum_c dR(lhs[r,c], v[r]) * g[r,c]; one wave per row
@@ -130,7 +161,7 @@ static int32_t bc_forward(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols, 
     set_error("broadcast op: unknown op %d", op);
     return SLHIP_EINVAL;
   }
-  hipLaunchKernelGGL((bc_fwd_kernel<BY_ROW_INDEX>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out);
+  bc_flat_launch<BY_ROW_INDEX, false>(ctx, op, len, cols, lhs, v, out, nullptr);
   return post_launch();
 }
 
@@ -148,8 +179,7 @@ static int32_t bc_backward(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols,
     return SLHIP_EINVAL;
   }
   if (lhs_grad) {
-    hipLaunchKernelGGL((bc_grad_lhs_kernel<BY_ROW_INDEX>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v,
-                       lhs_grad, g);
+    bc_flat_launch<BY_ROW_INDEX, true>(ctx, op, len, cols, lhs, v, lhs_grad, g);
     int32_t rc = post_launch();
     if (rc) return rc;
   }
