@@ -373,7 +373,9 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
   size_t cur_rows = rows;
   float* ws = (float*)ctx->workspace;
   size_t ws_left = ctx->workspace_bytes / sizeof(float);
-  while (cur_rows >= 8 && !(cur_rows * cols <= (1u << 18) && cur_rows <= 4096)) {
+  // (the last stage is quick for up to 256 rows of any length - 16 rows per lane, 16 columns per
+  // workgroup - and for small matrices of up to 4096 rows)
+  while (cur_rows >= 8 && !((cur_rows <= 256 && cur_rows * cols <= (1u << 22)) || (cur_rows * cols <= (1u << 18) && cur_rows <= 4096))) {
     const size_t n = cur_rows * cols, nv = n >> 2;
     size_t T = (size_t)ctx->num_cu * 512;
     if (T > nv / 16) T = nv / 16;
