@@ -28,10 +28,10 @@ sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # HBM-side bytes of one 4096^3 A*B launch, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
-# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (657069.8 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
+# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (651777.1 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
-GEMM_4096_TRAFFIC_BYTES = int((657069.8 * 2.0 + 65536.0) * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((651777.1 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 
@@ -171,6 +171,15 @@ def bench_bandwidth_suite(ctx, steps, warmup):
             out.append(bw_entry("max_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
             w, e = timed(ctx, lambda: ctx.call("slhip_sum_rows", rows, cols, xs.ptr, o1.ptr), steps, warmup)
             out.append(bw_entry("sum_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
+    # shapes off the beaten track, 2^27 elements each: rows of odd length, narrow and very wide matrices
+    for rows, cols in [(4026, 33333), (522247, 257), (13421772, 10), (134, 1000000)]:
+        ne = rows * cols
+        xs = x.view(0, ne)
+        ov = y.view(0, max(rows, cols))
+        for name, olen in (("sum_rows", cols), ("max_rows", cols), ("sum_cols", rows)):
+            fn = lambda name=name: ctx.call("slhip_" + name, rows, cols, xs.ptr, ov.ptr)
+            w, e = timed(ctx, fn, steps, warmup)
+            out.append(bw_entry("%s [%dx%d]" % (name, rows, cols), 4 * ne + 4 * olen, w, e)); log(out[-1])
     # fused elementwise chain on 2^28 elements per tensor: 4 reads + 1 write
     bb, cc, dd = ctx.uniform(n, -10, 10, 2, SEED), ctx.uniform(n, -10, 10, 3, SEED), ctx.uniform(n, -10, 10, 4, SEED)
     w, e = timed(ctx, lambda: ctx.call("slhip_ew_chain", n, x.ptr, bb.ptr, cc.ptr, dd.ptr, y.ptr), steps, warmup)
@@ -315,8 +324,8 @@ def main():
         log(suite["gemm_4096"])
     if "sweep" in parts:
         sweep = {}
-        for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (3584,) * 3, (4608,) * 3, (8192,) * 3, (8192, 2048, 784),
-                          (784, 2048, 8192)]:
+        for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (3584,) * 3, (4095,) * 3, (4608,) * 3, (8192,) * 3,
+                          (8192, 2048, 784), (784, 2048, 8192)]:
             st = max(3, args.steps // 4) if m >= 8192 and k >= 8192 else args.steps
             for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
                 r = bench_gemm(ctx, m, n, k, ta, tb, st, 2)
