@@ -745,6 +745,12 @@ def test_invalid_arguments_return_status_not_crash(hip):
     assert lib.slhip_sgemm(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, x.ptr, 0.0) == -4   # C aliases A
     assert lib.slhip_transpose(c.h, 4, 4, x.ptr, x.ptr, 0.0) == -4
     assert lib.slhip_ew_unary(c.h, 99, 0.0, 0.0, 4, x.ptr, x.ptr) == -1
+    assert lib.slhip_gemm_tail_policy(c.h, 7) == -1                      # unknown policies
+    assert lib.slhip_gemm_tile_policy(c.h, 2) == -1
+    assert lib.slhip_gemm_tail_policy(c.h, 0) == 0 and lib.slhip_gemm_tile_policy(c.h, 0) == 0
+    y = c.empty(16)
+    assert lib.slhip_sgemm_relu_mask(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, y.ptr, y.ptr, 0.0) == -4   # C aliases pre
+    y.free()
     x.free()
 
 
