@@ -286,6 +286,104 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
   }
 }
 
+// Short rows whose length is not a power of two (10, 100, 200 ... classes): with a few lanes per row
+// every row starts at a different phase of the cache lines and the wave's loads scatter (2.2-4.7
+// TB/s at 2^27 elements).  Here a workgroup streams a contiguous 16 KiB chunk of whole rows into LDS
+// with full-width loads, L lanes per row (shuffles only) work on it in place, and the chunk is
+// streamed out again.  The LDS index is skewed by one word per 32 (rows of even length would
+// otherwise pile onto the same banks).
+constexpr int SS_CHUNK = 4096;  // floats per workgroup and tensor
+__device__ __forceinline__ int ss_skew(int i) { return i + (i >> 5); }
+
+__device__ __forceinline__ void ss_load(float* buf, const float* __restrict__ src, int len) {
+  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
+    if (i + 3 < len) {
+      const float4 v = ld4s(src + i);
+      buf[ss_skew(i)] = v.x; buf[ss_skew(i + 1)] = v.y; buf[ss_skew(i + 2)] = v.z; buf[ss_skew(i + 3)] = v.w;
+    } else {
+      for (int e = i; e < len; ++e) buf[ss_skew(e)] = src[e];
+    }
+  }
+}
+
+template <int L>
+__global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int cols, int rpb, const float* __restrict__ x,
+                                                                float* __restrict__ out) {
+  __shared__ float buf[SS_CHUNK + SS_CHUNK / 32 + 4];
+  const size_t r0 = (size_t)blockIdx.x * rpb;
+  const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
+  const int len = nr * cols;
+  ss_load(buf, x + r0 * cols, len);
+  __syncthreads();
+  const int lane = threadIdx.x % L, group = threadIdx.x / L;
+  for (int rb = 0; rb < nr; rb += 256 / L) {  // the same trip count for every thread: the shuffles need whole groups
+    const int r = rb + group;
+    const bool active = r < nr;
+    const int base = r * cols;
+    float m = -__builtin_huge_valf();
+    if (active)
+      for (int c = lane; c < cols; c += L) m = fmaxf(m, buf[ss_skew(base + c)]);
+    m = wave_reduce<MaxOp, L>(m);
+    float sum = 0.0f;
+    if (active)
+      for (int c = lane; c < cols; c += L) {
+        const float e = expf(buf[ss_skew(base + c)] - m);
+        buf[ss_skew(base + c)] = e;
+        sum += e;
+      }
+    sum = wave_reduce<SumOp, L>(sum);
+    if (active)
+      for (int c = lane; c < cols; c += L) buf[ss_skew(base + c)] = buf[ss_skew(base + c)] / sum;
+  }
+  __syncthreads();
+  float* dst = out + r0 * cols;
+  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
+    if (i + 3 < len) st4s(dst + i, make_float4(buf[ss_skew(i)], buf[ss_skew(i + 1)], buf[ss_skew(i + 2)], buf[ss_skew(i + 3)]));
+    else
+      for (int e = i; e < len; ++e) dst[e] = buf[ss_skew(e)];
+  }
+}
+
+template <int L>
+__global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int cols, int rpb, float* x_grad,
+                                                                const float* __restrict__ out,
+                                                                const float* __restrict__ out_grad, float beta) {
+  __shared__ float sb[SS_CHUNK + SS_CHUNK / 32 + 4];
+  __shared__ float gb[SS_CHUNK + SS_CHUNK / 32 + 4];
+  const size_t r0 = (size_t)blockIdx.x * rpb;
+  const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
+  const int len = nr * cols;
+  ss_load(sb, out + r0 * cols, len);
+  ss_load(gb, out_grad + r0 * cols, len);
+  __syncthreads();
+  const int lane = threadIdx.x % L, group = threadIdx.x / L;
+  for (int rb = 0; rb < nr; rb += 256 / L) {
+    const int r = rb + group;
+    const bool active = r < nr;
+    const int base = r * cols;
+    float dot = 0.0f;
+    if (active)
+      for (int c = lane; c < cols; c += L) dot += sb[ss_skew(base + c)] * gb[ss_skew(base + c)];
+    dot = wave_reduce<SumOp, L>(dot);
+    if (active)
+      for (int c = lane; c < cols; c += L) sb[ss_skew(base + c)] = sb[ss_skew(base + c)] * (gb[ss_skew(base + c)] - dot);
+  }
+  __syncthreads();
+  float* dst = x_grad + r0 * cols;
+  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
+    if (i + 3 < len) {
+      float4 v = make_float4(sb[ss_skew(i)], sb[ss_skew(i + 1)], sb[ss_skew(i + 2)], sb[ss_skew(i + 3)]);
+      if (beta != 0.0f) {
+        const float4 o = ld4g(dst + i);
+        v.x = beta * o.x + v.x; v.y = beta * o.y + v.y; v.z = beta * o.z + v.z; v.w = beta * o.w + v.w;
+      }
+      st4g(dst + i, v);
+    } else {
+      for (int e = i; e < len; ++e) dst[e] = beta != 0.0f ? beta * dst[e] + sb[ss_skew(e)] : sb[ss_skew(e)];
+    }
+  }
+}
+
 struct SoftmaxCfg {
   int lanes;  // 0 = streaming fallback
   int items;
@@ -309,6 +407,28 @@ static SoftmaxCfg pick_cfg(size_t colsv, bool fwd) {
 template <bool FWD, bool VEC>
 static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, float* x_grad,
                                 const float* s, const float* g, float beta) {
+  // many short rows, not a power of two long (measured at 2^27 elements, forward / backward TB/s,
+  // lanes-per-row kernel -> this one: 10: 3.1 / 2.8 -> 4.8 / 3.9; 36: 2.2 / 2.9 -> 4.7 / 4.7; 100: 3.0 / 3.6 ->
+  // 4.4 / 4.3; from 200 on the lanes-per-row kernel is the faster one again)
+  if (cols >= 3 && cols <= 160 && (cols & (cols - 1)) != 0 && rows >= 1024) {
+    const int rpb = SS_CHUNK / (int)cols;
+    int lanes = 1;
+    while (lanes < 64 && lanes * 2 * rpb <= 256) lanes <<= 1;  // groups of `lanes` lanes, at least one per row of the chunk
+    const size_t blocks = (rows + rpb - 1) / rpb;
+    SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
+#define SL_SS(L)                                                                                                          \
+  case L:                                                                                                                 \
+    if (FWD)                                                                                                              \
+      hipLaunchKernelGGL((softmax_fwd_short_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, (int)cols, \
+                         rpb, x, out);                                                                                    \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((softmax_bwd_short_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, (int)cols, \
+                         rpb, x_grad, s, g, beta);                                                                        \
+    break;
+    switch (lanes) { SL_SS(1) SL_SS(2) SL_SS(4) SL_SS(8) SL_SS(16) SL_SS(32) SL_SS(64) }
+#undef SL_SS
+    return post_launch();
+  }
   const size_t colsv = cols / (VEC ? 4 : 1);
   SoftmaxCfg cfg = pick_cfg(colsv, FWD);
   if (cfg.lanes == 0) {

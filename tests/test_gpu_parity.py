@@ -334,7 +334,9 @@ SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (6
                   # odd row lengths: the scalar tail of the vector paths, register-resident and streaming
                   (6, 7), (5, 5), (300, 1001), (3, 4099), (3, 16387), (2, 40003), (4, 100001), (700, 6789),
                   # 1025..2048 vectors per row: the forward pass runs 512 lanes there, the backward pass 1024
-                  (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196)]
+                  (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196),
+                  # many short rows, not a power of two long: the LDS-staged kernels
+                  (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (4097, 37), (1024, 6)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=lambda s: "x".join(map(str, s)))
