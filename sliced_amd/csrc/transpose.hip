@@ -117,29 +117,62 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
   }
 }
 
-// Matrices with at most 32 columns (or rows): the tile above would be mostly empty.  One thread
-// per long-axis index walks the short axis; the strided side of every access pattern stays inside
-// a few cache lines that the neighbouring iterations reuse.
-template <bool ACC>
-__global__ __launch_bounds__(256) void transpose_few_cols_kernel(size_t rows, size_t cols, const float* __restrict__ x,
-                                                                 float* out) {
-  const size_t r = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (r >= rows) return;
-  for (size_t c = 0; c < cols; ++c) {
-    const float v = x[r * cols + c];
-    float* p = out + c * rows + r;  // coalesced over r
-    *p = ACC ? *p + v : v;
+// Matrices with few columns (or few rows): the tile above would be mostly empty.  A chunk of R whole
+// rows of the narrow matrix is one contiguous run of R*S floats (S = the short side) on the narrow
+// side and S runs of R floats on the other.  A workgroup moves one such chunk through LDS: both
+// sides are read and written with consecutive lanes on consecutive floats.  NARROW_IN: the input
+// is the narrow matrix [long x S]; else the input is [S x long] and the output is narrow.
+// The LDS index is skewed by one word per 32 (a power-of-two S would pile a column onto one bank).
+constexpr int TS_CHUNK = 8192;  // floats per workgroup
+__device__ __forceinline__ int ts_skew(int i) { return i + (i >> 5); }
+template <bool NARROW_IN, bool ACC>
+__global__ __launch_bounds__(256) void transpose_narrow_kernel(size_t long_side, int S, int R, const float* __restrict__ x,
+                                                               float* out) {
+  __shared__ float buf[TS_CHUNK + TS_CHUNK / 32 + 4];
+  const size_t l0 = (size_t)blockIdx.x * R;
+  const int nr = l0 + R <= long_side ? R : (int)(long_side - l0);
+  const int len = nr * S;
+  // LDS holds the chunk in the narrow matrix's order: element (l, s) at l*S + s.  Global memory is
+  // touched with dword-aligned float4 on both sides (scalar accesses stream at a third of the rate).
+  const int nr4 = nr & ~3, len4 = len & ~3;
+  if (NARROW_IN) {
+    const float* src = x + l0 * S;
+    for (int i = 4 * threadIdx.x; i < len4; i += 1024) {
+      const float4 v = ld4s(src + i);
+      buf[ts_skew(i)] = v.x; buf[ts_skew(i + 1)] = v.y; buf[ts_skew(i + 2)] = v.z; buf[ts_skew(i + 3)] = v.w;
+    }
+    for (int i = len4 + threadIdx.x; i < len; i += 256) buf[ts_skew(i)] = src[i];
+  } else {
+    for (int s = 0; s < S; ++s) {
+      const float* src = x + (size_t)s * long_side + l0;
+      for (int l = 4 * threadIdx.x; l < nr4; l += 1024) {
+        const float4 v = ld4s(src + l);
+        buf[ts_skew(l * S + s)] = v.x; buf[ts_skew((l + 1) * S + s)] = v.y;
+        buf[ts_skew((l + 2) * S + s)] = v.z; buf[ts_skew((l + 3) * S + s)] = v.w;
+      }
+      for (int l = nr4 + threadIdx.x; l < nr; l += 256) buf[ts_skew(l * S + s)] = src[l];
+    }
   }
-}
-template <bool ACC>
-__global__ __launch_bounds__(256) void transpose_few_rows_kernel(size_t rows, size_t cols, const float* __restrict__ x,
-                                                                 float* out) {
-  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= cols) return;
-  for (size_t r = 0; r < rows; ++r) {
-    const float v = x[r * cols + c];  // coalesced over c
-    float* p = out + c * rows + r;
-    *p = ACC ? *p + v : v;
+  __syncthreads();
+  if (NARROW_IN) {
+    for (int s = 0; s < S; ++s) {
+      float* dst = out + (size_t)s * long_side + l0;
+      for (int l = 4 * threadIdx.x; l < nr4; l += 1024) {
+        float4 v = make_float4(buf[ts_skew(l * S + s)], buf[ts_skew((l + 1) * S + s)], buf[ts_skew((l + 2) * S + s)],
+                               buf[ts_skew((l + 3) * S + s)]);
+        if (ACC) { const float4 o = ld4g(dst + l); v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
+        st4g(dst + l, v);
+      }
+      for (int l = nr4 + threadIdx.x; l < nr; l += 256) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + s)] : buf[ts_skew(l * S + s)];
+    }
+  } else {
+    float* dst = out + l0 * S;
+    for (int i = 4 * threadIdx.x; i < len4; i += 1024) {
+      float4 v = make_float4(buf[ts_skew(i)], buf[ts_skew(i + 1)], buf[ts_skew(i + 2)], buf[ts_skew(i + 3)]);
+      if (ACC) { const float4 o = ld4g(dst + i); v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
+      st4g(dst + i, v);
+    }
+    for (int i = len4 + threadIdx.x; i < len; i += 256) dst[i] = ACC ? dst[i] + buf[ts_skew(i)] : buf[ts_skew(i)];
   }
 }
 
@@ -169,16 +202,17 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     return post_launch();
   }
   if (cols <= 32 || rows <= 32) {
-    const size_t longer = cols <= 32 ? rows : cols;
-    SLHIP_REQUIRE((longer + 255) / 256 <= 0x7fffffffu, "matrix too large for one launch");
-    const dim3 g((unsigned)((longer + 255) / 256));
-    if (cols <= 32) {
-      if (acc) hipLaunchKernelGGL(transpose_few_cols_kernel<true>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
-      else hipLaunchKernelGGL(transpose_few_cols_kernel<false>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
-    } else {
-      if (acc) hipLaunchKernelGGL(transpose_few_rows_kernel<true>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
-      else hipLaunchKernelGGL(transpose_few_rows_kernel<false>, g, dim3(256), 0, ctx->stream, rows, cols, x, out);
-    }
+    const bool narrow_in = cols <= 32 && (rows > 32 || cols <= rows);  // which matrix has the short rows
+    const size_t long_side = narrow_in ? rows : cols;
+    const int S = (int)(narrow_in ? cols : rows);
+    const int R = TS_CHUNK / S;
+    const size_t blocks = (long_side + R - 1) / R;
+    SLHIP_REQUIRE(blocks <= 0x7fffffffu, "matrix too large for one launch");
+#define SL_TN(NI, A) \
+  hipLaunchKernelGGL((transpose_narrow_kernel<NI, A>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, long_side, S, R, x, out)
+    if (narrow_in) { if (acc) SL_TN(true, true); else SL_TN(true, false); }
+    else { if (acc) SL_TN(false, true); else SL_TN(false, false); }
+#undef SL_TN
     return post_launch();
   }
   const size_t tiles_r = (rows + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;
