@@ -201,8 +201,8 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     hipLaunchKernelGGL(axpy_copy_kernel, dim3((unsigned)((len + 63) / 64)), dim3(64), 0, ctx->stream, len, x, out);
     return post_launch();
   }
-  if (cols <= 32 || rows <= 32) {
-    const bool narrow_in = cols <= 32 && (rows > 32 || cols <= rows);  // which matrix has the short rows
+  if (cols <= 40 || rows <= 40) {  // measured: from a side of 48 on the tiled kernel is the faster one
+    const bool narrow_in = cols <= 40 && (rows > 40 || cols <= rows);  // which matrix has the short rows
     const size_t long_side = narrow_in ? rows : cols;
     const int S = (int)(narrow_in ? cols : rows);
     const int R = TS_CHUNK / S;

@@ -387,7 +387,10 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (4, 4096), (4096, 4), (1000, 1000), (1, 1 << 18), (1 << 18, 1),
              # rows / columns of odd length on the vector paths, and the few-rows / few-columns kernels
              (4097, 4097), (1234, 679), (300, 1001), (1001, 300), (100000, 7), (7, 100000), (33, 1000), (1000, 33),
-             (2, 5), (32, 70000), (259, 66)]
+             (2, 5), (32, 70000), (259, 66),
+             # the narrow-matrix kernel: chunk boundaries, sides 2..40, both directions, tiny and ragged long sides
+             (70001, 2), (2, 70001), (30000, 31), (31, 30000), (9999, 40), (40, 9999), (5000, 16), (16, 5003), (41, 3000),
+             (3000, 41), (3, 3), (40, 40), (17, 23)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
