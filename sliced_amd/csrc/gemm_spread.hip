@@ -60,30 +60,36 @@ __global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadA
 }
 
 // The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup
-// order), then beta / bias / relu as in the kernel's own epilogue.  Four workgroups per tile, 32
-// rows each.  Workgroup spread_first + w holds k tiles [w*U, (w+1)*U) of the tail's sequence, so
-// tile ti is covered by workgroups (ti*KT)/U .. ((ti+1)*KT - 1)/U, and it is the workgroup's run
-// number ti - (w*U)/KT (0 or 1, since U <= KT).
+// order), then beta / bias / relu as in the kernel's own epilogue.  Sixteen workgroups per tile,
+// 8 rows each, one float4 of the tile per thread - a tile of a long-K product can have hundreds of
+// partial tiles (64 x 64 x 1048576: one tile, 512 partials; four workgroups summing them one after
+// the other took 650 us of that product's 930).  Workgroup spread_first + w holds k tiles
+// [w*U, (w+1)*U) of the tail's sequence, so tile ti is covered by workgroups (ti*KT)/U ..
+// ((ti+1)*KT - 1)/U.  Only the first of them can have started in the tile before (U <= KT): its
+// partial of this tile is its run ti - (w*U)/KT; every later one's is its run 0.
 __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArgs sp) {
-  const unsigned ti = blockIdx.x >> 2, quarter = blockIdx.x & 3;
+  const unsigned ti = blockIdx.x >> 4, quarter = blockIdx.x & 15;
   unsigned tm, tn;
   tile_of_block(sp.first + ti, g.tiles_m, g.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
   const unsigned KT = sp.kt_total, U = sp.units;
   const unsigned w_first = (ti * KT) / U, w_last = ((ti + 1) * KT - 1) / U;
-  constexpr int PER = 32 * (BN / 4) / 256;  // float4 per thread
+  constexpr int PER = 8 * (BN / 4) / 256;  // float4 per thread: one
   float4 s[PER], c[PER], mk[PER];
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int f = threadIdx.x + 256 * e;
-    const int row_l = quarter * 32 + f / (BN / 4), c4 = f % (BN / 4);
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (unsigned w = w_first; w <= w_last; ++w) {
-      const unsigned run = ti - (w * U) / KT;
-      const float4 p = ld4(g.partial + ((size_t)2 * w + run) * SPREAD_SLOT + row_l * BN + 4 * c4);
-      if (w == w_first) sum = p;
-      else { sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w; }
+    const int row_l = quarter * 8 + f / (BN / 4), c4 = f % (BN / 4);
+    const float* p0 = g.partial + row_l * BN + 4 * c4;
+    float4 sum = ld4(p0 + ((size_t)2 * w_first + (ti - (w_first * U) / KT)) * SPREAD_SLOT);
+    auto add = [&](const float4& p) { sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w; };
+    unsigned w = w_first + 1;
+    for (; w + 3 <= w_last; w += 4) {  // four loads in flight, added in ascending order
+      const float4 q0 = ld4(p0 + (size_t)2 * w * SPREAD_SLOT), q1 = ld4(p0 + (size_t)2 * (w + 1) * SPREAD_SLOT),
+                   q2 = ld4(p0 + (size_t)2 * (w + 2) * SPREAD_SLOT), q3 = ld4(p0 + (size_t)2 * (w + 3) * SPREAD_SLOT);
+      add(q0); add(q1); add(q2); add(q3);
     }
+    for (; w <= w_last; ++w) add(ld4(p0 + (size_t)2 * w * SPREAD_SLOT));
     s[e] = sum;
     const size_t row = m0 + row_l, col = n0 + 4 * c4;
     c[e] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -101,7 +107,7 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int f = threadIdx.x + 256 * e;
-    const int row_l = quarter * 32 + f / (BN / 4), c4 = f % (BN / 4);
+    const int row_l = quarter * 8 + f / (BN / 4), c4 = f % (BN / 4);
     const size_t row = m0 + row_l, col = n0 + 4 * c4;
     if (row >= g.M || col >= g.N) continue;
     float v[4] = {s[e].x, s[e].y, s[e].z, s[e].w};
@@ -151,7 +157,7 @@ int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, con
 #undef SL_GEMM
   int32_t rc = post_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL(spread_fixup_kernel, dim3((unsigned)(4 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
+  hipLaunchKernelGGL(spread_fixup_kernel, dim3((unsigned)(16 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
   return post_launch();
 }
 
