@@ -291,15 +291,28 @@ int32_t bcast_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* a, c
   return post_launch();
 }
 
-// cce: one thread per row (rows are short: the class count)
-__global__ void cce_kernel(size_t rows, size_t cols, const float* __restrict__ p, const float* __restrict__ t,
-                           float* __restrict__ loss) {
-  size_t r = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (r >= rows) return;
+// cce: L lanes per row (a power of two up to 64, about 8 classes per lane), 256 / L rows per
+// workgroup; consecutive lanes read consecutive floats.  (One thread per row, the first version,
+// streamed [13M x 10] at 2.5 TB/s and [32768 x 4096] at 0.7.)
+template <int L>
+__global__ __launch_bounds__(256) void cce_kernel(size_t rows, size_t cols, const float* __restrict__ p,
+                                                  const float* __restrict__ t, float* __restrict__ loss) {
+  const size_t r = (size_t)blockIdx.x * (256 / L) + threadIdx.x / L;
+  const int lane = threadIdx.x % L;
   const float lo = (float)1e-7, hi = (float)(1.0 - 1e-7);
-  float s = 0.0f;
-  for (size_t c = 0; c < cols; ++c) s += fminf(fmaxf(p[r * cols + c], lo), hi) * t[r * cols + c];
-  loss[r] = -logf(s);
+  float s0 = 0.0f, s1 = 0.0f;
+  if (r < rows) {
+    const float* pr = p + r * cols;
+    const float* tr = t + r * cols;
+    size_t c = lane;
+    for (; c + L < cols; c += 2 * L) {
+      s0 += fminf(fmaxf(pr[c], lo), hi) * tr[c];
+      s1 += fminf(fmaxf(pr[c + L], lo), hi) * tr[c + L];
+    }
+    if (c < cols) s0 += fminf(fmaxf(pr[c], lo), hi) * tr[c];
+  }
+  const float s = wave_reduce<SumOp, L>(s0 + s1);
+  if (r < rows && lane == 0) loss[r] = -logf(s);
 }
 
 __global__ void onehot_kernel(size_t n, size_t classes, const float* __restrict__ cls, float* __restrict__ out) {
@@ -520,8 +533,13 @@ SLHIP_API int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const floa
   size_t len;
   SLHIP_REQUIRE(ctx && preds && targets && loss, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  hipLaunchKernelGGL(cce_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, ctx->stream, rows, cols, preds, targets,
-                     loss);
+  int lanes = 1;
+  while (lanes < 64 && (size_t)lanes * 8 < cols) lanes <<= 1;
+  SLHIP_REQUIRE(ceil_div(rows, 256 / lanes) <= 0x7fffffffu, "too many rows for one launch");
+#define SL_CCE(L) \
+  case L: hipLaunchKernelGGL((cce_kernel<L>), dim3(ceil_div(rows, 256 / L)), dim3(256), 0, ctx->stream, rows, cols, preds, targets, loss); break;
+  switch (lanes) { SL_CCE(1) SL_CCE(2) SL_CCE(4) SL_CCE(8) SL_CCE(16) SL_CCE(32) SL_CCE(64) }
+#undef SL_CCE
   return post_launch();
 }
 

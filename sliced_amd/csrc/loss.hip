@@ -65,49 +65,66 @@ __global__ __launch_bounds__(256) void mse_grad_kernel(size_t n, const float* __
 }
 
 // ---------------------------------------------------------------- softmax cross-entropy
-// One wave per row; the row is swept from global memory (it is short: a class count).
+// L lanes per row (a power of two up to 64, about 8 classes per lane), 256 / L rows per workgroup;
+// the row is swept from global memory three times (the second and third sweep hit the caches: a
+// workgroup's rows are a few KiB).  With one wave per row, whatever its length, rows of 10 classes
+// used 10 of 64 lanes: [13M x 10] streamed at 0.35 TB/s.
+template <int L>
 __global__ __launch_bounds__(256) void softmax_cce_kernel(size_t rows, size_t cols, const float* __restrict__ x,
                                                           const float* __restrict__ t, float* __restrict__ probs,
                                                           float* __restrict__ loss_rows) {
-  const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= rows) return;
-  const int lane = threadIdx.x & 63;
-  const float* xr = x + r * cols;
-  const float* tr = t + r * cols;
+  const size_t r = (size_t)blockIdx.x * (256 / L) + threadIdx.x / L;
+  const bool active = r < rows;
+  const int lane = threadIdx.x % L;
+  const float* xr = x + (active ? r : 0) * cols;
+  const float* tr = t + (active ? r : 0) * cols;
   float m = -__builtin_huge_valf();
-  for (size_t c = lane; c < cols; c += 64) m = fmaxf(m, xr[c]);
-  m = wave_reduce<MaxOp>(m);
+  if (active)
+    for (size_t c = lane; c < cols; c += L) m = fmaxf(m, xr[c]);
+  m = wave_reduce<MaxOp, L>(m);
   float s = 0.0f;
-  for (size_t c = lane; c < cols; c += 64) s += expf(xr[c] - m);
-  s = wave_reduce<SumOp>(s);
+  if (active)
+    for (size_t c = lane; c < cols; c += L) s += expf(xr[c] - m);
+  s = wave_reduce<SumOp, L>(s);
   const float lo = (float)1e-7, hi = (float)(1.0 - 1e-7);
   float acc = 0.0f;
-  for (size_t c = lane; c < cols; c += 64) {
-    const float p = expf(xr[c] - m) / s;
-    if (probs) probs[r * cols + c] = p;
-    acc += fminf(fmaxf(p, lo), hi) * tr[c];
-  }
-  acc = wave_reduce<SumOp>(acc);
-  if (lane == 0) loss_rows[r] = -logf(acc);
+  if (active)
+    for (size_t c = lane; c < cols; c += L) {
+      const float p = expf(xr[c] - m) / s;
+      if (probs) probs[r * cols + c] = p;
+      acc += fminf(fmaxf(p, lo), hi) * tr[c];
+    }
+  acc = wave_reduce<SumOp, L>(acc);
+  if (active && lane == 0) loss_rows[r] = -logf(acc);
 }
 
+template <int L>
 __global__ __launch_bounds__(256) void softmax_cce_grad_kernel(size_t rows, size_t cols, const float* __restrict__ p,
                                                                const float* __restrict__ t, float* __restrict__ lg,
                                                                float beta, const float* __restrict__ upstream) {
-  const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= rows) return;
-  const int lane = threadIdx.x & 63;
-  const float* pr = p + r * cols;
-  const float* tr = t + r * cols;
+  const size_t r = (size_t)blockIdx.x * (256 / L) + threadIdx.x / L;
+  const bool active = r < rows;
+  const int lane = threadIdx.x % L;
+  const float* pr = p + (active ? r : 0) * cols;
+  const float* tr = t + (active ? r : 0) * cols;
   float st = 0.0f;
-  for (size_t c = lane; c < cols; c += 64) st += tr[c];
-  st = wave_reduce<SumOp>(st);
+  if (active)
+    for (size_t c = lane; c < cols; c += L) st += tr[c];
+  st = wave_reduce<SumOp, L>(st);
   const float scale = upstream[0] / (float)rows;
-  for (size_t c = lane; c < cols; c += 64) {
-    const float g = (pr[c] * st - tr[c]) * scale;
-    float* dst = lg + r * cols + c;
-    *dst = beta != 0.0f ? beta * *dst + g : g;
-  }
+  if (active)
+    for (size_t c = lane; c < cols; c += L) {
+      const float g = (pr[c] * st - tr[c]) * scale;
+      float* dst = lg + r * cols + c;
+      *dst = beta != 0.0f ? beta * *dst + g : g;
+    }
+}
+
+// lanes per row for the row-wise loss kernels
+static int loss_lanes(size_t cols) {
+  int lanes = 1;
+  while (lanes < 64 && (size_t)lanes * 8 < cols) lanes <<= 1;
+  return lanes;
 }
 
 }  // namespace slhip
@@ -153,10 +170,22 @@ SLHIP_API int32_t slhip_softmax_cce(slhip_ctx* ctx, size_t rows, size_t cols, co
   size_t len;
   SLHIP_REQUIRE(ctx && logits && targets && loss_rows, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  const size_t blocks = (rows + 3) / 4;
+  // Long rows of a large batch: the register-resident softmax kernel followed by the cce pass moves
+  // 16 B per element at 6 TB/s; the fused kernel's three sweeps with two exponentials per element
+  // move 12 B at 2.6 ([32768 x 4096]: 0.62 ms fused, 0.35 ms as two kernels).  The fused kernel stays
+  // for what it was made for, the launch-bound training step with a few classes.
+  if (probs && cols >= 256 && len >= ((size_t)1 << 22)) {
+    int32_t rc = slhip_softmax(ctx, rows, cols, logits, probs);
+    if (rc) return rc;
+    return slhip_cce(ctx, rows, cols, probs, targets, loss_rows);
+  }
+  const int lanes = loss_lanes(cols);
+  const size_t blocks = (rows + 256 / lanes - 1) / (256 / lanes);
   SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-  hipLaunchKernelGGL(softmax_cce_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, logits, targets,
-                     probs, loss_rows);
+#define SL_SC(L) \
+  case L: hipLaunchKernelGGL((softmax_cce_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, logits, targets, probs, loss_rows); break;
+  switch (lanes) { SL_SC(1) SL_SC(2) SL_SC(4) SL_SC(8) SL_SC(16) SL_SC(32) SL_SC(64) }
+#undef SL_SC
   return post_launch();
 }
 
@@ -166,9 +195,12 @@ SLHIP_API int32_t slhip_softmax_cce_grad(slhip_ctx* ctx, size_t rows, size_t col
   size_t len;
   SLHIP_REQUIRE(ctx && probs && targets && logits_grad && upstream_dev, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  const size_t blocks = (rows + 3) / 4;
+  const int lanes = loss_lanes(cols);
+  const size_t blocks = (rows + 256 / lanes - 1) / (256 / lanes);
   SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-  hipLaunchKernelGGL(softmax_cce_grad_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, probs,
-                     targets, logits_grad, beta, upstream_dev);
+#define SL_SG(L) \
+  case L: hipLaunchKernelGGL((softmax_cce_grad_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, probs, targets, logits_grad, beta, upstream_dev); break;
+  switch (lanes) { SL_SG(1) SL_SG(2) SL_SG(4) SL_SG(8) SL_SG(16) SL_SG(32) SL_SG(64) }
+#undef SL_SG
   return post_launch();
 }

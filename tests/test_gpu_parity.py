@@ -584,7 +584,9 @@ def test_fused_mse_against_the_op_chain(hip, orc, n):
         assert np.array_equal(hip.mse_grad(x, y, xg0.copy(), up), want)
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (7, 3), (8192, 10), (300, 1000), (5, 70001)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(1, 1), (7, 3), (8192, 10), (300, 1000), (5, 70001), (3000, 100), (70000, 7),
+                                   (9000, 512), (1100, 4099)],  # the last two: softmax + cce as two kernels
+                         ids=lambda s: "x".join(map(str, s)))
 def test_fused_softmax_cross_entropy_against_the_op_chain(hip, orc, shape):
     rows, cols = shape
     n = rows * cols
