@@ -376,16 +376,39 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // the CU to itself, 1.25 / 1.8 / 2.3 us when two / three / four workgroups share the CU (4096^3
   // would run at 116 TFLOP/s that way), plus 5 us per launch; it has to beat the modelled time of
   // the best 128 x 128 plan by 8 %, the models being good to about that.
+  // The same small tiles with their k ranges spread over the chip (all of them: fewer tiles than
+  // workgroup slots), for outputs of a few small tiles and a long K - a 64 x 64 x 1048576 product
+  // uses a quarter of a 128 x 128 tile's matrix-core work: 320 us there, about a third of that here.
   bool small_tile = false;
   if (!(ta && tb)) {  // the doubly transposed form is not instantiated for the small tile
     const size_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+    static const double per_kt[5] = {0.0, 0.75, 1.25, 1.8, 2.3};
+    const size_t slots64 = (size_t)ctx->num_cu * 4;
+    const bool automatic = ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && best < 1e299;
+    // plan 1: one workgroup per small tile
+    double t_whole = 1e300;
+    if (tiles64 <= slots64) t_whole = (double)kt_total * per_kt[(tiles64 + ctx->num_cu - 1) / ctx->num_cu] + 5.0;
+    // plan 2: the k tiles of all small tiles dealt out evenly
+    double t_spread = 1e300;
+    size_t units64 = 0, workers64 = 0;
+    if (tiles64 < slots64 && kt_total >= 16 && kt_total < (1u << 20) && tiles64 * kt_total < (1u << 31)) {
+      const size_t total = tiles64 * kt_total;
+      units64 = (total + slots64 - 1) / slots64;
+      if (units64 < 8) units64 = 8;
+      if (units64 > kt_total) units64 = kt_total;
+      workers64 = (total + units64 - 1) / units64;
+      if (2 * workers64 * 64 * 64 * sizeof(float) <= ctx->workspace_bytes)
+        t_spread = (double)units64 * per_kt[(workers64 + ctx->num_cu - 1) / ctx->num_cu] + 5.0 + 4.0 +
+                   2.0 * (double)(tiles64 + workers64) * (64.0 * 64.0 * sizeof(float)) / 5.0e6;
+    }
+    bool spread64 = false;
     if (ctx->gemm_tile == SLHIP_TILE_64X64) {
       small_tile = true;
-    } else if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && best < 1e299 &&
-               tiles64 <= 4 * (size_t)ctx->num_cu) {
-      static const double per_kt[5] = {0.0, 0.75, 1.25, 1.8, 2.3};
-      const size_t share = (tiles64 + ctx->num_cu - 1) / ctx->num_cu;
-      small_tile = (double)kt_total * per_kt[share] + 5.0 < 0.92 * best;
+      spread64 = ctx->gemm_tail == SLHIP_TAIL_SPREAD && t_spread < 1e299;
+    } else if (automatic) {
+      const double t64 = t_whole < t_spread ? t_whole : t_spread;
+      small_tile = t64 < 0.92 * best;
+      spread64 = small_tile && t_spread < t_whole;
     }
     if (small_tile) {
       tiles_m = (M + 63) / 64; tiles_n = (N + 63) / 64;
@@ -393,6 +416,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
       splits = 1;
       spread_workers = 0;
+      if (spread64) {
+        sp.first = 0;
+        sp.units = (unsigned)units64;
+        sp.total = (unsigned)(tiles64 * kt_total);
+        spread_workers = workers64;
+      }
     }
   }
   const size_t tile_m = small_tile ? 64 : BM, tile_n = small_tile ? 64 : BN;
@@ -408,7 +437,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // every k tile of every workgroup complete, inside and 16-byte aligned: the kernel without the
   // clamped loops (k_chunk is a multiple of BK, so only the end of K can leave a partial tile)
   const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % tile_m == 0 && N % tile_n == 0 && K % BK == 0;
-  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, g, sp, spread_workers, tiles - sp.first);
+  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tiles - sp.first);
 
   dim3 grid((unsigned)tiles, (unsigned)splits);
 #define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                  \

@@ -10,10 +10,12 @@
 namespace slhip {
 
 // A workgroup of the spread tail: up to two runs of k tiles, each inside one tile of C, each
-// written as a raw partial tile (row-major 128 x 128) to workspace slot 2*w + run.
-template <bool TA, bool TB, int BK, bool ONLY_FAST>
-__device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp, float (*lds_a)[Cfg<BK, 128>::STAGE_FLOATS],
-                                                   float (*lds_b)[Cfg<BK, 128>::STAGE_FLOATS]) {
+// written as a raw partial tile (row-major, the tile's own size) to workspace slot 2*w + run.
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
+__device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp,
+                                                   float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
+                                                   float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS]) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
   const int r = lane & 31, h = lane >> 5;
@@ -27,69 +29,71 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
     u += (unsigned)(kb - ka);
     unsigned tm, tn;
     tile_of_block(sp.first + ti, g.tiles_m, g.tiles_n, tm, tn);
-    const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+    const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
 
-    floatx16 acc[2][2];
+    floatx16 acc[WM][WN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    gemm_k_range<TA, TB, BK, ONLY_FAST, 2, 2>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
+    gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
 
-    float* slot = g.partial + ((size_t)2 * w + run) * SPREAD_SLOT;
+    float* slot = g.partial + ((size_t)2 * w + run) * (TM * TN);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          slot[(wm * 64 + 32 * i + 8 * (v / 4) + 4 * h + (v % 4)) * BN + wn * 64 + 32 * j + r] = acc[i][j][v];
+          slot[(wm * 32 * WM + 32 * i + 8 * (v / 4) + 4 * h + (v % 4)) * TN + wn * 32 * WN + 32 * j + r] = acc[i][j][v];
   }
 }
 
-template <bool TA, bool TB, int BK, bool ONLY_FAST>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
 __global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadArgs sp) {
-  constexpr int STAGE = Cfg<BK, 128>::STAGE_FLOATS;
-  __shared__ __attribute__((aligned(16))) float lds_a[2][STAGE];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][STAGE];
-  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST>(g, sp, lds_a, lds_b);
-  else gemm_whole_tile<TA, TB, BK, ONLY_FAST, 2, 2>(g, lds_a, lds_b);
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<BK, 64 * WM>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 64 * WN>::STAGE_FLOATS];
+  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST, WM, WN>(g, sp, lds_a, lds_b);
+  else gemm_whole_tile<TA, TB, BK, ONLY_FAST, WM, WN>(g, lds_a, lds_b);
 }
 
 // The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup
-// order), then beta / bias / relu as in the kernel's own epilogue.  Sixteen workgroups per tile,
-// 8 rows each, one float4 of the tile per thread - a tile of a long-K product can have hundreds of
+// order), then beta / bias / relu as in the kernel's own epilogue.  One float4 of the tile per
+// thread (sixteen workgroups per 128 x 128 tile, four per 64 x 64 tile) - a tile of a long-K product can have hundreds of
 // partial tiles (64 x 64 x 1048576: one tile, 512 partials; four workgroups summing them one after
 // the other took 650 us of that product's 930).  Workgroup spread_first + w holds k tiles
 // [w*U, (w+1)*U) of the tail's sequence, so tile ti is covered by workgroups (ti*KT)/U ..
 // ((ti+1)*KT - 1)/U.  Only the first of them can have started in the tile before (U <= KT): its
 // partial of this tile is its run ti - (w*U)/KT; every later one's is its run 0.
+template <int TM, int TN>
 __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArgs sp) {
-  const unsigned ti = blockIdx.x >> 4, quarter = blockIdx.x & 15;
+  constexpr int PARTS = TM * TN / 4 / 256;  // workgroups per tile
+  constexpr int SLOT = TM * TN;
+  const unsigned ti = blockIdx.x / PARTS, part = blockIdx.x % PARTS;
   unsigned tm, tn;
   tile_of_block(sp.first + ti, g.tiles_m, g.tiles_n, tm, tn);
-  const size_t m0 = (size_t)tm * BM, n0 = (size_t)tn * BN;
+  const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
   const unsigned KT = sp.kt_total, U = sp.units;
   const unsigned w_first = (ti * KT) / U, w_last = ((ti + 1) * KT - 1) / U;
-  constexpr int PER = 8 * (BN / 4) / 256;  // float4 per thread: one
+  constexpr int PER = 1;  // float4 per thread
   float4 s[PER], c[PER], mk[PER];
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    const int f = threadIdx.x + 256 * e;
-    const int row_l = quarter * 8 + f / (BN / 4), c4 = f % (BN / 4);
-    const float* p0 = g.partial + row_l * BN + 4 * c4;
-    float4 sum = ld4(p0 + ((size_t)2 * w_first + (ti - (w_first * U) / KT)) * SPREAD_SLOT);
+    const int f = threadIdx.x + 256 * (int)part;
+    const int row_l = f / (TN / 4), c4 = f % (TN / 4);
+    const float* p0 = g.partial + row_l * TN + 4 * c4;
+    float4 sum = ld4(p0 + ((size_t)2 * w_first + (ti - (w_first * U) / KT)) * SLOT);
     auto add = [&](const float4& p) { sum.x += p.x; sum.y += p.y; sum.z += p.z; sum.w += p.w; };
     unsigned w = w_first + 1;
     for (; w + 3 <= w_last; w += 4) {  // four loads in flight, added in ascending order
-      const float4 q0 = ld4(p0 + (size_t)2 * w * SPREAD_SLOT), q1 = ld4(p0 + (size_t)2 * (w + 1) * SPREAD_SLOT),
-                   q2 = ld4(p0 + (size_t)2 * (w + 2) * SPREAD_SLOT), q3 = ld4(p0 + (size_t)2 * (w + 3) * SPREAD_SLOT);
+      const float4 q0 = ld4(p0 + (size_t)2 * w * SLOT), q1 = ld4(p0 + (size_t)2 * (w + 1) * SLOT),
+                   q2 = ld4(p0 + (size_t)2 * (w + 2) * SLOT), q3 = ld4(p0 + (size_t)2 * (w + 3) * SLOT);
       add(q0); add(q1); add(q2); add(q3);
     }
-    for (; w <= w_last; ++w) add(ld4(p0 + (size_t)2 * w * SPREAD_SLOT));
+    for (; w <= w_last; ++w) add(ld4(p0 + (size_t)2 * w * SLOT));
     s[e] = sum;
     const size_t row = m0 + row_l, col = n0 + 4 * c4;
     c[e] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -106,8 +110,8 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
   }
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    const int f = threadIdx.x + 256 * e;
-    const int row_l = quarter * 8 + f / (BN / 4), c4 = f % (BN / 4);
+    const int f = threadIdx.x + 256 * (int)part;
+    const int row_l = f / (TN / 4), c4 = f % (TN / 4);
     const size_t row = m0 + row_l, col = n0 + 4 * c4;
     if (row >= g.M || col >= g.N) continue;
     float v[4] = {s[e].x, s[e].y, s[e].z, s[e].w};
@@ -140,24 +144,31 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
   }
 }
 
-int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g, const SpreadArgs& sp,
-                           size_t workers, size_t tail_tiles) {
+int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
+                           const SpreadArgs& sp, size_t workers, size_t tail_tiles) {
   const dim3 grid((unsigned)(sp.first + workers));
-#define SL_GEMM(TA_, TB_)                                                                                              \
-  do {                                                                                                                 \
-    if (only_fast)                                                                                                     \
-      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, true>), grid, dim3(256), 0, ctx->stream, g, sp);       \
-    else                                                                                                               \
-      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, false>), grid, dim3(256), 0, ctx->stream, g, sp);      \
+#define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                          \
+  do {                                                                                                                        \
+    if (only_fast)                                                                                                            \
+      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, true, WM_, WN_>), grid, dim3(256), 0, ctx->stream, g, sp);    \
+    else                                                                                                                      \
+      hipLaunchKernelGGL((gemm_spread_kernel<TA_, TB_, GEMM_BK, false, WM_, WN_>), grid, dim3(256), 0, ctx->stream, g, sp);   \
+  } while (0)
+#define SL_GEMM(TA_, TB_)                      \
+  do {                                         \
+    if (small_tile) SL_GEMM3(TA_, TB_, 1, 1);  \
+    else SL_GEMM3(TA_, TB_, 2, 2);             \
   } while (0)
   if (!ta && !tb) SL_GEMM(false, false);
   else if (!ta && tb) SL_GEMM(false, true);
   else if (ta && !tb) SL_GEMM(true, false);
-  else SL_GEMM(true, true);
+  else SL_GEMM3(true, true, 2, 2);
 #undef SL_GEMM
+#undef SL_GEMM3
   int32_t rc = post_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL(spread_fixup_kernel, dim3((unsigned)(16 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
+  if (small_tile) hipLaunchKernelGGL((spread_fixup_kernel<64, 64>), dim3((unsigned)(4 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
+  else hipLaunchKernelGGL((spread_fixup_kernel<128, 128>), dim3((unsigned)(16 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
   return post_launch();
 }
 

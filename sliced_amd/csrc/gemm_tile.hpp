@@ -417,7 +417,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 }
 
 // Launches the spread-tail kernel and its fix-up (gemm_spread.hip).
-int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g, const SpreadArgs& sp,
-                           size_t workers, size_t tail_tiles);
+int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
+                           const SpreadArgs& sp, size_t workers, size_t tail_tiles);
 
 }  // namespace slhip

@@ -173,8 +173,27 @@ def test_gemm_small_tile(hip, orc):
             hip.gemm_tile_policy(hip.TILE_128X128)
             big = hip.sgemm(ta, tb, m, n, k, a, b)
             assert np.all(np.abs(got - big) <= 2 * bound)
+            # small tiles with their k ranges spread over the chip
+            if (k + 31) // 32 >= 16:
+                hip.gemm_tile_policy(hip.TILE_64X64)
+                hip.gemm_tail_policy(hip.TAIL_SPREAD)
+                sp = hip.sgemm(ta, tb, m, n, k, a, b)
+                assert np.all(np.abs(sp - exact) <= bound), np.max(np.abs(sp - exact) / bound)
+                assert np.array_equal(sp, hip.sgemm(ta, tb, m, n, k, a, b))
+                assert np.array_equal(hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0), sp + c0)
+                assert np.array_equal(hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre), np.where(pre >= 0, sp, 0 * sp))
+                hip.gemm_tail_policy(hip.TAIL_AUTO)
+        # the default policies on an output of one small tile and a long k
+        hip.gemm_tile_policy(hip.TILE_AUTO)
+        for (m, n, k, ta, tb) in [(64, 64, 200000, 1, 0), (60, 50, 70001, 0, 0), (64, 100, 50000, 0, 1)]:
+            say("small-tile spread, default policy", m, n, k, ta, tb)
+            a, b = gemm_operands(ta, tb, m, n, k)
+            exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+            got = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
     finally:
         hip.gemm_tile_policy(hip.TILE_AUTO)
+        hip.gemm_tail_policy(hip.TAIL_AUTO)
 
 
 def test_sgemm_relu_mask_equals_gemm_then_relu_grad(hip, orc):
