@@ -155,6 +155,7 @@ class HIP {
     if (g != grads_.end()) {  // the gradient lives and dies with its buffer
       const uint64_t gid = g->second.id;
       grads_.erase(g);
+      stale_.erase(gid);
       release(gid);
     }
   }
@@ -221,23 +222,43 @@ class HIP {
   size_t tape_len() const { return tape_.size(); }
 
   bool has_grad(uint64_t id) const { return grads_.count(id) != 0; }
-  Buffer grad(const Buffer& b) const {
+  // Gradient of `b` for reading (throws if none was ever written).
+  Buffer grad(const Buffer& b) {
     auto it = grads_.find(b.id);
     if (it == grads_.end()) throw Error("buffer " + std::to_string(b.id) + " has no gradient");
+    settle(it->second);
     return it->second;
   }
+  // Gradient of `b` for an op that accumulates into it: created zeroed if absent.
   Buffer grad_mut(const Buffer& b) {
-    auto it = grads_.find(b.id);
-    if (it != grads_.end()) return it->second;
-    Buffer g = pool_alloc(b.len);
-    grads_[b.id] = g;
+    Buffer g = grad_slot(b);
+    settle(g);
+    return g;
+  }
+  // Gradient of `b` for an op that writes it: `overwrite` = the op sets every element without
+  // reading any, so a pending zero fill of this gradient is dropped instead of run.
+  Buffer grad_out(const Buffer& b, bool overwrite) {
+    if (!overwrite) return grad_mut(b);
+    Buffer g = grad_slot(b);
+    stale_.erase(g.id);
     return g;
   }
   // All gradients live side by side in a few large slabs, so that zeroing them is one fill per
   // slab instead of one per gradient (17 launches per step for the three-layer MLP otherwise).
+  // Gradients of LAZY_ZERO_MIN floats and more have slabs of their own and are only marked: the
+  // fill runs when the gradient is next read or accumulated into, and not at all when an op
+  // overwrites it first - the activation gradients of a fused step, 64 MiB each for the classifier
+  // with batch 8192, are all written that way (41 us of fills a step otherwise).
   void zero_grad() {
     for (auto& sl : slabs_)
-      if (sl.used) check(slhip_memset(ctx_, sl.base, 0, sl.used * sizeof(float)), "slhip_memset");
+      if (!sl.lazy && sl.used) check(slhip_memset(ctx_, sl.base, 0, sl.used * sizeof(float)), "slhip_memset");
+    for (auto& kv : grads_)
+      if (kv.second.len >= LAZY_ZERO_MIN) stale_.insert(kv.second.id);
+  }
+  void drop_pending_zero(const Buffer& g) { stale_.erase(g.id); }  // the caller overwrites all of g
+  // Runs the zero fill that zero_grad() left pending for this buffer, if any.
+  void settle(const Buffer& g) {
+    if (!stale_.empty() && stale_.erase(g.id)) check(slhip_memset(ctx_, g.ptr, 0, g.len * sizeof(float)), "slhip_memset");
   }
   void run_tape() {
     for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
@@ -246,13 +267,13 @@ class HIP {
     relu_grad_done_.clear();
   }
   void backward(const Buffer& out) {
-    Buffer g = grad_mut(out);
+    Buffer g = grad_out(out, true);
     check(slhip_fill(ctx_, g.len, 1.0f, g.ptr), "slhip_fill");
     run_tape();
   }
   void backward_with(const Buffer& out, const Buffer& seed) {
     if (seed.len != out.len) throw Error("backward_with: seed length differs");
-    Buffer g = grad_mut(out);
+    Buffer g = grad_out(out, true);
     check(slhip_memcpy_d2d(ctx_, g.ptr, seed.ptr, g.len * sizeof(float)), "slhip_memcpy_d2d");
     run_tape();
   }
@@ -266,8 +287,9 @@ class HIP {
     uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
     add_grad_fn([=] {
       Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
-      float* lg = l.requires_grad ? grad_mut(l).ptr : nullptr;
-      float* rg = r.requires_grad ? grad_mut(r).ptr : nullptr;
+      const bool set = policy.gemm_beta == 0.0f;
+      float* lg = l.requires_grad ? grad_out(l, set).ptr : nullptr;
+      float* rg = r.requires_grad ? grad_out(r, set).ptr : nullptr;
       check(slhip_gemm_grad(ctx_, m, k, n, l.ptr, r.ptr, lg, rg, grad(o).ptr, policy.gemm_beta), "slhip_gemm_grad");
     });
     return out;
@@ -298,18 +320,19 @@ class HIP {
         g = grad(o);
       }
       check(slhip_add_row_mut_grad(ctx_, m, n, grad_mut(bb).ptr, g.ptr), "bias grad");
-      float* xg = xb.requires_grad ? grad_mut(xb).ptr : nullptr;
-      float* wg = wb.requires_grad ? grad_mut(wb).ptr : nullptr;
+      const bool set = policy.gemm_beta == 0.0f;
       auto producer = relu_pre_.find(xi);
-      if (policy.fuse_relu_grad && xg && producer != relu_pre_.end()) {
+      const bool into_pre = policy.fuse_relu_grad && xb.requires_grad && producer != relu_pre_.end();
+      float* xg = xb.requires_grad && !into_pre ? grad_out(xb, set).ptr : nullptr;
+      float* wg = wb.requires_grad ? grad_out(wb, set).ptr : nullptr;
+      if (into_pre) {
         // x is the ReLU output of a fused Linear that is still on the tape
         Buffer xp = lookup(producer->second);
         // written the way gemm_grad writes x.grad (policy.gemm_beta; SET by default): pre.grad is
         // zero at this point, and `0 + v` differs from `v` only in the sign of a zero
-        check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_mut(xp).ptr, policy.gemm_beta),
+        check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_out(xp, set).ptr, policy.gemm_beta),
               "slhip_sgemm_relu_mask");
         relu_grad_done_.insert(xi);
-        xg = nullptr;
       }
       check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
     });
@@ -431,7 +454,7 @@ class HIP {
     uint64_t xi = x.id, oi = out.id;
     add_grad_fn([=] {
       Buffer xb = lookup(xi), o = lookup(oi);
-      check(slhip_transpose(ctx_, cols, rows, grad(o).ptr, grad_mut(xb).ptr, policy.transpose_beta), "transpose_grad");
+      check(slhip_transpose(ctx_, cols, rows, grad(o).ptr, grad_out(xb, policy.transpose_beta == 0.0f).ptr, policy.transpose_beta), "transpose_grad");
     });
     return out;
   }
@@ -444,7 +467,7 @@ class HIP {
     uint64_t xi = x.id, oi = out.id;
     add_grad_fn([=] {
       Buffer xb = lookup(xi), o = lookup(oi);
-      check(slhip_softmax_grad(ctx_, samples, features, grad_mut(xb).ptr, o.ptr, grad(o).ptr, policy.softmax_beta),
+      check(slhip_softmax_grad(ctx_, samples, features, grad_out(xb, policy.softmax_beta == 0.0f).ptr, o.ptr, grad(o).ptr, policy.softmax_beta),
             "slhip_softmax_grad");
     });
     return out;
@@ -505,7 +528,7 @@ class HIP {
     uint64_t li = logits.id, ti = targets.id, pi = probs.id, oi = out.id;
     add_grad_fn([=] {
       Buffer l = lookup(li), t = lookup(ti), p = lookup(pi), o = lookup(oi);
-      check(slhip_softmax_cce_grad(ctx_, rows, cols, p.ptr, t.ptr, grad_mut(l).ptr, policy.softmax_beta, grad(o).ptr),
+      check(slhip_softmax_cce_grad(ctx_, rows, cols, p.ptr, t.ptr, grad_out(l, policy.softmax_beta == 0.0f).ptr, policy.softmax_beta, grad(o).ptr),
             "slhip_softmax_cce_grad");
     });
     return out;
@@ -558,29 +581,43 @@ class HIP {
   struct Slab {
     float* base;
     size_t cap, used;
+    bool lazy;  // holds the large gradients, which zero_grad() marks instead of filling
   };
+  static constexpr size_t LAZY_ZERO_MIN = size_t(1) << 20;
   Buffer pool_alloc(size_t len) {
     const size_t need = (len + 63) / 64 * 64;
-    if (slabs_.empty() || slabs_.back().used + need > slabs_.back().cap) {
-      size_t cap = slabs_.empty() ? (size_t(1) << 22) : slabs_.back().cap * 2;
+    const bool lazy = len >= LAZY_ZERO_MIN;
+    Slab* cur = nullptr;
+    size_t last_cap = 0;
+    for (auto& sl : slabs_)
+      if (sl.lazy == lazy) { cur = &sl; last_cap = sl.cap; }
+    if (!cur || cur->used + need > cur->cap) {
+      size_t cap = last_cap ? last_cap * 2 : (size_t(1) << 22);
       if (cap > (size_t(1) << 28)) cap = size_t(1) << 28;
       if (cap < need) cap = need;
-      Slab sl{nullptr, cap, 0};
+      Slab sl{nullptr, cap, 0, lazy};
       check(slhip_malloc(ctx_, cap * sizeof(float), (void**)&sl.base), "slhip_malloc");
       check(slhip_memset(ctx_, sl.base, 0, cap * sizeof(float)), "slhip_memset");
       slabs_.push_back(sl);
+      cur = &slabs_.back();
     }
-    Slab& sl = slabs_.back();
     Buffer b;
     b.dev = this;
     b.id = next_id_++;
     b.len = len;
-    b.ptr = sl.base + sl.used;
+    b.ptr = cur->base + cur->used;
     b.requires_grad = false;
     b.pooled = true;
-    sl.used += need;
+    cur->used += need;
     allocs_[b.id] = b;
     return b;
+  }
+  Buffer grad_slot(const Buffer& b) {
+    auto it = grads_.find(b.id);
+    if (it != grads_.end()) return it->second;
+    Buffer g = pool_alloc(b.len);  // out of a slab that was zeroed when it was created
+    grads_[b.id] = g;
+    return g;
   }
   Buffer scalar_scratch() {
     if (!scratch_.valid()) scratch_ = alloc(1, true);
@@ -595,6 +632,7 @@ class HIP {
   std::vector<Slab> slabs_;
   std::vector<std::function<void()>> tape_;
   std::unordered_map<uint64_t, uint64_t> relu_pre_;   // ReLU output of a fused Linear on the tape -> its pre-activation
+  std::unordered_set<uint64_t> stale_;                // large gradients with a zero fill pending since zero_grad()
   std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
   bool tape_enabled_ = true;
   std::vector<Buffer> cache_;
@@ -604,11 +642,13 @@ class HIP {
 
 inline std::vector<float> Buffer::read() const {
   std::vector<float> v(len);
+  dev->settle(*this);
   check(slhip_memcpy_d2h(dev->ctx(), v.data(), ptr, len * sizeof(float)), "slhip_memcpy_d2h");
   return v;
 }
 inline void Buffer::write(const float* host, size_t n) const {
   if (n != len) throw Error("write: length differs");
+  dev->drop_pending_zero(*this);
   check(slhip_memcpy_h2d(dev->ctx(), ptr, host, len * sizeof(float)), "slhip_memcpy_h2d");
 }
 inline Buffer Buffer::grad() const { return dev->grad(*this); }

@@ -297,6 +297,44 @@ def test_linear_fused_matches_unfused_tape(device):
         assert np.array_equal(a, c)
 
 
+def test_zero_grad_of_large_gradients_is_deferred_but_never_visible(device):
+    """Gradients of 2^20 floats and more are zeroed when next read or accumulated into, and not at
+    all when an op overwrites them first: whatever the order of calls, the values are those of
+    an immediate fill."""
+    n = (1 << 20) + 192
+    xv = rng.uniform(n, -2, 2, tag=0)
+    x = device.buffer(xv)
+    device.square(x).backward()
+    g = x.grad()                                       # handle kept across zero_grad
+    assert np.array_equal(g.read(), 2 * xv)
+    device.zero_grad()
+    assert not g.read().any()                          # read through the old handle
+    device.square(x).backward()                        # accumulating op: 0 + 2x, not 2x + 2x
+    assert np.array_equal(x.grad().read(), 2 * xv)
+    device.zero_grad()
+    device.square(x).backward()
+    device.square(x).backward()                        # second accumulation after one fill
+    assert np.array_equal(x.grad().read(), 4 * xv)
+
+    # overwriting op (gemm_grad with the default SET policy), then the accumulate policy
+    m, k, nn = 2048, 512, 8
+    a, b = device.buffer(rng.uniform(m * k, -1, 1, tag=1)), device.buffer(rng.uniform(k * nn, -1, 1, tag=2))
+    device.gemm(m, k, nn, a, b).backward()
+    first = a.grad().read()
+    assert first.any()
+    for _ in range(2):
+        device.zero_grad()
+        device.gemm(m, k, nn, a, b).backward()
+        assert np.array_equal(a.grad().read(), first)
+    device.set_grad_policy(gemm_beta=1.0)
+    device.zero_grad()
+    device.gemm(m, k, nn, a, b).backward()
+    assert np.array_equal(a.grad().read(), first)      # 0 + v
+    device.gemm(m, k, nn, a, b).backward()
+    assert np.allclose(a.grad().read(), 2 * first, rtol=1e-6, atol=0)
+    device.set_grad_policy()
+
+
 def test_relu_grad_fused_into_the_next_layers_input_gradient(device):
     # two fused Linear+ReLU layers and a plain one: with the ReLU gradients riding in the next
     # layer's input-gradient GEMM every gradient keeps its bits
