@@ -92,7 +92,9 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
   // with the fused Linear the ReLU gradients ride in the next layer's input-gradient GEMM
   dev.policy.fuse_relu_grad = fused;
 
-  // One training step.  Leaves the loss in loss_dev; reads it back unless `deferred`.
+  // One training step.  Reads the loss back unless `deferred`; then `loss_at` names the device
+  // scalar that holds it (the same one every step: op outputs are cached by call position).
+  Buffer loss_at = loss_dev;
   auto train_step = [&](bool deferred) -> float {
     dev.zero_grad();
     Matrix out;
@@ -108,7 +110,7 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
     float loss_val = 0.0f;
     if (fused_loss) {
       Buffer L = kind == 0 ? dev.mse_loss(out.data, y.data) : dev.softmax_cce_loss(batch, d_out, out.data, y.data);
-      if (deferred) dev.copy(L, 0, loss_dev, 0, 1);
+      if (deferred) loss_at = L;
       else loss_val = L.read()[0];
       L.backward();
     } else if (kind == 0) {
@@ -116,7 +118,7 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
       Matrix q = d.squared();
       Matrix s = q.as_dims(1, n_out).sum_cols();  // one row: the sum over every element
       Matrix L = s.mul(c);
-      if (deferred) dev.copy(L.data, 0, loss_dev, 0, 1);
+      if (deferred) loss_at = L.data;
       else loss_val = L.read()[0];
       L.backward();
     } else {
@@ -159,7 +161,7 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
       }
       recorded.run();
     }
-    dev.copy(loss_dev, 0, loss_log, it, 1);
+    dev.copy(loss_at, 0, loss_log, it, 1);
   }
   dev.sync();
   res.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();

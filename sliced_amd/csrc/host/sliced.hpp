@@ -156,6 +156,8 @@ class HIP {
       const uint64_t gid = g->second.id;
       grads_.erase(g);
       stale_.erase(gid);
+      ones_.erase(gid);
+      lazy_.erase(gid);
       release(gid);
     }
   }
@@ -233,6 +235,7 @@ class HIP {
   Buffer grad_mut(const Buffer& b) {
     Buffer g = grad_slot(b);
     settle(g);
+    ones_.erase(g.id);
     return g;
   }
   // Gradient of `b` for an op that writes it: `overwrite` = the op sets every element without
@@ -241,6 +244,7 @@ class HIP {
     if (!overwrite) return grad_mut(b);
     Buffer g = grad_slot(b);
     stale_.erase(g.id);
+    ones_.erase(g.id);
     return g;
   }
   // All gradients live side by side in a few large slabs, so that zeroing them is one fill per
@@ -252,13 +256,21 @@ class HIP {
   void zero_grad() {
     for (auto& sl : slabs_)
       if (!sl.lazy && sl.used) check(slhip_memset(ctx_, sl.base, 0, sl.used * sizeof(float)), "slhip_memset");
-    for (auto& kv : grads_)
-      if (kv.second.len >= LAZY_ZERO_MIN) stale_.insert(kv.second.id);
+    for (auto& kv : grads_) {
+      if (lazy_.count(kv.second.id)) stale_.insert(kv.second.id);
+      else ones_.erase(kv.second.id);
+    }
   }
-  void drop_pending_zero(const Buffer& g) { stale_.erase(g.id); }  // the caller overwrites all of g
+  void drop_pending_zero(const Buffer& g) {  // the caller overwrites all of g
+    stale_.erase(g.id);
+    ones_.erase(g.id);
+  }
   // Runs the zero fill that zero_grad() left pending for this buffer, if any.
   void settle(const Buffer& g) {
-    if (!stale_.empty() && stale_.erase(g.id)) check(slhip_memset(ctx_, g.ptr, 0, g.len * sizeof(float)), "slhip_memset");
+    if (!stale_.empty() && stale_.erase(g.id)) {
+      check(slhip_memset(ctx_, g.ptr, 0, g.len * sizeof(float)), "slhip_memset");
+      ones_.erase(g.id);
+    }
   }
   void run_tape() {
     for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
@@ -266,9 +278,17 @@ class HIP {
     relu_pre_.clear();
     relu_grad_done_.clear();
   }
+  // Seeds out's gradient with ones and runs the tape.  A seed gradient that backward() itself created
+  // lives with the deferred-zero gradients: while nothing else has written it since the last
+  // backward(), it still holds the ones, zero_grad() has only marked it, and the fill is skipped
+  // (one kernel less in every training step, recorded or not).
   void backward(const Buffer& out) {
-    Buffer g = grad_out(out, true);
-    check(slhip_fill(ctx_, g.len, 1.0f, g.ptr), "slhip_fill");
+    const bool fresh = !has_grad(out.id);
+    Buffer g = grad_slot(out, /*lazy=*/fresh);
+    const bool still_ones = ones_.count(g.id) != 0;
+    stale_.erase(g.id);
+    if (!still_ones) check(slhip_fill(ctx_, g.len, 1.0f, g.ptr), "slhip_fill");
+    ones_.insert(g.id);
     run_tape();
   }
   void backward_with(const Buffer& out, const Buffer& seed) {
@@ -584,9 +604,9 @@ class HIP {
     bool lazy;  // holds the large gradients, which zero_grad() marks instead of filling
   };
   static constexpr size_t LAZY_ZERO_MIN = size_t(1) << 20;
-  Buffer pool_alloc(size_t len) {
+  Buffer pool_alloc(size_t len, bool force_lazy = false) {
     const size_t need = (len + 63) / 64 * 64;
-    const bool lazy = len >= LAZY_ZERO_MIN;
+    const bool lazy = force_lazy || len >= LAZY_ZERO_MIN;
     Slab* cur = nullptr;
     size_t last_cap = 0;
     for (auto& sl : slabs_)
@@ -610,12 +630,13 @@ class HIP {
     b.pooled = true;
     cur->used += need;
     allocs_[b.id] = b;
+    if (lazy) lazy_.insert(b.id);
     return b;
   }
-  Buffer grad_slot(const Buffer& b) {
+  Buffer grad_slot(const Buffer& b, bool lazy = false) {
     auto it = grads_.find(b.id);
     if (it != grads_.end()) return it->second;
-    Buffer g = pool_alloc(b.len);  // out of a slab that was zeroed when it was created
+    Buffer g = pool_alloc(b.len, lazy);  // out of a slab that was zeroed when it was created
     grads_[b.id] = g;
     return g;
   }
@@ -632,6 +653,8 @@ class HIP {
   std::vector<Slab> slabs_;
   std::vector<std::function<void()>> tape_;
   std::unordered_map<uint64_t, uint64_t> relu_pre_;   // ReLU output of a fused Linear on the tape -> its pre-activation
+  std::unordered_set<uint64_t> lazy_;                 // gradients in the slabs that zero_grad() marks instead of filling
+  std::unordered_set<uint64_t> ones_;                 // gradients known to hold nothing but 1.0 (backward()'s seed)
   std::unordered_set<uint64_t> stale_;                // large gradients with a zero fill pending since zero_grad()
   std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
   bool tape_enabled_ = true;

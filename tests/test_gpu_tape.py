@@ -335,6 +335,29 @@ def test_zero_grad_of_large_gradients_is_deferred_but_never_visible(device):
     device.set_grad_policy()
 
 
+def test_backward_seed_is_refilled_after_another_op_wrote_it():
+    """backward() skips the fill of a seed gradient that still holds its ones; any other write to
+    that gradient (here: the buffer feeds a further op in one iteration) brings the fill back."""
+    from sliced_amd import host
+    dev = host.HIP(0, cached=True)
+    xv = rng.uniform(1000, 0.5, 1.5, tag=0)
+    x = dev.buffer(xv)
+    for epoch in range(6):
+        dev.begin_iteration()
+        dev.zero_grad()
+        sq = dev.square(x)
+        if epoch % 3 == 2:                              # sq is an inner node: its gradient is accumulated into
+            dev.square(sq).backward()
+            assert np.allclose(x.grad().read(), 4 * xv ** 3, rtol=1e-6, atol=0)
+        else:                                           # sq is the loss: its gradient is the seed
+            sq.backward()
+            assert np.array_equal(x.grad().read(), 2 * xv)
+            assert np.array_equal(sq.grad().read(), np.ones(1000, np.float32))
+    dev.zero_grad()
+    assert not sq.grad().read().any()
+    dev.close()
+
+
 def test_relu_grad_fused_into_the_next_layers_input_gradient(device):
     # two fused Linear+ReLU layers and a plain one: with the ReLU gradients riding in the next
     # layer's input-gradient GEMM every gradient keeps its bits
