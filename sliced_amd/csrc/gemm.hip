@@ -174,7 +174,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
   if (vec) {
     for (size_t i = tid; i < (mn >> 2); i += stride) {
       float4 s = ld4g(partial + 4 * i);
-      for (unsigned z = 1; z < splits; ++z) {
+      unsigned z = 1;
+      for (; z + 4 <= splits; z += 4) {  // four loads in flight, added in the same order as one by one
+        float4 p[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) p[u] = ld4g(partial + (size_t)(z + u) * mn + 4 * i);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { s.x += p[u].x; s.y += p[u].y; s.z += p[u].z; s.w += p[u].w; }
+      }
+      for (; z < splits; ++z) {
         float4 p = ld4g(partial + (size_t)z * mn + 4 * i);
         s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
       }
@@ -234,6 +242,14 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   g.m_fast = (aligned16(A) && aligned16(B)) ? M : 0;
   g.partial = (float*)ctx->workspace;
   const size_t mn_bytes = M * N * sizeof(float);
+
+  // HBM-bound skinny products with float4-friendly shapes: vector-ALU kernels of their own
+  {
+    int32_t rc = SLHIP_OK;
+    const int took = gemm_skinny_launch(ctx, ta, tb, g, &rc);
+    if (took == 1 || rc) return rc;
+    if (took == 2) return splitk_combine(ctx, g, g.splits);
+  }
 
   // Small and skinny (an output side <= 32, or K <= 16) products: wave-per-tile kernel.  "Small" is
   // <= 6e8 flop when the kernel can use its unchecked vector-load form (it then beats the tiled

@@ -1,0 +1,292 @@
+// Products with one very short dimension and a large streamed operand or result.  They are bound
+// by HBM, not by the matrix cores, so they run on the vector ALUs with every global access a
+// whole float4 per lane:
+//
+//   short K   (K <= 12, any form): C[M x N] is the large side (4 B written per 2K flop).  A thread
+//             keeps the K x 4 block of B for its four columns in registers and walks down the rows;
+//             the K values of A for a row are the same for the whole wave.  In a classifier this
+//             is the input gradient of the last layer, G[batch x classes] * W^T.
+//   narrow N  (N <= 16, A^T * B with A stored K x M): A is the large side and is read once, in
+//             rows of M contiguous floats; a lane keeps 4 x N accumulators for its four columns of
+//             A; the N values of B for a k are the same for the whole wave.  Sixteen waves of a
+//             workgroup interleave over the k range and add up through LDS in a fixed order;
+//             workgroups split K and leave partials in the workspace for the split-K combine.
+//             In a classifier this is the weight gradient of the last layer, H^T * G.
+//
+// Against the wave-per-tile MFMA kernel, which reads and writes 128-byte pieces per row
+// (MI355X, classifier with batch 8192, hidden 2048, 10 classes): input gradient with the ReLU
+// mask 33 -> 23 us (23 -> 14.5 without the mask), weight gradient with its combine 34.5 -> 29 us;
+// 4096 x 16 x 16384 (256 MiB of A) 116 -> 61 us, 1024 x 4 x 65536 112 -> 54 us.
+#include "gemm_tile.hpp"
+
+namespace slhip {
+
+// beyond 12 the wave-per-tile MFMA kernel is the faster one (4096 x 4096 x 16: 17.6 us against 19.3)
+constexpr int SHORT_K_MAX = 12;
+constexpr int SHORT_K_ROWS = 64;  // most rows of A a workgroup of the short-K kernel stages in LDS
+
+template <int KP, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_short_k_kernel(size_t M, size_t N, int K, const float* __restrict__ A,
+                                                           const float* __restrict__ B, float* C, float beta,
+                                                           const float* __restrict__ bias, int relu, float* pre_act,
+                                                           const float* mask, unsigned rows_per_block) {
+  // The rows of A this workgroup uses, zero-padded to KP columns: every lane of a wave reads the
+  // same row at the same time (one broadcast ds_read_b128 per four k).  Fetching them with
+  // wave-uniform global loads instead costs K load instructions per row and store.
+  __shared__ __attribute__((aligned(16))) float As[SHORT_K_ROWS][KP];
+  const size_t m0 = (size_t)blockIdx.y * rows_per_block;
+  const int rows = (int)(m0 + rows_per_block < M ? rows_per_block : M - m0);
+  for (int idx = threadIdx.x; idx < rows * KP; idx += 256) {
+    const int r = TA ? idx % rows : idx / KP, k = TA ? idx / rows : idx % KP;
+    float v = 0.0f;
+    if (k < K) v = TA ? A[(size_t)k * M + m0 + r] : A[(m0 + r) * (size_t)K + k];
+    As[r][k] = v;
+  }
+  const size_t n = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const bool active = n < N;
+  const size_t nc = active ? n : 0;
+  float b[KP][4];
+  if (TB) {
+    // B is stored N x K: the K x 4 block of a thread is 4K contiguous floats (16-byte aligned: n is
+    // a multiple of 4), K vector loads in flight together; float q*K + k of them is B[n + q][k].
+    // K is one of the four values that share this KP: each gets its own unrolled unpacking.
+    float f[KP * 4];
+#pragma unroll
+    for (int j = 0; j < KP; ++j) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (j < K) v = ld4g(B + nc * (size_t)K + 4 * j);
+      f[4 * j] = v.x; f[4 * j + 1] = v.y; f[4 * j + 2] = v.z; f[4 * j + 3] = v.w;
+    }
+    auto unpack = [&](auto kc) {
+      constexpr int KC = decltype(kc)::value;
+#pragma unroll
+      for (int k = 0; k < KP; ++k)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[k][q] = k < KC ? f[(q * KC + k) % (KP * 4)] : 0.0f;
+    };
+    switch (KP - K) {
+      case 0: unpack(std::integral_constant<int, KP>()); break;
+      case 1: unpack(std::integral_constant<int, KP - 1>()); break;
+      case 2: unpack(std::integral_constant<int, KP - 2>()); break;
+      default: unpack(std::integral_constant<int, KP - 3>()); break;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < KP; ++k) {
+      if (k < K) {
+        const float4 v = ld4g(B + (size_t)k * N + nc);
+        b[k][0] = v.x; b[k][1] = v.y; b[k][2] = v.z; b[k][3] = v.w;
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[k][q] = 0.0f;
+      }
+    }
+  }
+  float4 bi = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) bi = ld4g(bias + nc);
+  __syncthreads();
+  if (!active) return;
+  constexpr int R = 4;  // rows per pass: their mask / C reads are in flight together
+  for (int m = 0; m < rows; m += R) {
+    float acc[R][4];
+    size_t at[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int lr = m + r < rows ? m + r : rows - 1;  // a pass past the end repeats the last row and does not store it
+      at[r] = (m0 + lr) * N + n;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[r][q] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < KP; ++k) {
+        const float a = As[lr][k];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[r][q] = __builtin_fmaf(a, b[k][q], acc[r][q]);
+      }
+    }
+    // every read before the first store: C, pre_act and mask may be the same memory as far as the compiler knows
+    if (mask) {
+      float4 mk[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) mk[r] = ld4g(mask + at[r]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        acc[r][0] *= (mk[r].x >= 0.f ? 1.f : 0.f); acc[r][1] *= (mk[r].y >= 0.f ? 1.f : 0.f);
+        acc[r][2] *= (mk[r].z >= 0.f ? 1.f : 0.f); acc[r][3] *= (mk[r].w >= 0.f ? 1.f : 0.f);
+      }
+    }
+    if (beta != 0.0f) {
+      float4 cc[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) cc[r] = ld4g(C + at[r]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        acc[r][0] = beta * cc[r].x + acc[r][0]; acc[r][1] = beta * cc[r].y + acc[r][1];
+        acc[r][2] = beta * cc[r].z + acc[r][2]; acc[r][3] = beta * cc[r].w + acc[r][3];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (m + r >= rows) break;
+      float4 v = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+      if (bias) { v.x += bi.x; v.y += bi.y; v.z += bi.z; v.w += bi.w; }
+      if (pre_act) st4g(pre_act + at[r], v);
+      if (relu) {
+        v.x = (v.x >= 0.f ? 1.f : 0.f) * v.x; v.y = (v.y >= 0.f ? 1.f : 0.f) * v.y;
+        v.z = (v.z >= 0.f ? 1.f : 0.f) * v.z; v.w = (v.w >= 0.f ? 1.f : 0.f) * v.w;
+      }
+      st4g(C + at[r], v);
+    }
+  }
+}
+
+constexpr int NARROW_K_CHUNK = 1024;  // most k a workgroup of the narrow-N kernel covers (its slice of B sits in LDS)
+
+// dst = A^T * B over the k range of this workgroup (blockIdx.y), A stored K x M, B stored K x N.
+// U = loads of A in flight per lane.
+template <int NP, int U>
+__global__ __launch_bounds__(1024) void gemm_narrow_n_kernel(size_t M, int N, size_t K, const float* __restrict__ A,
+                                                             const float* __restrict__ B, float* __restrict__ dst,
+                                                             size_t k_chunk) {
+  // first the workgroup's slice of B, [k][NP] with zeros beyond N and beyond the slice's end: all
+  // lanes of a wave read the same row at the same time; then, the k loop done, the partial sums
+  // of the waves: [4][NP * 4][64]
+  __shared__ __attribute__((aligned(16))) float sh[NARROW_K_CHUNK * NP];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const size_t m = ((size_t)blockIdx.x * 64 + lane) * 4;
+  const bool active = m < M;
+  const size_t mc = active ? m : 0;
+  const size_t kbeg = (size_t)blockIdx.y * k_chunk;
+  const size_t kend = kbeg + k_chunk < K ? kbeg + k_chunk : K;
+  const int klen = (int)(kend - kbeg);
+  const int kpad = (klen + 16 * U - 1) / (16 * U) * (16 * U);  // whole passes: the rows beyond klen are zero
+  for (int idx = threadIdx.x; idx < kpad * NP; idx += 1024) {
+    const int k = idx / NP, n = idx % NP;
+    sh[idx] = (k < klen && n < N) ? B[(kbeg + k) * (size_t)N + n] : 0.0f;
+  }
+  __syncthreads();
+  float acc[NP][4];
+#pragma unroll
+  for (int n = 0; n < NP; ++n)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[n][q] = 0.0f;
+  // the sixteen waves take passes of U consecutive k in turn
+  for (int k0 = U * w; k0 < klen; k0 += 16 * U) {
+    float4 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k0 + u < klen ? k0 + u : klen - 1;  // past the end: any row, its B row is zero
+      a[u] = ld4s(A + (kbeg + kk) * M + mc);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int n = 0; n < NP; ++n) {
+        const float bv = sh[(k0 + u) * NP + n];
+        acc[n][0] = __builtin_fmaf(a[u].x, bv, acc[n][0]);
+        acc[n][1] = __builtin_fmaf(a[u].y, bv, acc[n][1]);
+        acc[n][2] = __builtin_fmaf(a[u].z, bv, acc[n][2]);
+        acc[n][3] = __builtin_fmaf(a[u].w, bv, acc[n][3]);
+      }
+    }
+  }
+  __syncthreads();  // B is done with: its memory takes the partial sums
+  float (*red)[NP * 4][64] = reinterpret_cast<float (*)[NP * 4][64]>(sh);
+  // Sixteen partial sums per output -> one, in a fixed order: waves 4j..4j+3 (j = 1, 2, 3) hand
+  // theirs to waves 0..3 in three rounds, then waves 1..3 hand theirs to wave 0.
+  for (int j = 1; j < 4; ++j) {
+    if ((w >> 2) == j) {
+#pragma unroll
+      for (int n = 0; n < NP; ++n)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) red[w & 3][n * 4 + q][lane] = acc[n][q];
+    }
+    __syncthreads();
+    if (w < 4) {
+#pragma unroll
+      for (int n = 0; n < NP; ++n)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[n][q] += red[w][n * 4 + q][lane];
+    }
+    __syncthreads();
+  }
+  if (w >= 1 && w < 4) {
+#pragma unroll
+    for (int n = 0; n < NP; ++n)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) red[w][n * 4 + q][lane] = acc[n][q];
+  }
+  __syncthreads();
+  if (w != 0 || !active) return;
+  float* out = dst + (size_t)blockIdx.y * M * (size_t)N + m * (size_t)N;
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int n = 0; n < NP; ++n)
+      if (n < N) out[(size_t)q * N + n] = ((acc[n][q] + red[1][n * 4 + q][lane]) + red[2][n * 4 + q][lane]) + red[3][n * 4 + q][lane];
+}
+
+// Returns 1 if a skinny kernel took the product (then *rc is its result), 0 if the caller should go on.
+// g carries the operands and the epilogue; g.splits is set for the caller's split-K combine.
+int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
+  const size_t M = g.M, N = g.N, K = g.K;
+  auto ok16 = [](const void* p) { return p == nullptr || aligned16(p); };
+  // short K: the result is the large side
+  if (K <= SHORT_K_MAX && N % 4 == 0 && N >= 64 && M * N >= (size_t(1) << 18) && aligned16(g.C) && ok16(g.mask) && ok16(g.pre_act) &&
+      ok16(g.bias) && aligned16(g.B)) {
+    const size_t gx = (N / 4 + 255) / 256;
+    // rows per workgroup: 64 (what its LDS holds; B's block is fetched once per workgroup) down to 16
+    // while that leaves fewer than two workgroups per CU
+    size_t rpb = SHORT_K_ROWS;
+    while (rpb > 16 && (M + rpb - 1) / rpb * gx < (size_t)ctx->num_cu * 2) rpb /= 2;
+    if ((M + rpb - 1) / rpb > 65535) return 0;
+    const dim3 grid((unsigned)gx, (unsigned)((M + rpb - 1) / rpb));
+#define SL_SK2(KP_, TA_, TB_)                                                                                         \
+  hipLaunchKernelGGL((gemm_short_k_kernel<KP_, TA_, TB_>), grid, dim3(256), 0, ctx->stream, M, N, (int)K, g.A, g.B, g.C, \
+                     g.beta, g.bias, g.relu, g.pre_act, g.mask, (unsigned)rpb)
+#define SL_SK(KP_)                       \
+  do {                                   \
+    if (!ta && !tb) SL_SK2(KP_, false, false); \
+    else if (!ta && tb) SL_SK2(KP_, false, true);  \
+    else if (ta && !tb) SL_SK2(KP_, true, false);  \
+    else SL_SK2(KP_, true, true);        \
+  } while (0)
+    if (K <= 4) SL_SK(4);
+    else if (K <= 8) SL_SK(8);
+    else SL_SK(12);
+#undef SL_SK
+#undef SL_SK2
+    *rc = post_launch();
+    return 1;
+  }
+  // narrow N: A (K x M) is the large side
+  if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22) && aligned16(g.A)) {
+    const size_t gx = (M / 4 + 63) / 64;
+    const size_t mn_bytes = M * N * sizeof(float);
+    // K splits: about one workgroup of sixteen waves per CU, each wave at least four passes of eight
+    // k, a workgroup at most NARROW_K_CHUNK k
+    size_t splits = ((size_t)ctx->num_cu + gx - 1) / gx;
+    const size_t most = K / 512;  // K >= 512 here
+    if (splits > most) splits = most;
+    if (splits < (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK) splits = (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK;
+    if (splits > 65535 || splits > ctx->workspace_bytes / mn_bytes) return 0;
+    size_t k_chunk = ((K + splits - 1) / splits + 127) / 128 * 128;
+    splits = (K + k_chunk - 1) / k_chunk;
+    const bool plain = splits == 1 && g.beta == 0.0f && !g.bias && !g.relu && !g.pre_act && !g.mask;
+    float* dst = plain ? g.C : g.partial;
+    const dim3 grid((unsigned)gx, (unsigned)splits);
+#define SL_NN(NP_, U_) \
+  hipLaunchKernelGGL((gemm_narrow_n_kernel<NP_, U_>), grid, dim3(1024), 0, ctx->stream, M, (int)N, K, g.A, g.B, dst, k_chunk)
+    if (N <= 4) SL_NN(4, 8);
+    else if (N <= 8) SL_NN(8, 8);
+    else if (N <= 12) SL_NN(12, 8);
+    else SL_NN(16, 4);
+#undef SL_NN
+    *rc = post_launch();
+    g.splits = plain ? 1 : (unsigned)splits;
+    g.k_chunk = k_chunk;
+    return plain || *rc ? 1 : 2;  // 2: partials are in the workspace, the caller combines them
+  }
+  return 0;
+}
+
+}  // namespace slhip

@@ -417,6 +417,10 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 }
 
 // Launches the spread-tail kernel and its fix-up (gemm_spread.hip).
+// gemm_skinny.hip: K <= 12, or A^T * B with N <= 16.  Returns 0 (not taken), 1 (done, *rc holds the
+// result) or 2 (partials of g.splits k ranges are in the workspace: the caller combines them).
+int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc);
+
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
                            const SpreadArgs& sp, size_t workers, size_t tail_tiles);
 

@@ -147,6 +147,42 @@ def test_gemm_spread_tail(hip, orc):
         hip.gemm_tail_policy(hip.TAIL_AUTO)
 
 
+def test_gemm_skinny_kernels(hip, orc):
+    """K <= 12 with a large result (vector-ALU kernel, rows of A staged in LDS) in all four forms with
+    every epilogue, and A^T * B with N <= 16 and a long K (A streamed once, k split over workgroups
+    and waves, partials combined in a fixed order)."""
+    for (m, n, k, ta, tb) in [(1031, 260, 10, 0, 1), (4100, 64, 1, 0, 0), (1500, 512, 12, 1, 0), (2050, 1028, 7, 1, 1),
+                              (8192, 2048, 10, 0, 1), (3000, 96, 4, 0, 1), (1111, 256, 9, 0, 0), (1024, 1024, 5, 0, 1),
+                              (1400, 200, 11, 0, 1), (1400, 200, 8, 1, 1)]:
+        say("short-K gemm", m, n, k, ta, tb)
+        a, b = gemm_operands(ta, tb, m, n, k)
+        exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+        got = hip.sgemm(ta, tb, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+        assert np.array_equal(hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre, c=c0.copy(), beta=1.0),
+                              c0 + np.where(pre >= 0, got, 0 * got))
+        if not ta and not tb:
+            bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+            out, pre_act = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+            pre_ref = orc.add_row(m, n, got, bias)
+            assert np.array_equal(pre_act, pre_ref)
+            assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+    for (m, n, k) in [(2048, 10, 8192), (1028, 1, 4133), (1028, 3, 4133), (4100, 4, 1000), (4100, 13, 1030), (1024, 16, 5000),
+                      (260, 8, 20000), (5000, 12, 900), (2052, 5, 2048), (1024, 9, 70000)]:
+        say("narrow-N gemm", m, n, k)
+        a, b = gemm_operands(1, 0, m, n, k)
+        exact, bound = gemm_bound(1, 0, m, n, k, a, b)
+        got = hip.sgemm(1, 0, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        assert np.array_equal(got, hip.sgemm(1, 0, m, n, k, a, b))          # same plan, same order of sums
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(1, 0, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+
+
 def test_gemm_small_tile(hip, orc):
     # 64 x 64 tiles (chosen by the cost model for products of a few hundred such tiles), forced here
     # so that edge tiles, rows of odd length, k remainders and the fused epilogues all run on them
