@@ -28,10 +28,10 @@ sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # HBM-side bytes of one 4096^3 A*B launch, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
-# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (656368.1 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
+# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (650615.9 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
-GEMM_4096_TRAFFIC_BYTES = int((656368.1 * 2.0 + 65536.0) * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((650615.9 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 
@@ -184,6 +184,12 @@ def bench_bandwidth_suite(ctx, steps, warmup):
     bb, cc, dd = ctx.uniform(n, -10, 10, 2, SEED), ctx.uniform(n, -10, 10, 3, SEED), ctx.uniform(n, -10, 10, 4, SEED)
     w, e = timed(ctx, lambda: ctx.call("slhip_ew_chain", n, x.ptr, bb.ptr, cc.ptr, dd.ptr, y.ptr), steps, warmup)
     out.append(bw_entry("ew_chain ((a+b)*c-d)^2^2 [2^28]", 20 * n, w, e)); log(out[-1])
+    # the classifier's last layer (config 5): products with a side of 10, bound by HBM rather than by the
+    # matrix cores; bytes = both operands and the result, each moved once
+    for m_, n_, k_, ta, tb, what in [(8192, 2048, 10, 0, 1, "A*Bt"), (2048, 10, 8192, 1, 0, "At*B"), (8192, 10, 2048, 0, 0, "A*B")]:
+        a_, b_, c_ = x.view(0, m_ * k_), x.view(m_ * k_, k_ * n_), y.view(0, m_ * n_)
+        w, e = timed(ctx, lambda: ctx.call("slhip_sgemm", ta, tb, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), steps, warmup)
+        out.append(bw_entry("gemm %s [%dx%dx%d]" % (what, m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_), w, e)); log(out[-1])
     w, e = timed(ctx, lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n), steps, warmup)
     out.append(bw_entry("device copy [1 GiB] (achievable line)", 8 * n, w, e)); log(out[-1])
     for b in (x, y, bb, cc, dd, vec_c, vec_r, one):
