@@ -47,20 +47,26 @@ inline void check(int32_t rc, const char* what) {
 class HIP;
 
 // A recorded op sequence (see HIP::record): run() replays it as one launch.
+class HIP;
 class Graph {
  public:
   Graph() = default;
-  Graph(slhip_ctx* ctx, slhip_graph* g) : ctx_(ctx), g_(g) {}
-  Graph(Graph&& o) noexcept : ctx_(o.ctx_), g_(o.g_) { o.g_ = nullptr; }
+  Graph(HIP* dev, slhip_ctx* ctx, slhip_graph* g, std::vector<uint64_t> seeds)
+      : dev_(dev), ctx_(ctx), g_(g), seeds_(std::move(seeds)) {}
+  Graph(Graph&& o) noexcept : dev_(o.dev_), ctx_(o.ctx_), g_(o.g_), seeds_(std::move(o.seeds_)) { o.g_ = nullptr; }
   Graph& operator=(Graph&& o) noexcept {
-    if (this != &o) { slhip_graph_destroy(g_); ctx_ = o.ctx_; g_ = o.g_; o.g_ = nullptr; }
+    if (this != &o) {
+      slhip_graph_destroy(g_);
+      dev_ = o.dev_; ctx_ = o.ctx_; g_ = o.g_; seeds_ = std::move(o.seeds_);
+      o.g_ = nullptr;
+    }
     return *this;
   }
   Graph(const Graph&) = delete;
   Graph& operator=(const Graph&) = delete;
   ~Graph() { slhip_graph_destroy(g_); }
   bool valid() const { return g_ != nullptr; }
-  void run() const { check(slhip_graph_launch(ctx_, g_), "slhip_graph_launch"); }
+  inline void run() const;
   size_t nodes() const {
     size_t n = 0;
     check(slhip_graph_node_count(g_, &n), "slhip_graph_node_count");
@@ -68,8 +74,10 @@ class Graph {
   }
 
  private:
+  HIP* dev_ = nullptr;
   slhip_ctx* ctx_ = nullptr;
   slhip_graph* g_ = nullptr;
+  std::vector<uint64_t> seeds_;  // seed gradients whose fill with ones backward() left out of the recording
 };
 
 struct Buffer {
@@ -206,16 +214,41 @@ class HIP {
   Graph record(F&& body) {
     check(slhip_graph_begin(ctx_), "slhip_graph_begin");
     slhip_graph* g = nullptr;
+    recording_ = true;
+    recorded_seeds_.clear();
     try {
       body();
     } catch (...) {
+      recording_ = false;
       slhip_graph_end(ctx_, &g);
       slhip_graph_destroy(g);
       tape_.clear();
       throw;
     }
+    recording_ = false;
     check(slhip_graph_end(ctx_, &g), "slhip_graph_end");
-    return Graph(ctx_, g);
+    return Graph(this, ctx_, g, std::move(recorded_seeds_));
+  }
+  // What a replay relies on without recording it: the host-side bookkeeping of zero_grad() and
+  // backward() ran when the step was recorded, not now.  Every fill that is pending on the host
+  // runs here, and every seed gradient whose fill the recording left out holds its ones again.
+  // In a loop that replays the same recording this finds nothing to do from the second replay on.
+  void before_replay(const std::vector<uint64_t>& seeds) {
+    for (uint64_t id : seeds) {
+      auto it = allocs_.find(id);
+      if (it == allocs_.end()) continue;
+      stale_.erase(id);
+      if (!ones_.count(id)) {
+        check(slhip_fill(ctx_, it->second.len, 1.0f, it->second.ptr), "slhip_fill");
+        ones_.insert(id);
+      }
+    }
+    const std::vector<uint64_t> pending(stale_.begin(), stale_.end());
+    for (uint64_t id : pending) {
+      auto it = allocs_.find(id);
+      if (it != allocs_.end()) settle(it->second);
+    }
+    stale_.clear();
   }
 
   // ---- autograd --------------------------------------------------------------------------
@@ -288,6 +321,7 @@ class HIP {
     const bool still_ones = ones_.count(g.id) != 0;
     stale_.erase(g.id);
     if (!still_ones) check(slhip_fill(ctx_, g.len, 1.0f, g.ptr), "slhip_fill");
+    else if (recording_) recorded_seeds_.push_back(g.id);
     ones_.insert(g.id);
     run_tape();
   }
@@ -653,6 +687,8 @@ class HIP {
   std::vector<Slab> slabs_;
   std::vector<std::function<void()>> tape_;
   std::unordered_map<uint64_t, uint64_t> relu_pre_;   // ReLU output of a fused Linear on the tape -> its pre-activation
+  bool recording_ = false;                            // inside record(): ops land in a graph
+  std::vector<uint64_t> recorded_seeds_;              // seed gradients the current recording relies on
   std::unordered_set<uint64_t> lazy_;                 // gradients in the slabs that zero_grad() marks instead of filling
   std::unordered_set<uint64_t> ones_;                 // gradients known to hold nothing but 1.0 (backward()'s seed)
   std::unordered_set<uint64_t> stale_;                // large gradients with a zero fill pending since zero_grad()
@@ -673,6 +709,10 @@ inline void Buffer::write(const float* host, size_t n) const {
   if (n != len) throw Error("write: length differs");
   dev->drop_pending_zero(*this);
   check(slhip_memcpy_h2d(dev->ctx(), ptr, host, len * sizeof(float)), "slhip_memcpy_h2d");
+}
+inline void Graph::run() const {
+  dev_->before_replay(seeds_);
+  check(slhip_graph_launch(ctx_, g_), "slhip_graph_launch");
 }
 inline Buffer Buffer::grad() const { return dev->grad(*this); }
 inline void Buffer::backward() const { dev->backward(*this); }
