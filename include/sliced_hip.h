@@ -276,6 +276,24 @@ int32_t slhip_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* pr
                        float* grad);
 int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* out);
 
+/* The ReLU mask of a fused Linear as one bit per element, packed 32 columns to a word, row-major
+ * [m][ceil(n / 32)] (bit c % 32 of word c / 32 of a row = pre-activation >= 0).  The backward pass
+ * of the reference needs the pre-activations only for that comparison (relu gradient
+ * src/matrix.rs:190-199; examples/sine_net.rs:32-40 chains gemm -> add_row_mut -> relu), so the
+ * pair below moves 1/32 of the bytes slhip_linear_fwd's pre_act and slhip_sgemm_relu_mask's pre do.
+ * slhip_linear_fwd_bits : out = relu(x·w + bias), bits = (x·w + bias >= 0); bias may be NULL.
+ * slhip_sgemm_relu_bits : c = beta*c + (op(a)·op(b)) * bit — what slhip_sgemm_relu_mask computes
+ *   from the float pre-activations, same values.
+ * slhip_relu_grad_bits  : x_grad += bit * out_grad, for a ReLU output that feeds something else
+ *   than a fused Linear.
+ * The two products run one workgroup per 128 x 128 tile of the result without splitting K. */
+int32_t slhip_linear_fwd_bits(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w,
+                              const float* bias, uint32_t* bits, float* out);
+int32_t slhip_sgemm_relu_bits(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
+                              const float* a, const float* b, const uint32_t* bits, float* c, float beta);
+int32_t slhip_relu_grad_bits(slhip_ctx* ctx, size_t rows, size_t cols, const uint32_t* bits, float* x_grad,
+                             const float* out_grad);
+
 /* Fused losses of the two example loops; every reference op they stand for stays available.
  * slhip_mse: loss_dev[0] = (sum_i (x_i - y_i)^2) * (1/n) — the chain sub, squared, sum_cols over one
  *   row, mul by the constant 1/n (loss tape of examples/sine_net.rs:150-156 summed on the device).

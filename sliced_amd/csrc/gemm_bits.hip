@@ -1,0 +1,213 @@
+// The ReLU mask as one bit per element.  A fused Linear's backward needs the pre-activations of
+// the layer below only for their sign; as floats they are written once by the forward pass and
+// read once by the input-gradient GEMM, 4 B each way per element, and that read sits at the very
+// end of a workgroup's life where nothing hides it (35-57 us per 64 MiB at batch 8192).  Here the
+// forward kernel writes the mask (pre >= 0) packed 32 columns to a word, row-major
+// [M][ceil(N / 32)], and the masked GEMM fetches the 128 words of its tile BEFORE its k loop:
+// four registers a lane, no latency left at the end.
+//
+// Both kernels are the 128 x 128 tile kernel of gemm.hip with another epilogue; they live in a
+// file of their own so that the plain kernel's code stays exactly as it is.  One workgroup per
+// tile, no K split: meant for outputs of a few hundred tiles and more (the caller decides).
+// A masked product with K <= 12 goes to the short-K vector kernel (gemm_skinny.hip) instead.
+//
+// Packing.  In accumulator block (i, j) of a wave, register v of lane (r, h) is row
+// 8*(v/4) + 4*h + v%4 and column r of a 32 x 32 block: a wave-wide ballot of one register is the
+// mask word of two rows (low half: h = 0, high half: h = 1).  Lane L < 32 keeps the word of row L
+// of the block, so a block's words leave (and arrive) as one access of 32 lanes.
+#include "gemm_tile.hpp"
+
+namespace slhip {
+
+__host__ __device__ constexpr int bits_row_of(int v, int h) { return 8 * (v / 4) + 4 * h + v % 4; }
+
+template <bool TA, bool TB, bool ONLY_FAST>
+__global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uint32_t* __restrict__ bits_in,
+                                                           uint32_t* __restrict__ bits_out, size_t W) {
+  constexpr int BK = GEMM_BK;
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<BK, 128>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 128>::STAGE_FLOATS];
+  unsigned tm, tn;
+  tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+  const size_t m0 = (size_t)tm * 128, n0 = (size_t)tn * 128;
+  const int ktiles = (int)((g.K + BK - 1) / BK);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int r = lane & 31, h = lane >> 5;
+
+  // the tile's mask words, in flight during the k loop
+  uint32_t mw[2][2] = {{0u, 0u}, {0u, 0u}};
+  if (bits_in) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const size_t row = m0 + wm * 64 + 32 * i + r, cw = (n0 + wn * 64 + 32 * j) >> 5;
+        if (h == 0 && row < g.M && cw < W) mw[i][j] = bits_in[row * W + cw];
+      }
+  }
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+  gemm_k_range<TA, TB, BK, ONLY_FAST, 2, 2>(g, 0, ktiles, 0, g.K, m0, n0, lds_a, lds_b, acc);
+
+  // every read (mask words, C for beta) before the first store
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const size_t col = n0 + wn * 64 + 32 * j + r;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float val = acc[i][j][v];
+        if (bits_in) {
+          const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)mw[i][j], bits_row_of(v, 0));
+          const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)mw[i][j], bits_row_of(v, 1));
+          val = ((((h ? hi : lo) >> r) & 1u) ? 1.0f : 0.0f) * val;
+        }
+        if (g.beta != 0.0f) {
+          const size_t row = m0 + wm * 64 + 32 * i + bits_row_of(v, h);
+          if (row < g.M && col < g.N) val = g.beta * g.C[row * g.N + col] + val;
+        }
+        acc[i][j][v] = val;
+      }
+    }
+  float bias_of[2] = {0.0f, 0.0f};
+  if (g.bias) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const size_t col = n0 + wn * 64 + 32 * j + r;
+      if (col < g.N) bias_of[j] = g.bias[col];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const size_t col = n0 + wn * 64 + 32 * j + r;
+      const bool cin = col < g.N;
+      const float bias = bias_of[j];
+      uint32_t word = 0u;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float val = acc[i][j][v];
+        if (g.bias) val = val + bias;
+        if (bits_out) {
+          const unsigned long long b = __ballot(val >= 0.0f && cin);
+          if (lane == bits_row_of(v, 0)) word = (uint32_t)b;
+          if (lane == bits_row_of(v, 1)) word = (uint32_t)(b >> 32);
+        }
+        if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
+        const size_t row = m0 + wm * 64 + 32 * i + bits_row_of(v, h);
+        if (row < g.M && cin) g.C[row * g.N + col] = val;
+      }
+      if (bits_out) {
+        const size_t row = m0 + wm * 64 + 32 * i + r, cw = (n0 + wn * 64 + 32 * j) >> 5;
+        if (h == 0 && row < g.M && cw < W) bits_out[row * W + cw] = word;
+      }
+    }
+}
+
+// x_grad += bit * out_grad: the ReLU gradient (src/matrix.rs:190-199) from the packed mask.
+__global__ __launch_bounds__(256) void relu_grad_bits_kernel(size_t rows, size_t cols, size_t W, const uint32_t* __restrict__ bits,
+                                                             float* x_grad, const float* __restrict__ out_grad) {
+  const size_t n = rows * cols;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    const size_t row = i / cols, col = i - row * cols;
+    const uint32_t bit = (bits[row * W + (col >> 5)] >> (col & 31)) & 1u;
+    x_grad[i] = x_grad[i] + (bit ? 1.0f : 0.0f) * out_grad[i];
+  }
+}
+
+static int32_t gemm_bits_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
+                             float* C, float beta, const float* bias, int relu, const uint32_t* bits_in, uint32_t* bits_out) {
+  GemmArgs g;
+  g.M = M; g.N = N; g.K = K; g.A = A; g.B = B; g.C = C; g.beta = beta;
+  g.bias = bias; g.relu = relu; g.pre_act = nullptr; g.mask = nullptr;
+  const size_t lda = ta ? M : K, ldb = tb ? K : N;
+  g.a_vec = lda % 4 == 0;
+  g.b_vec = ldb % 4 == 0;
+  g.m_fast = (aligned16(A) && aligned16(B)) ? M : 0;
+  g.partial = nullptr;
+  const size_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  if (tiles_m * tiles_n > 0x7fffffffu) {
+    set_error("gemm with bit mask: %zu x %zu tiles exceed one launch", tiles_m, tiles_n);
+    return SLHIP_EINVAL;
+  }
+  g.tiles_m = (unsigned)tiles_m; g.tiles_n = (unsigned)tiles_n;
+  g.splits = 1;
+  g.k_chunk = (K + GEMM_BK - 1) / GEMM_BK * GEMM_BK;
+  if (bits_in && !bits_out) {  // K <= 12: HBM-bound, the vector kernel reads the same words (8192 x 2048 x 10: 32 -> 16 us)
+    int32_t rc = SLHIP_OK;
+    if (gemm_short_k_launch(ctx, ta, tb, g, bits_in, &rc)) return rc;
+  }
+  const size_t W = (N + 31) / 32;
+  const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % BM == 0 && N % BN == 0 && K % GEMM_BK == 0;
+  const dim3 grid((unsigned)(tiles_m * tiles_n));
+#define SL_GB(TA_, TB_)                                                                                                      \
+  do {                                                                                                                       \
+    if (only_fast) hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, true>), grid, dim3(256), 0, ctx->stream, g, bits_in, bits_out, W); \
+    else hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, false>), grid, dim3(256), 0, ctx->stream, g, bits_in, bits_out, W);  \
+  } while (0)
+  if (!ta && !tb) SL_GB(false, false);
+  else if (!ta && tb) SL_GB(false, true);
+  else if (ta && !tb) SL_GB(true, false);
+  else SL_GB(true, true);
+#undef SL_GB
+  return post_launch();
+}
+
+static bool overlaps_bytes(const void* a, size_t na, const void* b, size_t nb) {
+  const char* p = (const char*)a;
+  const char* q = (const char*)b;
+  return p < q + nb && q < p + na;
+}
+
+}  // namespace slhip
+
+using namespace slhip;
+
+SLHIP_API int32_t slhip_linear_fwd_bits(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w,
+                                        const float* bias, uint32_t* bits, float* out) {
+  size_t mk, kn, mn;
+  SLHIP_REQUIRE(ctx && x && w && bits && out, "null argument");
+  SLHIP_REQUIRE(checked_len(m, k, &mk) && checked_len(k, n, &kn) && checked_len(m, n, &mn), "bad dims");
+  const size_t words = m * ((n + 31) / 32);
+  if (overlaps_bytes(out, mn * 4, x, mk * 4) || overlaps_bytes(out, mn * 4, w, kn * 4) || overlaps_bytes(bits, words * 4, out, mn * 4) ||
+      overlaps_bytes(bits, words * 4, x, mk * 4) || overlaps_bytes(bits, words * 4, w, kn * 4)) {
+    set_error("slhip_linear_fwd_bits: an output overlaps another operand");
+    return SLHIP_EALIAS;
+  }
+  return gemm_bits_run(ctx, false, false, m, n, k, x, w, out, 0.0f, bias, 1, nullptr, bits);
+}
+
+SLHIP_API int32_t slhip_sgemm_relu_bits(slhip_ctx* ctx, int32_t trans_a, int32_t trans_b, size_t m, size_t n, size_t k,
+                                        const float* a, const float* b, const uint32_t* bits, float* c, float beta) {
+  size_t mk, kn, mn;
+  SLHIP_REQUIRE(ctx && a && b && c && bits, "null argument");
+  SLHIP_REQUIRE(checked_len(m, k, &mk) && checked_len(k, n, &kn) && checked_len(m, n, &mn), "bad dims");
+  const size_t words = m * ((n + 31) / 32);
+  if (overlaps_bytes(c, mn * 4, a, mk * 4) || overlaps_bytes(c, mn * 4, b, kn * 4) || overlaps_bytes(c, mn * 4, bits, words * 4)) {
+    set_error("slhip_sgemm_relu_bits: C overlaps an input");
+    return SLHIP_EALIAS;
+  }
+  return gemm_bits_run(ctx, trans_a != 0, trans_b != 0, m, n, k, a, b, c, beta, nullptr, 0, bits, nullptr);
+}
+
+SLHIP_API int32_t slhip_relu_grad_bits(slhip_ctx* ctx, size_t rows, size_t cols, const uint32_t* bits, float* x_grad,
+                                       const float* out_grad) {
+  size_t len;
+  SLHIP_REQUIRE(ctx && bits && x_grad && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  size_t blocks = (len + 255) / 256;
+  const size_t cap = (size_t)ctx->num_cu * 32;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(relu_grad_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, (cols + 31) / 32, bits,
+                     x_grad, out_grad);
+  return post_launch();
+}

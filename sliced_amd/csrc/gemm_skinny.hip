@@ -29,7 +29,8 @@ template <int KP, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_short_k_kernel(size_t M, size_t N, int K, const float* __restrict__ A,
                                                            const float* __restrict__ B, float* C, float beta,
                                                            const float* __restrict__ bias, int relu, float* pre_act,
-                                                           const float* mask, unsigned rows_per_block) {
+                                                           const float* mask, const uint32_t* __restrict__ bits,
+                                                           unsigned rows_per_block) {
   // The rows of A this workgroup uses, zero-padded to KP columns: every lane of a wave reads the
   // same row at the same time (one broadcast ds_read_b128 per four k).  Fetching them with
   // wave-uniform global loads instead costs K load instructions per row and store.
@@ -89,11 +90,12 @@ __global__ __launch_bounds__(256) void gemm_short_k_kernel(size_t M, size_t N, i
   constexpr int R = 4;  // rows per pass: their mask / C reads are in flight together
   for (int m = 0; m < rows; m += R) {
     float acc[R][4];
-    size_t at[R];
+    size_t at[R], row[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int lr = m + r < rows ? m + r : rows - 1;  // a pass past the end repeats the last row and does not store it
-      at[r] = (m0 + lr) * N + n;
+      row[r] = m0 + lr;
+      at[r] = row[r] * N + n;
 #pragma unroll
       for (int q = 0; q < 4; ++q) acc[r][q] = 0.0f;
 #pragma unroll
@@ -112,6 +114,18 @@ __global__ __launch_bounds__(256) void gemm_short_k_kernel(size_t M, size_t N, i
       for (int r = 0; r < R; ++r) {
         acc[r][0] *= (mk[r].x >= 0.f ? 1.f : 0.f); acc[r][1] *= (mk[r].y >= 0.f ? 1.f : 0.f);
         acc[r][2] *= (mk[r].z >= 0.f ? 1.f : 0.f); acc[r][3] *= (mk[r].w >= 0.f ? 1.f : 0.f);
+      }
+    }
+    if (bits) {  // the mask packed 32 columns to a word, row-major: the thread's four columns share a word
+      const size_t W = (N + 31) >> 5;
+      uint32_t mk[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) mk[r] = bits[row[r] * W + (n >> 5)];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t four = mk[r] >> (n & 31);
+        acc[r][0] *= ((four & 1u) ? 1.f : 0.f); acc[r][1] *= ((four & 2u) ? 1.f : 0.f);
+        acc[r][2] *= ((four & 4u) ? 1.f : 0.f); acc[r][3] *= ((four & 8u) ? 1.f : 0.f);
       }
     }
     if (beta != 0.0f) {
@@ -227,22 +241,23 @@ __global__ __launch_bounds__(1024) void gemm_narrow_n_kernel(size_t M, int N, si
 
 // Returns 1 if a skinny kernel took the product (then *rc is its result), 0 if the caller should go on.
 // g carries the operands and the epilogue; g.splits is set for the caller's split-K combine.
-int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
+// The short-K kernel if the product qualifies (returns 1, *rc = launch status), else 0.
+int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const uint32_t* bits, int32_t* rc) {
   const size_t M = g.M, N = g.N, K = g.K;
   auto ok16 = [](const void* p) { return p == nullptr || aligned16(p); };
-  // short K: the result is the large side
-  if (K <= SHORT_K_MAX && N % 4 == 0 && N >= 64 && M * N >= (size_t(1) << 18) && aligned16(g.C) && ok16(g.mask) && ok16(g.pre_act) &&
-      ok16(g.bias) && aligned16(g.B)) {
-    const size_t gx = (N / 4 + 255) / 256;
-    // rows per workgroup: 64 (what its LDS holds; B's block is fetched once per workgroup) down to 16
-    // while that leaves fewer than two workgroups per CU
-    size_t rpb = SHORT_K_ROWS;
-    while (rpb > 16 && (M + rpb - 1) / rpb * gx < (size_t)ctx->num_cu * 2) rpb /= 2;
-    if ((M + rpb - 1) / rpb > 65535) return 0;
-    const dim3 grid((unsigned)gx, (unsigned)((M + rpb - 1) / rpb));
+  if (!(K <= SHORT_K_MAX && N % 4 == 0 && N >= 64 && M * N >= (size_t(1) << 18) && aligned16(g.C) && ok16(g.mask) &&
+        ok16(g.pre_act) && ok16(g.bias) && aligned16(g.B)))
+    return 0;
+  const size_t gx = (N / 4 + 255) / 256;
+  // rows per workgroup: 64 (what its LDS holds; B's block is fetched once per workgroup) down to 16
+  // while that leaves fewer than two workgroups per CU
+  size_t rpb = SHORT_K_ROWS;
+  while (rpb > 16 && (M + rpb - 1) / rpb * gx < (size_t)ctx->num_cu * 2) rpb /= 2;
+  if ((M + rpb - 1) / rpb > 65535) return 0;
+  const dim3 grid((unsigned)gx, (unsigned)((M + rpb - 1) / rpb));
 #define SL_SK2(KP_, TA_, TB_)                                                                                         \
   hipLaunchKernelGGL((gemm_short_k_kernel<KP_, TA_, TB_>), grid, dim3(256), 0, ctx->stream, M, N, (int)K, g.A, g.B, g.C, \
-                     g.beta, g.bias, g.relu, g.pre_act, g.mask, (unsigned)rpb)
+                     g.beta, g.bias, g.relu, g.pre_act, g.mask, bits, (unsigned)rpb)
 #define SL_SK(KP_)                       \
   do {                                   \
     if (!ta && !tb) SL_SK2(KP_, false, false); \
@@ -250,14 +265,19 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
     else if (ta && !tb) SL_SK2(KP_, true, false);  \
     else SL_SK2(KP_, true, true);        \
   } while (0)
-    if (K <= 4) SL_SK(4);
-    else if (K <= 8) SL_SK(8);
-    else SL_SK(12);
+  if (K <= 4) SL_SK(4);
+  else if (K <= 8) SL_SK(8);
+  else SL_SK(12);
 #undef SL_SK
 #undef SL_SK2
-    *rc = post_launch();
-    return 1;
-  }
+  *rc = post_launch();
+  return 1;
+}
+
+int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
+  const size_t M = g.M, N = g.N, K = g.K;
+  // short K: the result is the large side
+  if (gemm_short_k_launch(ctx, ta, tb, g, nullptr, rc)) return 1;
   // narrow N: A (K x M) is the large side
   if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22) && aligned16(g.A)) {
     const size_t gx = (M / 4 + 63) / 64;

@@ -40,6 +40,9 @@ SLH_API int slh_set_grad_policy(void* dev, float gemm_beta, float softmax_beta, 
 SLH_API int slh_set_fuse_relu_grad(void* dev, int on) {
   return guard([&] { ((HIP*)dev)->policy.fuse_relu_grad = on != 0; });
 }
+SLH_API int slh_set_relu_bits(void* dev, int on) {
+  return guard([&] { ((HIP*)dev)->policy.relu_bits = on != 0; });
+}
 SLH_API int slh_buffer_from(void* dev, const float* host, size_t len, uint64_t* id) {
   return guard([&] { *id = ((HIP*)dev)->from(host, len).id; });
 }

@@ -91,6 +91,7 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
 
   // with the fused Linear the ReLU gradients ride in the next layer's input-gradient GEMM
   dev.policy.fuse_relu_grad = fused;
+  dev.policy.relu_bits = fused;
 
   // One training step.  Reads the loss back unless `deferred`; then `loss_at` names the device
   // scalar that holds it (the same one every step: op outputs are cached by call position).

@@ -107,6 +107,11 @@ struct GradPolicy {
   // one kernel instead of GEMM + elementwise pass, equal values (a zero may change its sign).  Off by
   // default: it is only the sequence the tape would run when that ReLU output feeds nothing else.
   bool fuse_relu_grad = false;
+  // With fuse_relu_grad: a fused Linear + ReLU whose output has 2^22 elements or more keeps the
+  // ReLU mask as one bit per element (slhip_linear_fwd_bits) instead of the pre-activations, and
+  // the consumer's input-gradient GEMM reads those bits (slhip_sgemm_relu_bits): 1/32 of the bytes
+  // both ways, equal values.  The pre-activation buffer then only names the gradient.
+  bool relu_bits = false;
 };
 
 class HIP {
@@ -309,6 +314,7 @@ class HIP {
     for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
     tape_.clear();
     relu_pre_.clear();
+    relu_bits_.clear();
     relu_grad_done_.clear();
   }
   // Seeds out's gradient with ones and runs the tape.  A seed gradient that backward() itself created
@@ -356,10 +362,16 @@ class HIP {
     expect(x, m * k, "linear x"); expect(w, k * n, "linear w"); expect(bias, n, "linear bias");
     Buffer pre = relu ? retrieve(m * n) : Buffer();
     Buffer out = retrieve(m * n);
-    check(slhip_linear_fwd(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, relu ? 1 : 0, relu ? pre.ptr : nullptr, out.ptr),
-          "slhip_linear_fwd");
-    uint64_t xi = x.id, wi = w.id, bi = bias.id, oi = out.id, pi = relu ? pre.id : 0;
+    const bool as_bits = relu && policy.fuse_relu_grad && policy.relu_bits && m * n >= (size_t(1) << 22);
+    Buffer mask = as_bits ? retrieve(m * ((n + 31) / 32)) : Buffer();
+    if (as_bits)
+      check(slhip_linear_fwd_bits(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, (uint32_t*)mask.ptr, out.ptr), "slhip_linear_fwd_bits");
+    else
+      check(slhip_linear_fwd(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, relu ? 1 : 0, relu ? pre.ptr : nullptr, out.ptr),
+            "slhip_linear_fwd");
+    uint64_t xi = x.id, wi = w.id, bi = bias.id, oi = out.id, pi = relu ? pre.id : 0, mi = as_bits ? mask.id : 0;
     if (relu) relu_pre_[oi] = pi;
+    if (as_bits) relu_bits_[oi] = mi;
     add_grad_fn([=] {
       Buffer xb = lookup(xi), wb = lookup(wi), bb = lookup(bi), o = lookup(oi);
       Buffer g;
@@ -367,8 +379,11 @@ class HIP {
         Buffer p = lookup(pi);
         Buffer pg = grad_mut(p);
         relu_pre_.erase(oi);
-        if (!relu_grad_done_.erase(oi))  // else the consumer's backward has written pre.grad already
-          check(slhip_ew_unary_grad(ctx_, SLHIP_RELU, 0.0f, p.len, p.ptr, pg.ptr, grad(o).ptr), "relu grad");
+        relu_bits_.erase(oi);
+        if (!relu_grad_done_.erase(oi)) {  // else the consumer's backward has written pre.grad already
+          if (mi) check(slhip_relu_grad_bits(ctx_, m, n, (const uint32_t*)lookup(mi).ptr, pg.ptr, grad(o).ptr), "relu grad");
+          else check(slhip_ew_unary_grad(ctx_, SLHIP_RELU, 0.0f, p.len, p.ptr, pg.ptr, grad(o).ptr), "relu grad");
+        }
         g = pg;
       } else {
         g = grad(o);
@@ -384,8 +399,14 @@ class HIP {
         Buffer xp = lookup(producer->second);
         // written the way gemm_grad writes x.grad (policy.gemm_beta; SET by default): pre.grad is
         // zero at this point, and `0 + v` differs from `v` only in the sign of a zero
-        check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_out(xp, set).ptr, policy.gemm_beta),
-              "slhip_sgemm_relu_mask");
+        auto packed = relu_bits_.find(xi);
+        if (packed != relu_bits_.end())
+          check(slhip_sgemm_relu_bits(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, (const uint32_t*)lookup(packed->second).ptr,
+                                      grad_out(xp, set).ptr, policy.gemm_beta),
+                "slhip_sgemm_relu_bits");
+        else
+          check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_out(xp, set).ptr, policy.gemm_beta),
+                "slhip_sgemm_relu_mask");
         relu_grad_done_.insert(xi);
       }
       check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
@@ -692,6 +713,7 @@ class HIP {
   std::unordered_set<uint64_t> lazy_;                 // gradients in the slabs that zero_grad() marks instead of filling
   std::unordered_set<uint64_t> ones_;                 // gradients known to hold nothing but 1.0 (backward()'s seed)
   std::unordered_set<uint64_t> stale_;                // large gradients with a zero fill pending since zero_grad()
+  std::unordered_map<uint64_t, uint64_t> relu_bits_;  // ... -> its packed mask, where the forward kept bits instead
   std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
   bool tape_enabled_ = true;
   std::vector<Buffer> cache_;

@@ -115,6 +115,10 @@ class HIP:
     def set_grad_policy(self, gemm_beta=0.0, softmax_beta=0.0, transpose_beta=0.0):
         _ck(lib().slh_set_grad_policy(self.h, _f(gemm_beta), _f(softmax_beta), _f(transpose_beta)))
 
+    def set_relu_bits(self, on):
+        """With set_fuse_relu_grad: large fused Linear + ReLU layers keep their ReLU mask as bits."""
+        _ck(lib().slh_set_relu_bits(self.h, C.c_int(1 if on else 0)))
+
     def set_fuse_relu_grad(self, on):
         """Fused Linear layers write their input gradient through the previous layer's ReLU gradient."""
         _ck(lib().slh_set_fuse_relu_grad(self.h, C.c_int(1 if on else 0)))

@@ -326,6 +326,33 @@ def linear_fwd(m, k, n, x, w, bias, relu=False, want_pre_act=False):
         return do.numpy()
 
 
+def linear_fwd_bits(m, k, n, x, w, bias):
+    """relu(x·w + bias) and the packed mask (x·w + bias >= 0): uint32 [m][ceil(n / 32)]."""
+    words = m * ((n + 31) // 32)
+    with _Scope() as s:
+        dx, dw, db, do, dbits = s.up(x), s.up(w), s.up(bias), s.empty(m * n), s.zeros(words)
+        s.c.call("slhip_linear_fwd_bits", m, k, n, dx.ptr, dw.ptr, _ptr(db), dbits.ptr, do.ptr)
+        return do.numpy(), dbits.numpy().view(np.uint32).reshape(m, -1)
+
+
+def sgemm_relu_bits(ta, tb, m, n, k, a, b, bits, c=None, beta=0.0):
+    """c = beta*c + (op(a)·op(b)) * bit."""
+    with _Scope() as s:
+        da, db = s.up(a), s.up(b)
+        dbits = s.up(np.ascontiguousarray(bits, np.uint32).ravel().view(np.float32))
+        dc = s.up(c) if c is not None else s.empty(m * n)
+        s.c.call("slhip_sgemm_relu_bits", int(ta), int(tb), m, n, k, da.ptr, db.ptr, dbits.ptr, dc.ptr, float(beta))
+        return dc.numpy()
+
+
+def relu_grad_bits(rows, cols, bits, x_grad, out_grad):
+    with _Scope() as s:
+        dbits = s.up(np.ascontiguousarray(bits, np.uint32).ravel().view(np.float32))
+        dx, dg = s.up(x_grad), s.up(out_grad)
+        s.c.call("slhip_relu_grad_bits", rows, cols, dbits.ptr, dx.ptr, dg.ptr)
+        return dx.numpy()
+
+
 # ---- softmax & co ----------------------------------------------------------------------
 def softmax(samples, features, x):
     with _Scope() as s:

@@ -882,3 +882,45 @@ def test_recorded_sequence_replays_like_eager_calls(hip, orc):
     assert lib.slhip_graph_destroy(g) == 0
     for z in (da, dw, db, y, s, col, keep, scratch):
         z.free()
+
+
+def test_relu_mask_as_bits_equals_the_float_mask(hip, orc):
+    """slhip_linear_fwd_bits / slhip_sgemm_relu_bits / slhip_relu_grad_bits against the float forms
+    (linear_fwd with pre-activations, sgemm_relu_mask, the relu gradient): the same values within the
+    GEMM bound, a mask that agrees with the exact pre-activations wherever their sign is not within
+    that bound of zero, and outputs that are zero exactly where the mask is clear."""
+    for (m, k, n) in [(256, 96, 128), (300, 70, 200), (129, 33, 97), (1024, 784, 2048), (520, 64, 36)]:
+        say("bit mask forward", m, k, n)
+        x = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
+        w = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
+        bias = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+        out, bits = hip.linear_fwd_bits(m, k, n, x, w, bias)
+        exact, bound = gemm_bound(0, 0, m, n, k, x, w)
+        pre_ref = exact.reshape(m, n) + bias.astype(np.float64)
+        out = out.reshape(m, n)
+        unpacked = ((bits[:, np.arange(n) // 32] >> (np.arange(n) % 32).astype(np.uint32)) & 1).astype(bool)
+        sure = np.abs(pre_ref) > bound.reshape(m, n) + 1e-6          # sign not in doubt
+        assert np.array_equal(unpacked[sure], (pre_ref >= 0)[sure])
+        assert np.all(np.abs(out - np.where(unpacked, pre_ref, 0)) <= bound.reshape(m, n) + 1e-6)
+        assert np.all(out[~unpacked] == 0) and np.all(out[unpacked] >= 0)
+        if n % 32:                                                    # bits beyond the last column stay clear
+            assert not np.any(bits[:, -1] >> np.uint32(n % 32))
+    for (m, n, k, ta, tb) in [(256, 128, 96, 0, 1), (300, 200, 70, 0, 1), (129, 97, 33, 0, 0), (1024, 2048, 512, 0, 1),
+                              (1031, 260, 10, 0, 1), (4100, 64, 3, 1, 0), (2050, 1028, 7, 1, 1), (700, 512, 12, 0, 0),
+                              (200, 130, 64, 1, 0), (140, 260, 40, 1, 1)]:
+        say("bit mask backward", m, n, k, ta, tb)
+        a, b = gemm_operands(ta, tb, m, n, k)
+        exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        keep = (pre >= 0).reshape(m, n)
+        words = (n + 31) // 32
+        bits = np.zeros((m, words), np.uint32)
+        for c in range(n):
+            bits[:, c // 32] |= keep[:, c].astype(np.uint32) << np.uint32(c % 32)
+        got = hip.sgemm_relu_bits(ta, tb, m, n, k, a, b, bits)
+        assert np.all(np.abs(got - np.where(keep.ravel(), exact, 0)) <= bound)
+        assert np.all(got[~keep.ravel()] == 0)
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_bits(ta, tb, m, n, k, a, b, bits, c=c0.copy(), beta=1.0), c0 + got)
+        g = rng.uniform(m * n, -1, 1, tag=5, seed=SEED)
+        assert np.array_equal(hip.relu_grad_bits(m, n, bits, c0.copy(), g), c0 + np.where(keep.ravel(), g, 0 * g))

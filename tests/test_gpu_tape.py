@@ -384,6 +384,42 @@ def test_relu_grad_fused_into_the_next_layers_input_gradient(device):
         assert np.array_equal(a, c)
 
 
+def test_relu_mask_kept_as_bits_gives_the_same_gradients(device):
+    """Layers of 2^22 outputs and more keep their ReLU mask as bits when the policy allows it: the
+    gradients equal those of the float path up to the order in which the GEMM plans add (the bit
+    kernels run whole tiles unsplit) and the few mask bits that order decides, and a ReLU output that feeds something else than a fused
+    Linear takes the unpacking elementwise gradient."""
+    m, d0, d1, d2, d3 = 2048, 64, 2048, 2080, 10
+    x = rng.uniform(m * d0, -1, 1, tag=0)
+    ws = [rng.uniform(a * b, -0.1, 0.1, tag=10 + i) for i, (a, b) in enumerate([(d0, d1), (d1, d2), (d2, d3)])]
+    bs = [rng.uniform(b, -0.5, 0.5, tag=20 + i) for i, b in enumerate([d1, d2, d3])]
+    res = []
+    try:
+        device.set_fuse_relu_grad(True)
+        for bits in (False, True):
+            device.set_relu_bits(bits)
+            for tail in ("linear", "square"):
+                xb = device.buffer(x)
+                wb = [device.buffer(w) for w in ws]
+                bb = [device.buffer(b) for b in bs]
+                h1 = device.linear(m, d0, d1, xb, wb[0], bb[0], True)
+                h2 = device.linear(m, d1, d2, h1, wb[1], bb[1], True)
+                out = device.linear(m, d2, d3, h2, wb[2], bb[2], False) if tail == "linear" else device.square(h2)
+                out.backward()
+                res.append([out.read(), xb.grad().read()] + [w.grad().read() for w in wb[:2]] + [b.grad().read() for b in bb[:2]])
+    finally:
+        device.set_fuse_relu_grad(False)
+        device.set_relu_bits(False)
+    for ref, got in ((res[0], res[2]), (res[1], res[3])):
+        assert np.abs(ref[1]).max() > 0
+        for a, c in zip(ref, got):
+            # the two paths add in different orders, so a pre-activation within rounding of zero may
+            # land on the other side of it: a handful of mask bits, each worth one term of a sum
+            scale = np.abs(a).max()
+            off = np.abs(a - c) > 1e-3 * scale          # three chained products of K up to 2080: 1e-5 * sqrt(K) each
+            assert off.mean() <= 1e-3 and np.max(np.abs(a - c)) <= 5e-2 * scale, (off.mean(), np.max(np.abs(a - c)), scale)
+
+
 def test_errors_surface_as_exceptions(device):
     from sliced_amd import host
     a = device.buffer([1, 2, 3])
