@@ -28,10 +28,10 @@ sys.path.insert(0, ROOT)
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # HBM-side bytes of one 4096^3 A*B launch, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` runs of
-# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (645235.8 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
+# this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (646261.4 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
-GEMM_4096_TRAFFIC_BYTES = int((645235.8 * 2.0 + 65536.0) * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((646261.4 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 
