@@ -812,6 +812,11 @@ def test_invalid_arguments_return_status_not_crash(hip):
     assert lib.slhip_gemm_tail_policy(c.h, 0) == 0 and lib.slhip_gemm_tile_policy(c.h, 0) == 0
     y = c.empty(16)
     assert lib.slhip_sgemm_relu_mask(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, y.ptr, y.ptr, 0.0) == -4   # C aliases pre
+    assert lib.slhip_sgemm_relu_bits(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, y.ptr, y.ptr, 0.0) == -4   # C aliases the bits
+    assert lib.slhip_sgemm_relu_bits(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, None, y.ptr, 0.0) == -1
+    assert lib.slhip_linear_fwd_bits(c.h, 2, 2, 2, x.ptr, x.ptr, None, y.ptr, y.ptr) == -4        # bits alias out
+    assert lib.slhip_linear_fwd_bits(c.h, 2, 0, 2, x.ptr, x.ptr, None, y.ptr, x.ptr) == -1        # zero dimension
+    assert lib.slhip_relu_grad_bits(c.h, 2, 2, None, y.ptr, x.ptr) == -1
     y.free()
     x.free()
 
