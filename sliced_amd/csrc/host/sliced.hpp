@@ -370,8 +370,8 @@ class HIP {
       check(slhip_linear_fwd(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, relu ? 1 : 0, relu ? pre.ptr : nullptr, out.ptr),
             "slhip_linear_fwd");
     uint64_t xi = x.id, wi = w.id, bi = bias.id, oi = out.id, pi = relu ? pre.id : 0, mi = as_bits ? mask.id : 0;
-    if (relu) relu_pre_[oi] = pi;
-    if (as_bits) relu_bits_[oi] = mi;
+    if (relu && tape_enabled_) relu_pre_[oi] = pi;  // entries live until run_tape()
+    if (as_bits && tape_enabled_) relu_bits_[oi] = mi;
     add_grad_fn([=] {
       Buffer xb = lookup(xi), wb = lookup(wi), bb = lookup(bi), o = lookup(oi);
       Buffer g;
