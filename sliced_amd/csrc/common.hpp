@@ -80,6 +80,10 @@ inline int32_t post_launch() {
   return SLHIP_OK;
 }
 
+// Blocks for `a` items at `b` per block.  The count is computed in size_t; launch sites check
+// grid_fits() first, because a count cast to unsigned would wrap and cover part of the data.
+constexpr size_t MAX_GRID = 0x7fffffffu;
+inline bool grid_fits(size_t a, size_t b) { return (a + b - 1) / b <= MAX_GRID; }
 inline unsigned ceil_div(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }
 
 // ------------------------------------------------------------------ device helpers

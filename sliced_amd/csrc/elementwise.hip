@@ -535,7 +535,7 @@ SLHIP_API int32_t slhip_cce(slhip_ctx* ctx, size_t rows, size_t cols, const floa
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
   int lanes = 1;
   while (lanes < 64 && (size_t)lanes * 8 < cols) lanes <<= 1;
-  SLHIP_REQUIRE(ceil_div(rows, 256 / lanes) <= 0x7fffffffu, "too many rows for one launch");
+  SLHIP_REQUIRE(grid_fits(rows, 256 / lanes), "too many rows for one launch");
 #define SL_CCE(L) \
   case L: hipLaunchKernelGGL((cce_kernel<L>), dim3(ceil_div(rows, 256 / L)), dim3(256), 0, ctx->stream, rows, cols, preds, targets, loss); break;
   switch (lanes) { SL_CCE(1) SL_CCE(2) SL_CCE(4) SL_CCE(8) SL_CCE(16) SL_CCE(32) SL_CCE(64) }
@@ -556,6 +556,7 @@ SLHIP_API int32_t slhip_onehot(slhip_ctx* ctx, size_t n, size_t classes, const f
   size_t len;
   SLHIP_REQUIRE(ctx && cls && out, "null argument");
   SLHIP_REQUIRE(checked_len(n, classes, &len), "bad dims");
+  SLHIP_REQUIRE(grid_fits(len, 256), "too many elements for one launch");
   hipLaunchKernelGGL(onehot_kernel, dim3(ceil_div(len, 256)), dim3(256), 0, ctx->stream, n, classes, cls, out);
   return post_launch();
 }

@@ -113,6 +113,37 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
     }
 }
 
+// Products the tiled kernel's loads are not written for: an output side of at most 32 or K of at most
+// 16 (its clamped vector loads assume an x-contiguous operand at least one float4 wide, and the plain
+// GEMM keeps such shapes away from it as well).  One lane per element of C, 64 columns of one row per
+// wave, the k range walked in order: slow and safe - nothing that trains a layer this narrow keeps
+// its mask as bits, but the entry points accept the shapes.
+template <bool TA, bool TB>
+__global__ __launch_bounds__(64) void gemm_bits_small_kernel(GemmArgs g, const uint32_t* __restrict__ bits_in,
+                                                             uint32_t* __restrict__ bits_out, size_t W) {
+  const size_t cblocks = (g.N + 63) / 64;
+  const size_t row = blockIdx.x / cblocks, cb = blockIdx.x % cblocks;
+  const int lane = threadIdx.x;
+  const size_t col = cb * 64 + lane;
+  const bool in = col < g.N;
+  const size_t cc = in ? col : g.N - 1;
+  const float* ap = TA ? g.A + row : g.A + row * g.K;
+  const float* bp = TB ? g.B + cc * g.K : g.B + cc;
+  const size_t astep = TA ? g.M : 1, bstep = TB ? 1 : g.N;
+  float val = 0.0f;
+  for (size_t k = 0; k < g.K; ++k) val = val + ap[k * astep] * bp[k * bstep];
+  if (bits_in) val = (((bits_in[row * W + (cc >> 5)] >> (cc & 31)) & 1u) ? 1.0f : 0.0f) * val;
+  if (g.beta != 0.0f && in) val = g.beta * g.C[row * g.N + col] + val;
+  if (g.bias) val = val + g.bias[cc];
+  if (bits_out) {
+    const unsigned long long b = __ballot(val >= 0.0f && in);
+    const size_t cw = cb * 2 + (lane >> 5);
+    if ((lane & 31) == 0 && cw < W) bits_out[row * W + cw] = (uint32_t)(lane ? b >> 32 : b);
+  }
+  if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
+  if (in) g.C[row * g.N + col] = val;
+}
+
 // x_grad += bit * out_grad: the ReLU gradient (src/matrix.rs:190-199) from the packed mask.
 __global__ __launch_bounds__(256) void relu_grad_bits_kernel(size_t rows, size_t cols, size_t W, const uint32_t* __restrict__ bits,
                                                              float* x_grad, const float* __restrict__ out_grad) {
@@ -147,6 +178,21 @@ static int32_t gemm_bits_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t 
     if (gemm_short_k_launch(ctx, ta, tb, g, bits_in, &rc)) return rc;
   }
   const size_t W = (N + 31) / 32;
+  if (M <= 32 || N <= 32 || K <= 16) {
+    const size_t blocks = M * ((N + 63) / 64);
+    if (blocks > 0x7fffffffu) {
+      set_error("gemm with bit mask: %zu x %zu is too large for the narrow-shape kernel", M, N);
+      return SLHIP_EINVAL;
+    }
+#define SL_GBS(TA_, TB_) \
+  hipLaunchKernelGGL((gemm_bits_small_kernel<TA_, TB_>), dim3((unsigned)blocks), dim3(64), 0, ctx->stream, g, bits_in, bits_out, W)
+    if (!ta && !tb) SL_GBS(false, false);
+    else if (!ta && tb) SL_GBS(false, true);
+    else if (ta && !tb) SL_GBS(true, false);
+    else SL_GBS(true, true);
+#undef SL_GBS
+    return post_launch();
+  }
   const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % BM == 0 && N % BN == 0 && K % GEMM_BK == 0;
   const dim3 grid((unsigned)(tiles_m * tiles_n));
 #define SL_GB(TA_, TB_)                                                                                                      \

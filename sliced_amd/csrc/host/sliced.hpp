@@ -227,7 +227,7 @@ class HIP {
       recording_ = false;
       slhip_graph_end(ctx_, &g);
       slhip_graph_destroy(g);
-      tape_.clear();
+      clear_tape();
       throw;
     }
     recording_ = false;
@@ -310,12 +310,23 @@ class HIP {
       ones_.erase(g.id);
     }
   }
-  void run_tape() {
-    for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
+  // After a backward pass, finished or failed, the device holds no tape: a closure that throws
+  // (a released buffer, a refused launch) must not leave the rest behind for the next pass to replay.
+  void clear_tape() {
     tape_.clear();
     relu_pre_.clear();
     relu_bits_.clear();
     relu_grad_done_.clear();
+    relu_uses_.clear();
+  }
+  void run_tape() {
+    try {
+      for (size_t i = tape_.size(); i-- > 0;) tape_[i]();
+    } catch (...) {
+      clear_tape();
+      throw;
+    }
+    clear_tape();
   }
   // Seeds out's gradient with ones and runs the tape.  A seed gradient that backward() itself created
   // lives with the deferred-zero gradients: while nothing else has written it since the last
@@ -342,6 +353,7 @@ class HIP {
   // GemmMayGrad::gemm  src/ops.rs:250-289
   Buffer gemm(size_t m, size_t k, size_t n, const Buffer& lhs, const Buffer& rhs) {
     expect(lhs, m * k, "gemm lhs"); expect(rhs, k * n, "gemm rhs");
+    used(lhs, rhs);
     Buffer out = retrieve(m * n);
     check(slhip_gemm(ctx_, m, k, n, lhs.ptr, rhs.ptr, out.ptr), "slhip_gemm");
     uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
@@ -360,9 +372,11 @@ class HIP {
   // (examples/sine_net.rs:32-40, src/matrix.rs:169-190), merged into one.
   Buffer linear(size_t m, size_t k, size_t n, const Buffer& x, const Buffer& w, const Buffer& bias, bool relu) {
     expect(x, m * k, "linear x"); expect(w, k * n, "linear w"); expect(bias, n, "linear bias");
+    used(x, w, bias);
     Buffer pre = relu ? retrieve(m * n) : Buffer();
     Buffer out = retrieve(m * n);
-    const bool as_bits = relu && policy.fuse_relu_grad && policy.relu_bits && m * n >= (size_t(1) << 22);
+    // (layers narrower than 64 outputs keep the float mask: the bit kernels' tile path starts there)
+    const bool as_bits = relu && policy.fuse_relu_grad && policy.relu_bits && m * n >= (size_t(1) << 22) && n >= 64 && k > 16;
     Buffer mask = as_bits ? retrieve(m * ((n + 31) / 32)) : Buffer();
     if (as_bits)
       check(slhip_linear_fwd_bits(ctx_, m, k, n, x.ptr, w.ptr, bias.ptr, (uint32_t*)mask.ptr, out.ptr), "slhip_linear_fwd_bits");
@@ -391,7 +405,11 @@ class HIP {
       check(slhip_add_row_mut_grad(ctx_, m, n, grad_mut(bb).ptr, g.ptr), "bias grad");
       const bool set = policy.gemm_beta == 0.0f;
       auto producer = relu_pre_.find(xi);
-      const bool into_pre = policy.fuse_relu_grad && xb.requires_grad && producer != relu_pre_.end();
+      auto uses = relu_uses_.find(xi);
+      // only when this Linear is the ReLU output's single reader: any other consumer adds its own
+      // term to x.grad, which the producer's ReLU gradient then has to pick up the unfused way
+      const bool into_pre = policy.fuse_relu_grad && xb.requires_grad && producer != relu_pre_.end() &&
+                            uses != relu_uses_.end() && uses->second == 1;
       float* xg = xb.requires_grad && !into_pre ? grad_out(xb, set).ptr : nullptr;
       float* wg = wb.requires_grad ? grad_out(wb, set).ptr : nullptr;
       if (into_pre) {
@@ -417,6 +435,7 @@ class HIP {
   // RowOpMayGrad::add_row  src/ops.rs:323-356
   Buffer add_row(size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
     expect(lhs, rows * cols, "add_row lhs"); expect(rhs, cols, "add_row rhs");
+    used(lhs, rhs);
     Buffer out = retrieve(rows * cols);
     check(slhip_add_row(ctx_, rows, cols, lhs.ptr, rhs.ptr, out.ptr), "slhip_add_row");
     uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
@@ -429,6 +448,7 @@ class HIP {
   // RowOpMayGrad::add_row_mut  src/ops.rs:358-374 — in place; lhs keeps its id and gradient
   void add_row_mut(size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
     expect(lhs, rows * cols, "add_row_mut lhs"); expect(rhs, cols, "add_row_mut rhs");
+    used(lhs, rhs);
     check(slhip_add_row(ctx_, rows, cols, lhs.ptr, rhs.ptr, lhs.ptr), "slhip_add_row");
     uint64_t li = lhs.id, ri = rhs.id;
     add_grad_fn([=] {
@@ -442,6 +462,7 @@ class HIP {
   // src/ops2/row_op/grad.rs:12-41, src/ops2/col_op/grad.rs:12-27): both sides accumulate.
   Buffer bcast_op(bool by_row_index, int op, size_t rows, size_t cols, const Buffer& lhs, const Buffer& rhs) {
     expect(lhs, rows * cols, "row/col op lhs"); expect(rhs, by_row_index ? rows : cols, "row/col op rhs");
+    used(lhs, rhs);
     Buffer out = retrieve(rows * cols);
     check((by_row_index ? slhip_col_op : slhip_row_op)(ctx_, op, rows, cols, lhs.ptr, rhs.ptr, out.ptr), "row/col op");
     uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
@@ -460,6 +481,7 @@ class HIP {
 
   // Diagflat::diagflat + DiagflatGrad (src/ops2/diagflat/mod.rs, grad/cpu.rs:34-38)
   Buffer diagflat(const Buffer& x) {
+    used(x);
     Buffer out = retrieve(x.len * x.len);
     check(slhip_diagflat(ctx_, x.len, x.ptr, out.ptr), "slhip_diagflat");
     uint64_t xi = x.id, oi = out.id;
@@ -472,6 +494,7 @@ class HIP {
 
   // Onehot::onehot + onehot_grad (src/ops2/onehot/cpu.rs:40-44, grad/cpu.rs:3-12)
   Buffer onehot(size_t classes, const Buffer& cls) {
+    used(cls);
     Buffer out = retrieve(cls.len * classes);
     check(slhip_onehot(ctx_, cls.len, classes, cls.ptr, out.ptr), "slhip_onehot");
     uint64_t ci = cls.id, oi = out.id;
@@ -485,14 +508,23 @@ class HIP {
   // BinaryOpsMayGrad::{add,sub,mul}  src/ops.rs:115-171
   Buffer binary(int op, const Buffer& lhs, const Buffer& rhs) {
     if (lhs.len != rhs.len) throw Error("binary op: lengths differ");
+    used(lhs, rhs);
     Buffer out = retrieve(lhs.len);
     check(slhip_ew_binary(ctx_, op, lhs.len, lhs.ptr, rhs.ptr, out.ptr), "slhip_ew_binary");
     uint64_t li = lhs.id, ri = rhs.id, oi = out.id;
     add_grad_fn([=] {
       Buffer l = lookup(li), r = lookup(ri), o = lookup(oi);
       // the reference touches both gradients whatever requires_grad says (src/ops.rs:118-128)
-      check(slhip_ew_binary_grad(ctx_, op, l.len, l.ptr, r.ptr, grad_mut(l).ptr, grad_mut(r).ptr, grad(o).ptr),
-            "slhip_ew_binary_grad");
+      float* lg = grad_mut(l).ptr;
+      float* rg = grad_mut(r).ptr;
+      if (lg == rg) {
+        // x op x: slice_binary_grad adds the lhs term, then the rhs term, into the one gradient
+        // (src/ops2/binary_ew/grad/cpu_stack.rs:55-58); two one-sided calls keep that order
+        check(slhip_ew_binary_grad(ctx_, op, l.len, l.ptr, r.ptr, lg, nullptr, grad(o).ptr), "slhip_ew_binary_grad");
+        check(slhip_ew_binary_grad(ctx_, op, l.len, l.ptr, r.ptr, nullptr, rg, grad(o).ptr), "slhip_ew_binary_grad");
+      } else {
+        check(slhip_ew_binary_grad(ctx_, op, l.len, l.ptr, r.ptr, lg, rg, grad(o).ptr), "slhip_ew_binary_grad");
+      }
     });
     return out;
   }
@@ -502,6 +534,7 @@ class HIP {
 
   // apply_fn + add_unary_grad: square (src/ops.rs:25-45), pow (:64-77), relu (src/matrix.rs:169-190)
   Buffer unary(int op, const Buffer& x, float p = 0.0f, float q = 0.0f, bool with_grad = true) {
+    used(x);
     Buffer out = retrieve(x.len);
     check(slhip_ew_unary(ctx_, op, p, q, x.len, x.ptr, out.ptr), "slhip_ew_unary");
     if (with_grad) {
@@ -524,6 +557,7 @@ class HIP {
   // TransposeMayGrad::transpose  src/ops.rs:207-220
   Buffer transpose(size_t rows, size_t cols, const Buffer& x) {
     expect(x, rows * cols, "transpose");
+    used(x);
     Buffer out = retrieve(x.len);
     check(slhip_transpose(ctx_, rows, cols, x.ptr, out.ptr, 0.0f), "slhip_transpose");
     uint64_t xi = x.id, oi = out.id;
@@ -537,6 +571,7 @@ class HIP {
   // SoftmaxMayGrad::softmax  src/ops.rs:751-778
   Buffer softmax(size_t samples, size_t features, const Buffer& x) {
     expect(x, samples * features, "softmax");
+    used(x);
     Buffer out = retrieve(x.len);
     check(slhip_softmax(ctx_, samples, features, x.ptr, out.ptr), "slhip_softmax");
     uint64_t xi = x.id, oi = out.id;
@@ -554,6 +589,7 @@ class HIP {
   enum Red { SUM_ROWS, SUM_COLS, MAX_ROWS, MAX_COLS, MEAN_ROWS, MEAN_COLS };
   Buffer reduce(Red kind, size_t rows, size_t cols, const Buffer& x) {
     expect(x, rows * cols, "reduction");
+    used(x);
     const bool over_rows = kind == SUM_ROWS || kind == MAX_ROWS || kind == MEAN_ROWS;
     Buffer out = retrieve(over_rows ? cols : rows);
     typedef int32_t (*Fwd)(slhip_ctx*, size_t, size_t, const float*, float*);
@@ -582,6 +618,7 @@ class HIP {
   // mean squared error == sub, squared, sum_cols over one row, mul by 1/n
   Buffer mse_loss(const Buffer& x, const Buffer& y) {
     if (x.len != y.len) throw Error("mse_loss: lengths differ");
+    used(x, y);
     Buffer out = retrieve(1);
     check(slhip_mse(ctx_, x.len, x.ptr, y.ptr, out.ptr), "slhip_mse");
     uint64_t xi = x.id, yi = y.id, oi = out.id;
@@ -595,6 +632,7 @@ class HIP {
   // == softmax on the tape + cce / cce_grad + backward_with of examples/nn.rs:124-152,229-233
   Buffer softmax_cce_loss(size_t rows, size_t cols, const Buffer& logits, const Buffer& targets) {
     expect(logits, rows * cols, "softmax_cce logits"); expect(targets, rows * cols, "softmax_cce targets");
+    used(logits, targets);
     Buffer probs = retrieve(rows * cols);
     Buffer per_row = retrieve(rows);
     Buffer out = retrieve(1);
@@ -646,6 +684,15 @@ class HIP {
   }
 
  private:
+  // Every op's forward reports the buffers it reads.  What is counted: the consumers of a fused
+  // Linear's ReLU output, because GradPolicy::fuse_relu_grad may skip that output's own gradient
+  // only while exactly one op (the next fused Linear) reads it.
+  void used(const Buffer& b) {
+    if (!tape_enabled_ || relu_pre_.empty()) return;
+    if (relu_pre_.count(b.id)) ++relu_uses_[b.id];
+  }
+  template <class... Rest>
+  void used(const Buffer& b, const Rest&... rest) { used(b); used(rest...); }
   static void expect(const Buffer& b, size_t len, const char* what) {
     if (!b.valid() || b.len != len)
       throw Error(std::string(what) + ": buffer length " + std::to_string(b.len) + " != " + std::to_string(len));
@@ -715,6 +762,7 @@ class HIP {
   std::unordered_set<uint64_t> stale_;                // large gradients with a zero fill pending since zero_grad()
   std::unordered_map<uint64_t, uint64_t> relu_bits_;  // ... -> its packed mask, where the forward kept bits instead
   std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
+  std::unordered_map<uint64_t, unsigned> relu_uses_;  // ReLU output of a fused Linear on the tape -> ops that read it so far
   bool tape_enabled_ = true;
   std::vector<Buffer> cache_;
   size_t cursor_ = 0;

@@ -138,6 +138,7 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const 
     tpr = 1;
     while (tpr < 64 && (size_t)tpr * 4 < per_seg) tpr <<= 1;
   }
+  SLHIP_REQUIRE(grid_fits(rows, tpr == 0 ? 1 : 256 / tpr), "too many rows for one launch");
 #define SL_RR(T)                                                                                              \
   case T: {                                                                                                   \
     unsigned rpb = T == 0 ? 1 : 256 / (T == 0 ? 1 : T);                                                       \
@@ -277,6 +278,7 @@ static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, 
   else if (cols >= 16 && rows * 16 <= 4096) cw = 16;
   else if (cols >= 4 && rows * 4 <= 4096) cw = 4;
   else if (rows > 4096) cw = cols >= 16 ? 16 : cols >= 4 ? 4 : 1;  // long inputs: coalescing matters more
+  SLHIP_REQUIRE(grid_fits(cols, cw), "too many columns for one launch");
 #define SL_CF(CW_)                                                                                                    \
   hipLaunchKernelGGL((colreduce_final_kernel<Op, CW_>), dim3(ceil_div(cols, CW_)), dim3(256), 0, ctx->stream, rows, cols, \
                      x, out, fin)
@@ -543,6 +545,7 @@ SLHIP_API int32_t slhip_max_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, 
     tpr = 1;
     while (tpr < 64 && (size_t)tpr * 8 < cols) tpr <<= 1;
   }
+  SLHIP_REQUIRE(grid_fits(rows, tpr == 0 ? 1 : 256 / tpr), "too many rows for one launch");
 #define SL_MCG(T)                                                                                          \
   case T: {                                                                                                \
     unsigned rpb = T == 0 ? 1 : 256 / (T == 0 ? 1 : T);                                                    \

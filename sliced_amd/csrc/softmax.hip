@@ -431,6 +431,7 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
   }
   const size_t colsv = cols / (VEC ? 4 : 1);
   SoftmaxCfg cfg = pick_cfg(colsv, FWD);
+  SLHIP_REQUIRE(rows <= MAX_GRID, "too many rows for one launch");
   if (cfg.lanes == 0) {
     if (FWD) hipLaunchKernelGGL(softmax_fwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x, out);
     else hipLaunchKernelGGL(softmax_bwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta);

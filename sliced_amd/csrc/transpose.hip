@@ -190,8 +190,8 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
   SLHIP_REQUIRE(ctx && x && out, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
   SLHIP_REQUIRE(beta == 0.0f || beta == 1.0f, "beta must be 0 (set) or 1 (accumulate)");
-  if (x == out) {
-    set_error("slhip_transpose: in-place transpose is not supported");
+  if (x < out + len && out < x + len) {  // the same buffer, or any partial overlap
+    set_error("slhip_transpose: out overlaps x (in-place transpose is not supported)");
     return SLHIP_EALIAS;
   }
   const bool acc = beta != 0.0f;

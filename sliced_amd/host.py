@@ -130,6 +130,10 @@ class HIP:
     def zeros(self, n):
         return self._out(lib().slh_buffer_zeros, _sz(n))
 
+    def release(self, buf):
+        """Frees a buffer and its gradient; closures on the tape that still name it will throw."""
+        _ck(lib().slh_buffer_release(self.h, _u64(buf.id)))
+
     def begin_iteration(self):
         _ck(lib().slh_begin_iteration(self.h))
 

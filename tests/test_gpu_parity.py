@@ -894,7 +894,9 @@ def test_relu_mask_as_bits_equals_the_float_mask(hip, orc):
     (linear_fwd with pre-activations, sgemm_relu_mask, the relu gradient): the same values within the
     GEMM bound, a mask that agrees with the exact pre-activations wherever their sign is not within
     that bound of zero, and outputs that are zero exactly where the mask is clear."""
-    for (m, k, n) in [(256, 96, 128), (300, 70, 200), (129, 33, 97), (1024, 784, 2048), (520, 64, 36)]:
+    # the last six: an output side of at most 32 or a short K, which the tile loads are not written for
+    for (m, k, n) in [(256, 96, 128), (300, 70, 200), (129, 33, 97), (1024, 784, 2048), (520, 64, 36),
+                      (300, 40, 1), (257, 70, 2), (130, 33, 3), (520, 64, 20), (20, 100, 200), (300, 8, 200)]:
         say("bit mask forward", m, k, n)
         x = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
         w = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
@@ -912,7 +914,9 @@ def test_relu_mask_as_bits_equals_the_float_mask(hip, orc):
             assert not np.any(bits[:, -1] >> np.uint32(n % 32))
     for (m, n, k, ta, tb) in [(256, 128, 96, 0, 1), (300, 200, 70, 0, 1), (129, 97, 33, 0, 0), (1024, 2048, 512, 0, 1),
                               (1031, 260, 10, 0, 1), (4100, 64, 3, 1, 0), (2050, 1028, 7, 1, 1), (700, 512, 12, 0, 0),
-                              (200, 130, 64, 1, 0), (140, 260, 40, 1, 1)]:
+                              (200, 130, 64, 1, 0), (140, 260, 40, 1, 1),
+                              (300, 3, 40, 0, 0), (300, 1, 70, 0, 0), (3, 200, 40, 1, 0), (2, 130, 64, 1, 1),
+                              (520, 20, 64, 0, 1), (1, 1, 33, 0, 0), (40, 2, 17, 1, 1)]:
         say("bit mask backward", m, n, k, ta, tb)
         a, b = gemm_operands(ta, tb, m, n, k)
         exact, bound = gemm_bound(ta, tb, m, n, k, a, b)

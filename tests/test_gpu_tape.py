@@ -429,6 +429,70 @@ def test_errors_surface_as_exceptions(device):
         a.grad()                                 # no gradient was ever written
 
 
+def test_self_products_are_differentiable(device, orc):
+    """x*x, x+x, x-x: both gradient terms land in the one gradient, lhs term first
+    (slice_binary_grad, src/ops2/binary_ew/grad/cpu_stack.rs:55-58)."""
+    xv = np.array([1, -2, 3, 0.5, -7], np.float32)
+    for op, name, want in ((device.mul, "mul", 2 * xv), (device.add, "add", np.full(5, 2, np.float32)),
+                           (device.sub, "sub", np.zeros(5, np.float32))):
+        say("self", name)
+        x = device.buffer(xv)
+        out = op(x, x)
+        out.backward()
+        lg, rg = np.zeros(5, np.float32), np.zeros(5, np.float32)
+        code = {"add": orc.ADD, "sub": orc.SUB, "mul": orc.MUL}[name]
+        orc.binary_ew_grad(code, xv, xv, lg, rg, np.ones(5, np.float32))
+        eq(x.grad(), lg + rg)
+        eq(x.grad(), want)
+
+
+def test_relu_output_with_two_readers_keeps_its_own_gradient(device):
+    """With the ReLU gradient folded into the next layer's input-gradient GEMM switched on, a ReLU
+    output that a second op reads as well must still collect that op's term: the fold is taken
+    only for a single reader, and both settings give the same gradients."""
+    m, d0, d1, d2 = 160, 48, 96, 80
+    x = rng.uniform(m * d0, -1, 1, tag=0)
+    w1, w2 = rng.uniform(d0 * d1, -0.5, 0.5, tag=1), rng.uniform(d1 * d2, -0.5, 0.5, tag=2)
+    b1, b2 = rng.uniform(d1, -0.5, 0.5, tag=3), rng.uniform(d2, -0.5, 0.5, tag=4)
+    res = []
+    try:
+        for fuse in (False, True):
+            device.set_fuse_relu_grad(fuse)
+            device.set_grad_policy(gemm_beta=1.0)           # accumulate, so both readers' terms add up
+            xb, w1b, w2b, b1b, b2b = (device.buffer(v) for v in (x, w1, w2, b1, b2))
+            h1 = device.linear(m, d0, d1, xb, w1b, b1b, True)
+            y = device.linear(m, d1, d2, h1, w2b, b2b, False)   # reader 1: a fused Linear
+            s = device.square(h1)                                # reader 2
+            ys = device.sum_cols(d2, y)
+            ss = device.sum_cols(d1, s)
+            tot = device.add(ys, ss)
+            tot.backward()
+            res.append([h1.grad().read(), xb.grad().read(), w1b.grad().read(), b1b.grad().read()])
+    finally:
+        device.set_fuse_relu_grad(False)
+        device.set_grad_policy()
+    h1g = res[1][0]
+    # h1.grad holds both terms: 2*h1 from the square and the rows of W2 summed from the Linear
+    assert np.abs(h1g).max() > 0
+    for a, c in zip(*res):
+        assert np.array_equal(a, c)
+
+
+def test_failed_backward_leaves_no_tape_behind(device):
+    from sliced_amd import host
+    a, b = device.buffer([1, 2, 3]), device.buffer([4, 5, 6])
+    out = device.mul(a, b)
+    device.release(a)                        # the closure on the tape now names a buffer that is gone
+    with pytest.raises(host.HostError):
+        out.backward()
+    assert device.tape_len() == 0
+    c, d = device.buffer([1, 2, 3]), device.buffer([4, 5, 6])
+    out2 = device.mul(c, d)
+    out2.backward()                          # must not replay the stale closure
+    eq(c.grad(), [4, 5, 6])
+    eq(d.grad(), [1, 2, 3])
+
+
 # --------------------------------------------------------------------------- training loops
 def loss_parity(got, ref, tol):
     rel = np.abs(got - ref) / np.maximum(np.abs(ref), 1e-30)
