@@ -176,6 +176,16 @@ int32_t slhip_max_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x,
 int32_t slhip_max_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*rows*/);
 int32_t slhip_mean_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*cols*/);
 int32_t slhip_mean_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*rows*/);
+/* slhip_sum_rows for callers that cannot allocate device memory, or may not have a library do it
+ * on their behalf: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same kernels, same result bits as
+ * slhip_sum_rows; the partial sums of its streaming stages live in a file-scope device array of
+ * 4 MiB that every GPU the library runs on holds until the process ends, instead of the context
+ * workspace.  The call itself allocates and frees nothing.  Limit: cols <= 131072 (any number of
+ * rows); wider matrices return SLHIP_EWORKSPACE.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (two contexts, two streams) race; calls on one context
+ * are ordered by its stream.  The array needs no clearing between calls. */
+int32_t slhip_sum_rows_static(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out /*cols*/);
 int32_t slhip_sum(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);
 int32_t slhip_max(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);
 int32_t slhip_mean(slhip_ctx* ctx, size_t len, const float* x, float* out_dev /*1*/);

@@ -52,6 +52,7 @@ PROTOTYPES = {
     "slhip_sgemm_relu_bits": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_relu_grad_bits": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_sum_rows": [c_vp, c_sz, c_sz, c_vp, c_vp],
+    "slhip_sum_rows_static": [c_vp, c_sz, c_sz, c_vp, c_vp],
     "slhip_sum_cols": [c_vp, c_sz, c_sz, c_vp, c_vp],
     "slhip_max_rows": [c_vp, c_sz, c_sz, c_vp, c_vp],
     "slhip_max_cols": [c_vp, c_sz, c_sz, c_vp, c_vp],

@@ -22,6 +22,7 @@ struct slhip_ctx {
   bool capturing = false;        // between slhip_graph_begin and slhip_graph_end
   int gemm_tail = 0;             // SLHIP_TAIL_*: how the tiled GEMM treats a partly filled last round
   int gemm_tile = 0;             // SLHIP_TILE_*: tile of C per workgroup of the tiled GEMM
+  float* static_scratch = nullptr;  // this device's copy of the file-scope scratch array of reduce.hip
 };
 
 struct slhip_event {
@@ -40,6 +41,9 @@ constexpr int WAVE = 64;
 constexpr size_t DEFAULT_WORKSPACE_BYTES = size_t(256) << 20;
 
 void set_error(const char* fmt, ...);
+// reduce.hip: resolves the device address of the file-scope scratch array for `device`, which must
+// be the current device.  Called once per context by slhip_init.
+int32_t static_scratch_resolve(int device, float** ptr);
 int32_t hip_fail(hipError_t e, const char* what);
 
 #define SLHIP_CHECK_HIP(expr)                                   \

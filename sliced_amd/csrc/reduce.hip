@@ -340,7 +340,7 @@ __global__ __launch_bounds__(1024) void fullreduce_final_kernel(size_t n, const 
 }
 
 template <class Op>
-static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin) {
+static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin, float* part) {
   const bool vec = true;
   size_t items = vec ? (n >> 2) + 1 : n;
   size_t blocks = (items + 256 * 16 - 1) / (256 * 16);
@@ -353,7 +353,6 @@ static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, 
     hipLaunchKernelGGL((fullreduce_final_kernel<Op>), dim3(1), dim3(1024), 0, ctx->stream, n, x, out, fin);
     return post_launch();
   }
-  float* part = (float*)ctx->workspace;
   if (vec)
     hipLaunchKernelGGL((fullreduce_kernel<Op, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
   else
@@ -364,10 +363,12 @@ static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, 
   return post_launch();
 }
 
-// out[c] = reduce over the strided axis.
+// out[c] = reduce over the strided axis.  ws / ws_left: where the partial results of the streaming
+// stages go (the context workspace, or the static scratch array), in floats.
 template <class Op>
-static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
-  if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin);
+static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin, float* ws,
+                           size_t ws_left) {
+  if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin, ws);  // at most 4 partials per CU
   // one row: the reduction over rows is that row itself
   if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, cols * sizeof(float));
   // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
@@ -377,8 +378,6 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
   const size_t unit = cols / (cols % 4 == 0 ? 4 : cols % 2 == 0 ? 2 : 1);
   const float* cur = x;
   size_t cur_rows = rows;
-  float* ws = (float*)ctx->workspace;
-  size_t ws_left = ctx->workspace_bytes / sizeof(float);
   // (the last stage is quick for up to 256 rows of any length - 16 rows per lane, 16 columns per
   // workgroup - and for small matrices of up to 4096 rows)
   while (cur_rows >= 8 && !((cur_rows <= 256 && cur_rows * cols <= (1u << 22)) || (cur_rows * cols <= (1u << 18) && cur_rows <= 4096))) {
@@ -398,6 +397,46 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
     ws_left -= 4 * T;
   }
   return colreduce_final_launch<Op>(ctx, cur_rows, cols, cur, out, fin);
+}
+
+template <class Op>
+static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
+  return reduce_rows<Op>(ctx, rows, cols, x, out, fin, (float*)ctx->workspace, ctx->workspace_bytes / sizeof(float));
+}
+template <class Op>
+static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin) {
+  return reduce_all<Op>(ctx, n, x, out, fin, (float*)ctx->workspace);
+}
+
+// ---------------------------------------------------------------------------------------
+// Scratch memory for callers that cannot allocate (slhip_sum_rows_static): the partial results of
+// the streaming stages in a file-scope device array instead of the context workspace.  Every GPU
+// holds its own copy of the array at its own address; in host code the array's name is only a
+// stand-in for the symbol, so the address is asked for once per device and everything below works
+// with that pointer.  Nothing in it has to start at zero: each stage writes all the partials the
+// next stage reads.
+// ---------------------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_FLOATS = size_t(1) << 20;  // 4 MiB per GPU, held until the process ends
+static __device__ __align__(256) float static_scratch[STATIC_SCRATCH_FLOATS];
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+static float* g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];  // device address per ordinal, 0 = not asked yet
+
+int32_t static_scratch_resolve(int device, float** ptr) {
+  if (device < 0 || device >= STATIC_SCRATCH_MAX_DEVICES) {
+    set_error("device ordinal %d beyond the %d this library keeps scratch addresses for", device, STATIC_SCRATCH_MAX_DEVICES);
+    return SLHIP_EINVAL;
+  }
+  if (!g_static_scratch[device]) {
+    void* p = nullptr;
+    SLHIP_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)));
+    if (!p) {
+      set_error("hipGetSymbolAddress returned no address for the static scratch array");
+      return SLHIP_EINVAL;
+    }
+    g_static_scratch[device] = (float*)p;
+  }
+  *ptr = g_static_scratch[device];
+  return SLHIP_OK;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -487,6 +526,22 @@ SLHIP_API int32_t slhip_mean_cols(slhip_ctx* ctx, size_t rows, size_t cols, cons
 SLHIP_API int32_t slhip_sum_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
   SL_DIMS_OK();
   return reduce_rows<SumOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0});
+}
+// The widest matrix whose streaming stages fit the static scratch array whatever its height: a stage
+// keeps 4 partials for each of its T <= 512 * (number of CUs) threads, T a multiple of
+// cols / gcd(cols, 4), and a stage runs only if it at least halves its input; with cols <= 131072 and
+// 256 CUs the first stage needs at most 2^19 floats and every later one at most half of the one
+// before, so all of them fit the 2^20 floats.
+constexpr size_t STATIC_MAX_COLS = 131072;
+SLHIP_API int32_t slhip_sum_rows_static(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
+  SL_DIMS_OK();
+  if (cols > STATIC_MAX_COLS) {
+    set_error("slhip_sum_rows_static: %zu columns; the static scratch serves at most %zu (use slhip_sum_rows)", cols,
+              STATIC_MAX_COLS);
+    return SLHIP_EWORKSPACE;
+  }
+  SLHIP_REQUIRE(ctx->static_scratch, "the context has no static scratch address");
+  return reduce_rows<SumOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0}, ctx->static_scratch, STATIC_SCRATCH_FLOATS);
 }
 SLHIP_API int32_t slhip_max_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
   SL_DIMS_OK();

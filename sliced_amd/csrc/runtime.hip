@@ -104,6 +104,15 @@ static int32_t make_ctx(int32_t ordinal, hipStream_t external, bool use_external
     return hip_fail(e, "hipMalloc(workspace)");
   }
   c->workspace_bytes = DEFAULT_WORKSPACE_BYTES;
+  // the device is current (hipSetDevice above): every GPU holds its own copy of the static scratch
+  // array at its own address
+  const int32_t rc = static_scratch_resolve(ordinal, &c->static_scratch);
+  if (rc != SLHIP_OK) {
+    (void)hipFree(c->workspace);
+    if (c->owns_stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+    return rc;
+  }
   *out = c;
   return SLHIP_OK;
 }

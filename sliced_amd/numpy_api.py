@@ -77,6 +77,12 @@ def sum_rows(cols, x):
     return _reduce("slhip_sum_rows", x.size // cols, cols, x, cols)
 
 
+def sum_rows_static(cols, x):
+    """slhip_sum_rows_static: the same reduction with its partial sums in the library's static scratch array."""
+    x = _f32(x)
+    return _reduce("slhip_sum_rows_static", x.size // cols, cols, x, cols)
+
+
 def sum_cols(cols, x):
     x = _f32(x)
     return _reduce("slhip_sum_cols", x.size // cols, cols, x, x.size // cols)

@@ -1,0 +1,65 @@
+"""slhip_sum_rows_static, the entry point that allocates nothing (its partial sums live in a
+file-scope device array), against slhip_sum_rows through the C ABI: the same kernels, so the same
+bits.  Two calls in a row share the array, the second on a smaller input; shapes cover the
+one-kernel form, one and two streaming stages, rows of odd length, a single column and a single row.
+This file is collected last on purpose, so that a failure here hides no other test."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from sliced_amd import rng
+
+pytestmark = pytest.mark.gpu
+SEED = 0x51CED
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def test_static_scratch_variant_matches_sum_rows(hip, orc):
+    shapes = [(8192, 4096), (2048, 1000), (16384, 2049), (300, 77), (1 << 20, 10), (64, 131072), (1 << 21, 1),
+              (1, 5000), (4096, 64), (37, 3)]
+    for i, (rows, cols) in enumerate(shapes):
+        say("sum_rows_static", rows, cols)
+        x = rng.uniform(rows * cols, -10, 10, tag=i, seed=SEED)
+        want = hip.sum_rows(cols, x)
+        got = hip.sum_rows_static(cols, x)
+        assert np.array_equal(got, want), (rows, cols)
+        # and against the CPU restatement of the reference, on the backward-error scale of a sum
+        if rows * cols <= (1 << 24):
+            ref = orc.sum_rows(cols, x)
+            scale = np.abs(x.reshape(rows, cols).astype(np.float64)).sum(axis=0)
+            assert np.all(np.abs(got.astype(np.float64) - ref) <= 2e-6 * scale + 1e-30), (rows, cols)
+
+
+def test_two_calls_in_a_row_second_smaller(hip):
+    """Back-to-back calls on one context share the scratch array; the second, smaller input must not
+    see anything the first left there."""
+    c = hip.ctx()
+    big = rng.uniform(16384 * 4096, -10, 10, tag=20, seed=SEED)
+    small = rng.uniform(2048 * 1000, -10, 10, tag=21, seed=SEED)
+    want_big, want_small = hip.sum_rows(4096, big), hip.sum_rows(1000, small)
+    dbig, dsmall = c.array(big), c.array(small)
+    obig, osmall = c.empty(4096), c.empty(1000)
+    say("static, 16384 x 4096 then 2048 x 1000, no wait in between")
+    c.call("slhip_sum_rows_static", 16384, 4096, dbig.ptr, obig.ptr)
+    c.call("slhip_sum_rows_static", 2048, 1000, dsmall.ptr, osmall.ptr)
+    assert np.array_equal(obig.numpy(), want_big)
+    assert np.array_equal(osmall.numpy(), want_small)
+    for b in (dbig, dsmall, obig, osmall):
+        b.free()
+
+
+def test_static_variant_rejects_what_does_not_fit(hip):
+    c = hip.ctx()
+    x = c.zeros(2 * 131076)
+    out = c.empty(131076)
+    rc = c.lib.slhip_sum_rows_static(c.h, 2, 131076, x.ptr, out.ptr)
+    assert rc == -3
+    assert b"131072" in c.lib.slhip_last_error_string()
+    assert c.lib.slhip_sum_rows_static(c.h, 0, 4, x.ptr, out.ptr) == -1
+    assert c.lib.slhip_sum_rows_static(c.h, 2, 4, None, out.ptr) == -1
+    x.free()
+    out.free()
