@@ -34,7 +34,7 @@ def big(hip):
     d.free()
 
 
-def test_reductions_16384_squared_against_oracle(big, orc):
+def test_reductions_16384_squared_against_oracle(big, orc, deviations):
     c, R, C, d, x = big
     out_r, out_c = c.empty(R), c.empty(C)
     say("max_cols / max_rows 16384^2 (bit-exact, with ties)")
@@ -51,16 +51,23 @@ def test_reductions_16384_squared_against_oracle(big, orc):
     got, ref = out_r.numpy(), orc.sum_cols(C, x)
     assert np.all(np.abs(got - exact) <= 1e-6 * abs_r)
     assert np.all(np.abs(got - ref) <= 1e-6 * abs_r + np.abs(ref - exact))
+    deviations("sum_cols [16384x16384]", "max |gpu-oracle| / sum|x|", np.max(np.abs(got.astype(np.float64) - ref) / abs_r), 1e-6)
     c.call("slhip_sum_rows", R, C, d.ptr, out_c.ptr)
     exact = X.sum(0, dtype=np.float64)
     got, ref = out_c.numpy(), orc.sum_rows(C, x)
     assert np.all(np.abs(got - exact) <= 1e-6 * abs_c)
     assert np.all(np.abs(got - ref) <= 1e-6 * abs_c + np.abs(ref - exact))
+    deviations("sum_rows [16384x16384]", "max |gpu-oracle| / sum|x|", np.max(np.abs(got.astype(np.float64) - ref) / abs_c), 1e-6)
     say("mean over 2^28")
     one = c.empty(1)
     c.call("slhip_mean", R * C, d.ptr, one.ptr)
     tot = X.sum(dtype=np.float64)
     assert abs(float(one.numpy()[0]) - tot / x.size) <= 1e-6 * abs_r.sum() / x.size + 1e-7 * abs(tot / x.size)
+    mean_ref = float(orc.mean(x))             # the reference's sequential f32 sum over 2^28 values, divided
+    # (the reference's sequential f32 sum of 2^28 terms is itself several 1e-6 of sum|x| from exact)
+    deviations("mean [2^28]", "|gpu-oracle| / mean|x|", abs(float(one.numpy()[0]) - mean_ref) / (abs_r.sum() / x.size), 2e-5)
+    deviations("mean [2^28]", "|oracle-f64| / mean|x| (the reference's own)", abs(mean_ref - tot / x.size) / (abs_r.sum() / x.size), 2e-5)
+    deviations("mean [2^28]", "|gpu-f64| / mean|x|", abs(float(one.numpy()[0]) - tot / x.size) / (abs_r.sum() / x.size), 1e-6)
     # degenerate shapes of the same tensor: [1 x 2^28] and [2^28 x 1]
     say("degenerate shapes")
     m = float(x.max())
@@ -123,9 +130,17 @@ def test_elementwise_chain_2_28_against_oracle(big, orc):
         z.free()
 
 
+# Ceilings of the direct softmax deviation per row length, with margin over what was measured.  The
+# reference's softmax divides by a sequential f32 sum of `cols` exponentials, which is itself up to
+# 1.5e-5 (rows of 4096) from the exact sum; the GPU result stays within 1e-6 of the exact value, so
+# the direct deviation IS the reference's rounding (both are recorded below).
+SOFTMAX_DIRECT = {128: 5e-6, 1024: 2e-5, 4096: 5e-5, 16384: 2e-4}
+SOFTMAX_GRAD_DIRECT = {128: 5e-6, 1024: 1e-5, 4096: 2e-5, 16384: 5e-5}
+
+
 @pytest.mark.parametrize("shape", [(32768, 4096), (1 << 20, 128), (1 << 17, 1024), (1 << 13, 16384)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_softmax_full_size(hip, orc, shape):
+def test_softmax_full_size(hip, orc, deviations, shape):
     rows, cols = shape
     n = rows * cols
     c = hip.ctx()
@@ -143,6 +158,13 @@ def test_softmax_full_size(hip, orc, shape):
     assert np.max(np.abs(s - exact) / np.maximum(exact, 1e-300)) <= 1e-6
     assert np.all(np.abs(s - ref) <= 1e-6 * exact + np.abs(ref - exact))
     assert np.max(np.abs(s.reshape(rows, cols).sum(1, dtype=np.float64) - 1.0)) <= 1e-6
+    # the direct deviation from the reference's five-pass f32 result: what remains beyond 1e-6 for long
+    # rows is the rounding of the reference's own sequential sum of `cols` exponentials
+    nz = ref > 0
+    cfg = "softmax [%dx%d]" % (rows, cols)
+    deviations(cfg, "max |gpu-oracle| / oracle", np.max(np.abs(s[nz].astype(np.float64) - ref[nz]) / ref[nz]), SOFTMAX_DIRECT[cols])
+    deviations(cfg, "max |oracle-f64| / f64 (the reference's own)", np.max(np.abs(ref[nz] - exact[nz]) / exact[nz]), SOFTMAX_DIRECT[cols])
+    deviations(cfg, "max |gpu-f64| / f64", np.max(np.abs(s[nz] - exact[nz]) / exact[nz]), 1e-6)
     c.call("slhip_softmax_grad", rows, cols, dxg.ptr, ds.ptr, dg.ptr, 0.0)
     got = dxg.numpy()
     S, G = s.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
@@ -151,6 +173,10 @@ def test_softmax_full_size(hip, orc, shape):
     assert np.all(np.abs(got - exact_b) <= bound)
     ob = orc.softmax_grad(rows, cols, s, g)
     assert np.all(np.abs(got - ob) <= bound + np.abs(ob - exact_b))
+    # (the oracle's closed form sums <s, g> sequentially in f32 over `cols` terms: again its own rounding)
+    deviations(cfg + " grad", "max |gpu-oracle| / (|s|(|g|+sum|s||g|))", np.max(np.abs(got.astype(np.float64) - ob) / (bound * 1e6)), SOFTMAX_GRAD_DIRECT[cols])
+    deviations(cfg + " grad", "max |oracle-f64| / same scale (the reference's own)", np.max(np.abs(ob - exact_b) / (bound * 1e6)), SOFTMAX_GRAD_DIRECT[cols])
+    deviations(cfg + " grad", "max |gpu-f64| / same scale", np.max(np.abs(got - exact_b) / (bound * 1e6)), 1e-6)
     # a constant upstream gradient gives zero
     c.call("slhip_fill", n, 1.0, dg.ptr)
     c.call("slhip_softmax_grad", rows, cols, dxg.ptr, ds.ptr, dg.ptr, 0.0)
