@@ -269,6 +269,34 @@ int32_t slhip_ew_unary_grad(slhip_ctx* ctx, int32_t op, float p, size_t n, const
 int32_t slhip_ew_chain(slhip_ctx* ctx, size_t n, const float* a, const float* b, const float* c,
                        const float* d, float* out);
 
+/* A chain of elementwise ops as ONE pass: what the tape's blanket wrappers (BinaryOpsMayGrad,
+ * SquareMayGrad, PowMayGrad ..., src/ops.rs:20-187) produce when they are chained, e.g.
+ * examples/chained_perf.rs:86-90 (square, add, mul, mul, add), with the intermediates kept in
+ * registers.  A program has up to SLHIP_EW_MAX_OPS instructions over up to SLHIP_EW_MAX_INPUTS
+ * input buffers of n floats.  Register j < 4 is input j; register 4 + i is the result of
+ * instruction i; an instruction reads registers below its own; the program's result is that of
+ * its last instruction.  op is a binary code (SLHIP_ADD .. SLHIP_DIV, reads src0 and src1) or
+ * SLHIP_EW_UNARY | a unary code (reads src0; p and q as in slhip_ew_unary).  Results have the bits
+ * of the same ops run one after the other through slhip_ew_binary / slhip_ew_unary.
+ * slhip_ew_program_grad: input_grads[j] += d result / d input j * out_grad for every non-null
+ * entry, the intermediates recomputed, every instruction's terms added in the order the
+ * single-op gradient calls would add them (last instruction first, lhs before rhs).  An
+ * instruction flagged SLHIP_EW_NOGRAD passes no gradient on (exp and clip have no gradient
+ * function in the reference, src/ops.rs:394-408,419-425).  out may alias an input; the
+ * gradients must be distinct buffers. */
+enum { SLHIP_EW_MAX_INPUTS = 4, SLHIP_EW_MAX_OPS = 8 };
+enum { SLHIP_EW_UNARY = 0x10 };  /* or-ed into slhip_ew_insn.op */
+enum { SLHIP_EW_NOGRAD = 0x1 };  /* slhip_ew_insn.flags */
+typedef struct slhip_ew_insn {
+  uint8_t op, src0, src1, flags;
+  float p, q;
+} slhip_ew_insn;
+int32_t slhip_ew_program(slhip_ctx* ctx, size_t n, size_t n_inputs, const float* const* inputs, size_t n_ops,
+                         const slhip_ew_insn* prog, float* out);
+int32_t slhip_ew_program_grad(slhip_ctx* ctx, size_t n, size_t n_inputs, const float* const* inputs,
+                              float* const* input_grads, size_t n_ops, const slhip_ew_insn* prog,
+                              const float* out_grad);
+
 /* ---------------------------------------------------------------- training helpers -
  * Host loops of the examples that a device-resident training loop needs as kernels.
  *   sgd_step : p[i] -= g[i]·lr                       (examples/sine_net.rs:105-116)

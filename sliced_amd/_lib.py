@@ -78,6 +78,8 @@ PROTOTYPES = {
     "slhip_ew_unary": [c_vp, c_i32, C.c_float, C.c_float, c_sz, c_vp, c_vp],
     "slhip_ew_unary_grad": [c_vp, c_i32, C.c_float, c_sz, c_vp, c_vp, c_vp],
     "slhip_ew_chain": [c_vp, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
+    "slhip_ew_program": [c_vp, c_sz, c_sz, c_vp, c_sz, c_vp, c_vp],
+    "slhip_ew_program_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_sz, c_vp, c_vp],
     "slhip_sgd_step": [c_vp, c_sz, c_vp, c_vp, C.c_float],
     "slhip_row_op": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_row_op_grad": [c_vp, c_i32, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],

@@ -43,11 +43,73 @@ SLH_API int slh_set_fuse_relu_grad(void* dev, int on) {
 SLH_API int slh_set_relu_bits(void* dev, int on) {
   return guard([&] { ((HIP*)dev)->policy.relu_bits = on != 0; });
 }
+// Elementwise ops are deferred and chains of them launched as one kernel (GradPolicy::fuse_elementwise).
+SLH_API int slh_set_fuse_elementwise(void* dev, int on) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    d->run();
+    d->policy.fuse_elementwise = on != 0;
+  });
+}
+SLH_API int slh_run(void* dev) {  // launches whatever is deferred: the lazy device's `run()`
+  return guard([&] { ((HIP*)dev)->run(); });
+}
+SLH_API size_t slh_deferred(void* dev) { return ((HIP*)dev)->deferred(); }
+SLH_API int slh_enable_tape(void* dev, int on) {
+  return guard([&] { ((HIP*)dev)->enable_tape(on != 0); });
+}
+SLH_API int slh_device_ctx(void* dev, void** ctx) {  // the slhip context the device issues its ops on
+  return guard([&] { *ctx = (void*)((HIP*)dev)->ctx(); });
+}
+// Records body-less helper for tests: begins / ends a recording around ops issued through this API.
+SLH_API int slh_record_begin(void* dev) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    d->run();
+    check(slhip_graph_begin(d->ctx()), "slhip_graph_begin");
+  });
+}
+SLH_API int slh_record_end(void* dev, size_t* nodes) {
+  return guard([&] {
+    HIP* d = (HIP*)dev;
+    d->run();
+    slhip_graph* g = nullptr;
+    check(slhip_graph_end(d->ctx(), &g), "slhip_graph_end");
+    check(slhip_graph_node_count(g, nodes), "slhip_graph_node_count");
+    check(slhip_graph_launch(d->ctx(), g), "slhip_graph_launch");  // the recorded ops have not run yet: run them once
+    check(slhip_sync(d->ctx()), "slhip_sync");
+    slhip_graph_destroy(g);
+  });
+}
+// The two elementwise chains of the reference's examples written against Matrix, method by method:
+// which == 0: ((a + b) * c - d).pow(2).squared()      (the bandwidth suite's chain; a, b, c, d)
+// which == 1: square(x) * x + (b + x) * b              (examples/chained_perf.rs:86-90; a = x, b = b)
+SLH_API int slh_matrix_chain(void* dev, int which, size_t rows, size_t cols, uint64_t a, uint64_t b, uint64_t c,
+                             uint64_t d, uint64_t* out) {
+  return guard([&] {
+    HIP* dv = (HIP*)dev;
+    if (which == 0) {
+      Matrix A(dv->lookup(a), rows, cols), B(dv->lookup(b), rows, cols), C(dv->lookup(c), rows, cols),
+          D(dv->lookup(d), rows, cols);
+      *out = A.add(B).mul(C).sub(D).pow(2.0f).squared().data.id;
+    } else {
+      Matrix X(dv->lookup(a), rows, cols), B(dv->lookup(b), rows, cols);
+      Matrix squared = X.squared();
+      Matrix add = B.add(X);
+      Matrix mul_b = add.mul(B);
+      Matrix mul = squared.mul(X);
+      *out = mul.add(mul_b).data.id;
+    }
+  });
+}
 SLH_API int slh_buffer_from(void* dev, const float* host, size_t len, uint64_t* id) {
   return guard([&] { *id = ((HIP*)dev)->from(host, len).id; });
 }
 SLH_API int slh_buffer_zeros(void* dev, size_t len, uint64_t* id) {
   return guard([&] { *id = ((HIP*)dev)->alloc(len, true).id; });
+}
+SLH_API int slh_buffer_ptr(void* dev, uint64_t id, void** ptr) {  // the device address, for callers that fill it themselves
+  return guard([&] { *ptr = (void*)((HIP*)dev)->lookup(id).ptr; });
 }
 SLH_API int slh_buffer_len(void* dev, uint64_t id, size_t* len) {
   return guard([&] { *len = ((HIP*)dev)->lookup(id).len; });

@@ -25,6 +25,7 @@
 #pragma once
 #include <cstdint>
 #include <cstdio>
+#include <algorithm>
 #include <functional>
 #include <stdexcept>
 #include <string>
@@ -112,6 +113,16 @@ struct GradPolicy {
   // the consumer's input-gradient GEMM reads those bits (slhip_sgemm_relu_bits): 1/32 of the bytes
   // both ways, equal values.  The pre-activation buffer then only names the gradient.
   bool relu_bits = false;
+  // Elementwise ops (binary, unary) are not launched when they are issued but when something
+  // needs their result; by then the tape knows which intermediates of a chain nothing else reads
+  // and launches each such chain as ONE kernel (slhip_ew_program), its backward as one kernel too
+  // (slhip_ew_program_grad, which recomputes the intermediates) - the device-side form of what the
+  // reference's lazy devices do with an op queue (`Autograd<Lazy<Base>>`, examples/sine_net.rs:178).
+  // Values and leaf gradients have the bits of the op-by-op sequence.  What differs: the gradient
+  // BUFFER of an intermediate that was fused away is never written (reading it throws), and an
+  // intermediate that is read later is computed then, from what its inputs hold at that time.
+  // Off by default, like every other departure from the reference's eager CPU device.
+  bool fuse_elementwise = false;
 };
 
 class HIP {
@@ -129,7 +140,10 @@ class HIP {
   HIP& operator=(const HIP&) = delete;
 
   slhip_ctx* ctx() const { return ctx_; }
-  void sync() { check(slhip_sync(ctx_), "slhip_sync"); }
+  void sync() {
+    run();
+    check(slhip_sync(ctx_), "slhip_sync");
+  }
 
   // ---- buffers ---------------------------------------------------------------------------
   Buffer alloc(size_t len, bool zero = true) {
@@ -160,6 +174,8 @@ class HIP {
     it->second.requires_grad = v;
   }
   void release(uint64_t id) {
+    if (pending_.count(id) || !pending_order_.empty()) run();
+    virtual_.erase(id);
     auto it = allocs_.find(id);
     if (it == allocs_.end()) return;
     if (!it->second.pooled) check(slhip_free(ctx_, it->second.ptr), "slhip_free");  // pool memory stays with the pool
@@ -181,6 +197,8 @@ class HIP {
     if (!cached_) return alloc(len, zero);
     if (cursor_ < cache_.size() && cache_[cursor_].len == len) {
       Buffer b = cache_[cursor_++];
+      if (pending_.count(b.id)) run();  // last iteration's deferred op into this very buffer
+      virtual_.erase(b.id);             // whatever it stood for, the op at hand overwrites it
       if (zero) check(slhip_memset(ctx_, b.ptr, 0, len * sizeof(float)), "slhip_memset");
       return b;
     }
@@ -217,12 +235,14 @@ class HIP {
   // Graph is in use.
   template <class F>
   Graph record(F&& body) {
+    run();  // what was deferred before the recording belongs before it
     check(slhip_graph_begin(ctx_), "slhip_graph_begin");
     slhip_graph* g = nullptr;
     recording_ = true;
     recorded_seeds_.clear();
     try {
       body();
+      run();  // deferred elementwise ops of the body are part of the recording
     } catch (...) {
       recording_ = false;
       slhip_graph_end(ctx_, &g);
@@ -239,6 +259,7 @@ class HIP {
   // runs here, and every seed gradient whose fill the recording left out holds its ones again.
   // In a loop that replays the same recording this finds nothing to do from the second replay on.
   void before_replay(const std::vector<uint64_t>& seeds) {
+    run();
     for (uint64_t id : seeds) {
       auto it = allocs_.find(id);
       if (it == allocs_.end()) continue;
@@ -255,6 +276,39 @@ class HIP {
     }
     stale_.clear();
   }
+
+  // ---- deferred elementwise ops (GradPolicy::fuse_elementwise) ------------------------------
+  // Launches everything that is deferred (the lazy device's `dev.run()`, examples/sine_net.rs:205).
+  // Every op that is not elementwise, every read-back, backward() and record() call it themselves.
+  void run() {
+    if (pending_order_.empty() || flushing_) return;
+    flushing_ = true;
+    std::vector<uint64_t> order;
+    order.swap(pending_order_);
+    try {
+      // group roots first, in the order they were issued: nodes that end a chain or have several
+      // readers; a root's group pulls in the single-reader nodes below it
+      for (uint64_t id : order) {
+        auto it = pending_.find(id);
+        if (it != pending_.end() && it->second.readers != 1) emit_group(id);
+      }
+      for (uint64_t id : order)
+        if (pending_.count(id)) emit_group(id);
+    } catch (...) {
+      flushing_ = false;
+      pending_.clear();
+      throw;
+    }
+    pending_.clear();
+    flushing_ = false;
+  }
+  // Makes b's memory hold b's value: launches what is deferred, and computes b now if it was an
+  // intermediate that a fused chain kept in registers.
+  void ready(const Buffer& b) {
+    run();
+    if (!virtual_.empty() && virtual_.count(b.id)) materialise(b.id);
+  }
+  size_t deferred() const { return pending_order_.size(); }
 
   // ---- autograd --------------------------------------------------------------------------
   void add_grad_fn(std::function<void()> f) { if (tape_enabled_) tape_.push_back(std::move(f)); }
@@ -292,6 +346,7 @@ class HIP {
   // overwrites it first - the activation gradients of a fused step, 64 MiB each for the classifier
   // with batch 8192, are all written that way (41 us of fills a step otherwise).
   void zero_grad() {
+    run();
     for (auto& sl : slabs_)
       if (!sl.lazy && sl.used) check(slhip_memset(ctx_, sl.base, 0, sl.used * sizeof(float)), "slhip_memset");
     for (auto& kv : grads_) {
@@ -318,6 +373,8 @@ class HIP {
     relu_bits_.clear();
     relu_grad_done_.clear();
     relu_uses_.clear();
+    pending_.clear();
+    pending_order_.clear();
   }
   void run_tape() {
     try {
@@ -333,6 +390,7 @@ class HIP {
   // backward(), it still holds the ones, zero_grad() has only marked it, and the fill is skipped
   // (one kernel less in every training step, recorded or not).
   void backward(const Buffer& out) {
+    run();
     const bool fresh = !has_grad(out.id);
     Buffer g = grad_slot(out, /*lazy=*/fresh);
     const bool still_ones = ones_.count(g.id) != 0;
@@ -344,6 +402,8 @@ class HIP {
   }
   void backward_with(const Buffer& out, const Buffer& seed) {
     if (seed.len != out.len) throw Error("backward_with: seed length differs");
+    run();
+    ready(seed);
     Buffer g = grad_out(out, true);
     check(slhip_memcpy_d2d(ctx_, g.ptr, seed.ptr, g.len * sizeof(float)), "slhip_memcpy_d2d");
     run_tape();
@@ -508,6 +568,8 @@ class HIP {
   // BinaryOpsMayGrad::{add,sub,mul}  src/ops.rs:115-171
   Buffer binary(int op, const Buffer& lhs, const Buffer& rhs) {
     if (lhs.len != rhs.len) throw Error("binary op: lengths differ");
+    if (op < SLHIP_ADD || op > SLHIP_DIV) throw Error("binary op: unknown op code");
+    if (policy.fuse_elementwise) return defer(EwNode{0, lhs.id, rhs.id, op, false, 0.0f, 0.0f, true, lhs.len}, lhs, rhs);
     used(lhs, rhs);
     Buffer out = retrieve(lhs.len);
     check(slhip_ew_binary(ctx_, op, lhs.len, lhs.ptr, rhs.ptr, out.ptr), "slhip_ew_binary");
@@ -534,6 +596,8 @@ class HIP {
 
   // apply_fn + add_unary_grad: square (src/ops.rs:25-45), pow (:64-77), relu (src/matrix.rs:169-190)
   Buffer unary(int op, const Buffer& x, float p = 0.0f, float q = 0.0f, bool with_grad = true) {
+    if (op < SLHIP_SQUARE || op > SLHIP_SIGMOID) throw Error("unary op: unknown op code");
+    if (policy.fuse_elementwise) return defer(EwNode{0, x.id, 0, op, true, p, q, with_grad, x.len}, x, x);
     used(x);
     Buffer out = retrieve(x.len);
     check(slhip_ew_unary(ctx_, op, p, q, x.len, x.ptr, out.ptr), "slhip_ew_unary");
@@ -649,6 +713,7 @@ class HIP {
 
   // Mean::mean  src/ops2/mean/mod.rs:15-17 — a host scalar, not on the tape
   float mean(const Buffer& x) {
+    ready(x);
     Buffer s = scalar_scratch();
     check(slhip_mean(ctx_, x.len, x.ptr, s.ptr), "slhip_mean");
     float v;
@@ -659,15 +724,20 @@ class HIP {
   // The same reduction left on the device (for recorded sequences, which cannot read back)
   void mean_to(const Buffer& x, const Buffer& out) {
     expect(out, 1, "mean_to out");
+    ready(x);
+    ready(out);
     check(slhip_mean(ctx_, x.len, x.ptr, out.ptr), "slhip_mean");
   }
   void copy(const Buffer& src, size_t src_off, const Buffer& dst, size_t dst_off, size_t n) {
     if (src_off + n > src.len || dst_off + n > dst.len) throw Error("copy: range outside the buffer");
+    ready(src);
+    ready(dst);
     check(slhip_memcpy_d2d(ctx_, dst.ptr + dst_off, src.ptr + src_off, n * sizeof(float)), "slhip_memcpy_d2d");
   }
 
   // SGD of the examples (examples/sine_net.rs:105-116): value -= grad * lr, on the device
   void sgd_step(const Buffer& p, float lr) {
+    ready(p);
     check(slhip_sgd_step(ctx_, p.len, p.ptr, grad(p).ptr, lr), "slhip_sgd_step");
   }
   // the same for a whole parameter list in one launch
@@ -675,6 +745,7 @@ class HIP {
     std::vector<float*> p;
     std::vector<const float*> g;
     std::vector<size_t> n;
+    run();
     for (const Buffer& b : params) {
       p.push_back(b.ptr);
       g.push_back(grad(b).ptr);
@@ -688,11 +759,180 @@ class HIP {
   // Linear's ReLU output, because GradPolicy::fuse_relu_grad may skip that output's own gradient
   // only while exactly one op (the next fused Linear) reads it.
   void used(const Buffer& b) {
+    ready(b);
+    count_use(b);
+  }
+  void count_use(const Buffer& b) {
     if (!tape_enabled_ || relu_pre_.empty()) return;
     if (relu_pre_.count(b.id)) ++relu_uses_[b.id];
   }
   template <class... Rest>
   void used(const Buffer& b, const Rest&... rest) { used(b); used(rest...); }
+  // One deferred elementwise op.  ids, not pointers: the closures resolve buffers when they run.
+  struct EwNode {
+    uint64_t out, a, b;  // b = 0 for a unary op
+    int op;
+    bool unary;
+    float p, q;
+    bool with_grad;
+    size_t len;
+    size_t tape_slot = SIZE_MAX;  // where its gradient closure goes on the tape, if anywhere
+    unsigned readers = 0;         // deferred ops that read `out` so far
+    uint64_t seq = 0;             // order of issue
+  };
+  Buffer defer(EwNode n, const Buffer& lhs, const Buffer& rhs) {
+    count_use(lhs);
+    if (!n.unary) count_use(rhs);
+    // an input that an earlier chain kept in registers is computed now: it has a second reader
+    if (!virtual_.empty()) {
+      if (virtual_.count(n.a)) materialise(n.a);
+      if (!n.unary && virtual_.count(n.b)) materialise(n.b);
+    }
+    Buffer out = retrieve(n.len);
+    n.out = out.id;
+    n.seq = ++ew_seq_;
+    if (tape_enabled_ && n.with_grad) {
+      n.tape_slot = tape_.size();
+      tape_.push_back([] {});
+    }
+    auto reads = [&](uint64_t id) {
+      auto it = pending_.find(id);
+      if (it != pending_.end()) ++it->second.readers;
+    };
+    reads(n.a);
+    if (!n.unary) reads(n.b);
+    pending_[n.out] = n;
+    pending_order_.push_back(n.out);
+    if (pending_order_.size() >= 1024) run();  // bounds the host-side bookkeeping of very long chains
+    return out;
+  }
+  void launch_single(const EwNode& n) {
+    Buffer a = lookup(n.a), o = lookup(n.out);
+    if (n.unary) check(slhip_ew_unary(ctx_, n.op, n.p, n.q, n.len, a.ptr, o.ptr), "slhip_ew_unary");
+    else check(slhip_ew_binary(ctx_, n.op, n.len, a.ptr, lookup(n.b).ptr, o.ptr), "slhip_ew_binary");
+  }
+  // The gradient step of one elementwise op, as the op-by-op tape runs it.
+  void single_grad(const EwNode& n) {
+    Buffer a = lookup(n.a), o = lookup(n.out);
+    if (n.unary) {
+      check(slhip_ew_unary_grad(ctx_, n.op, n.p, n.len, a.ptr, grad_mut(a).ptr, grad(o).ptr), "slhip_ew_unary_grad");
+      return;
+    }
+    Buffer b = lookup(n.b);
+    // the reference touches both gradients whatever requires_grad says (src/ops.rs:118-128)
+    float* lg = grad_mut(a).ptr;
+    float* rg = grad_mut(b).ptr;
+    if (lg == rg) {
+      // x op x: slice_binary_grad adds the lhs term, then the rhs term, into the one gradient
+      // (src/ops2/binary_ew/grad/cpu_stack.rs:55-58); two one-sided calls keep that order
+      check(slhip_ew_binary_grad(ctx_, n.op, n.len, a.ptr, b.ptr, lg, nullptr, grad(o).ptr), "slhip_ew_binary_grad");
+      check(slhip_ew_binary_grad(ctx_, n.op, n.len, a.ptr, b.ptr, nullptr, rg, grad(o).ptr), "slhip_ew_binary_grad");
+    } else {
+      check(slhip_ew_binary_grad(ctx_, n.op, n.len, a.ptr, b.ptr, lg, rg, grad(o).ptr), "slhip_ew_binary_grad");
+    }
+  }
+  // Computes a fused-away intermediate into its buffer after all (somebody reads it).
+  void materialise(uint64_t id) {
+    auto it = virtual_.find(id);
+    if (it == virtual_.end()) return;
+    const EwNode n = it->second;
+    virtual_.erase(it);
+    materialise(n.a);
+    if (!n.unary) materialise(n.b);
+    launch_single(n);
+  }
+  // Launches the chain that ends in `root`: the root and, below it, every deferred op whose result
+  // only this chain reads, as long as the program stays within 8 instructions and 4 inputs.
+  void emit_group(uint64_t root) {
+    std::vector<uint64_t> ops{root}, leaves;
+    std::function<bool(uint64_t)> expand = [&](uint64_t id) -> bool {
+      const EwNode n = pending_.at(id);
+      const uint64_t srcs[2] = {n.a, n.unary ? 0 : n.b};
+      for (uint64_t src : srcs) {
+        if (!src || std::find(ops.begin(), ops.end(), src) != ops.end()) continue;
+        auto it = pending_.find(src);
+        if (it != pending_.end() && it->second.readers == 1 && ops.size() < SLHIP_EW_MAX_OPS) {
+          const std::vector<uint64_t> ops_before = ops, leaves_before = leaves;
+          ops.push_back(src);
+          if (expand(src)) continue;
+          ops = ops_before;        // does not fit: src is computed on its own and read as an input
+          leaves = leaves_before;
+        }
+        if (std::find(leaves.begin(), leaves.end(), src) == leaves.end()) {
+          if (leaves.size() == SLHIP_EW_MAX_INPUTS) return false;
+          leaves.push_back(src);
+        }
+      }
+      return true;
+    };
+    if (!expand(root)) {
+      const EwNode n = pending_.at(root);
+      ops.assign(1, root);
+      leaves.assign(1, n.a);
+      if (!n.unary && n.b != n.a) leaves.push_back(n.b);
+    }
+    for (uint64_t leaf : leaves)
+      if (pending_.count(leaf)) emit_group(leaf);  // an input that is itself deferred comes first
+    std::vector<EwNode> group;
+    for (uint64_t id : ops) group.push_back(pending_.at(id));
+    std::sort(group.begin(), group.end(), [](const EwNode& x, const EwNode& y) { return x.seq < y.seq; });
+    for (uint64_t id : ops) pending_.erase(id);
+    const EwNode last = group.back();  // the root: issued after everything it reads
+    if (group.size() == 1) {
+      launch_single(last);
+      if (last.tape_slot != SIZE_MAX) tape_[last.tape_slot] = [this, last] { single_grad(last); };
+      return;
+    }
+    // registers: input j -> j, instruction i -> 4 + i
+    std::vector<slhip_ew_insn> prog;
+    auto reg_of = [&](uint64_t id) -> uint8_t {
+      for (size_t j = 0; j < leaves.size(); ++j)
+        if (leaves[j] == id) return (uint8_t)j;
+      for (size_t i = 0; i < group.size(); ++i)
+        if (group[i].out == id) return (uint8_t)(SLHIP_EW_MAX_INPUTS + i);
+      throw Error("elementwise fusion: operand outside its group");
+    };
+    for (const EwNode& n : group) {
+      slhip_ew_insn in;
+      in.op = (uint8_t)(n.unary ? (SLHIP_EW_UNARY | n.op) : n.op);
+      in.src0 = reg_of(n.a);
+      in.src1 = n.unary ? in.src0 : reg_of(n.b);
+      in.flags = n.with_grad ? 0 : SLHIP_EW_NOGRAD;
+      in.p = n.p;
+      in.q = n.q;
+      prog.push_back(in);
+    }
+    std::vector<const float*> in_ptrs;
+    for (uint64_t leaf : leaves) in_ptrs.push_back(lookup(leaf).ptr);
+    check(slhip_ew_program(ctx_, last.len, in_ptrs.size(), in_ptrs.data(), prog.size(), prog.data(), lookup(last.out).ptr),
+          "slhip_ew_program");
+    for (size_t i = 0; i + 1 < group.size(); ++i) virtual_[group[i].out] = group[i];
+    if (last.tape_slot == SIZE_MAX) return;
+    tape_[last.tape_slot] = [this, group, leaves, prog] {
+      const EwNode& root_node = group.back();
+      // Another op has read an intermediate after all and left a gradient for it: that term has to
+      // flow on through the intermediate's own gradient step, so the chain runs backwards op by op.
+      bool touched = false;
+      for (size_t i = 0; i + 1 < group.size(); ++i) touched = touched || has_grad(group[i].out);
+      if (touched) {
+        for (size_t i = 0; i + 1 < group.size(); ++i) materialise(group[i].out);
+        for (size_t i = group.size(); i-- > 0;)
+          if (group[i].with_grad && has_grad(group[i].out)) single_grad(group[i]);
+        return;
+      }
+      std::vector<const float*> ins;
+      std::vector<float*> grads;
+      for (uint64_t leaf : leaves) {
+        Buffer l = lookup(leaf);
+        ins.push_back(l.ptr);
+        grads.push_back(grad_mut(l).ptr);
+      }
+      check(slhip_ew_program_grad(ctx_, root_node.len, ins.size(), ins.data(), grads.data(), prog.size(), prog.data(),
+                                  grad(lookup(root_node.out)).ptr),
+            "slhip_ew_program_grad");
+    };
+  }
+
   static void expect(const Buffer& b, size_t len, const char* what) {
     if (!b.valid() || b.len != len)
       throw Error(std::string(what) + ": buffer length " + std::to_string(b.len) + " != " + std::to_string(len));
@@ -763,6 +1003,11 @@ class HIP {
   std::unordered_map<uint64_t, uint64_t> relu_bits_;  // ... -> its packed mask, where the forward kept bits instead
   std::unordered_set<uint64_t> relu_grad_done_;       // ReLU outputs whose pre-activation gradient a consumer has written
   std::unordered_map<uint64_t, unsigned> relu_uses_;  // ReLU output of a fused Linear on the tape -> ops that read it so far
+  std::unordered_map<uint64_t, EwNode> pending_;      // deferred elementwise ops by the buffer they will write
+  std::vector<uint64_t> pending_order_;               // ... in the order they were issued
+  std::unordered_map<uint64_t, EwNode> virtual_;      // intermediates a launched chain kept in registers: how to compute them
+  uint64_t ew_seq_ = 0;
+  bool flushing_ = false;
   bool tape_enabled_ = true;
   std::vector<Buffer> cache_;
   size_t cursor_ = 0;
@@ -771,12 +1016,14 @@ class HIP {
 
 inline std::vector<float> Buffer::read() const {
   std::vector<float> v(len);
+  dev->ready(*this);
   dev->settle(*this);
   check(slhip_memcpy_d2h(dev->ctx(), v.data(), ptr, len * sizeof(float)), "slhip_memcpy_d2h");
   return v;
 }
 inline void Buffer::write(const float* host, size_t n) const {
   if (n != len) throw Error("write: length differs");
+  dev->ready(*this);
   dev->drop_pending_zero(*this);
   check(slhip_memcpy_h2d(dev->ctx(), ptr, host, len * sizeof(float)), "slhip_memcpy_h2d");
 }

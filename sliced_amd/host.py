@@ -41,6 +41,7 @@ def lib():
         _h = C.CDLL(LIB_PATH)
         _h.slh_last_error.restype = C.c_char_p
         _h.slh_tape_len.restype = C.c_size_t
+        _h.slh_deferred.restype = C.c_size_t
     return _h
 
 
@@ -122,6 +123,40 @@ class HIP:
     def set_fuse_relu_grad(self, on):
         """Fused Linear layers write their input gradient through the previous layer's ReLU gradient."""
         _ck(lib().slh_set_fuse_relu_grad(self.h, C.c_int(1 if on else 0)))
+
+    def set_fuse_elementwise(self, on):
+        """Elementwise ops are deferred; chains whose intermediates nothing else reads run as one kernel."""
+        _ck(lib().slh_set_fuse_elementwise(self.h, C.c_int(1 if on else 0)))
+
+    def run(self):
+        """Launches whatever is deferred (the lazy device's `run()`)."""
+        _ck(lib().slh_run(self.h))
+
+    def deferred(self):
+        return lib().slh_deferred(self.h)
+
+    def enable_tape(self, on):
+        _ck(lib().slh_enable_tape(self.h, C.c_int(1 if on else 0)))
+
+    def ctx_handle(self):
+        """The slhip context this device issues its ops on (for event timing on the same stream)."""
+        p = C.c_void_p()
+        _ck(lib().slh_device_ctx(self.h, C.byref(p)))
+        return p
+
+    def record_begin(self):
+        _ck(lib().slh_record_begin(self.h))
+
+    def record_end(self):
+        """Ends the recording, runs it once, returns its number of kernel nodes."""
+        n = _sz()
+        _ck(lib().slh_record_end(self.h, C.byref(n)))
+        return n.value
+
+    def matrix_chain(self, which, rows, cols, a, b, c=None, d=None):
+        """which 0: ((a+b)*c-d).pow(2).squared(); which 1: square(x)*x + (b+x)*b with x = a - written against Matrix."""
+        c, d = c or a, d or a
+        return self._out(lib().slh_matrix_chain, int(which), _sz(rows), _sz(cols), _u64(a.id), _u64(b.id), _u64(c.id), _u64(d.id))
 
     def buffer(self, data):
         a = np.ascontiguousarray(data, dtype=np.float32).ravel()
@@ -298,6 +333,65 @@ def mlp_train(kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmu
     if info is not None:
         info["graph_nodes"] = nodes.value
     return losses, secs.value
+
+
+def bench_chain(n, iters=20, warmup=5, with_backward=True):
+    """The bandwidth suite's chain ((a+b)*c-d) -> pow 2 -> square on n elements per tensor, issued op by
+    op against the tape (add, mul, sub, pow, square), once with every op launched as it is issued and
+    once with elementwise fusion switched on (one kernel for the chain, one for its backward).  Times
+    are medians of per-iteration HIP-event pairs on the device's own stream; GB/s of the 20
+    algorithmic bytes per element (4 reads, 1 write) forward, of 52 (4 inputs, the seed, 4 gradients
+    read and written) for forward + backward."""
+    import statistics
+    L = _lib.load()
+    out = {"elements": n}
+    for label, fuse in (("op_by_op_tape", False), ("fused_tape", True)):
+        dev = HIP(0, cached=True)
+        dev.set_fuse_elementwise(fuse)
+        ctx = dev.ctx_handle()
+        bufs = []
+        for tag in range(4):
+            b = dev.zeros(n)
+            p = C.c_void_p()
+            _ck(lib().slh_buffer_ptr(dev.h, _u64(b.id), C.byref(p)))
+            _lib.check(L.slhip_rand_uniform(ctx, 0x51CED, tag + 1, -10.0, 10.0, n, p), "slhip_rand_uniform")
+            bufs.append(b)
+        a, b, c, d = bufs
+
+        def chain():
+            dev.begin_iteration()
+            return dev.square(dev.pow(dev.sub(dev.mul(dev.add(a, b), c), d), 2.0))
+
+        def timed(body):
+            ms = []
+            for it in range(warmup + iters):
+                e0, e1 = C.c_void_p(), C.c_void_p()
+                L.slhip_event_create(ctx, C.byref(e0)); L.slhip_event_create(ctx, C.byref(e1))
+                L.slhip_event_record(ctx, e0)
+                body()
+                L.slhip_event_record(ctx, e1)
+                t = C.c_float()
+                _lib.check(L.slhip_event_elapsed_ms(e0, e1, C.byref(t)), "slhip_event_elapsed_ms")
+                L.slhip_event_destroy(e0); L.slhip_event_destroy(e1)
+                if it >= warmup:
+                    ms.append(t.value)
+            return statistics.median(ms)
+
+        dev.enable_tape(False)
+        fwd = timed(lambda: (chain(), dev.run()))
+        out["ms_" + label] = fwd
+        out["GBps_" + label] = 20.0 * n / fwd / 1e6
+        if with_backward:
+            dev.enable_tape(True)
+
+            def step():
+                dev.zero_grad()
+                chain().backward()
+            both = timed(step)
+            out["ms_fwd_bwd_" + label] = both
+            out["GBps_fwd_bwd_" + label] = (20.0 + 52.0) * n / both / 1e6
+        dev.close()
+    return out
 
 
 C1 = dict(kind=0, batch=1024, d_in=1, d_h=64, d_out=1, lr=0.01, steps=200)

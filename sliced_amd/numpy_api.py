@@ -233,6 +233,53 @@ def unary_grad(op, x, x_grad, out_grad, p=0.0):
     return x_grad
 
 
+EW_UNARY, EW_NOGRAD = 0x10, 0x1
+INSN = np.dtype([("op", "u1"), ("src0", "u1"), ("src1", "u1"), ("flags", "u1"), ("p", "f4"), ("q", "f4")])
+
+
+def ew_insn(prog):
+    """[(op, src0, src1, flags, p, q), ...] -> the packed slhip_ew_insn array."""
+    arr = np.zeros(len(prog), INSN)
+    for i, t in enumerate(prog):
+        t = tuple(t) + (0,) * (6 - len(t))
+        arr[i] = t
+    return arr
+
+
+def _ptr_array(bufs):
+    import ctypes as C
+    arr = (C.c_void_p * len(bufs))(*[b.ptr if b is not None else None for b in bufs])
+    return arr
+
+
+def ew_program(inputs, prog):
+    """slhip_ew_program: the program's result over the input arrays."""
+    import ctypes as C
+    ins = [_f32(x) for x in inputs]
+    code = ew_insn(prog)
+    with _Scope() as s:
+        d = [s.up(x) for x in ins]
+        out = s.empty(ins[0].size)
+        ptrs = _ptr_array(d)
+        s.c.call("slhip_ew_program", ins[0].size, len(d), C.cast(ptrs, C.c_void_p), len(code), code.ctypes.data, out.ptr)
+        return out.numpy()
+
+
+def ew_program_grad(inputs, grads, prog, out_grad):
+    """slhip_ew_program_grad: grads[j] (None = skipped) after the call."""
+    import ctypes as C
+    ins = [_f32(x) for x in inputs]
+    code = ew_insn(prog)
+    with _Scope() as s:
+        d = [s.up(x) for x in ins]
+        g = [s.up(x) for x in grads]
+        og = s.up(out_grad)
+        ip, gp = _ptr_array(d), _ptr_array(g)
+        s.c.call("slhip_ew_program_grad", ins[0].size, len(d), C.cast(ip, C.c_void_p), C.cast(gp, C.c_void_p), len(code),
+                 code.ctypes.data, og.ptr)
+        return [b.numpy() if b is not None else None for b in g]
+
+
 def ew_chain(a, b, c, d):
     a = _f32(a)
     with _Scope() as s:
