@@ -1,23 +1,32 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X array-op hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-suite] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-suite] [--no-cpu] [--only parts]
 
 Headline (the JSON line's `value`): f32 GEMM TFLOP/s at M=N=K=4096, C = A·B, operands seeded
-U(-1,1) and resident in HBM before the timed region.  One step = one pass of the kernel.
+U(-1,1) and resident in HBM before the timed region.  One step = one pass of the kernel; W untimed
+launches, then exactly K launches between two stream synchronisations.
+
 The same line carries
-  roofline     - the GEMM kernel against the fp32 matrix peak, from HIP-event timing of the same
-                 launches on the stream they run on;
-  cpu_baseline - the CPU oracle's sgemm (a restatement of the reference's CPU path) timed on this
-                 host's cores on one pass of the same 4096^3 product;
-  suite        - the other workloads of the metric: A·Bᵀ / Aᵀ·B, the reductions, softmax fwd/bwd,
-                 transpose, the fused elementwise chain (GB/s of ALGORITHMIC bytes against 8 TB/s)
-                 and MLP training steps/s.
-Only one GPU is used; --gpus above 1 is refused.
+  roofline     - the GEMM kernel against the fp32 matrix peak: `achieved` is the flop count divided
+                 by the average launch duration of those K launches, from HIP events on the stream they
+                 run on.  Beside it: the median of per-launch event pairs (`achieved_median`), the same
+                 with the caches swept before every launch, the other two forms, the GEMM sweep, every
+                 bandwidth-bound op of the metric as GB/s of ALGORITHMIC bytes against 8 TB/s
+                 (`ops`, and flat `GBps: <op>` / `frac: <op>` keys), and the MLP training loops in
+                 steps/s (`mlp`, flat `steps/s: <loop>` keys);
+  cpu_baseline - the CPU side on this host's cores: the oracle's sgemm (a restatement of the
+                 reference's loops; `kind: port`) on one pass of the same 4096^3 product, the same
+                 product through numpy's bundled OpenBLAS (the reference's CPU GEMM is a CBLAS sgemm),
+                 the streaming ops and the two training loops.
+Bandwidth ops and sweep entries are timed as the median of per-launch HIP-event pairs over at least
+20 launches after at least 5 warm-ups; operands below 512 MiB have the caches swept (a 1 GiB fill)
+between launches, outside the event pair.  Only one GPU is used; --gpus above 1 is refused.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -31,9 +40,11 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # this program (profiles/hbm_traffic_gemm_and_bandwidth_suite.md): (646261.4 KiB x 2.0 + 65536 KiB x 1.0) x 1024,
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
+# A counter run cannot happen inside this program; the figure is that profile's, not this run's.
 GEMM_4096_TRAFFIC_BYTES = int((646261.4 * 2.0 + 65536.0) * 1024)
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
+MIN_ITERS, MIN_WARMUP = 20, 5
 
 
 def log(*a):
@@ -41,7 +52,8 @@ def log(*a):
 
 
 def timed(ctx, fn, steps, warmup):
-    """(wall ms per step with sync on both sides, HIP-event ms per launch)."""
+    """(wall ms per step with a stream sync on both sides, HIP-event ms per launch averaged over the
+    same launches)."""
     for _ in range(warmup):
         fn()
     ctx.sync()
@@ -59,6 +71,33 @@ def timed(ctx, fn, steps, warmup):
     return wall, ev
 
 
+def pair_times(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
+    """HIP-event milliseconds of every one of `iters` launches of fn(), each between its own pair of
+    events on the stream it runs on, after `warmup` untimed launches.  sweep: a 1 GiB scratch buffer
+    that is filled between launches, outside the pairs, to push the operands out of L2 and the
+    memory-side cache."""
+    iters, warmup = max(iters, MIN_ITERS), max(warmup, MIN_WARMUP)
+    for _ in range(warmup):
+        fn()
+    ev = [(ctx.event(), ctx.event()) for _ in range(iters)]
+    for a, b in ev:
+        if sweep is not None:
+            ctx.call("slhip_fill", sweep.n, 1.0, sweep.ptr)
+        ctx.record(a)
+        fn()
+        ctx.record(b)
+    ctx.sync()
+    ms = [ctx.elapsed_ms(a, b) for a, b in ev]
+    for a, b in ev:
+        ctx.lib.slhip_event_destroy(a)
+        ctx.lib.slhip_event_destroy(b)
+    return ms
+
+
+def median_ms(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
+    return statistics.median(pair_times(ctx, fn, iters, warmup, sweep))
+
+
 def spin_up(ctx, seconds=0.4):
     """Untimed: keep the matrix cores busy until the clocks have ramped (the first launches after
     an idle period run at about 2.0 instead of 2.4 GHz).  Uses the At*B kernel so that a profile of
@@ -74,35 +113,22 @@ def spin_up(ctx, seconds=0.4):
         x.free()
 
 
-def timed_cold(ctx, fn, steps, scratch):
-    """HIP-event ms per launch with the caches (L2 and the 256 MiB memory-side cache) swept between
-    launches by a fill of a 1 GiB scratch buffer; the sweep is outside the event pair."""
-    e0, e1 = ctx.event(), ctx.event()
-    total = 0.0
-    for _ in range(steps):
-        ctx.call("slhip_fill", scratch.n, 1.0, scratch.ptr)
-        ctx.record(e0)
-        fn()
-        ctx.record(e1)
-        total += ctx.elapsed_ms(e0, e1)
-    ctx.lib.slhip_event_destroy(e0)
-    ctx.lib.slhip_event_destroy(e1)
-    return total / steps
-
-
-def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, cold_scratch=None):
+def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headline=False):
     a = ctx.uniform(m * k, -1, 1, 0, SEED)
     b = ctx.uniform(k * n, -1, 1, 1, SEED)
     c = ctx.zeros(m * n)
     fn = lambda: ctx.call("slhip_sgemm", ta, tb, m, n, k, a.ptr, b.ptr, c.ptr, beta)
-    wall, ev = timed(ctx, fn, steps, warmup)
     flop = 2.0 * m * n * k
-    res = {"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
-           "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS}
-    if cold_scratch is not None:
-        cold = timed_cold(ctx, fn, max(5, steps // 2), cold_scratch)
-        res["ms_kernel_caches_swept"] = cold
-        res["tflops_kernel_caches_swept"] = flop / cold / 1e9
+    res = {}
+    if headline:
+        wall, ev = timed(ctx, fn, steps, warmup)
+        res.update({"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
+                    "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS})
+    med = median_ms(ctx, fn, steps, warmup)
+    res.update({"ms_median": med, "tflops_median": flop / med / 1e9, "frac_median": flop / med / 1e9 / FP32_MATRIX_PEAK_TFLOPS})
+    if sweep is not None:
+        cold = median_ms(ctx, fn, steps, warmup, sweep)
+        res.update({"ms_median_caches_swept": cold, "tflops_median_caches_swept": flop / cold / 1e9})
     for x in (a, b, c):
         x.free()
     return res
@@ -126,78 +152,97 @@ def shader_clock_mhz():
     return best
 
 
-def bw_entry(name, algo_bytes, wall, ev):
-    gbs = algo_bytes / ev / 1e6
-    return {"op": name, "algorithmic_bytes": algo_bytes, "ms_wall": wall, "ms_kernel": ev, "GBps": gbs,
-            "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+def bw_entry(ctx, name, algo_bytes, fn, iters, sweep=None):
+    ms = pair_times(ctx, fn, iters, MIN_WARMUP, sweep)
+    med = statistics.median(ms)
+    gbs = algo_bytes / med / 1e6
+    e = {"op": name, "algorithmic_bytes": algo_bytes, "ms_median": med, "ms_min": min(ms), "ms_max": max(ms),
+         "launches": len(ms), "caches_swept": sweep is not None, "GBps": gbs, "frac": gbs / HBM_PEAK_GBS}
+    log(e)
+    return e
 
 
-def bench_bandwidth_suite(ctx, steps, warmup):
+def bench_bandwidth_suite(ctx, iters):
     out = []
     R = C = 16384
     n = R * C
     x = ctx.uniform(n, -10, 10, 0, SEED)
     vec_c, vec_r, one = ctx.empty(C), ctx.empty(R), ctx.empty(1)
     y = ctx.empty(n)
+    add = lambda *a, **k: out.append(bw_entry(ctx, *a, **k))
+    # config 4: reductions, mean and transpose on [16384 x 16384]
     for name, outbuf, olen in [("sum_rows", vec_c, C), ("sum_cols", vec_r, R), ("max_rows", vec_c, C),
                                ("max_cols", vec_r, R)]:
-        fn = lambda name=name, outbuf=outbuf: ctx.call("slhip_" + name, R, C, x.ptr, outbuf.ptr)
-        w, e = timed(ctx, fn, steps, warmup)
-        out.append(bw_entry("%s [16384x16384]" % name, 4 * n + 4 * olen, w, e))
-        log(out[-1])
-    w, e = timed(ctx, lambda: ctx.call("slhip_mean", n, x.ptr, one.ptr), steps, warmup)
-    out.append(bw_entry("mean [2^28]", 4 * n + 4, w, e)); log(out[-1])
-    w, e = timed(ctx, lambda: ctx.call("slhip_transpose", R, C, x.ptr, y.ptr, 0.0), steps, warmup)
-    out.append(bw_entry("transpose [16384x16384]", 8 * n, w, e)); log(out[-1])
-    # degenerate 1-D shapes of the same tensor
+        add("%s [16384x16384]" % name, 4 * n + 4 * olen,
+            lambda name=name, outbuf=outbuf: ctx.call("slhip_" + name, R, C, x.ptr, outbuf.ptr), iters)
+    add("mean [2^28]", 4 * n + 4, lambda: ctx.call("slhip_mean", n, x.ptr, one.ptr), iters)
+    add("transpose [16384x16384]", 8 * n, lambda: ctx.call("slhip_transpose", R, C, x.ptr, y.ptr, 0.0), iters)
+    # config 4: the degenerate shapes of the same tensor - the reducing direction ...
     N1 = 1 << 28
-    for name, rows, cols, olen in [("sum_cols", 1, N1, 1), ("sum_rows", N1, 1, 1), ("max_cols", 1, N1, 1),
-                                   ("max_rows", N1, 1, 1)]:
-        fn = lambda name=name, rows=rows, cols=cols: ctx.call("slhip_" + name, rows, cols, x.ptr, one.ptr)
-        w, e = timed(ctx, fn, steps, warmup)
-        out.append(bw_entry("%s [%dx%d]" % (name, rows, cols), 4 * n + 4 * olen, w, e)); log(out[-1])
-    # softmax forward / backward, [32768 x 4096] and the row-length sweep at 2^27 elements
+    for name, rows, cols in [("sum_cols", 1, N1), ("sum_rows", N1, 1), ("max_cols", 1, N1), ("max_rows", N1, 1)]:
+        add("%s [%dx%d] -> 1" % (name, rows, cols), 4 * n + 4,
+            lambda name=name, rows=rows, cols=cols: ctx.call("slhip_" + name, rows, cols, x.ptr, one.ptr), iters)
+    # ... and the copy direction (2^28 outputs), and the transposes of a vector
+    for name, rows, cols in [("sum_rows", 1, N1), ("max_rows", 1, N1), ("sum_cols", N1, 1), ("max_cols", N1, 1)]:
+        add("%s [%dx%d] -> 2^28" % (name, rows, cols), 8 * n,
+            lambda name=name, rows=rows, cols=cols: ctx.call("slhip_" + name, rows, cols, x.ptr, y.ptr), iters)
+    for rows, cols in [(1, N1), (N1, 1)]:
+        add("transpose [%dx%d]" % (rows, cols), 8 * n,
+            lambda rows=rows, cols=cols: ctx.call("slhip_transpose", rows, cols, x.ptr, y.ptr, 0.0), iters)
+    # config 3: softmax forward / backward, [32768 x 4096] and the row-length sweep at 2^27 elements
     for rows, cols in [(32768, 4096), (1 << 20, 128), (1 << 17, 1024), (1 << 13, 16384)]:
         ne = rows * cols
         xs, g, s = x.view(0, ne), x.view(ne, ne), y.view(0, ne)
         xg = y.view(ne, ne)
-        w, e = timed(ctx, lambda: ctx.call("slhip_softmax", rows, cols, xs.ptr, s.ptr), steps, warmup)
-        out.append(bw_entry("softmax fwd [%dx%d]" % (rows, cols), 8 * ne, w, e)); log(out[-1])
-        w, e = timed(ctx, lambda: ctx.call("slhip_softmax_grad", rows, cols, xg.ptr, s.ptr, g.ptr, 0.0), steps, warmup)
-        out.append(bw_entry("softmax bwd [%dx%d]" % (rows, cols), 12 * ne, w, e)); log(out[-1])
+        add("softmax fwd [%dx%d]" % (rows, cols), 8 * ne, lambda: ctx.call("slhip_softmax", rows, cols, xs.ptr, s.ptr), iters)
+        add("softmax bwd [%dx%d]" % (rows, cols), 12 * ne,
+            lambda: ctx.call("slhip_softmax_grad", rows, cols, xg.ptr, s.ptr, g.ptr, 0.0), iters)
         if cols == 4096:
-            o1 = vec_c.view(0, cols)
-            w, e = timed(ctx, lambda: ctx.call("slhip_max_rows", rows, cols, xs.ptr, o1.ptr), steps, warmup)
-            out.append(bw_entry("max_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
-            w, e = timed(ctx, lambda: ctx.call("slhip_sum_rows", rows, cols, xs.ptr, o1.ptr), steps, warmup)
-            out.append(bw_entry("sum_rows [32768x4096]", 4 * ne + 4 * cols, w, e)); log(out[-1])
+            for name, o1, olen in (("max_rows", vec_c.view(0, cols), cols), ("sum_rows", vec_c.view(0, cols), cols),
+                                   ("max_cols", vec_r.view(0, R), rows), ("sum_cols", vec_r.view(0, R), rows)):
+                if olen > o1.n:
+                    o1 = y.view(ne, olen)
+                add("%s [32768x4096]" % name, 4 * ne + 4 * olen,
+                    lambda name=name, o1=o1: ctx.call("slhip_" + name, rows, cols, xs.ptr, o1.ptr), iters)
     # shapes off the beaten track, 2^27 elements each: rows of odd length, narrow and very wide matrices
     for rows, cols in [(4026, 33333), (522247, 257), (13421772, 10), (134, 1000000)]:
         ne = rows * cols
         xs = x.view(0, ne)
         ov = y.view(0, max(rows, cols))
         for name, olen in (("sum_rows", cols), ("max_rows", cols), ("sum_cols", rows)):
-            fn = lambda name=name: ctx.call("slhip_" + name, rows, cols, xs.ptr, ov.ptr)
-            w, e = timed(ctx, fn, steps, warmup)
-            out.append(bw_entry("%s [%dx%d]" % (name, rows, cols), 4 * ne + 4 * olen, w, e)); log(out[-1])
-    # fused elementwise chain on 2^28 elements per tensor: 4 reads + 1 write
+            add("%s [%dx%d]" % (name, rows, cols), 4 * ne + 4 * olen,
+                lambda name=name: ctx.call("slhip_" + name, rows, cols, xs.ptr, ov.ptr), iters)
+    # config 4: the elementwise chain on 2^28 elements per tensor: 4 reads + 1 write
     bb, cc, dd = ctx.uniform(n, -10, 10, 2, SEED), ctx.uniform(n, -10, 10, 3, SEED), ctx.uniform(n, -10, 10, 4, SEED)
-    w, e = timed(ctx, lambda: ctx.call("slhip_ew_chain", n, x.ptr, bb.ptr, cc.ptr, dd.ptr, y.ptr), steps, warmup)
-    out.append(bw_entry("ew_chain ((a+b)*c-d)^2^2 [2^28]", 20 * n, w, e)); log(out[-1])
+    add("ew_chain ((a+b)*c-d)^2^2 [2^28], hand-fused kernel", 20 * n,
+        lambda: ctx.call("slhip_ew_chain", n, x.ptr, bb.ptr, cc.ptr, dd.ptr, y.ptr), iters)
+    for b in (bb, cc, dd):
+        b.free()
     # the classifier's last layer (config 5): products with a side of 10, bound by HBM rather than by the
-    # matrix cores; bytes = both operands and the result, each moved once
+    # matrix cores; bytes = both operands and the result, each moved once.  64 MiB operands: caches swept
+    sweep = ctx.empty(1 << 28)
     for m_, n_, k_, ta, tb, what in [(8192, 2048, 10, 0, 1, "A*Bt"), (2048, 10, 8192, 1, 0, "At*B"), (8192, 10, 2048, 0, 0, "A*B")]:
         a_, b_, c_ = x.view(0, m_ * k_), x.view(m_ * k_, k_ * n_), y.view(0, m_ * n_)
-        w, e = timed(ctx, lambda: ctx.call("slhip_sgemm", ta, tb, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), steps, warmup)
-        out.append(bw_entry("gemm %s [%dx%dx%d]" % (what, m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_), w, e)); log(out[-1])
-    w, e = timed(ctx, lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n), steps, warmup)
-    out.append(bw_entry("device copy [1 GiB] (achievable line)", 8 * n, w, e)); log(out[-1])
-    for b in (x, y, bb, cc, dd, vec_c, vec_r, one):
+        add("gemm %s [%dx%dx%d]" % (what, m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_),
+            lambda: ctx.call("slhip_sgemm", ta, tb, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), iters, sweep=sweep)
+    sweep.free()
+    add("device copy [1 GiB] (achievable line)", 8 * n, lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n), iters)
+    for b in (x, y, vec_c, vec_r, one):
         b.free()
     return out
 
 
-def bench_mlp(ctx, steps_c5, steps_c1):
+def bench_tape_chain(ctx_unused, iters):
+    """Config 4's chain written op by op against the host tape (add, mul, sub, pow 2, square), which
+    fuses it into one launch where the intermediates have a single reader."""
+    try:
+        from sliced_amd import host
+        return host.bench_chain(1 << 28, iters)
+    except Exception as e:  # the host layer is optional for the kernel benchmark
+        return {"skipped": "%s" % e}
+
+
+def bench_mlp(steps_c5, steps_c1):
     try:
         from sliced_amd import host
     except Exception as e:  # the host layer is optional for the kernel benchmark
@@ -209,38 +254,70 @@ def cpu_baseline(m, n, k):
     import oracle
     cores = oracle.max_threads()
     oracle.set_threads(cores)
-    rs = np.random.RandomState(1)
-    a = rs.uniform(-1, 1, m * k).astype(np.float32)
-    b = rs.uniform(-1, 1, k * n).astype(np.float32)
+    from sliced_amd import rng
+    a = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)        # the very operands the GPU multiplies
+    b = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
     oracle.gemm(64, 64, 64, a[:4096], b[:4096])        # load + warm
     t0 = time.perf_counter()
     oracle.gemm(m, n, k, a, b)
     dt = time.perf_counter() - t0
     res = {"value": 2.0 * m * n * k / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-           "sample": "one pass of the same %dx%dx%d f32 product by the CPU oracle's blocked sgemm "
-                     "(sequential-k f32, no FMA), %.2f s on %d threads" % (m, n, k, dt, cores)}
+           "sample": "one pass of the same %dx%dx%d product, oracle sgemm (sequential-k f32, no FMA), %.2f s, %d threads"
+                     % (m, n, k, dt, cores)}
     oracle.set_threads(1)
     ms = 1024
     t0 = time.perf_counter()
     oracle.gemm(ms, ms, ms, a[:ms * ms], b[:ms * ms])
     dt1 = time.perf_counter() - t0
     res["single_thread_TFLOPs_at_1024"] = 2.0 * ms ** 3 / dt1 / 1e12
+    res.update(cblas_row(m, n, k, a, b))
     res["ops"] = cpu_streaming_ops(oracle, cores)
     res["mlp"] = cpu_mlp_steps(oracle, cores)
+    for loop, row in res["mlp"].items():
+        if isinstance(row, dict):
+            for key, v in row.items():
+                if key.startswith("steps_per_s"):
+                    res["%s %s" % (loop.split(" ")[0], key)] = v
     return res
+
+
+def cblas_row(m, n, k, a, b):
+    """The same product through a CBLAS sgemm - what the reference's CPU device calls
+    (src/ops2/gemm/cpu_stack.rs:39 -> custos GenericBlas -> cblas_sgemm): numpy's f32 matmul runs on
+    the OpenBLAS that numpy bundles, on as many threads as that library chooses to use."""
+    A, B = a.reshape(m, k), b.reshape(k, n)
+    np.matmul(A[:256], B)                               # load + warm the library's threads
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        np.matmul(A, B)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    threads, lib = None, "OpenBLAS bundled with numpy %s" % np.__version__
+    try:
+        from threadpoolctl import threadpool_info
+        for info in threadpool_info():
+            if info.get("user_api") == "blas":
+                threads = info.get("num_threads")
+                lib = "%s %s (numpy %s)" % (info.get("internal_api"), info.get("version"), np.__version__)
+    except Exception:
+        pass
+    return {"cblas_TFLOPs": 2.0 * m * n * k / best / 1e12, "cblas_threads": threads,
+            "cblas_sample": "best of 3 passes of the same %dx%dx%d f32 product, np.matmul -> cblas_sgemm of %s, %.3f s"
+                            % (m, n, k, lib, best)}
 
 
 def cpu_mlp_steps(oracle, cores):
     """Steps per second of the oracle's training loop (the reference's op sequence on the host) on the
-    two MLP configurations: all 200 steps of the sine fit, a bounded sample of 2 steps of the
-    classifier (260 GFLOP each), on one thread (the reference is single-threaded) and on every core."""
+    two MLP configurations: all 200 steps of the sine fit, a bounded sample of the classifier's steps
+    (260 GFLOP each), on one thread (the reference's loops are single-threaded) and on every core."""
     try:
         from sliced_amd import host
     except Exception as e:  # configurations and seeded data live beside the host layer's bindings
         return {"skipped": "host layer not built: %s" % e}
     out = {}
     for name, cfg, steps_by_threads in (("C1 sine fit 1-64-64-1 batch 1024", host.C1, {1: 200, cores: 200}),
-                                        ("C5 classifier 784-2048-2048-10 batch 8192", host.C5, {1: 1, cores: 2})):
+                                        ("C5 classifier 784-2048-2048-10 batch 8192", host.C5, {1: 2, cores: 6})):
         x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
         row = {}
         for th, steps in steps_by_threads.items():
@@ -292,7 +369,7 @@ def main():
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--size", type=int, default=4096)
-    ap.add_argument("--only", default="", help="comma list of suite parts to run: gemm,sweep,bandwidth,mlp")
+    ap.add_argument("--only", default="", help="comma list of suite parts to run: gemm,sweep,bandwidth,chain,mlp")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus %d refused); the hot path has no "
@@ -305,44 +382,71 @@ def main():
     M = N = K = args.size
 
     spin_up(ctx)
-    head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup)
-    log("gemm NN", head)
-    suite = {}
+    head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup, headline=True)
+    log("gemm A*B", head)
+    roof = {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": head["frac_of_peak"], "traffic": GEMM_4096_TRAFFIC_BYTES if M == 4096 else None,
+            "traffic_source": "profiles/hbm_traffic_gemm_and_bandwidth_suite.md (rocprofv3 --pmc of this program, not this run)",
+            "achieved_median": head["tflops_median"], "frac_median": head["frac_median"],
+            "timing": "achieved: average over the timed launches; *_median and every op below: median of per-launch "
+                      "HIP-event pairs, >= %d launches after >= %d warm-ups" % (MIN_ITERS, MIN_WARMUP)}
     # the clock while the matrix cores are busy: queue 0.3 s of launches, sample, then wait
     a, b, c = ctx.uniform(M * K, -1, 1, 0, SEED), ctx.uniform(K * N, -1, 1, 1, SEED), ctx.zeros(M * N)
     for _ in range(min(200, int(300 / max(head["ms_kernel"], 0.01)) + 1)):
         ctx.call("slhip_sgemm", 0, 0, M, N, K, a.ptr, b.ptr, c.ptr, 0.0)
     time.sleep(0.15)
-    suite["shader_clock_mhz_under_gemm_load"] = shader_clock_mhz()
+    roof["shader_clock_mhz_under_gemm_load"] = shader_clock_mhz()
     ctx.sync()
     for x in (a, b, c):
         x.free()
-    log("sclk under load:", suite["shader_clock_mhz_under_gemm_load"])
-    parts = set(args.only.split(",")) if args.only else {"gemm", "sweep", "bandwidth", "mlp"}
+    log("sclk under load:", roof["shader_clock_mhz_under_gemm_load"])
+    parts = set(args.only.split(",")) if args.only else {"gemm", "sweep", "bandwidth", "chain", "mlp"}
     if args.no_suite:
         parts = set()
+    iters = max(MIN_ITERS, args.steps)
     if "gemm" in parts:
-        scratch = ctx.empty(1 << 28)
-        suite["gemm_4096"] = {"A*B": bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup, cold_scratch=scratch),
-                              "A*Bt": bench_gemm(ctx, M, N, K, 0, 1, args.steps, args.warmup, cold_scratch=scratch),
-                              "At*B": bench_gemm(ctx, M, N, K, 1, 0, args.steps, args.warmup, cold_scratch=scratch)}
-        scratch.free()
-        log(suite["gemm_4096"])
+        sweep_buf = ctx.empty(1 << 28)
+        forms = {}
+        for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
+            r = bench_gemm(ctx, M, N, K, ta, tb, iters, MIN_WARMUP, sweep=sweep_buf)
+            forms[form] = r
+            roof["TFLOPs: %d^3 %s" % (M, form)] = r["tflops_median"]
+            roof["TFLOPs: %d^3 %s, caches swept" % (M, form)] = r["tflops_median_caches_swept"]
+            log(form, r)
+        roof["achieved_caches_swept"] = forms["A*B"]["tflops_median_caches_swept"]
+        roof["gemm_forms"] = forms
+        sweep_buf.free()
     if "sweep" in parts:
         sweep = {}
         for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (3584,) * 3, (4095,) * 3, (4608,) * 3, (8192,) * 3,
                           (8192, 2048, 784), (784, 2048, 8192)]:
-            st = max(3, args.steps // 4) if m >= 8192 and k >= 8192 else args.steps
             for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
-                r = bench_gemm(ctx, m, n, k, ta, tb, st, 2)
-                sweep["%dx%dx%d %s" % (m, n, k, form)] = {"tflops": r["tflops_kernel"], "frac": r["frac_of_peak"]}
-                log(m, n, k, form, sweep["%dx%dx%d %s" % (m, n, k, form)])
-        suite["gemm_sweep"] = sweep
+                r = bench_gemm(ctx, m, n, k, ta, tb, iters, MIN_WARMUP)
+                key = "%dx%dx%d %s" % (m, n, k, form)
+                sweep[key] = {"tflops": r["tflops_median"], "frac": r["frac_median"], "ms": r["ms_median"]}
+                roof["TFLOPs: " + key] = r["tflops_median"]
+                log(key, sweep[key])
+        roof["gemm_sweep"] = sweep
     if "bandwidth" in parts:
-        suite["bandwidth"] = bench_bandwidth_suite(ctx, max(5, args.steps // 2), 2)
+        ops = bench_bandwidth_suite(ctx, iters)
+        roof["ops"] = ops
+        for e in ops:
+            roof["GBps: " + e["op"]] = round(e["GBps"], 1)
+    ctx.close()
+    if "chain" in parts:
+        ch = bench_tape_chain(None, iters)
+        log("tape chain", ch)
+        roof["tape_chain"] = ch
+        for key in ("GBps_fused_tape", "GBps_op_by_op_tape"):
+            if key in ch:
+                roof["GBps: ew chain [2^28], " + key[5:].replace("_", " ")] = round(ch[key], 1)
     if "mlp" in parts:
-        suite["mlp"] = bench_mlp(ctx, 50, 200)
-        log(suite["mlp"])
+        mlp = bench_mlp(50, 200)
+        log(mlp)
+        roof["mlp"] = mlp
+        for loop, row in mlp.items():
+            if isinstance(row, dict) and "steps_per_s" in row:
+                roof["steps/s: " + loop] = round(row["steps_per_s"], 1)
 
     cpu = None
     if not args.no_cpu:
@@ -364,14 +468,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
                    "kernel": "gemm_kernel<false,false,32,true,2,2>: 128x128 tiles, BK=32, v_mfma_f32_32x32x2_f32"},
-        "roofline": {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": head["frac_of_peak"],
-                     "traffic": GEMM_4096_TRAFFIC_BYTES if M == 4096 else None},
+        "roofline": roof,
         "cpu_baseline": cpu,
-        "suite": suite,
     }
     print(json.dumps(line))
-    ctx.close()
 
 
 if __name__ == "__main__":
