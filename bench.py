@@ -74,7 +74,7 @@ def timed(ctx, fn, steps, warmup):
 def pair_times(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
     """HIP-event milliseconds of every one of `iters` launches of fn(), each between its own pair of
     events on the stream it runs on, after `warmup` untimed launches.  sweep: a 1 GiB scratch buffer
-    that is filled between launches, outside the pairs, to push the operands out of L2 and the
+    that is read through between launches, outside the pairs, to push the operands out of L2 and the
     memory-side cache."""
     iters, warmup = max(iters, MIN_ITERS), max(warmup, MIN_WARMUP)
     for _ in range(warmup):
@@ -82,7 +82,10 @@ def pair_times(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
     ev = [(ctx.event(), ctx.event()) for _ in range(iters)]
     for a, b in ev:
         if sweep is not None:
-            ctx.call("slhip_fill", sweep.n, 1.0, sweep.ptr)
+            # a READ of the scratch: it pushes the operands out and leaves no dirty lines behind whose
+            # write-back the timed kernel would have to wait for (a fill as the sweep costs a 64 MiB
+            # read 4 us more than this)
+            ctx.call("slhip_max", sweep.n - 1, sweep.ptr, sweep.view(sweep.n - 1, 1).ptr)
         ctx.record(a)
         fn()
         ctx.record(b)

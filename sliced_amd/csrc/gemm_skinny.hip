@@ -13,6 +13,15 @@
 //             workgroups split K and leave partials in the workspace for the split-K combine.
 //             In a classifier this is the weight gradient of the last layer, H^T * G.
 //
+//   narrow N, A row-major (N <= 16, A * B with A stored M x K): A is the large side again, but now
+//             the reduction runs along its contiguous axis.  The 16-block matrix instruction
+//             (v_mfma_f32_4x4x1: sixteen independent 4 x 4 x 1 products per issue) takes block b as
+//             a k position: lane (b, i) loads a float4 of row i at k = 64 s + 4 b, so a load
+//             instruction of a wave reads 256 contiguous bytes of each of four rows; B's column
+//             groups wait in LDS in the order the B operand wants them; the sixteen blocks'
+//             partial sums meet in four butterfly steps per row group.  In a classifier this is
+//             the forward product of the last layer, H * W.
+//
 // Against the wave-per-tile MFMA kernel, which reads and writes 128-byte pieces per row
 // (MI355X, classifier with batch 8192, hidden 2048, 10 classes): input gradient with the ReLU
 // mask 33 -> 23 us (23 -> 14.5 without the mask), weight gradient with its combine 34.5 -> 29 us;
@@ -239,6 +248,141 @@ __global__ __launch_bounds__(1024) void gemm_narrow_n_kernel(size_t M, int N, si
       if (n < N) out[(size_t)q * N + n] = ((acc[n][q] + red[1][n * 4 + q][lane]) + red[2][n * 4 + q][lane]) + red[3][n * 4 + q][lane];
 }
 
+// C = A * B for a narrow B: A stored M x K (K a multiple of 4), B stored K x N, N <= 4 * G.
+// A workgroup of eight waves stages a k chunk of B in LDS once ([column group][k / 4][column][k % 4],
+// zero beyond N and K, so that the B operand of lane (b, j) for four consecutive k is one
+// ds_read_b128 and a wave's reads are 1 KiB contiguous); a wave takes groups of four rows, issues
+// ALL its loads of a chunk before the first multiply (32 float4 per lane for a chunk of 2048 k:
+// the workgroup's whole share of A is in flight at once) and multiplies them as they arrive.
+constexpr int ROWS_NARROW_KC = 2048;  // k per chunk: 16 KiB of LDS per column of B's groups
+typedef float rn_f4 __attribute__((ext_vector_type(4)));
+
+template <int G>
+__global__ __launch_bounds__(512) void gemm_rows_narrow_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) float rn_b[];  // [G][KC / 4][4][4]
+  constexpr int KC = ROWS_NARROW_KC, KQ = KC / 4, STEPS = KC / 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int b = lane >> 2, ij = lane & 3;  // block of the matrix instruction; row (A operand) or column (B operand, result) in it
+  const size_t M = g.M, K = g.K;
+  const int N = (int)g.N;
+  const size_t groups = (M + 3) / 4;
+  const size_t chunks = (K + KC - 1) / KC;
+  for (size_t grp0 = (size_t)blockIdx.x * 8; grp0 < groups; grp0 += (size_t)gridDim.x * 8) {
+    const size_t grp = grp0 + w;
+    const bool have = grp < groups;
+    const size_t row = have ? (grp * 4 + ij < M ? grp * 4 + ij : M - 1) : 0;
+    rn_f4 acc[G];
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi) acc[gi] = rn_f4{0.f, 0.f, 0.f, 0.f};
+    for (size_t ch = 0; ch < chunks; ++ch) {
+      const size_t k0 = ch * KC;
+      const int klen = (int)(k0 + KC < K ? KC : K - k0);
+      // B's chunk is staged on the first pass, and again whenever the chunk changes (K > KC), BEFORE
+      // the loads of A are issued: a wave's loads return in order, so a load of B behind the loads of A
+      // would not be usable before all of A has arrived.  A thread takes four whole rows of B
+      // (k = thread + 512 r): N loads each, contiguous across the threads and all in flight together,
+      // then 4 * G scattered LDS writes per row, which also lay down the zeros beyond N and K.
+      if (grp0 == (size_t)blockIdx.x * 8 || chunks > 1) {
+        float f[KC / 512][4 * G];
+#pragma unroll
+        for (int r = 0; r < KC / 512; ++r) {
+          const int k = threadIdx.x + 512 * r;
+#pragma unroll
+          for (int n = 0; n < 4 * G; ++n) f[r][n] = (k < klen && n < N) ? g.B[(k0 + k) * (size_t)N + n] : 0.0f;
+        }
+        __syncthreads();  // the previous chunk is done with
+#pragma unroll
+        for (int r = 0; r < KC / 512; ++r) {
+          const int k = threadIdx.x + 512 * r;
+#pragma unroll
+          for (int n = 0; n < 4 * G; ++n) rn_b[(((n >> 2) * KQ + (k >> 2)) * 4 + (n & 3)) * 4 + (k & 3)] = f[r][n];
+        }
+        __syncthreads();
+      }
+      // this lane's share of the chunk in batches of LOADS float4, every batch in flight at once
+      // (16 KiB per wave and batch; with all 32 in flight the accumulators and B's fragments no
+      // longer fit beside them, and a spill's reload in this loop waits for every load of A that is
+      // still in flight)
+      constexpr int LOADS = 16;
+      if (have) {
+#pragma unroll 1
+        for (int s0 = 0; s0 < STEPS && 64 * s0 < klen; s0 += LOADS) {
+          float4 a[LOADS];
+#pragma unroll
+          for (int u = 0; u < LOADS; ++u) {
+            const int k = 64 * (s0 + u) + 4 * b;
+            a[u] = ld4s(g.A + row * K + k0 + (k < klen ? k : klen - 4));
+          }
+#pragma unroll
+          for (int u = 0; u < LOADS; ++u) {
+            const int s = s0 + u;
+            float4 av = a[u];
+            if (64 * s + 4 * b >= klen) av = make_float4(0.f, 0.f, 0.f, 0.f);  // past the end of K: B's zeros alone would not tame an inf
+            float4 bv[G];
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) bv[gi] = ld4(rn_b + ((gi * KQ + 16 * s + b) * 4 + ij) * 4);
+            // consecutive instructions use different accumulators
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) acc[gi] = __builtin_amdgcn_mfma_f32_4x4x1f32(av.x, bv[gi].x, acc[gi], 0, 0, 0);
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) acc[gi] = __builtin_amdgcn_mfma_f32_4x4x1f32(av.y, bv[gi].y, acc[gi], 0, 0, 0);
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) acc[gi] = __builtin_amdgcn_mfma_f32_4x4x1f32(av.z, bv[gi].z, acc[gi], 0, 0, 0);
+#pragma unroll
+            for (int gi = 0; gi < G; ++gi) acc[gi] = __builtin_amdgcn_mfma_f32_4x4x1f32(av.w, bv[gi].w, acc[gi], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (!have) continue;
+    // register v of lane (b, j) in group gi: the sum over block b's k positions for row v, column
+    // 4 gi + j.  Four butterfly steps add the sixteen blocks, in the same order on every lane.
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float x = acc[gi][v];
+        x += __shfl_xor(x, 4, WAVE);
+        x += __shfl_xor(x, 8, WAVE);
+        x += __shfl_xor(x, 16, WAVE);
+        x += __shfl_xor(x, 32, WAVE);
+        acc[gi][v] = x;
+      }
+    if (b != 0) continue;
+    // lanes 0..3 hold everything: every read (mask, C for beta) before the first store
+    float val[G][4];
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const size_t r = grp * 4 + v;
+        const int c = 4 * gi + ij;
+        float x = acc[gi][v];
+        if (r < M && c < N) {
+          const size_t at = r * (size_t)N + c;
+          if (g.mask) x = (g.mask[at] >= 0.0f ? 1.0f : 0.0f) * x;
+          if (g.beta != 0.0f) x = g.beta * g.C[at] + x;
+          if (g.bias) x = x + g.bias[c];
+        }
+        val[gi][v] = x;
+      }
+#pragma unroll
+    for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const size_t r = grp * 4 + v;
+        const int c = 4 * gi + ij;
+        if (r < M && c < N) {
+          const size_t at = r * (size_t)N + c;
+          float x = val[gi][v];
+          if (g.pre_act) g.pre_act[at] = x;
+          if (g.relu) x = (x >= 0.0f ? 1.0f : 0.0f) * x;
+          g.C[at] = x;
+        }
+      }
+  }
+}
+
 // Returns 1 if a skinny kernel took the product (then *rc is its result), 0 if the caller should go on.
 // g carries the operands and the epilogue; g.splits is set for the caller's split-K combine.
 // The short-K kernel if the product qualifies (returns 1, *rc = launch status), else 0.
@@ -278,6 +422,33 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
   const size_t M = g.M, N = g.N, K = g.K;
   // short K: the result is the large side
   if (gemm_short_k_launch(ctx, ta, tb, g, nullptr, rc)) return 1;
+  // narrow N, A row-major: A (M x K) is the large side, the reduction runs along its rows
+  if (!ta && !tb && N <= 16 && K % 4 == 0 && K >= 256 && M >= 32 && M * K >= (size_t(1) << 22)) {
+    const int G = (int)((N + 3) / 4);
+    const size_t lds = (size_t)ROWS_NARROW_KC * 4 * G * sizeof(float);
+    const size_t groups8 = ((M + 3) / 4 + 7) / 8;  // workgroups' worth of row groups
+    // one workgroup per CU (its chunk of B takes 32 KiB of LDS per column group), each looping
+    // over its share of the rows
+    const size_t blocks = groups8 < (size_t)ctx->num_cu ? groups8 : (size_t)ctx->num_cu;
+    const dim3 grid((unsigned)blocks);
+#define SL_RN(G_)                                                                                                        \
+  do {                                                                                                                   \
+    static bool sized = false;                                                                                           \
+    if (!sized) {                                                                                                        \
+      (void)hipFuncSetAttribute((const void*)gemm_rows_narrow_kernel<G_>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                ROWS_NARROW_KC * 16 * G_);                                                              \
+      sized = true;                                                                                                      \
+    }                                                                                                                    \
+    hipLaunchKernelGGL((gemm_rows_narrow_kernel<G_>), grid, dim3(512), lds, ctx->stream, g);                             \
+  } while (0)
+    if (G == 1) SL_RN(1);
+    else if (G == 2) SL_RN(2);
+    else if (G == 3) SL_RN(3);
+    else SL_RN(4);
+#undef SL_RN
+    *rc = post_launch();
+    return 1;
+  }
   // narrow N: A (K x M) is the large side
   if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22) && aligned16(g.A)) {
     const size_t gx = (M / 4 + 63) / 64;

@@ -183,6 +183,38 @@ def test_gemm_skinny_kernels(hip, orc):
         assert np.array_equal(hip.sgemm(1, 0, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
 
 
+def test_gemm_rows_narrow_kernel(hip, orc):
+    """A * B with N <= 16 and a large row-major A (the classifier head's forward product): the
+    sixteen-block matrix-instruction kernel.  N in {1, 3, 10, 16} and the sizes between, K a multiple
+    of 4 that is not one of 64, shorter than a chunk, longer than one and than two, M not a multiple
+    of 4 or of the workgroup's 32 rows, every epilogue, and a row of A that holds an inf (it must not
+    leak into other rows through the zero padding)."""
+    for (m, n, k) in [(8192, 10, 2048), (2049, 1, 2048), (4099, 3, 2052), (33000, 16, 260), (1030, 13, 4100), (2048, 8, 6148),
+                      (4096, 5, 1024), (16385, 12, 256), (3001, 10, 2000), (70000, 2, 64 * 5 + 4)]:
+        say("rows-narrow gemm", m, n, k)
+        a, b = gemm_operands(0, 0, m, n, k)
+        exact, bound = gemm_bound(0, 0, m, n, k, a, b)
+        got = hip.sgemm(0, 0, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        assert np.all(np.abs(got - orc.gemm(m, n, k, a, b)) <= bound)
+        assert np.array_equal(got, hip.sgemm(0, 0, m, n, k, a, b))          # same order of sums on every run
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(0, 0, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(0, 0, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+        bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+        out, pre_act = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+        pre_ref = orc.add_row(m, n, got, bias)
+        assert np.array_equal(pre_act, pre_ref)
+        assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+    m, n, k = 4100, 10, 1000
+    a, b = gemm_operands(0, 0, m, n, k)
+    a = a.copy()
+    a[7 * k + 999] = np.inf          # the last element of row 7: the vector after it is another lane's padding
+    got = hip.sgemm(0, 0, m, n, k, a, b).reshape(m, n)
+    assert np.all(np.isinf(got[7])) and np.all(np.isfinite(np.delete(got, 7, axis=0)))
+
+
 def test_gemm_small_tile(hip, orc):
     # 64 x 64 tiles (chosen by the cost model for products of a few hundred such tiles), forced here
     # so that edge tiles, rows of odd length, k remainders and the fused epilogues all run on them
