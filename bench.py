@@ -20,8 +20,10 @@ The same line carries
                  product through numpy's bundled OpenBLAS (the reference's CPU GEMM is a CBLAS sgemm),
                  the streaming ops and the two training loops.
 Bandwidth ops and sweep entries are timed as the median of per-launch HIP-event pairs over at least
-20 launches after at least 5 warm-ups; operands below 512 MiB have the caches swept (a 1 GiB fill)
-between launches, outside the event pair.  Only one GPU is used; --gpus above 1 is refused.
+20 launches after at least 5 warm-ups; operands below 512 MiB have the caches swept (a read of a
+1 GiB scratch) between launches, outside the event pair.  A per-launch pair contains the launch gap
+(about 6 us: `fill of one element` in the list); the GEMM sweep therefore also reports the rate of
+launches queued back to back inside one pair.  Only one GPU is used; --gpus above 1 is refused.
 """
 import argparse
 import json
@@ -116,7 +118,7 @@ def spin_up(ctx, seconds=0.4):
         x.free()
 
 
-def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headline=False):
+def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headline=False, back_to_back=False):
     a = ctx.uniform(m * k, -1, 1, 0, SEED)
     b = ctx.uniform(k * n, -1, 1, 1, SEED)
     c = ctx.zeros(m * n)
@@ -129,6 +131,11 @@ def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headli
                     "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS})
     med = median_ms(ctx, fn, steps, warmup)
     res.update({"ms_median": med, "tflops_median": flop / med / 1e9, "frac_median": flop / med / 1e9 / FP32_MATRIX_PEAK_TFLOPS})
+    if back_to_back:
+        # launches queued one behind the other inside ONE event pair: the launch gap of about 6 us
+        # that every per-launch pair contains overlaps with the kernel before it
+        _, ev = timed(ctx, fn, steps, warmup)
+        res.update({"ms_back_to_back": ev, "tflops_back_to_back": flop / ev / 1e9})
     if sweep is not None:
         cold = median_ms(ctx, fn, steps, warmup, sweep)
         res.update({"ms_median_caches_swept": cold, "tflops_median_caches_swept": flop / cold / 1e9})
@@ -228,6 +235,14 @@ def bench_bandwidth_suite(ctx, iters):
         a_, b_, c_ = x.view(0, m_ * k_), x.view(m_ * k_, k_ * n_), y.view(0, m_ * n_)
         add("gemm %s [%dx%dx%d]" % (what, m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_),
             lambda: ctx.call("slhip_sgemm", ta, tb, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), iters, sweep=sweep)
+    # what a launch costs in this way of timing, and what a plain streaming kernel reaches on operands
+    # of the head products' size (64 MiB) timed the same way: the lines those three stand against
+    add("fill of one element (the launch floor of a per-launch event pair)", 4, lambda: ctx.call("slhip_fill", 1, 1.0, one.ptr), iters)
+    n64 = 1 << 23
+    add("device copy [64 MiB of traffic] (achievable line at the head products' size)", 8 * n64,
+        lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n64), iters, sweep=sweep)
+    add("sum [64 MiB read] (achievable line for a reduction at that size)", 8 * n64,
+        lambda: ctx.call("slhip_sum", 2 * n64, x.ptr, one.ptr), iters, sweep=sweep)
     sweep.free()
     add("device copy [1 GiB] (achievable line)", 8 * n, lambda: ctx.call("slhip_memcpy_d2d", y.ptr, x.ptr, 4 * n), iters)
     for b in (x, y, vec_c, vec_r, one):
@@ -424,10 +439,12 @@ def main():
         for (m, n, k) in [(512,) * 3, (1024,) * 3, (2048,) * 3, (3584,) * 3, (4095,) * 3, (4608,) * 3, (8192,) * 3,
                           (8192, 2048, 784), (784, 2048, 8192)]:
             for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
-                r = bench_gemm(ctx, m, n, k, ta, tb, iters, MIN_WARMUP)
+                r = bench_gemm(ctx, m, n, k, ta, tb, iters, MIN_WARMUP, back_to_back=True)
                 key = "%dx%dx%d %s" % (m, n, k, form)
-                sweep[key] = {"tflops": r["tflops_median"], "frac": r["frac_median"], "ms": r["ms_median"]}
-                roof["TFLOPs: " + key] = r["tflops_median"]
+                sweep[key] = {"tflops": r["tflops_median"], "frac": r["frac_median"], "ms": r["ms_median"],
+                              "tflops_back_to_back": r["tflops_back_to_back"], "ms_back_to_back": r["ms_back_to_back"]}
+                roof["TFLOPs: " + key] = round(r["tflops_median"], 2)
+                roof["TFLOPs, launches back to back: " + key] = round(r["tflops_back_to_back"], 2)
                 log(key, sweep[key])
         roof["gemm_sweep"] = sweep
     if "bandwidth" in parts:
