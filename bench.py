@@ -260,12 +260,12 @@ def bench_tape_chain(ctx_unused, iters):
         return {"skipped": "%s" % e}
 
 
-def bench_mlp(steps_c5, steps_c1):
+def bench_mlp(steps_c5, steps_c1, graph=True):
     try:
         from sliced_amd import host
     except Exception as e:  # the host layer is optional for the kernel benchmark
         return {"skipped": "host layer not built: %s" % e}
-    return host.bench_mlp(steps_c5, steps_c1)
+    return host.bench_mlp(steps_c5, steps_c1, graph=graph)
 
 
 def cpu_baseline(m, n, k):
@@ -386,6 +386,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="leave out the MLP variants that replay a recorded step (for runs under a kernel tracer, "
+                         "which has crashed inside hipGraphLaunch; the kernels of a step are the same either way)")
     ap.add_argument("--size", type=int, default=4096)
     ap.add_argument("--only", default="", help="comma list of suite parts to run: gemm,sweep,bandwidth,chain,mlp")
     args = ap.parse_args()
@@ -461,7 +464,7 @@ def main():
             if key in ch:
                 roof["GBps: ew chain [2^28], " + key[5:].replace("_", " ")] = round(ch[key], 1)
     if "mlp" in parts:
-        mlp = bench_mlp(50, 200)
+        mlp = bench_mlp(50, 200, graph=not args.no_graph)
         log(mlp)
         roof["mlp"] = mlp
         for loop, row in mlp.items():

@@ -169,6 +169,20 @@ extern "C" {
         pre_act: *mut f32,
         out: *mut f32,
     ) -> i32;
+    pub fn slhip_linear_grad(
+        ctx: *mut SlhipCtx,
+        m: usize,
+        k: usize,
+        n: usize,
+        x: *const f32,
+        w: *const f32,
+        x_grad: *mut f32,
+        relu_pre: *const f32,
+        w_grad: *mut f32,
+        bias_grad: *mut f32,
+        out_grad: *const f32,
+        beta: f32,
+    ) -> i32;
     pub fn slhip_sum_rows(ctx: *mut SlhipCtx, rows: usize, cols: usize, x: *const f32, out: *mut f32) -> i32;
     pub fn slhip_sum_cols(ctx: *mut SlhipCtx, rows: usize, cols: usize, x: *const f32, out: *mut f32) -> i32;
     pub fn slhip_max_rows(ctx: *mut SlhipCtx, rows: usize, cols: usize, x: *const f32, out: *mut f32) -> i32;

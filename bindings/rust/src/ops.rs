@@ -423,6 +423,17 @@ impl<Mods: Retrieve<Self, f32> + 'static> HIP<Mods> {
         check(unsafe { slhip_linear_fwd(self.ctx, m, k, n, x.ptr(), w.ptr(), bias.ptr(), relu as i32, pre, out.ptr_mut()) }).unwrap();
         out
     }
+    /// The backward pass of that Linear: the gradients `gemm` (src/ops2/gemm/grad/cpu_stack.rs:36,39) and
+    /// `add_row_mut` (src/ops2/row_op/grad/cpu.rs:42-50) leave on the tape, for small layers as one launch.
+    /// `relu_pre`: pre-activations of the ReLU that produced `x`; its gradient is then taken on the way.
+    #[allow(clippy::too_many_arguments)]
+    pub fn linear_grad(&self, m: usize, k: usize, n: usize, x: &Buf<Mods>, w: &Buf<Mods>, x_grad: Option<&mut Buf<Mods>>, relu_pre: Option<&Buf<Mods>>, w_grad: Option<&mut Buf<Mods>>, bias_grad: Option<&mut Buf<Mods>>, out_grad: &Buf<Mods>) {
+        let xg = x_grad.map_or(core::ptr::null_mut(), |b| b.ptr_mut());
+        let wg = w_grad.map_or(core::ptr::null_mut(), |b| b.ptr_mut());
+        let bg = bias_grad.map_or(core::ptr::null_mut(), |b| b.ptr_mut());
+        let pre = relu_pre.map_or(core::ptr::null(), |b| b.ptr());
+        check(unsafe { slhip_linear_grad(self.ctx, m, k, n, x.ptr(), w.ptr(), xg, pre, wg, bg, out_grad.ptr(), GRAD_BETA) }).unwrap();
+    }
     /// `cce` of examples/nn.rs:124-138 on the device: loss[r] = -ln sum_c clip(p, 1e-7, 1 - 1e-7) * t.
     pub fn cce(&self, rows: usize, cols: usize, preds: &Buf<Mods>, targets: &Buf<Mods>) -> Buf<Mods> {
         let mut loss = self.retrieve(rows, (preds, targets)).unwrap();

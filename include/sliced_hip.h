@@ -165,6 +165,21 @@ int32_t slhip_gemm_grad(slhip_ctx* ctx, size_t m, size_t k, size_t n, const floa
  * pre_act (may be NULL) receives the value before relu, which the relu gradient needs. */
 int32_t slhip_linear_fwd(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w,
                          const float* bias, int32_t relu, float* pre_act, float* out);
+/* The whole backward pass of that Linear layer, out_grad[m×n] given - the closures that gemm
+ * (GemmGrad, src/ops2/gemm/grad/cpu_stack.rs:36,39) and add_row_mut (add_row_mut_grad,
+ * src/ops2/row_op/grad/cpu.rs:42-50) leave on the tape, and optionally the ReLU closure of the layer
+ * before (src/matrix.rs:169-190):
+ *     x_grad[m×k]  = beta·x_grad + (out_grad·wᵀ) ⊙ (relu_pre >= 0)     (relu_pre NULL: no mask)
+ *     w_grad[k×n]  = beta·w_grad + xᵀ·out_grad
+ *     bias_grad[n] += Σ_r out_grad[r,·]
+ * x_grad, w_grad and bias_grad may each be NULL (that result is skipped).  Layers of up to 2^25
+ * flop whose operands stay below 2^18 elements run as ONE launch (such steps are bound by launch
+ * latency); every other shape runs the same kernels as slhip_add_row_mut_grad, slhip_sgemm /
+ * slhip_sgemm_relu_mask and slhip_sgemm called one after the other.  x_grad and w_grad have the bits
+ * of those calls either way; bias_grad is summed in another order in the single launch.  No
+ * gradient may overlap an input. */
+int32_t slhip_linear_grad(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w, float* x_grad,
+                          const float* relu_pre, float* w_grad, float* bias_grad, const float* out_grad, float beta);
 
 /* ---------------------------------------------------------------- reductions -------
  * SumRows/SumCols (src/ops2/sum/mod.rs:19-25), MaxRows/MaxCols (src/ops2/max/mod.rs:20-26),

@@ -48,6 +48,7 @@ PROTOTYPES = {
     "slhip_gemm": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_gemm_grad": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_linear_fwd": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp],
+    "slhip_linear_grad": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_linear_fwd_bits": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp],
     "slhip_sgemm_relu_bits": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_relu_grad_bits": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],

@@ -42,26 +42,55 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 // hide latency and measured 15-20 % slower with 2, 4 or 8 (8192x10x2048: 41 us against 48).
 // FULL = every k range is a whole number of groups and the k-contiguous operands are float4
 // loadable: no bounds checks, and a k-contiguous operand comes in as one float4 per group.
-template <bool TA, bool TB, int NG, bool FULL>
-__global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
-  extern __shared__ float red[];  // [waves][16][64]
-  const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6, nw = blockDim.x >> 6;
+// COLSUM (the At*B form only): the workgroups of tile row 0 also add the column sums of B over
+// this launch's k range to colsum[N] - the bias gradient of a Linear layer, whose weight gradient
+// xT*g reads the very same g.  `nw` = waves that share this tile's k range; a workgroup may hold
+// more (the pair kernel below), the others only keep the barrier company.
+template <bool TA, bool TB, int NG, bool FULL, bool COLSUM>
+__device__ __forceinline__ void wave_tile(const GemmArgs& g, float* red, const unsigned tile, const unsigned ky, const int nw,
+                                          float* colsum) {
+  const int lane = threadIdx.x & 63, wk = threadIdx.x >> 6;
   const int r = lane & 31, h = lane >> 5;
-  const size_t tm = blockIdx.x / g.tiles_n, tn = blockIdx.x % g.tiles_n;
+  const size_t tm = tile / g.tiles_n, tn = tile % g.tiles_n;
   const size_t m0 = tm * 32, n0 = tn * 32;
-  const size_t kbeg = (size_t)blockIdx.y * g.k_chunk;
+  const size_t kbeg = (size_t)ky * g.k_chunk;
   const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
   const size_t groups = (kend - kbeg + 7) / 8, per = (groups + nw - 1) / nw;
-  const size_t gbeg = wk * per, gend = gbeg + per < groups ? gbeg + per : groups;
+  const size_t gbeg = (size_t)wk * per < groups ? (size_t)wk * per : groups;
+  const size_t gend = gbeg + per < groups ? gbeg + per : groups;  // empty for waves past nw
   // rows / columns past the edge are clamped: they compute copies that are never stored
   const size_t row = m0 + r < g.M ? m0 + r : g.M - 1, col = n0 + r < g.N ? n0 + r : g.N - 1;
   const float* ap = TA ? g.A + row : g.A + row * g.K;
   const float* bp = TB ? g.B + col * g.K : g.B + col;
   const size_t astep = TA ? g.M : 1, bstep = TB ? 1 : g.N;
 
+  // Accumulator register v of lane (r, h): row 8*(v/4) + 4*h + v%4, column r.  With several waves to
+  // a tile, register v is finished by the wave with v % nw == wk (nw is a power of two).  What the
+  // epilogue reads from memory (bias, ReLU mask, C for beta) is requested here, ahead of the k
+  // loop: asked for after it, each of these loads would put one more trip to memory on the
+  // critical path of a kernel that is a handful of such trips long.
+  const bool raw = g.splits > 1;
+  const size_t c = n0 + r;
+  auto idx_of = [&](int v) { return (m0 + 8 * (v / 4) + 4 * h + (v % 4)) * g.N + c; };
+  bool mine[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) mine[v] = (v & (nw - 1)) == wk && m0 + 8 * (v / 4) + 4 * h + (v % 4) < g.M && c < g.N;
+  float bias = 0.0f, mask_v[16], c_old[16];
+  const bool with_mask = !raw && g.mask != nullptr, with_c = !raw && g.beta != 0.0f;
+  if (!raw && g.bias && c < g.N) bias = g.bias[c];
+  if (with_mask) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mask_v[v] = mine[v] ? g.mask[idx_of(v)] : 0.0f;
+  }
+  if (with_c) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) c_old[v] = mine[v] ? g.C[idx_of(v)] : 0.0f;
+  }
+
   floatx16 acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  float cs = 0.0f;  // COLSUM: this lane's share of column n0 + r (its half of every group of 8 k)
   // NG groups of 8 k at a time: all 8*NG loads are issued before the first MFMA needs one
   auto run_groups = [&](size_t gi, auto ng_tag) {
     constexpr int N = decltype(ng_tag)::value;
@@ -99,6 +128,12 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
     for (int u = 0; u < N; ++u)
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
+    if (COLSUM) {
+#pragma unroll
+      for (int u = 0; u < N; ++u)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) cs += b[u][t];
+    }
   };
   size_t gi = gbeg;
   for (; gi + NG <= gend; gi += NG) run_groups(gi, std::integral_constant<int, NG>());
@@ -106,26 +141,30 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
     for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>());
   for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>());
 
+  const bool sums = COLSUM && colsum != nullptr && tm == 0;
+  if (sums) cs += __shfl_xor(cs, 32);  // the two halves of every group of 8 k
   if (nw > 1) {
+    if (wk < nw) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red[(wk * 16 + v) * 64 + lane] = acc[v];
+      for (int v = 0; v < 16; ++v) red[(wk * 16 + v) * 64 + lane] = acc[v];
+      if (sums && h == 0) red[nw * 16 * 64 + wk * 32 + r] = cs;
+    }
     __syncthreads();
   }
-  // accumulator register v of lane (r, h): row 8*(v/4) + 4*h + v%4, column r; the waves share
-  // the 16 registers out between them
-  const bool raw = g.splits > 1;
-  float* dst = raw ? g.partial + (size_t)blockIdx.y * g.M * g.N : g.C;
-  const size_t c = n0 + r;
+  if (wk >= nw) return;
+  if (sums && wk == 0 && h == 0 && n0 + r < g.N) {
+    float t = cs;
+    if (nw > 1) {
+      t = red[nw * 16 * 64 + r];
+      for (int w = 1; w < nw; ++w) t += red[nw * 16 * 64 + w * 32 + r];
+    }
+    colsum[n0 + r] += t;
+  }
+  float* dst = raw ? g.partial + (size_t)ky * g.M * g.N : g.C;
   if (c >= g.N) return;
-  const float bias = (!raw && g.bias) ? g.bias[c] : 0.0f;
-  // Register v goes to the wave with v % nw == wk (nw is a power of two).  As in the tiled kernel's
-  // epilogue, every read (LDS partials, C for beta) comes before the first store.
   float val[16];
-  bool mine[16];
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    const size_t rr = m0 + 8 * (v / 4) + 4 * h + (v % 4);
-    mine[v] = (v & (nw - 1)) == wk && rr < g.M;
     val[v] = acc[v];
     if (nw > 1 && mine[v]) {
       float t = red[v * 64 + lane];
@@ -133,17 +172,14 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
       val[v] = t;
     }
   }
-  auto idx_of = [&](int v) { return (m0 + 8 * (v / 4) + 4 * h + (v % 4)) * g.N + c; };
   if (!raw) {
-    if (g.mask) {
+    if (with_mask) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (mine[v]) val[v] = (g.mask[idx_of(v)] >= 0.0f ? 1.0f : 0.0f) * val[v];
+      for (int v = 0; v < 16; ++v) val[v] = (mask_v[v] >= 0.0f ? 1.0f : 0.0f) * val[v];
     }
-    if (g.beta != 0.0f) {
+    if (with_c) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        if (mine[v]) val[v] = g.beta * g.C[idx_of(v)] + val[v];
+      for (int v = 0; v < 16; ++v) val[v] = g.beta * c_old[v] + val[v];
     }
     if (g.bias) {
 #pragma unroll
@@ -162,6 +198,25 @@ __global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
 #pragma unroll
   for (int v = 0; v < 16; ++v)
     if (mine[v]) dst[idx_of(v)] = val[v];
+}
+
+template <bool TA, bool TB, int NG, bool FULL>
+__global__ __launch_bounds__(1024) void gemm_wave_kernel(GemmArgs g) {
+  extern __shared__ float red[];  // [waves][16][64]
+  wave_tile<TA, TB, NG, FULL, false>(g, red, blockIdx.x, blockIdx.y, blockDim.x >> 6, nullptr);
+}
+
+// Both products of a small Linear layer's backward pass in one launch: workgroups below `tiles_x`
+// compute tiles of x.grad = g*wT (optionally masked by a ReLU's pre-activation), the others tiles of
+// w.grad = xT*g, and those of its first tile row the bias gradient as well.  Each product keeps the
+// plan (waves per tile, order of its sums) that a launch of its own would use, so the results are
+// the same bits; what is saved is two launches per layer of a step that is all launch latency.
+template <bool FULLX, bool FULLW>
+__global__ __launch_bounds__(512) void gemm_wave_pair_kernel(GemmArgs gx, GemmArgs gw, float* colsum, unsigned tiles_x, int nw_x,
+                                                             int nw_w) {
+  extern __shared__ float red[];  // [waves][16][64] + [waves][32]
+  if (blockIdx.x < tiles_x) wave_tile<false, true, 8, FULLX, false>(gx, red, blockIdx.x, 0, nw_x, nullptr);
+  else wave_tile<true, false, 8, FULLW, true>(gw, red, blockIdx.x - tiles_x, 0, nw_w, colsum);
 }
 
 // C = sum_z partial[z] (z ascending) + beta*C, then bias / relu.
@@ -231,6 +286,38 @@ static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) 
   return post_launch();
 }
 
+// Plan of the wave-per-tile kernel for an M x N x K product: waves per workgroup (at most 8 for
+// small problems, where 16 measured 10-15 % slower, at most 16 for large skinny ones, where 8
+// did), each keeping >= 4 groups of 8 k; then whole-grid splits of K until the chip has about 8
+// waves per CU.  A split of a large problem keeps >= 8 groups per wave.  A split of a small one
+// keeps >= 32: up to there the extra groups of an unsplit wave (about 1.2 us per 8) cost less than
+// the combine kernel that a split brings (3-4 us, and one more node in a recorded step).
+// Returns whether the problem counts as small (<= 2^25 flop).
+static bool wave_plan(const slhip_ctx* ctx, size_t M, size_t N, size_t K, unsigned* nw_out, size_t* splits_out,
+                      size_t* k_chunk_out) {
+  const double flop = 2.0 * (double)M * (double)N * (double)K;
+  const size_t tiles = ((M + 31) / 32) * ((N + 31) / 32), groups = (K + 7) / 8;
+  const size_t mn_bytes = M * N * sizeof(float);
+  unsigned nw = 1;
+  const bool small = flop <= 33554432.0;
+  while (nw < (small ? 8u : 16u) && groups >= (size_t)nw * 2 * 4) nw *= 2;
+  size_t splits = 1;
+  const size_t want = (size_t)ctx->num_cu * 8;
+  if (tiles * nw < want) {
+    splits = (want + tiles * nw - 1) / (tiles * nw);
+    const size_t most = groups / ((size_t)nw * (small ? 32 : 8));
+    if (splits > most) splits = most;
+    if (splits > 64) splits = 64;
+    if (splits > ctx->workspace_bytes / mn_bytes) splits = ctx->workspace_bytes / mn_bytes;
+    if (splits < 1) splits = 1;
+  }
+  const size_t k_chunk = ((K + splits - 1) / splits + 7) / 8 * 8;
+  *nw_out = nw;
+  *k_chunk_out = k_chunk;
+  *splits_out = (K + k_chunk - 1) / k_chunk;
+  return small;
+}
+
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
                         float* C, float beta, const float* bias, int relu, float* pre_act, const float* mask) {
   GemmArgs g;
@@ -263,28 +350,10 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       return SLHIP_EINVAL;
     }
     g.tiles_m = (unsigned)wt_m; g.tiles_n = (unsigned)wt_n;
-    const size_t tiles = wt_m * wt_n, groups = (K + 7) / 8;
-    // waves per workgroup (at most 8 for small problems, where 16 measured 10-15 % slower, at
-    // most 16 for large skinny ones, where 8 did): each keeps >= 4 groups of k; then
-    // whole-grid splits of K until the chip has about 8 waves per CU.  A split of a large problem
-    // keeps >= 8 groups per wave.  A split of a small one keeps >= 32: up to there the extra
-    // groups of an unsplit wave (about 1.2 us per 8) cost less than the combine kernel that a
-    // split brings (3-4 us, and one more node in a recorded step)
-    unsigned nw = 1;
-    const bool small = flop <= 33554432.0;
-    while (nw < (small ? 8u : 16u) && groups >= (size_t)nw * 2 * 4) nw *= 2;
-    size_t splits = 1;
-    const size_t want = (size_t)ctx->num_cu * 8;
-    if (tiles * nw < want) {
-      splits = (want + tiles * nw - 1) / (tiles * nw);
-      const size_t most = groups / ((size_t)nw * (small ? 32 : 8));
-      if (splits > most) splits = most;
-      if (splits > 64) splits = 64;
-      if (splits > ctx->workspace_bytes / mn_bytes) splits = ctx->workspace_bytes / mn_bytes;
-      if (splits < 1) splits = 1;
-    }
-    size_t k_chunk = ((K + splits - 1) / splits + 7) / 8 * 8;
-    splits = (K + k_chunk - 1) / k_chunk;
+    const size_t tiles = wt_m * wt_n;
+    unsigned nw;
+    size_t splits, k_chunk;
+    const bool small = wave_plan(ctx, M, N, K, &nw, &splits, &k_chunk);
     g.splits = (unsigned)splits;
     g.k_chunk = k_chunk;
     dim3 wgrid((unsigned)tiles, (unsigned)splits);
@@ -543,6 +612,92 @@ SLHIP_API int32_t slhip_gemm_grad(slhip_ctx* ctx, size_t m, size_t k, size_t n, 
     if (rc) return rc;
   }
   return SLHIP_OK;
+}
+
+namespace slhip {
+
+// Both gradient products (and the bias gradient) of a small layer as one launch of the pair
+// kernel.  Returns false, with nothing launched, unless both products are small problems of the
+// wave-per-tile kernel that need no k split and no skinny kernel would take either.
+static bool linear_grad_pair(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w, float* x_grad,
+                             const float* relu_pre, float* w_grad, float* bias_grad, const float* g, float beta, int32_t* rc) {
+  if (!w_grad) return false;
+  const size_t lim = size_t(1) << 18;  // below every skinny kernel's threshold
+  if (m * k >= lim || k * n >= lim || m * n >= lim || 2.0 * (double)m * (double)k * (double)n > 33554432.0) return false;
+  if (m == 0 || k == 0 || n == 0) return false;
+  GemmArgs gx, gw;
+  unsigned nwx = 1, nww = 1;
+  size_t splits = 1, k_chunk = 0, tiles_x = 0;
+  // x.grad[m x k] = g[m x n] * wT (w stored k x n)
+  if (x_grad) {
+    gx.M = m; gx.N = k; gx.K = n; gx.A = g; gx.B = w; gx.C = x_grad; gx.beta = beta;
+    gx.bias = nullptr; gx.relu = 0; gx.pre_act = nullptr; gx.mask = relu_pre;
+    gx.a_vec = n % 4 == 0; gx.b_vec = n % 4 == 0;
+    gx.m_fast = 0; gx.partial = nullptr;
+    wave_plan(ctx, m, k, n, &nwx, &splits, &k_chunk);
+    if (splits != 1) return false;
+    gx.splits = 1; gx.k_chunk = k_chunk;
+    gx.tiles_m = (unsigned)((m + 31) / 32); gx.tiles_n = (unsigned)((k + 31) / 32);
+    tiles_x = (size_t)gx.tiles_m * gx.tiles_n;
+  } else {
+    gx = GemmArgs();
+  }
+  // w.grad[k x n] = xT * g (x stored m x k)
+  gw.M = k; gw.N = n; gw.K = m; gw.A = x; gw.B = g; gw.C = w_grad; gw.beta = beta;
+  gw.bias = nullptr; gw.relu = 0; gw.pre_act = nullptr; gw.mask = nullptr;
+  gw.a_vec = k % 4 == 0; gw.b_vec = n % 4 == 0;
+  gw.m_fast = 0; gw.partial = nullptr;
+  wave_plan(ctx, k, n, m, &nww, &splits, &k_chunk);
+  if (splits != 1 || nwx > 8 || nww > 8) return false;
+  gw.splits = 1; gw.k_chunk = k_chunk;
+  gw.tiles_m = (unsigned)((k + 31) / 32); gw.tiles_n = (unsigned)((n + 31) / 32);
+  const size_t tiles_w = (size_t)gw.tiles_m * gw.tiles_n;
+  // the unchecked form of each product, as gemm_run decides it: whole groups of 8 k and float4
+  // loads of the k-contiguous operands (g and w rows for x.grad; none for w.grad)
+  const bool fullx = n % 8 == 0 && gx.a_vec && gx.b_vec, fullw = m % 8 == 0;
+  const unsigned nw = nwx > nww ? nwx : nww;
+  const size_t lds = nw > 1 ? ((size_t)nw * 16 * 64 + (size_t)nw * 32) * sizeof(float) : 0;
+  const dim3 grid((unsigned)(tiles_x + tiles_w));
+#define SL_PAIR(FX_, FW_)                                                                                                \
+  hipLaunchKernelGGL((gemm_wave_pair_kernel<FX_, FW_>), grid, dim3(64 * nw), lds, ctx->stream, gx, gw, bias_grad, (unsigned)tiles_x, \
+                     (int)nwx, (int)nww)
+  if (fullx && fullw) SL_PAIR(true, true);
+  else if (fullx) SL_PAIR(true, false);
+  else if (fullw) SL_PAIR(false, true);
+  else SL_PAIR(false, false);
+#undef SL_PAIR
+  *rc = post_launch();
+  return true;
+}
+
+}  // namespace slhip
+
+SLHIP_API int32_t slhip_linear_grad(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w, float* x_grad,
+                                    const float* relu_pre, float* w_grad, float* bias_grad, const float* out_grad, float beta) {
+  size_t mk, kn, mn;
+  SLHIP_REQUIRE(ctx && x && w && out_grad, "null argument");
+  SLHIP_REQUIRE(checked_len(m, k, &mk) && checked_len(k, n, &kn) && checked_len(m, n, &mn), "bad dims");
+  SLHIP_REQUIRE(!relu_pre || x_grad, "a ReLU mask without x_grad");
+  if ((x_grad && (overlaps(x_grad, mk, out_grad, mn) || overlaps(x_grad, mk, w, kn) || overlaps(x_grad, mk, x, mk))) ||
+      (w_grad && (overlaps(w_grad, kn, out_grad, mn) || overlaps(w_grad, kn, x, mk) || overlaps(w_grad, kn, w, kn))) ||
+      (bias_grad && overlaps(bias_grad, n, out_grad, mn))) {
+    set_error("slhip_linear_grad: a gradient overlaps an input");
+    return SLHIP_EALIAS;
+  }
+  int32_t rc = SLHIP_OK;
+  if (linear_grad_pair(ctx, m, k, n, x, w, x_grad, relu_pre, w_grad, bias_grad, out_grad, beta, &rc)) return rc;
+  // the same three results op by op, in the order the tape's own closures run them
+  if (bias_grad) {
+    rc = slhip_add_row_mut_grad(ctx, m, n, bias_grad, out_grad);
+    if (rc) return rc;
+  }
+  if (x_grad) {
+    rc = relu_pre ? slhip_sgemm_relu_mask(ctx, 0, 1, m, k, n, out_grad, w, relu_pre, x_grad, beta)
+                  : slhip_sgemm(ctx, 0, 1, m, k, n, out_grad, w, x_grad, beta);
+    if (rc) return rc;
+  }
+  if (w_grad) rc = slhip_sgemm(ctx, 1, 0, k, n, m, x, out_grad, w_grad, beta);
+  return rc;
 }
 
 SLHIP_API int32_t slhip_linear_fwd(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* x, const float* w,

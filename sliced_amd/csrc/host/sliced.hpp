@@ -462,7 +462,7 @@ class HIP {
       } else {
         g = grad(o);
       }
-      check(slhip_add_row_mut_grad(ctx_, m, n, grad_mut(bb).ptr, g.ptr), "bias grad");
+      float* bg = grad_mut(bb).ptr;
       const bool set = policy.gemm_beta == 0.0f;
       auto producer = relu_pre_.find(xi);
       auto uses = relu_uses_.find(xi);
@@ -472,22 +472,30 @@ class HIP {
                             uses != relu_uses_.end() && uses->second == 1;
       float* xg = xb.requires_grad && !into_pre ? grad_out(xb, set).ptr : nullptr;
       float* wg = wb.requires_grad ? grad_out(wb, set).ptr : nullptr;
-      if (into_pre) {
-        // x is the ReLU output of a fused Linear that is still on the tape
+      auto packed = into_pre ? relu_bits_.find(xi) : relu_bits_.end();
+      if (into_pre && packed != relu_bits_.end()) {
+        // x is the ReLU output of a fused Linear that is still on the tape, its mask one bit an element
         Buffer xp = lookup(producer->second);
-        // written the way gemm_grad writes x.grad (policy.gemm_beta; SET by default): pre.grad is
-        // zero at this point, and `0 + v` differs from `v` only in the sign of a zero
-        auto packed = relu_bits_.find(xi);
-        if (packed != relu_bits_.end())
-          check(slhip_sgemm_relu_bits(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, (const uint32_t*)lookup(packed->second).ptr,
-                                      grad_out(xp, set).ptr, policy.gemm_beta),
-                "slhip_sgemm_relu_bits");
-        else
-          check(slhip_sgemm_relu_mask(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, xp.ptr, grad_out(xp, set).ptr, policy.gemm_beta),
-                "slhip_sgemm_relu_mask");
+        check(slhip_add_row_mut_grad(ctx_, m, n, bg, g.ptr), "bias grad");
+        check(slhip_sgemm_relu_bits(ctx_, 0, 1, m, k, n, g.ptr, wb.ptr, (const uint32_t*)lookup(packed->second).ptr,
+                                    grad_out(xp, set).ptr, policy.gemm_beta),
+              "slhip_sgemm_relu_bits");
+        relu_grad_done_.insert(xi);
+        check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, nullptr, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
+        return;
+      }
+      const float* pre = nullptr;
+      if (into_pre) {
+        // the same with the float pre-activations as the mask.  x.grad goes to pre.grad, written the
+        // way gemm_grad writes x.grad (policy.gemm_beta; SET by default): pre.grad is zero at this
+        // point, and `0 + v` differs from `v` only in the sign of a zero
+        Buffer xp = lookup(producer->second);
+        pre = xp.ptr;
+        xg = grad_out(xp, set).ptr;
         relu_grad_done_.insert(xi);
       }
-      check(slhip_gemm_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, wg, g.ptr, policy.gemm_beta), "slhip_gemm_grad");
+      // bias, input and weight gradient: one launch for small layers, else the three kernels in turn
+      check(slhip_linear_grad(ctx_, m, k, n, xb.ptr, wb.ptr, xg, pre, wg, bg, g.ptr, policy.gemm_beta), "slhip_linear_grad");
     });
     return out;
   }

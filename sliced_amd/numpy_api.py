@@ -379,6 +379,19 @@ def linear_fwd(m, k, n, x, w, bias, relu=False, want_pre_act=False):
         return do.numpy()
 
 
+def linear_grad(m, k, n, x, w, out_grad, x_grad=None, relu_pre=None, w_grad=None, bias_grad=None, beta=0.0):
+    """The backward pass of a Linear layer (slhip_linear_grad): the gradients that are given (as their
+    values before the call) come back updated in place, the others are skipped."""
+    with _Scope() as s:
+        dx, dw, dg = s.up(x), s.up(w), s.up(out_grad)
+        dxg, dpre, dwg, dbg = s.up(x_grad), s.up(relu_pre), s.up(w_grad), s.up(bias_grad)
+        s.c.call("slhip_linear_grad", m, k, n, dx.ptr, dw.ptr, _ptr(dxg), _ptr(dpre), _ptr(dwg), _ptr(dbg), dg.ptr, float(beta))
+        for host, dev in ((x_grad, dxg), (w_grad, dwg), (bias_grad, dbg)):
+            if host is not None:
+                host[:] = dev.numpy().reshape(host.shape)
+    return x_grad, w_grad, bias_grad
+
+
 def linear_fwd_bits(m, k, n, x, w, bias):
     """relu(x·w + bias) and the packed mask (x·w + bias >= 0): uint32 [m][ceil(n / 32)]."""
     words = m * ((n + 31) // 32)

@@ -324,6 +324,49 @@ def test_linear_fwd_fused_equals_gemm_bias_relu(hip, orc):
         assert np.array_equal(out2, pre_ref)
 
 
+def test_linear_grad_one_launch_equals_the_three_ops(hip, orc):
+    """slhip_linear_grad: x.grad and w.grad carry the bits of slhip_sgemm / slhip_sgemm_relu_mask called on
+    their own (small layers run both products in one launch, each with the plan of its own launch);
+    the bias gradient is a sum in another order: within 1e-6 * sum|g| of the oracle's add_row_mut_grad.
+    Shapes: the sine fit's three layers, ragged ones, one that needs the wave kernel's checked form,
+    one too large for the single launch (it takes the three kernels in turn)."""
+    for (m, k, n) in [(1024, 1, 64), (1024, 64, 64), (1024, 64, 1), (1000, 37, 13), (7, 5, 3), (33, 65, 31), (200, 96, 40),
+                      (4096, 63, 17), (8192, 256, 10)]:
+        for beta in (0.0, 1.0):
+            for masked in (False, True):
+                say("linear_grad", m, k, n, "beta", beta, "masked", masked)
+                x = rng.uniform(m * k, -1, 1, tag=0, seed=SEED)
+                w = rng.uniform(k * n, -1, 1, tag=1, seed=SEED)
+                g = rng.normal(m * n, 1.0, tag=2, seed=SEED)
+                pre = rng.normal(m * k, 1.0, tag=3, seed=SEED) if masked else None
+                xg0 = rng.uniform(m * k, -1, 1, tag=4, seed=SEED)
+                wg0 = rng.uniform(k * n, -1, 1, tag=5, seed=SEED)
+                bg0 = rng.uniform(n, -1, 1, tag=6, seed=SEED)
+                xg, wg, bg = xg0.copy(), wg0.copy(), bg0.copy()
+                hip.linear_grad(m, k, n, x, w, g, x_grad=xg, relu_pre=pre, w_grad=wg, bias_grad=bg, beta=beta)
+                if masked:
+                    xg_ref = hip.sgemm_relu_mask(0, 1, m, k, n, g, w, pre, c=xg0.copy(), beta=beta)
+                else:
+                    xg_ref = hip.sgemm(0, 1, m, k, n, g, w, c=xg0.copy(), beta=beta)
+                wg_ref = hip.sgemm(1, 0, k, n, m, x, g, c=wg0.copy(), beta=beta)
+                assert np.array_equal(xg, np.asarray(xg_ref).ravel())
+                assert np.array_equal(wg, np.asarray(wg_ref).ravel())
+                bg_ref = bg0.copy()
+                orc.add_row_mut_grad(m, n, bg_ref, g)
+                bound = 1e-6 * (np.abs(g.reshape(m, n)).sum(axis=0) + np.abs(bg0)) + 1e-30
+                assert np.all(np.abs(bg - bg_ref) <= bound), np.abs(bg - bg_ref).max()
+                exact = bg0.astype(np.float64) + g.reshape(m, n).astype(np.float64).sum(axis=0)
+                assert np.all(np.abs(bg - exact) <= bound)
+                # a layer whose input needs no gradient: only w.grad and the bias gradient
+                wg2, bg2 = wg0.copy(), bg0.copy()
+                hip.linear_grad(m, k, n, x, w, g, w_grad=wg2, bias_grad=bg2, beta=beta)
+                assert np.array_equal(wg2, wg)
+                assert np.array_equal(bg2, bg)
+    with pytest.raises(Exception):
+        hip.linear_grad(4, 4, 4, np.zeros(16, np.float32), np.zeros(16, np.float32), np.zeros(16, np.float32),
+                        relu_pre=np.zeros(16, np.float32), w_grad=np.zeros(16, np.float32))
+
+
 # --------------------------------------------------------------------------- reductions
 RED_SHAPES = [(1, 1), (1, 5), (5, 1), (3, 4), (7, 13), (64, 64), (33, 1000), (1000, 33), (257, 4096), (4096, 257),
               (16, 40000), (40000, 16), (2, 300001), (300001, 2), (1, 1 << 20), (1 << 20, 1), (2048, 2048),
