@@ -54,6 +54,7 @@ pub const SLHIP_TAIL_SPREAD: i32 = 2;
 pub const SLHIP_TILE_AUTO: i32 = 0;
 pub const SLHIP_TILE_128X128: i32 = 1;
 pub const SLHIP_TILE_64X64: i32 = 3;
+pub const SLHIP_TILE_128X128_WIDE: i32 = 4;
 
 /// Elementwise programs (slhip_ew_program): limits, the unary marker or-ed into `op`, the flag
 /// that stops the gradient at an instruction.

@@ -524,6 +524,15 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % tile_m == 0 && N % tile_n == 0 && K % BK == 0;
   if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tiles - sp.first);
 
+  // One workgroup per CU at most (and the 128 x 128 tile): the eight-wave kernel
+  const bool wide_fits = !small_tile && !(ta && tb);
+  if (wide_fits && (ctx->gemm_tile == SLHIP_TILE_128X128_WIDE ||
+                    (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && tiles * splits <= (size_t)ctx->num_cu))) {
+    int32_t rc = gemm_wide_launch(ctx, ta, tb, only_fast, g);
+    if (rc || splits == 1) return rc;
+    return splitk_combine(ctx, g, splits);
+  }
+
   dim3 grid((unsigned)tiles, (unsigned)splits);
 #define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                  \
   do {                                                                                                                \
@@ -588,7 +597,9 @@ SLHIP_API int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy) {
 
 SLHIP_API int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy) {
   SLHIP_REQUIRE(ctx, "null argument");
-  SLHIP_REQUIRE(policy == SLHIP_TILE_AUTO || policy == SLHIP_TILE_128X128 || policy == SLHIP_TILE_64X64, "unknown policy");
+  SLHIP_REQUIRE(policy == SLHIP_TILE_AUTO || policy == SLHIP_TILE_128X128 || policy == SLHIP_TILE_64X64 ||
+                    policy == SLHIP_TILE_128X128_WIDE,
+                "unknown policy");
   ctx->gemm_tile = policy;
   return SLHIP_OK;
 }

@@ -4,9 +4,10 @@
 // on purpose: the plain kernel's k loop gains or loses about 1.5 % with the code the compiler
 // happens to place around it, and a kernel added to its file moved it.
 //
-// A workgroup is 4 waves in a 2 x 2 grid; every wave owns WM x WN accumulators of 32 x 32, so the
-// workgroup's tile of C is (64*WM) x (64*WN): 128 x 128 for large products, 128 x 64 and 64 x 64
-// for products whose 128 x 128 grid would leave most of the chip idle.
+// A workgroup is WGM x WGN waves (2 x 2 unless said otherwise); every wave owns WM x WN
+// accumulators of 32 x 32, so the workgroup's tile of C is (32*WM*WGM) x (32*WN*WGN): 128 x 128
+// for large products, 64 x 64 for products whose 128 x 128 grid would leave most of the chip idle,
+// and 128 x 128 on eight waves (2 x 4, each 64 x 32) for grids that give a CU a single workgroup.
 #pragma once
 #include <type_traits>
 
@@ -19,13 +20,13 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int BM = 128, BN = 128;
 constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form at 2048^3 and above
 
-// One operand tile: XT rows or columns of the operand (64 or 128) by BK of k.
-template <int BK, int XT>
+// One operand tile: XT rows or columns of the operand (64 or 128) by BK of k, staged by NT threads.
+template <int BK, int XT, int NT = 256>
 struct Cfg {
   static constexpr int KC_PITCH = BK + 4;  // [x][k] layout, k contiguous
   static constexpr int XC_PITCH = XT + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
   static constexpr int STAGE_FLOATS = XT * KC_PITCH > BK * XC_PITCH ? XT * KC_PITCH : BK * XC_PITCH;
-  static constexpr int NV = BK * XT / 4 / 256;  // float4 per thread per operand tile
+  static constexpr int NV = BK * XT / 4 / NT;  // float4 per thread per operand tile
 };
 
 struct GemmArgs {
@@ -57,9 +58,9 @@ struct SpreadArgs {
 constexpr size_t SPREAD_SLOT = (size_t)BM * BN;  // floats of one partial tile in the workspace
 
 // Operand tile held in registers between the global load and the LDS store.
-template <int BK, int XT>
+template <int BK, int XT, int NT = 256>
 struct Frag {
-  float4 v[Cfg<BK, XT>::NV];
+  float4 v[Cfg<BK, XT, NT>::NV];
 };
 
 // How a k tile is fetched from global memory.
@@ -82,13 +83,13 @@ struct Frag {
 enum { LOAD_FAST = 0, LOAD_VCLAMP = 1, LOAD_SCALAR = 2, LOAD_XCLAMP = 3 };
 
 // k-contiguous source: element (x, k) at src[x*ld + k]; tile XT x BK.
-template <int BK, int XT, int MODE>
-__device__ __forceinline__ void load_kc(Frag<BK, XT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+template <int BK, int XT, int MODE, int NT = 256>
+__device__ __forceinline__ void load_kc(Frag<BK, XT, NT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
-  constexpr int VPR = BK / 4, RPP = 256 / VPR;  // float4 per row, rows per pass
+  constexpr int VPR = BK / 4, RPP = NT / VPR;  // float4 per row, rows per pass
   const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) {
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) {
     const size_t x = x0 + xr + RPP * p, k = k0 + 4 * kq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + x * ld + k);
@@ -113,23 +114,23 @@ __device__ __forceinline__ void load_kc(Frag<BK, XT>& f, const float* __restrict
     }
   }
 }
-template <int BK, int XT>
-__device__ __forceinline__ void store_kc(const Frag<BK, XT>& f, float* lds) {
-  constexpr int VPR = BK / 4, RPP = 256 / VPR;
+template <int BK, int XT, int NT = 256>
+__device__ __forceinline__ void store_kc(const Frag<BK, XT, NT>& f, float* lds) {
+  constexpr int VPR = BK / 4, RPP = NT / VPR;
   const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK, XT>::KC_PITCH + 4 * kq, f.v[p]);
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(lds + (xr + RPP * p) * Cfg<BK, XT>::KC_PITCH + 4 * kq, f.v[p]);
 }
 
 // x-contiguous source: element (x, k) at src[k*ld + x]; tile BK x XT.  LOAD_VCLAMP relies on
 // X % 4 == 0 (implied by ld % 4 == 0, ld being X here): a float4 is inside or outside as a whole.
-template <int BK, int XT, int MODE>
-__device__ __forceinline__ void load_xc(Frag<BK, XT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
+template <int BK, int XT, int MODE, int NT = 256>
+__device__ __forceinline__ void load_xc(Frag<BK, XT, NT>& f, const float* __restrict__ src, size_t ld, size_t X, size_t Kend,
                                         size_t x0, size_t k0) {
-  constexpr int XQ = XT / 4, KR = 256 / XQ;  // float4 per k-row (32 or 16), k-rows per pass (8 or 16)
+  constexpr int XQ = XT / 4, KR = NT / XQ;  // float4 per k-row (32 or 16), k-rows per pass (8 or 16)
   const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) {
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) {
     const size_t k = k0 + kr + KR * p, x = x0 + 4 * xq;
     if (MODE == LOAD_FAST) {
       f.v[p] = ld4(src + k * ld + x);
@@ -153,12 +154,12 @@ __device__ __forceinline__ void load_xc(Frag<BK, XT>& f, const float* __restrict
     }
   }
 }
-template <int BK, int XT>
-__device__ __forceinline__ void store_xc(const Frag<BK, XT>& f, float* lds) {
-  constexpr int XQ = XT / 4, KR = 256 / XQ;
+template <int BK, int XT, int NT = 256>
+__device__ __forceinline__ void store_xc(const Frag<BK, XT, NT>& f, float* lds) {
+  constexpr int XQ = XT / 4, KR = NT / XQ;
   const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
 #pragma unroll
-  for (int p = 0; p < Cfg<BK, XT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
 }
 
 // MFMA fragments of one 8-wide k group for the NI 32-row blocks of this wave's rows (or columns).
@@ -220,33 +221,34 @@ constexpr int PIN_SMALL[2][2] = {{0, 0}, {0, 0}};      // the 64 x 64 tile's loo
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
 // ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
 // kernel's throughput.
-template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST, int WM, int WN>
+template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
 __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
-                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
-                                           float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
-  constexpr int TM = 64 * WM, TN = 64 * WN;  // the workgroup's tile of C
+                                           size_t m0, size_t n0, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
+                                           float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
+  constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;  // the workgroup's tile of C
+  constexpr int NT = 64 * WGM * WGN;                      // its threads
   constexpr int KSTEPS = BK / 8;
   constexpr int REFILL_AT = (TA && !TB) ? KSTEPS - 1 : (KSTEPS > 1 ? 1 : 0);
   if (kt_begin >= kt_end) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
   // A is KC ([m][k], ld = K) unless transposed ([k][m], ld = M); B is XC ([k][n], ld = N)
   // unless transposed ([n][k], ld = K).
   const size_t lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
 
-  Frag<BK, TM> fa;
-  Frag<BK, TN> fb;
+  Frag<BK, TM, NT> fa;
+  Frag<BK, TN, NT> fb;
   auto load_stage = [&](int kt) {
     const size_t k0 = kbeg + (size_t)kt * BK;
-    if (TA) load_xc<BK, TM, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    else load_kc<BK, TM, MODE>(fa, g.A, lda, g.M, kend, m0, k0);
-    if (TB) load_kc<BK, TN, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
-    else load_xc<BK, TN, MODE>(fb, g.B, ldb, g.N, kend, n0, k0);
+    if (TA) load_xc<BK, TM, MODE, NT>(fa, g.A, lda, g.M, kend, m0, k0);
+    else load_kc<BK, TM, MODE, NT>(fa, g.A, lda, g.M, kend, m0, k0);
+    if (TB) load_kc<BK, TN, MODE, NT>(fb, g.B, ldb, g.N, kend, n0, k0);
+    else load_xc<BK, TN, MODE, NT>(fb, g.B, ldb, g.N, kend, n0, k0);
   };
   auto store_stage = [&](int s) {
-    if (TA) store_xc<BK, TM>(fa, lds_a[s]); else store_kc<BK, TM>(fa, lds_a[s]);
-    if (TB) store_kc<BK, TN>(fb, lds_b[s]); else store_xc<BK, TN>(fb, lds_b[s]);
+    if (TA) store_xc<BK, TM, NT>(fa, lds_a[s]); else store_kc<BK, TM, NT>(fa, lds_a[s]);
+    if (TB) store_kc<BK, TN, NT>(fb, lds_b[s]); else store_xc<BK, TN, NT>(fb, lds_b[s]);
   };
 
   // Software pipeline over the k tiles.  While tile kt is multiplied out of LDS stage s:
@@ -264,7 +266,7 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   if (kt_begin + 1 < kt_end) load_stage(kt_begin + 1);
   __syncthreads();
 
-  constexpr bool BIG = WM == 2 && WN == 2;
+  constexpr bool BIG = WM == 2 && WN == 2 && WGM == 2 && WGN == 2;
   if (MODE == LOAD_FAST) pin_loop_start<!BIG ? PIN_SMALL[TA][TB] : ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
   if (MODE == LOAD_XCLAMP) pin_loop_start<BIG ? PIN_XCLAMP[TA][TB] : PIN_SMALL[TA][TB]>();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
@@ -312,16 +314,16 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 // ONLY_FAST: the host has checked that every k tile of every tile qualifies for LOAD_FAST (M and N
 // multiples of 128, every k chunk a multiple of BK, operands float4-loadable and 16-byte aligned);
 // the kernel then contains that one loop and nothing else.
-template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
 __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, size_t kbeg, size_t kend, size_t m0,
-                                             size_t n0, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
-                                             float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
+                                             size_t n0, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
+                                             float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
   if (ONLY_FAST) {
-    gemm_tiles<TA, TB, BK, LOAD_FAST, true, WM, WN>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+    gemm_tiles<TA, TB, BK, LOAD_FAST, true, WM, WN, WGM, WGN>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
     return;
   }
   const bool vec = g.a_vec && g.b_vec;
-  const bool fast = vec && m0 + 64 * WM <= g.m_fast && n0 + 64 * WN <= g.N;
+  const bool fast = vec && m0 + 32 * WM * WGM <= g.m_fast && n0 + 32 * WN * WGN <= g.N;
   const int kfull = (int)((kend - kbeg) / BK);             // complete k tiles of the chunk
   const int before_last = (int)((g.K - 1 - kbeg) / BK);    // k tiles that end before index K - 1
   int e1 = fast ? (kb < kfull ? kb : kfull) : ka;
@@ -332,18 +334,18 @@ __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, 
     if (e2 < e1) e2 = e1;
   }
   const int e3 = vec ? kb : e2;
-  gemm_tiles<TA, TB, BK, LOAD_FAST, false, WM, WN>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false, WM, WN>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false, WM, WN>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false, WM, WN>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_FAST, false, WM, WN, WGM, WGN>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false, WM, WN, WGM, WGN>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false, WM, WN, WGM, WGN>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false, WM, WN, WGM, WGN>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 }
 
 // A workgroup that computes one whole tile of C (or, with g.splits > 1, one k chunk of it as a raw
 // partial product): blockIdx.x = tile, blockIdx.y = k chunk.
-template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
-__device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
-                                                float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS]) {
-  constexpr int TM = 64 * WM, TN = 64 * WN;
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
+__device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
+                                                float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS]) {
+  constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;
   unsigned tm, tn;
   tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
   const size_t m0 = (size_t)tm * TM, n0 = (size_t)tn * TN;
@@ -352,7 +354,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
 
   floatx16 acc[WM][WN];
@@ -363,7 +365,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's (32*WM) x (32*WN) tile.
@@ -423,6 +425,9 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
 // The K <= 12 kernel alone, with the mask of the product given as bits (row-major, 32 columns to a
 // word) or NULL.  Returns 1 if it took the product (*rc = launch status), else 0.
 int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const uint32_t* bits, int32_t* rc);
+
+// gemm_wide.hip: the 128 x 128 tile on eight waves, g planned as for the four-wave kernel.
+int32_t gemm_wide_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
 
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
                            const SpreadArgs& sp, size_t workers, size_t tail_tiles);

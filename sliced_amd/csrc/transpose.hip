@@ -1,7 +1,7 @@
 // Matrix transpose through a padded LDS tile: out[c*rows + r] = x[r*cols + c].
 //
 // A tile covers 256 input rows x 64 input columns.  It is read with streaming float4 loads
-// along the input rows (256-byte pieces), staged in LDS with a row pitch of 65 words, and written
+// along the input rows (256-byte pieces), staged in LDS (rows permuted and skewed so that neither side meets bank conflicts), and written
 // with streaming float4 stores along the output rows: every output row of the tile receives 256
 // consecutive floats, a full 1 KiB burst.  Workgroups are numbered down the input rows first, so
 // that neighbouring workgroups extend each other's output bursts.  On MI355X the long write
@@ -21,7 +21,14 @@ constexpr int TC = 64;   // input columns per tile
 template <bool VEC_LD, bool VEC_ST, bool ACC>
 __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols, const float* __restrict__ x,
                                                         float* out, unsigned tiles_r, unsigned group) {
-  __shared__ float tile[TR][TC + 1];
+  // Tile element (r, c) lives at ((r % 4) * 64 + r / 4) * 65 + c + 17 * (r % 4).  The store side of
+  // the kernel has lane l fetch rows 4l .. 4l+3 of one column: with plain [r][c] rows, whatever the
+  // pitch, lanes 8 apart meet on the same bank (four to a bank); here lane l's four rows sit 65 words
+  // from lane l+1's, one bank further on.  The 17 * (r % 4) skew keeps the load side, where a wave
+  // writes four consecutive rows at a time (vector form) or 64 (scalar form reads them back), on
+  // distinct banks as well.
+  __shared__ float tile_mem[TR * (TC + 1) + 52];
+  auto tile = [&](int r, int c) -> float& { return tile_mem[((r & 3) * (TR / 4) + (r >> 2)) * (TC + 1) + c + 17 * (r & 3)]; };
   // tiles are walked in groups of `group` tile rows, row index fastest (group = tiles_r: straight
   // down the rows, column by column)
   const unsigned tiles_c = gridDim.x / tiles_r, in_group = group * tiles_c;
@@ -58,10 +65,10 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 #pragma unroll
     for (int p = 0; p < TR / 16; ++p) {
       const int rr = ly + 16 * p;
-      tile[rr][4 * lx + 0] = v[p].x;
-      tile[rr][4 * lx + 1] = v[p].y;
-      tile[rr][4 * lx + 2] = v[p].z;
-      tile[rr][4 * lx + 3] = v[p].w;
+      tile(rr, 4 * lx + 0) = v[p].x;
+      tile(rr, 4 * lx + 1) = v[p].y;
+      tile(rr, 4 * lx + 2) = v[p].z;
+      tile(rr, 4 * lx + 3) = v[p].w;
     }
   } else {
     const int lx = t & 63, ly = t >> 6;  // 64 columns, 4 rows per pass
@@ -69,7 +76,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
     for (int p = 0; p < TR / 4; ++p) {
       const int rr = ly + 4 * p;
       const size_t r = r0 + rr, c = c0 + lx;
-      tile[rr][lx] = (r < rows && c < cols) ? x[r * cols + c] : 0.0f;
+      tile(rr, lx) = (r < rows && c < cols) ? x[r * cols + c] : 0.0f;
     }
   }
   __syncthreads();
@@ -91,7 +98,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
       const int cc = ly + 4 * p;  // input column = output row
       const size_t oc = c0 + cc;
       if (oc < cols && orow0 < rows) {
-        float4 v = make_float4(tile[4 * lx + 0][cc], tile[4 * lx + 1][cc], tile[4 * lx + 2][cc], tile[4 * lx + 3][cc]);
+        float4 v = make_float4(tile(4 * lx + 0, cc), tile(4 * lx + 1, cc), tile(4 * lx + 2, cc), tile(4 * lx + 3, cc));
         float* p_out = out + oc * rows + orow0;
         if (orow0 + 3 < rows) {
           if (ACC) { v.x += old[p].x; v.y += old[p].y; v.z += old[p].z; v.w += old[p].w; }
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
     for (int p = 0; p < TC; ++p) {  // one output row per pass, 256 consecutive floats
       const size_t oc = c0 + p, orow = r0 + t;
       if (oc < cols && orow < rows) {
-        float v = tile[t][p];
+        float v = tile(t, p);
         float* p_out = out + oc * rows + orow;
         if (ACC) v += *p_out;
         *p_out = v;

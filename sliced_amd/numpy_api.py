@@ -335,7 +335,7 @@ def gemm_tail_policy(policy):
     ctx().call("slhip_gemm_tail_policy", int(policy))
 
 
-TILE_AUTO, TILE_128X128, TILE_64X64 = 0, 1, 3
+TILE_AUTO, TILE_128X128, TILE_64X64, TILE_128X128_WIDE = 0, 1, 3, 4
 
 
 def gemm_tile_policy(policy):

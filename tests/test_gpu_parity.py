@@ -264,6 +264,42 @@ def test_gemm_small_tile(hip, orc):
         hip.gemm_tail_policy(hip.TAIL_AUTO)
 
 
+def test_gemm_eight_wave_tile(hip, orc):
+    # The 128 x 128 tile on eight waves (chosen on its own when the tile grid gives a CU at most one
+    # workgroup), forced here so that edge tiles, rows of odd length, k remainders, one to five k
+    # tiles (the pipeline's prologue cases), k splits and the fused
+    # epilogues all run on it.  With whole tiles and no k split it sums in the four-wave kernel's order.
+    shapes = [(1000, 1000, 512, 0, 0), (1024, 1024, 1024, 0, 1), (999, 1001, 515, 1, 0), (640, 384, 300, 0, 0),
+              (129, 257, 4099, 0, 1), (2048, 192, 777, 1, 0), (130, 2000, 333, 0, 0), (256, 256, 32, 0, 0),
+              (256, 256, 64, 1, 0), (256, 384, 96, 0, 1), (256, 256, 130, 0, 0), (384, 256, 160, 1, 0),
+              (2048, 2048, 2048, 0, 0)]
+    try:
+        for (m, n, k, ta, tb) in shapes:
+            say("eight-wave gemm", m, n, k, ta, tb)
+            a, b = gemm_operands(ta, tb, m, n, k)
+            exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+            hip.gemm_tile_policy(hip.TILE_128X128_WIDE)
+            hip.gemm_tail_policy(hip.TAIL_WHOLE)
+            got = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+            c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+            assert np.array_equal(hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+            pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+            assert np.array_equal(hip.sgemm_relu_mask(ta, tb, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+            if not ta and not tb:
+                bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+                out, pre_act = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+                pre_ref = orc.add_row(m, n, got, bias)
+                assert np.array_equal(pre_act, pre_ref)
+                assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+            hip.gemm_tile_policy(hip.TILE_128X128)
+            four = hip.sgemm(ta, tb, m, n, k, a, b)
+            assert np.array_equal(got, four)       # the same k order per element, split or not
+    finally:
+        hip.gemm_tile_policy(hip.TILE_AUTO)
+        hip.gemm_tail_policy(hip.TAIL_AUTO)
+
+
 def test_sgemm_relu_mask_equals_gemm_then_relu_grad(hip, orc):
     # every kernel that has the epilogue: wave per tile, tiled, split K, spread tail
     shapes = [(64, 64, 64, 0, 1), (1024, 64, 64, 0, 1), (100, 37, 19, 0, 0), (256, 256, 4096, 0, 1), (640, 384, 300, 0, 1),
@@ -883,7 +919,7 @@ def test_invalid_arguments_return_status_not_crash(hip):
     assert lib.slhip_transpose(c.h, 4, 4, x.ptr, x.ptr, 0.0) == -4
     assert lib.slhip_ew_unary(c.h, 99, 0.0, 0.0, 4, x.ptr, x.ptr) == -1
     assert lib.slhip_gemm_tail_policy(c.h, 7) == -1                      # unknown policies
-    assert lib.slhip_gemm_tile_policy(c.h, 2) == -1
+    assert lib.slhip_gemm_tile_policy(c.h, 2) == -1 and lib.slhip_gemm_tile_policy(c.h, 5) == -1
     assert lib.slhip_gemm_tail_policy(c.h, 0) == 0 and lib.slhip_gemm_tile_policy(c.h, 0) == 0
     y = c.empty(16)
     assert lib.slhip_sgemm_relu_mask(c.h, 0, 0, 2, 2, 2, x.ptr, x.ptr, y.ptr, y.ptr, 0.0) == -4   # C aliases pre
