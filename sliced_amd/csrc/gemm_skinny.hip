@@ -162,90 +162,132 @@ __global__ __launch_bounds__(256) void gemm_short_k_kernel(size_t M, size_t N, i
   }
 }
 
-constexpr int NARROW_K_CHUNK = 1024;  // most k a workgroup of the narrow-N kernel covers (its slice of B sits in LDS)
-
-// dst = A^T * B over the k range of this workgroup (blockIdx.y), A stored K x M, B stored K x N.
-// U = loads of A in flight per lane.
-template <int NP, int U>
-__global__ __launch_bounds__(1024) void gemm_narrow_n_kernel(size_t M, int N, size_t K, const float* __restrict__ A,
-                                                             const float* __restrict__ B, float* __restrict__ dst,
-                                                             size_t k_chunk) {
-  // first the workgroup's slice of B, [k][NP] with zeros beyond N and beyond the slice's end: all
-  // lanes of a wave read the same row at the same time; then, the k loop done, the partial sums
-  // of the waves: [4][NP * 4][64]
-  __shared__ __attribute__((aligned(16))) float sh[NARROW_K_CHUNK * NP];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+// partial[z] = A^T * B over the k range of workgroup z = blockIdx.y: A stored K x M, B stored K x N,
+// N <= NP <= 16.  A lane owns four columns of A and 4 x NP sums; a wave walks down its share of the
+// k range with eight float4 loads of A per batch, 1 KiB contiguous per load and wave, the next
+// batch requested before the current one is multiplied and the first before anything else: the
+// workgroup's slice of B (one contiguous run of k_chunk * N floats) goes into LDS as [k][NP] rows,
+// zero beyond N and beyond the end of K, behind those loads.  In the loop a row of B is NP / 4
+// broadcast ds_read_b128.  The eight waves of a workgroup then add their sums in wave order
+// through LDS (one barrier) and wave 0 writes them as [M][NP] rows - the 4 x NP sums of a lane are
+// contiguous there, NP float4 stores; narrow_n_combine_kernel adds the workgroups' partials in a
+// fixed order.
+constexpr int NARROW_WAVES = 8;      // waves per workgroup
+constexpr int NARROW_BATCH = 8;      // rows of A per batch and wave
+constexpr int NARROW_K_CHUNK = 512;  // most k per workgroup (its rows of B sit in LDS)
+template <int NP>
+__global__ __launch_bounds__(64 * NARROW_WAVES) void gemm_narrow_n_kernel(size_t M, int N, size_t K, const float* __restrict__ A,
+                                                                          const float* __restrict__ B,
+                                                                          float* __restrict__ partial, size_t k_chunk) {
+  constexpr int U = NP > 12 ? NARROW_BATCH / 2 : NARROW_BATCH, Q = NP / 4;  // sixteen columns: 64 sums a lane, half the batch
+  __shared__ __attribute__((aligned(16))) float4 red[NARROW_WAVES - 1][NP][64];
+  __shared__ __attribute__((aligned(16))) float bsh[NARROW_K_CHUNK * NP];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const size_t m = ((size_t)blockIdx.x * 64 + lane) * 4;
   const bool active = m < M;
-  const size_t mc = active ? m : 0;
+  // lanes past the last column read the last whole vector of the row again and are never stored
+  const size_t mc = active ? m : M - 4;
   const size_t kbeg = (size_t)blockIdx.y * k_chunk;
   const size_t kend = kbeg + k_chunk < K ? kbeg + k_chunk : K;
   const int klen = (int)(kend - kbeg);
-  const int kpad = (klen + 16 * U - 1) / (16 * U) * (16 * U);  // whole passes: the rows beyond klen are zero
-  for (int idx = threadIdx.x; idx < kpad * NP; idx += 1024) {
-    const int k = idx / NP, n = idx % NP;
-    sh[idx] = (k < klen && n < N) ? B[(kbeg + k) * (size_t)N + n] : 0.0f;
-  }
-  __syncthreads();
-  float acc[NP][4];
+  const int per_wave = (int)(k_chunk / NARROW_WAVES);  // a multiple of 2 * U
+  const int k_first = w * per_wave, k_last = k_first + per_wave;  // relative to kbeg; rows from klen on are zero in LDS
+  float4 acc[NP];
 #pragma unroll
-  for (int n = 0; n < NP; ++n)
+  for (int n = 0; n < NP; ++n) acc[n] = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto load_batch = [&](float4 (&a)[U], int k0) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) acc[n][q] = 0.0f;
-  // the sixteen waves take passes of U consecutive k in turn
-  for (int k0 = U * w; k0 < klen; k0 += 16 * U) {
-    float4 a[U];
+    for (int u = 0; u < U; ++u) a[u] = ld4s(A + (kbeg + (k0 + u < klen ? k0 + u : klen - 1)) * M + mc);
+  };
+  auto multiply_batch = [&](const float4 (&a)[U], int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kk = k0 + u < klen ? k0 + u : klen - 1;  // past the end: any row, its B row is zero
-      a[u] = ld4s(A + (kbeg + kk) * M + mc);
-    }
+      const float4* brow = reinterpret_cast<const float4*>(bsh + (size_t)(k0 + u) * NP);  // wave-uniform
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+      for (int q = 0; q < Q; ++q) {
+        const float4 bq = brow[q];
+        const float bv[4] = {bq.x, bq.y, bq.z, bq.w};
 #pragma unroll
-      for (int n = 0; n < NP; ++n) {
-        const float bv = sh[(k0 + u) * NP + n];
-        acc[n][0] = __builtin_fmaf(a[u].x, bv, acc[n][0]);
-        acc[n][1] = __builtin_fmaf(a[u].y, bv, acc[n][1]);
-        acc[n][2] = __builtin_fmaf(a[u].z, bv, acc[n][2]);
-        acc[n][3] = __builtin_fmaf(a[u].w, bv, acc[n][3]);
+        for (int j = 0; j < 4; ++j) {
+          acc[4 * q + j].x = __builtin_fmaf(a[u].x, bv[j], acc[4 * q + j].x);
+          acc[4 * q + j].y = __builtin_fmaf(a[u].y, bv[j], acc[4 * q + j].y);
+          acc[4 * q + j].z = __builtin_fmaf(a[u].z, bv[j], acc[4 * q + j].z);
+          acc[4 * q + j].w = __builtin_fmaf(a[u].w, bv[j], acc[4 * q + j].w);
+        }
       }
     }
-  }
-  __syncthreads();  // B is done with: its memory takes the partial sums
-  float (*red)[NP * 4][64] = reinterpret_cast<float (*)[NP * 4][64]>(sh);
-  // Sixteen partial sums per output -> one, in a fixed order: waves 4j..4j+3 (j = 1, 2, 3) hand
-  // theirs to waves 0..3 in three rounds, then waves 1..3 hand theirs to wave 0.
-  for (int j = 1; j < 4; ++j) {
-    if ((w >> 2) == j) {
-#pragma unroll
-      for (int n = 0; n < NP; ++n)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) red[w & 3][n * 4 + q][lane] = acc[n][q];
+  };
+  float4 a0[U], a1[U];
+  const bool any = k_first < klen;
+  if (any) load_batch(a0, k_first);
+  {
+    const float* bsrc = B + kbeg * (size_t)N;
+    const int rows = (int)k_chunk;
+    for (int idx = threadIdx.x; idx < rows * NP; idx += 64 * NARROW_WAVES) {
+      const int k = idx / NP, n = idx % NP;
+      bsh[idx] = (k < klen && n < N) ? bsrc[k * N + n] : 0.0f;
     }
-    __syncthreads();
-    if (w < 4) {
-#pragma unroll
-      for (int n = 0; n < NP; ++n)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) acc[n][q] += red[w][n * 4 + q][lane];
-    }
-    __syncthreads();
   }
-  if (w >= 1 && w < 4) {
+  __syncthreads();
+  if (any) {
+    for (int k0 = k_first; k0 < k_last; k0 += 2 * U) {
+      load_batch(a1, k0 + U);
+      multiply_batch(a0, k0);
+      if (k0 + 2 * U < k_last) load_batch(a0, k0 + 2 * U);
+      multiply_batch(a1, k0 + U);
+    }
+  }
+  if (w > 0) {
 #pragma unroll
-    for (int n = 0; n < NP; ++n)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) red[w][n * 4 + q][lane] = acc[n][q];
+    for (int n = 0; n < NP; ++n) red[w - 1][n][lane] = acc[n];
   }
   __syncthreads();
   if (w != 0 || !active) return;
-  float* out = dst + (size_t)blockIdx.y * M * (size_t)N + m * (size_t)N;
+  for (int v = 0; v < NARROW_WAVES - 1; ++v) {
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
+    for (int n = 0; n < NP; ++n) {
+      const float4 t = red[v][n][lane];
+      acc[n].x += t.x; acc[n].y += t.y; acc[n].z += t.z; acc[n].w += t.w;
+    }
+  }
+  // element e of the lane's 4 x NP run: row e / NP of its four, column e % NP (M is a multiple of 4)
+  float* out = partial + ((size_t)blockIdx.y * M + m) * NP;
+  auto elem = [&](int e) {
+    const float4 s = acc[e % NP];
+    const int q = e / NP;
+    return q == 0 ? s.x : q == 1 ? s.y : q == 2 ? s.z : s.w;
+  };
 #pragma unroll
-    for (int n = 0; n < NP; ++n)
-      if (n < N) out[(size_t)q * N + n] = ((acc[n][q] + red[1][n * 4 + q][lane]) + red[2][n * 4 + q][lane]) + red[3][n * 4 + q][lane];
+  for (int t = 0; t < NP; ++t) st4g(out + 4 * t, make_float4(elem(4 * t), elem(4 * t + 1), elem(4 * t + 2), elem(4 * t + 3)));
+}
+
+// C = sum_z partial[z] (z ascending; partial[z] is [M][NP]) + beta*C, then bias / pre-activation / relu.
+template <int NP>
+__global__ __launch_bounds__(256) void narrow_n_combine_kernel(size_t M, int N, unsigned splits, const float* __restrict__ partial,
+                                                               float* C, float beta, const float* __restrict__ bias, int relu,
+                                                               float* pre_act, const float* __restrict__ mask) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * (size_t)N) return;
+  const size_t row = i / N, n = i % N;
+  const float* p = partial + row * NP + n;
+  const size_t step = M * NP;
+  float s = p[0];
+  unsigned z = 1;
+  for (; z + 8 <= splits; z += 8) {  // eight loads in flight, added in the same order as one by one
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = p[(size_t)(z + u) * step];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += t[u];
+  }
+  for (; z < splits; ++z) s += p[(size_t)z * step];
+  if (mask) s *= (mask[i] >= 0.f ? 1.f : 0.f);
+  if (beta != 0.0f) s = beta * C[i] + s;
+  if (bias) s += bias[n];
+  if (pre_act) pre_act[i] = s;
+  if (relu) s = (s >= 0.f ? 1.f : 0.f) * s;
+  C[i] = s;
 }
 
 // C = A * B for a narrow B: A stored M x K (K a multiple of 4), B stored K x N, N <= 4 * G.
@@ -450,32 +492,40 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
     return 1;
   }
   // narrow N: A (K x M) is the large side
-  if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22) && aligned16(g.A)) {
+  if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22)) {
+    const int NP = (int)((N + 3) / 4 * 4);
     const size_t gx = (M / 4 + 63) / 64;
-    const size_t mn_bytes = M * N * sizeof(float);
-    // K splits: about one workgroup of sixteen waves per CU, each wave at least four passes of eight
-    // k, a workgroup at most NARROW_K_CHUNK k
+    // K splits: one workgroup of eight waves per CU (its LDS holds seven waves' sums), every wave
+    // whole double batches; the partials (splits x M x NP floats) stay a small fraction of A
+    constexpr size_t GRAIN = (size_t)NARROW_WAVES * 2 * NARROW_BATCH;  // 128 k
     size_t splits = ((size_t)ctx->num_cu + gx - 1) / gx;
-    const size_t most = K / 512;  // K >= 512 here
+    const size_t most = K / GRAIN;  // K >= 512 here
     if (splits > most) splits = most;
     if (splits < (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK) splits = (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK;
-    if (splits > 65535 || splits > ctx->workspace_bytes / mn_bytes) return 0;
-    size_t k_chunk = ((K + splits - 1) / splits + 127) / 128 * 128;
+    if (splits > 65535) splits = 65535;
+    const size_t part_bytes = M * NP * sizeof(float);
+    if (splits > ctx->workspace_bytes / part_bytes) splits = ctx->workspace_bytes / part_bytes;
+    if (splits < 1) return 0;
+    const size_t k_chunk = ((K + splits - 1) / splits + GRAIN - 1) / GRAIN * GRAIN;
     splits = (K + k_chunk - 1) / k_chunk;
-    const bool plain = splits == 1 && g.beta == 0.0f && !g.bias && !g.relu && !g.pre_act && !g.mask;
-    float* dst = plain ? g.C : g.partial;
+    if (gx > 0x7fffffffu) return 0;
     const dim3 grid((unsigned)gx, (unsigned)splits);
-#define SL_NN(NP_, U_) \
-  hipLaunchKernelGGL((gemm_narrow_n_kernel<NP_, U_>), grid, dim3(1024), 0, ctx->stream, M, (int)N, K, g.A, g.B, dst, k_chunk)
-    if (N <= 4) SL_NN(4, 8);
-    else if (N <= 8) SL_NN(8, 8);
-    else if (N <= 12) SL_NN(12, 8);
-    else SL_NN(16, 4);
+    const size_t outs = M * N;
+    const dim3 cgrid((unsigned)((outs + 255) / 256));
+#define SL_NN(NP_)                                                                                                           \
+  do {                                                                                                                       \
+    hipLaunchKernelGGL((gemm_narrow_n_kernel<NP_>), grid, dim3(64 * NARROW_WAVES), 0, ctx->stream, M, (int)N, K, g.A, g.B,   \
+                       g.partial, k_chunk);                                                                                  \
+    hipLaunchKernelGGL((narrow_n_combine_kernel<NP_>), cgrid, dim3(256), 0, ctx->stream, M, (int)N, (unsigned)splits,        \
+                       (const float*)g.partial, g.C, g.beta, g.bias, g.relu, g.pre_act, g.mask);                             \
+  } while (0)
+    if (NP == 4) SL_NN(4);
+    else if (NP == 8) SL_NN(8);
+    else if (NP == 12) SL_NN(12);
+    else SL_NN(16);
 #undef SL_NN
     *rc = post_launch();
-    g.splits = plain ? 1 : (unsigned)splits;
-    g.k_chunk = k_chunk;
-    return plain || *rc ? 1 : 2;  // 2: partials are in the workspace, the caller combines them
+    return 1;
   }
   return 0;
 }

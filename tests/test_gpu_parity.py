@@ -150,7 +150,8 @@ def test_gemm_spread_tail(hip, orc):
 def test_gemm_skinny_kernels(hip, orc):
     """K <= 12 with a large result (vector-ALU kernel, rows of A staged in LDS) in all four forms with
     every epilogue, and A^T * B with N <= 16 and a long K (A streamed once, k split over workgroups
-    and waves, partials combined in a fixed order)."""
+    and waves, partials combined in a fixed order): N in {1, 3, 10, 16} and between, K odd, K shorter
+    and longer than a workgroup's chunk, M not a multiple of the 256 columns of a workgroup."""
     for (m, n, k, ta, tb) in [(1031, 260, 10, 0, 1), (4100, 64, 1, 0, 0), (1500, 512, 12, 1, 0), (2050, 1028, 7, 1, 1),
                               (8192, 2048, 10, 0, 1), (3000, 96, 4, 0, 1), (1111, 256, 9, 0, 0), (1024, 1024, 5, 0, 1),
                               (1400, 200, 11, 0, 1), (1400, 200, 8, 1, 1)]:
@@ -181,6 +182,9 @@ def test_gemm_skinny_kernels(hip, orc):
         assert np.array_equal(got, hip.sgemm(1, 0, m, n, k, a, b))          # same plan, same order of sums
         c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
         assert np.array_equal(hip.sgemm(1, 0, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(1, 0, m, n, k, a, b, pre, c=c0.copy(), beta=1.0),
+                              c0 + np.where(pre >= 0, got, 0 * got))
 
 
 def test_gemm_rows_narrow_kernel(hip, orc):
