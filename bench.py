@@ -103,19 +103,18 @@ def median_ms(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
     return statistics.median(pair_times(ctx, fn, iters, warmup, sweep))
 
 
-def spin_up(ctx, seconds=0.4):
-    """Untimed: keep the matrix cores busy until the clocks have ramped (the first launches after
-    an idle period run at about 2.0 instead of 2.4 GHz).  Uses the At*B kernel so that a profile of
-    this program attributes only the timed 4096^3 launches to the headline A*B kernel."""
-    n = 2048
-    a, b, c = ctx.uniform(n * n, -1, 1, 0, SEED), ctx.uniform(n * n, -1, 1, 1, SEED), ctx.zeros(n * n)
+def spin_up(ctx, a, b, c, n, seconds=1.0):
+    """Untimed: keep the matrix cores under the headline's own load until clocks and power state have
+    settled (the first launches after an idle period run at about 2.0 instead of 2.4 GHz, and a lighter
+    spin-up kernel, or operand set-up between spin-up and timing, left the first timed block 2-4 % slow
+    in some runs).  Uses the A*Bt kernel on the headline's own operands, right before the headline's
+    warm-up launches, so that a profile of this program attributes only the headline's own warm-up
+    and timed launches to the headline A*B kernel."""
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < seconds:
         for _ in range(20):
-            ctx.call("slhip_sgemm", 1, 0, n, n, n, a.ptr, b.ptr, c.ptr, 0.0)
+            ctx.call("slhip_sgemm", 0, 1, n, n, n, a.ptr, b.ptr, c.ptr, 0.0)
         ctx.sync()
-    for x in (a, b, c):
-        x.free()
 
 
 def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headline=False, back_to_back=False):
@@ -126,6 +125,8 @@ def bench_gemm(ctx, m, n, k, ta, tb, steps, warmup, beta=0.0, sweep=None, headli
     flop = 2.0 * m * n * k
     res = {}
     if headline:
+        if m == n == k:
+            spin_up(ctx, a, b, c, m)
         wall, ev = timed(ctx, fn, steps, warmup)
         res.update({"ms_wall": wall, "ms_kernel": ev, "tflops_wall": flop / wall / 1e9, "tflops_kernel": flop / ev / 1e9,
                     "frac_of_peak": flop / ev / 1e9 / FP32_MATRIX_PEAK_TFLOPS})
@@ -402,7 +403,6 @@ def main():
     log("device:", ctx.name())
     M = N = K = args.size
 
-    spin_up(ctx)
     head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup, headline=True)
     log("gemm A*B", head)
     roof = {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
