@@ -326,7 +326,8 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   const size_t lda = ta ? M : K, ldb = tb ? K : N;
   g.a_vec = lda % 4 == 0;  // dword-aligned vector loads: the leading dimension decides, not the base
   g.b_vec = ldb % 4 == 0;
-  g.m_fast = (aligned16(A) && aligned16(B)) ? M : 0;
+  // (the fast loop addresses a tile panel with 32-bit byte offsets: 127 rows of the leading dimension)
+  g.m_fast = (aligned16(A) && aligned16(B) && lda < (size_t(1) << 22) && ldb < (size_t(1) << 22)) ? M : 0;
   g.partial = (float*)ctx->workspace;
   const size_t mn_bytes = M * N * sizeof(float);
 

@@ -163,7 +163,7 @@ static int32_t gemm_bits_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t 
   const size_t lda = ta ? M : K, ldb = tb ? K : N;
   g.a_vec = lda % 4 == 0;
   g.b_vec = ldb % 4 == 0;
-  g.m_fast = (aligned16(A) && aligned16(B)) ? M : 0;
+  g.m_fast = (aligned16(A) && aligned16(B) && lda < (size_t(1) << 22) && ldb < (size_t(1) << 22)) ? M : 0;  // 32-bit tile offsets
   g.partial = nullptr;
   const size_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   if (tiles_m * tiles_n > 0x7fffffffu) {

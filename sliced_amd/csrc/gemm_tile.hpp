@@ -162,6 +162,39 @@ __device__ __forceinline__ void store_xc(const Frag<BK, XT, NT>& f, float* lds) 
   for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
 }
 
+// LOAD_FAST as scalar base + 32-bit vector offset.  tile_offsets: the byte offset of each of this
+// thread's float4 from the tile's first element at a k tile's first k, for a k-contiguous (KC) or
+// an x-contiguous source - the same thread -> element map as load_kc / load_xc, which store_kc /
+// store_xc rely on.  The host only lets LOAD_FAST run when these fit 32 bits (leading dimension
+// below 2^22).  load_panel: the NV loads of a stage from the panel that starts at `panel`, a
+// wave-uniform address: `global_load_dwordx4 v, v_offset, s[base]`.
+template <int BK, int XT, int NT, bool KC>
+__device__ __forceinline__ void tile_offsets(unsigned* off, size_t ld) {
+  if (KC) {
+    constexpr int VPR = BK / 4, RPP = NT / VPR;
+    const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
+#pragma unroll
+    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) off[p] = (unsigned)(((size_t)(xr + RPP * p) * ld + 4 * kq) * sizeof(float));
+  } else {
+    constexpr int XQ = XT / 4, KR = NT / XQ;
+    const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
+#pragma unroll
+    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) off[p] = (unsigned)(((size_t)(kr + KR * p) * ld + 4 * xq) * sizeof(float));
+  }
+}
+template <int BK, int XT, int NT>
+__device__ __forceinline__ void load_panel(Frag<BK, XT, NT>& f, const float* panel, unsigned* off) {
+  const char* base = reinterpret_cast<const char*>(panel);
+#pragma unroll
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) {
+    // the empty asm keeps the 32 -> 64 bit extension of the offset next to the load: hoisted out of
+    // the loop it leaves a 64-bit vector add per load behind, kept here the pair folds into the
+    // load's scalar-base addressing mode
+    asm volatile("" : "+v"(off[p]));
+    f.v[p] = ld4(reinterpret_cast<const float*>(base + (size_t)off[p]));
+  }
+}
+
 // MFMA fragments of one 8-wide k group for the NI 32-row blocks of this wave's rows (or columns).
 // KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's rows/cols in the tile.
 template <bool KC, int BK, int XT, int NI>
@@ -196,14 +229,16 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = local / gsize;
 }
 
-// Where the k loop's code starts relative to a 32-byte boundary is worth up to 4 % of the kernel's
+// Where the k loop's code starts relative to a 32-byte boundary is worth up to 1.5 % of the kernel's
 // speed, repeatably: measured on 4096^3 with the start 0 / 8 / 16 / 24 bytes past a boundary
-// (TFLOP/s): A*B 132.3 / 134.9 / 134.2 / 131.1, A*Bt 139.9 / 139.0 / 141.1 / 139.8, At*B 134.1 /
-// 128.8 / 130.4 / 129.8; odd multiples of 4 bytes were never best, 64-byte alignment adds nothing.
-// Left to chance the start moves whenever code earlier in the file changes, so it is pinned,
-// per form, for the two loops that large products spend their time in.  The best offset is a
-// property of the loop's code: after a change to the loop or to what precedes it in gemm_tiles,
-// measure the four offsets again.  P = offset in units of 8 bytes.
+// (TFLOP/s, launches back to back): A*B 135.4 / 136.2 / 135.4 / 134.6, A*Bt 140.0 / 141.4 / 141.2 /
+// 140.8, At*B 137.4 / 136.9 / 136.8 / 136.7; the eight-wave tile at 2048^3: A*B 126.4 / 127.7 /
+// 127.5 / 126.9, A*Bt 133.5 / 133.5 / 132.8 / 132.6, At*B 119.4 / 119.8 / 119.4 / 119.5.  (With
+// 64-bit vector address arithmetic still in the loop the spread was up to 4 %.)  Left to chance the
+// start moves whenever code earlier in the file changes, so it is pinned, per form, for the loops
+// that large products spend their time in.  The best offset is a property of the loop's code:
+// after a change to the loop or to what precedes it in gemm_tiles, measure the four offsets
+// again.  P = offset in units of 8 bytes.
 template <int P>
 __device__ __forceinline__ void pin_loop_start() {
   static_assert(P >= 0 && P < 4, "offset is 0, 8, 16 or 24 bytes");
@@ -212,9 +247,10 @@ __device__ __forceinline__ void pin_loop_start() {
   if (P == 2) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
   if (P == 3) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
 }
-constexpr int PIN_ONLY_FAST[2][2] = {{1, 2}, {0, 1}};  // [TA][TB]; the kernel that holds no other loop
+constexpr int PIN_ONLY_FAST[2][2] = {{1, 1}, {0, 1}};  // [TA][TB]; the kernel that holds no other loop
 constexpr int PIN_FAST[2][2] = {{1, 1}, {0, 1}};       // the same loop in the kernel that holds all four
 constexpr int PIN_XCLAMP[2][2] = {{1, 2}, {1, 1}};
+constexpr int PIN_WIDE[2][2] = {{1, 1}, {1, 1}};       // the eight-wave tile
 constexpr int PIN_SMALL[2][2] = {{0, 0}, {0, 0}};      // the 64 x 64 tile's loops: no offset differs by more than 2 %
 
 // The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
@@ -229,6 +265,15 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   constexpr int NT = 64 * WGM * WGN;                      // its threads
   constexpr int KSTEPS = BK / 8;
   constexpr int REFILL_AT = (TA && !TB) ? KSTEPS - 1 : (KSTEPS > 1 ? 1 : 0);
+  // The fast loop of the four-wave 128 x 128 tile refills the two operands in different k-groups
+  // (A's stores and loads in one, B's in another) for A*B and A*Bt: the memory instructions of a
+  // refill, issued in one run, hold the wave's MFMA issue up behind them.  Measured at 4096^3 with
+  // everything in group 1 / the split below (TFLOP/s, launches back to back): A*B 134.5 / 136.0,
+  // A*Bt 137.4 / 141.2; At*B is best with everything in the last group (137.1 against 131-134 for
+  // every split), and so is the eight-wave tile (2048^3: 127.9 / 133.5 / 120.2 unsplit).  Interleaving
+  // store A, load A, store B, load B inside ONE group is the worst order (2048^3: 114).
+  constexpr bool SPLIT_REFILL = MODE == LOAD_FAST && KSTEPS == 4 && WM == 2 && WN == 2 && WGM == 2 && WGN == 2 && !TA;
+  constexpr int REFILL_A = TB ? 1 : 2, REFILL_B = 3;
   if (kt_begin >= kt_end) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -239,7 +284,27 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 
   Frag<BK, TM, NT> fa;
   Frag<BK, TN, NT> fb;
+  // LOAD_FAST: the address of a load is a scalar base (the tile panel at k tile kt, advanced by the
+  // scalar unit) plus a per-thread 32-bit byte offset that never changes, so the loop holds no
+  // vector arithmetic for its sixteen loads.  As per-thread 64-bit pointers every load cost two
+  // 64-bit vector adds per k tile, and vector ALU work in this loop is paid for in matrix-core time.
+  // (The buffer-descriptor form of the same idea is out: this compiler lowers the 128-bit raw buffer
+  // load builtin to a 32-bit load.)
+  unsigned off_a[Cfg<BK, TM, NT>::NV], off_b[Cfg<BK, TN, NT>::NV];
+  const float* base_a = nullptr;
+  const float* base_b = nullptr;
+  if (MODE == LOAD_FAST) {
+    tile_offsets<BK, TM, NT, !TA>(off_a, lda);
+    tile_offsets<BK, TN, NT, TB>(off_b, ldb);
+    base_a = TA ? g.A + kbeg * lda + m0 : g.A + m0 * lda + kbeg;
+    base_b = TB ? g.B + n0 * ldb + kbeg : g.B + kbeg * ldb + n0;
+  }
   auto load_stage = [&](int kt) {
+    if (MODE == LOAD_FAST) {
+      load_panel<BK, TM, NT>(fa, base_a + (size_t)kt * (TA ? BK * lda : BK), off_a);
+      load_panel<BK, TN, NT>(fb, base_b + (size_t)kt * (TB ? BK : BK * ldb), off_b);
+      return;
+    }
     const size_t k0 = kbeg + (size_t)kt * BK;
     if (TA) load_xc<BK, TM, MODE, NT>(fa, g.A, lda, g.M, kend, m0, k0);
     else load_kc<BK, TM, MODE, NT>(fa, g.A, lda, g.M, kend, m0, k0);
@@ -267,7 +332,9 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   __syncthreads();
 
   constexpr bool BIG = WM == 2 && WN == 2 && WGM == 2 && WGN == 2;
-  if (MODE == LOAD_FAST) pin_loop_start<!BIG ? PIN_SMALL[TA][TB] : ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
+  constexpr bool WIDE = WGM * WGN == 8;
+  if (MODE == LOAD_FAST)
+    pin_loop_start<WIDE ? PIN_WIDE[TA][TB] : !BIG ? PIN_SMALL[TA][TB] : ONLY_FAST ? PIN_ONLY_FAST[TA][TB] : PIN_FAST[TA][TB]>();
   if (MODE == LOAD_XCLAMP) pin_loop_start<BIG ? PIN_XCLAMP[TA][TB] : PIN_SMALL[TA][TB]>();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int s = (kt - kt_begin) & 1;
@@ -281,7 +348,17 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
         read_frag<!TA, BK, TM, WM>(a[nxt], lds_a[s], wm * 32 * WM, kk8 + 1, r, h);
         read_frag<TB, BK, TN, WN>(b[nxt], lds_b[s], wn * 32 * WN, kk8 + 1, r, h);
       }
-      if (kk8 == REFILL_AT) {
+      if (SPLIT_REFILL) {
+        // each operand's LDS stores and loads in a k-group of their own (table REFILL_SPLIT)
+        if (kk8 == REFILL_A) {
+          if (kt + 1 < kt_end) { if (TA) store_xc<BK, TM, NT>(fa, lds_a[s ^ 1]); else store_kc<BK, TM, NT>(fa, lds_a[s ^ 1]); }
+          if (kt + 2 < kt_end) load_panel<BK, TM, NT>(fa, base_a + (size_t)(kt + 2) * (TA ? BK * lda : BK), off_a);
+        }
+        if (kk8 == REFILL_B) {
+          if (kt + 1 < kt_end) { if (TB) store_kc<BK, TN, NT>(fb, lds_b[s ^ 1]); else store_xc<BK, TN, NT>(fb, lds_b[s ^ 1]); }
+          if (kt + 2 < kt_end) load_panel<BK, TN, NT>(fb, base_b + (size_t)(kt + 2) * (TB ? BK : BK * ldb), off_b);
+        }
+      } else if (kk8 == REFILL_AT) {
         // stage s^1 was last read in the previous iteration, which ended with a barrier
         if (kt + 1 < kt_end) store_stage(s ^ 1);
         if (kt + 2 < kt_end) load_stage(kt + 2);
