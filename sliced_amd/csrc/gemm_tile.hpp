@@ -162,27 +162,35 @@ __device__ __forceinline__ void store_xc(const Frag<BK, XT, NT>& f, float* lds) 
   for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
 }
 
-// LOAD_FAST as scalar base + 32-bit vector offset.  tile_offsets: the byte offset of each of this
-// thread's float4 from the tile's first element at a k tile's first k, for a k-contiguous (KC) or
-// an x-contiguous source - the same thread -> element map as load_kc / load_xc, which store_kc /
-// store_xc rely on.  The host only lets LOAD_FAST run when these fit 32 bits (leading dimension
-// below 2^22).  load_panel: the NV loads of a stage from the panel that starts at `panel`, a
-// wave-uniform address: `global_load_dwordx4 v, v_offset, s[base]`.
-template <int BK, int XT, int NT, bool KC>
-__device__ __forceinline__ void tile_offsets(unsigned* off, size_t ld) {
+// LOAD_FAST and LOAD_XCLAMP as scalar base + 32-bit vector offset.  tile_offsets: the byte offset of
+// each of this thread's float4 from the tile's first element at a k tile's first k, for a
+// k-contiguous (KC) or an x-contiguous source - the same thread -> element map as load_kc / load_xc,
+// which store_kc / store_xc rely on.  CLAMP (LOAD_XCLAMP): a row or a vector of columns that starts
+// outside the operand is fetched from inside it instead (the last row; the tile's first columns) -
+// its values only reach rows and columns of C that are never stored.  The offsets fit 32 bits for
+// leading dimensions below 2^22, which is checked where these modes are chosen.  load_panel: the NV
+// loads of a stage from the panel that starts at `panel`, a wave-uniform address:
+// `global_load_dwordx4 v, v_offset, s[base]`.
+template <int BK, int XT, int NT, bool KC, bool CLAMP>
+__device__ __forceinline__ void tile_offsets(unsigned* off, size_t ld, size_t x0, size_t X) {
   if (KC) {
     constexpr int VPR = BK / 4, RPP = NT / VPR;
     const int kq = threadIdx.x % VPR, xr = threadIdx.x / VPR;
 #pragma unroll
-    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) off[p] = (unsigned)(((size_t)(xr + RPP * p) * ld + 4 * kq) * sizeof(float));
+    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) {
+      size_t xi = xr + RPP * p;
+      if (CLAMP && x0 + xi >= X) xi = X - 1 - x0;
+      off[p] = (unsigned)((xi * ld + 4 * kq) * sizeof(float));
+    }
   } else {
     constexpr int XQ = XT / 4, KR = NT / XQ;
     const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
+    const size_t xi = (CLAMP && x0 + 4 * xq >= X) ? 0 : 4 * xq;
 #pragma unroll
-    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) off[p] = (unsigned)(((size_t)(kr + KR * p) * ld + 4 * xq) * sizeof(float));
+    for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) off[p] = (unsigned)(((size_t)(kr + KR * p) * ld + xi) * sizeof(float));
   }
 }
-template <int BK, int XT, int NT>
+template <int BK, int XT, int NT, bool ALIGNED>
 __device__ __forceinline__ void load_panel(Frag<BK, XT, NT>& f, const float* panel, unsigned* off) {
   const char* base = reinterpret_cast<const char*>(panel);
 #pragma unroll
@@ -191,7 +199,8 @@ __device__ __forceinline__ void load_panel(Frag<BK, XT, NT>& f, const float* pan
     // the loop it leaves a 64-bit vector add per load behind, kept here the pair folds into the
     // load's scalar-base addressing mode
     asm volatile("" : "+v"(off[p]));
-    f.v[p] = ld4(reinterpret_cast<const float*>(base + (size_t)off[p]));
+    const float* at = reinterpret_cast<const float*>(base + (size_t)off[p]);
+    f.v[p] = ALIGNED ? ld4(at) : ld4g(at);
   }
 }
 
@@ -272,7 +281,7 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   // A*Bt 137.4 / 141.2; At*B is best with everything in the last group (137.1 against 131-134 for
   // every split), and so is the eight-wave tile (2048^3: 127.9 / 133.5 / 120.2 unsplit).  Interleaving
   // store A, load A, store B, load B inside ONE group is the worst order (2048^3: 114).
-  constexpr bool SPLIT_REFILL = MODE == LOAD_FAST && KSTEPS == 4 && WM == 2 && WN == 2 && WGM == 2 && WGN == 2 && !TA;
+  constexpr bool SPLIT_REFILL = (MODE == LOAD_FAST || MODE == LOAD_XCLAMP) && KSTEPS == 4 && WM == 2 && WN == 2 && WGM == 2 && WGN == 2 && !TA;
   constexpr int REFILL_A = TB ? 1 : 2, REFILL_B = 3;
   if (kt_begin >= kt_end) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -284,7 +293,7 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 
   Frag<BK, TM, NT> fa;
   Frag<BK, TN, NT> fb;
-  // LOAD_FAST: the address of a load is a scalar base (the tile panel at k tile kt, advanced by the
+  // LOAD_FAST and LOAD_XCLAMP: the address of a load is a scalar base (the tile panel at k tile kt, advanced by the
   // scalar unit) plus a per-thread 32-bit byte offset that never changes, so the loop holds no
   // vector arithmetic for its sixteen loads.  As per-thread 64-bit pointers every load cost two
   // 64-bit vector adds per k tile, and vector ALU work in this loop is paid for in matrix-core time.
@@ -293,16 +302,18 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   unsigned off_a[Cfg<BK, TM, NT>::NV], off_b[Cfg<BK, TN, NT>::NV];
   const float* base_a = nullptr;
   const float* base_b = nullptr;
-  if (MODE == LOAD_FAST) {
-    tile_offsets<BK, TM, NT, !TA>(off_a, lda);
-    tile_offsets<BK, TN, NT, TB>(off_b, ldb);
+  constexpr bool PANEL = MODE == LOAD_FAST || MODE == LOAD_XCLAMP;
+  constexpr bool ALIGNED = MODE == LOAD_FAST;
+  if (PANEL) {
+    tile_offsets<BK, TM, NT, !TA, MODE == LOAD_XCLAMP>(off_a, lda, m0, g.M);
+    tile_offsets<BK, TN, NT, TB, MODE == LOAD_XCLAMP>(off_b, ldb, n0, g.N);
     base_a = TA ? g.A + kbeg * lda + m0 : g.A + m0 * lda + kbeg;
     base_b = TB ? g.B + n0 * ldb + kbeg : g.B + kbeg * ldb + n0;
   }
   auto load_stage = [&](int kt) {
-    if (MODE == LOAD_FAST) {
-      load_panel<BK, TM, NT>(fa, base_a + (size_t)kt * (TA ? BK * lda : BK), off_a);
-      load_panel<BK, TN, NT>(fb, base_b + (size_t)kt * (TB ? BK : BK * ldb), off_b);
+    if (PANEL) {
+      load_panel<BK, TM, NT, ALIGNED>(fa, base_a + (size_t)kt * (TA ? BK * lda : BK), off_a);
+      load_panel<BK, TN, NT, ALIGNED>(fb, base_b + (size_t)kt * (TB ? BK : BK * ldb), off_b);
       return;
     }
     const size_t k0 = kbeg + (size_t)kt * BK;
@@ -352,11 +363,11 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
         // each operand's LDS stores and loads in a k-group of their own (table REFILL_SPLIT)
         if (kk8 == REFILL_A) {
           if (kt + 1 < kt_end) { if (TA) store_xc<BK, TM, NT>(fa, lds_a[s ^ 1]); else store_kc<BK, TM, NT>(fa, lds_a[s ^ 1]); }
-          if (kt + 2 < kt_end) load_panel<BK, TM, NT>(fa, base_a + (size_t)(kt + 2) * (TA ? BK * lda : BK), off_a);
+          if (kt + 2 < kt_end) load_panel<BK, TM, NT, ALIGNED>(fa, base_a + (size_t)(kt + 2) * (TA ? BK * lda : BK), off_a);
         }
         if (kk8 == REFILL_B) {
           if (kt + 1 < kt_end) { if (TB) store_kc<BK, TN, NT>(fb, lds_b[s ^ 1]); else store_xc<BK, TN, NT>(fb, lds_b[s ^ 1]); }
-          if (kt + 2 < kt_end) load_panel<BK, TN, NT>(fb, base_b + (size_t)(kt + 2) * (TB ? BK : BK * ldb), off_b);
+          if (kt + 2 < kt_end) load_panel<BK, TN, NT, ALIGNED>(fb, base_b + (size_t)(kt + 2) * (TB ? BK : BK * ldb), off_b);
         }
       } else if (kk8 == REFILL_AT) {
         // stage s^1 was last read in the previous iteration, which ended with a barrier
@@ -406,7 +417,9 @@ __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, 
   int e1 = fast ? (kb < kfull ? kb : kfull) : ka;
   if (e1 < ka) e1 = ka;
   int e2 = e1;
-  if (!fast) {
+  // (the x-clamped loop addresses a tile panel with 32-bit byte offsets, like the fast one)
+  const bool narrow_ld = (TA ? g.M : g.K) < (size_t(1) << 22) && (TB ? g.K : g.N) < (size_t(1) << 22);
+  if (!fast && narrow_ld) {
     e2 = kb < before_last ? kb : before_last;
     if (e2 < e1) e2 = e1;
   }
