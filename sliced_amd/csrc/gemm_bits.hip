@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const size_t row = m0 + wm * 64 + 32 * i + r, cw = (n0 + wn * 64 + 32 * j) >> 5;
+        const size_t row = m0 + block_of<2>(wm, i) + r, cw = (n0 + block_of<2>(wn, j)) >> 5;
         if (h == 0 && row < g.M && cw < W) mw[i][j] = bits_in[row * W + cw];
       }
   }
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + wn * 64 + 32 * j + r;
+      const size_t col = n0 + block_of<2>(wn, j) + r;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         float val = acc[i][j][v];
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
           val = ((((h ? hi : lo) >> r) & 1u) ? 1.0f : 0.0f) * val;
         }
         if (g.beta != 0.0f) {
-          const size_t row = m0 + wm * 64 + 32 * i + bits_row_of(v, h);
+          const size_t row = m0 + block_of<2>(wm, i) + bits_row_of(v, h);
           if (row < g.M && col < g.N) val = g.beta * g.C[row * g.N + col] + val;
         }
         acc[i][j][v] = val;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
   if (g.bias) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + wn * 64 + 32 * j + r;
+      const size_t col = n0 + block_of<2>(wn, j) + r;
       if (col < g.N) bias_of[j] = g.bias[col];
     }
   }
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + wn * 64 + 32 * j + r;
+      const size_t col = n0 + block_of<2>(wn, j) + r;
       const bool cin = col < g.N;
       const float bias = bias_of[j];
       uint32_t word = 0u;
@@ -103,11 +103,11 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
           if (lane == bits_row_of(v, 1)) word = (uint32_t)(b >> 32);
         }
         if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
-        const size_t row = m0 + wm * 64 + 32 * i + bits_row_of(v, h);
+        const size_t row = m0 + block_of<2>(wm, i) + bits_row_of(v, h);
         if (row < g.M && cin) g.C[row * g.N + col] = val;
       }
       if (bits_out) {
-        const size_t row = m0 + wm * 64 + 32 * i + r, cw = (n0 + wn * 64 + 32 * j) >> 5;
+        const size_t row = m0 + block_of<2>(wm, i) + r, cw = (n0 + block_of<2>(wn, j)) >> 5;
         if (h == 0 && row < g.M && cw < W) bits_out[row * W + cw] = word;
       }
     }

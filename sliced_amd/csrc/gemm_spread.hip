@@ -48,7 +48,7 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
       for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          slot[(wm * 32 * WM + 32 * i + 8 * (v / 4) + 4 * h + (v % 4)) * TN + wn * 32 * WN + 32 * j + r] = acc[i][j][v];
+          slot[(block_of<2>(wm, i) + 8 * (v / 4) + 4 * h + (v % 4)) * TN + block_of<2>(wn, j) + r] = acc[i][j][v];
   }
 }
 

@@ -24,10 +24,27 @@ constexpr int GEMM_BK = 32;  // measured against 16: 3-10 % faster on every form
 template <int BK, int XT, int NT = 256>
 struct Cfg {
   static constexpr int KC_PITCH = BK + 4;  // [x][k] layout, k contiguous
-  static constexpr int XC_PITCH = XT + 4;  // [k][x] layout, x contiguous; pitch keeps float4 alignment
+  // [k][x] layout, x contiguous: rows of exactly XT words, and element (k, x) sits at column
+  // x ^ 32 when bit 2 of k is set (xc_index).  An MFMA fragment read takes k = 8g + 4h + t for
+  // the lanes' halves h = 0, 1: the swizzle puts the two halves on different banks, where padding
+  // the rows did before - but with rows of 128 words every fragment address of a k tile is the
+  // lane's base plus a multiple of 64 words, which ds_read2st64_b32 takes as an immediate.  With
+  // padded rows (pitch 132) the four k of a group needed a base register each, computed in the
+  // loop: 9 vector adds per k tile, paid for in matrix-core time (A*B 135.3 -> 139.5 TFLOP/s
+  // with the adds taken out).
+  static constexpr int XC_PITCH = XT;
   static constexpr int STAGE_FLOATS = XT * KC_PITCH > BK * XC_PITCH ? XT * KC_PITCH : BK * XC_PITCH;
   static constexpr int NV = BK * XT / 4 / NT;  // float4 per thread per operand tile
 };
+
+__device__ __forceinline__ int xc_swizzle(int k) { return ((k >> 2) & 1) << 5; }
+
+// The 32-wide block of rows (or columns) of the workgroup's tile that wave coordinate w (of WG
+// along this side) owns as its i-th: blocks are dealt out to the waves in turn, so a wave's blocks
+// lie 32 * WG apart - a multiple of 64 for the two-by-two grid, which the fragment addressing
+// above relies on.
+template <int WG>
+__device__ __forceinline__ constexpr int block_of(int w, int i) { return 32 * (w + WG * i); }
 
 struct GemmArgs {
   size_t M, N, K;
@@ -158,8 +175,10 @@ template <int BK, int XT, int NT = 256>
 __device__ __forceinline__ void store_xc(const Frag<BK, XT, NT>& f, float* lds) {
   constexpr int XQ = XT / 4, KR = NT / XQ;
   const int xq = threadIdx.x % XQ, kr = threadIdx.x / XQ;
+  static_assert(KR % 8 == 0, "bit 2 of a thread's rows kr + KR*p is that of kr: one swizzle per thread");
+  float* at = lds + kr * Cfg<BK, XT>::XC_PITCH + ((4 * xq) ^ xc_swizzle(kr));
 #pragma unroll
-  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(lds + (kr + KR * p) * Cfg<BK, XT>::XC_PITCH + 4 * xq, f.v[p]);
+  for (int p = 0; p < Cfg<BK, XT, NT>::NV; ++p) st4(at + KR * p * Cfg<BK, XT>::XC_PITCH, f.v[p]);
 }
 
 // LOAD_FAST and LOAD_XCLAMP as scalar base + 32-bit vector offset.  tile_offsets: the byte offset of
@@ -205,17 +224,20 @@ __device__ __forceinline__ void load_panel(Frag<BK, XT, NT>& f, const float* pan
 }
 
 // MFMA fragments of one 8-wide k group for the NI 32-row blocks of this wave's rows (or columns).
-// KC = true: lds is [x][k]; false: [k][x].  x_base = first of the wave's rows/cols in the tile.
-template <bool KC, int BK, int XT, int NI>
-__device__ __forceinline__ void read_frag(float (&out)[NI][4], const float* lds, int x_base, int kk8, int r, int h) {
+// KC = true: lds is [x][k]; false: [k][x] (swizzled, see Cfg).  w = the wave's coordinate along this
+// side of the WG-wide wave grid.
+template <bool KC, int BK, int XT, int NI, int WG>
+__device__ __forceinline__ void read_frag(float (&out)[NI][4], const float* lds, int w, int kk8, int r, int h) {
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     if (KC) {
-      float4 t = ld4(lds + (x_base + 32 * i + r) * Cfg<BK, XT>::KC_PITCH + kk8 * 8 + 4 * h);
+      float4 t = ld4(lds + (block_of<WG>(w, i) + r) * Cfg<BK, XT>::KC_PITCH + kk8 * 8 + 4 * h);
       out[i][0] = t.x; out[i][1] = t.y; out[i][2] = t.z; out[i][3] = t.w;
     } else {
+      // bit 2 of k = 8*kk8 + 4*h + t is h: one swizzle for the lane, folded into its base address
+      const float* lane_base = lds + 4 * h * Cfg<BK, XT>::XC_PITCH + ((block_of<WG>(w, 0) ^ (h << 5)) + r);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) out[i][t] = lds[(kk8 * 8 + 4 * h + t) * Cfg<BK, XT>::XC_PITCH + x_base + 32 * i + r];
+      for (int t = 0; t < 4; ++t) out[i][t] = lane_base[(kk8 * 8 + t) * Cfg<BK, XT>::XC_PITCH + 32 * WG * i];
     }
   }
 }
@@ -350,17 +372,17 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int s = (kt - kt_begin) & 1;
     float a[2][WM][4], b[2][WN][4];
-    read_frag<!TA, BK, TM, WM>(a[0], lds_a[s], wm * 32 * WM, 0, r, h);
-    read_frag<TB, BK, TN, WN>(b[0], lds_b[s], wn * 32 * WN, 0, r, h);
+    read_frag<!TA, BK, TM, WM, WGM>(a[0], lds_a[s], wm, 0, r, h);
+    read_frag<TB, BK, TN, WN, WGN>(b[0], lds_b[s], wn, 0, r, h);
 #pragma unroll
     for (int kk8 = 0; kk8 < KSTEPS; ++kk8) {
       const int cur = kk8 & 1, nxt = cur ^ 1;
       if (kk8 + 1 < KSTEPS) {
-        read_frag<!TA, BK, TM, WM>(a[nxt], lds_a[s], wm * 32 * WM, kk8 + 1, r, h);
-        read_frag<TB, BK, TN, WN>(b[nxt], lds_b[s], wn * 32 * WN, kk8 + 1, r, h);
+        read_frag<!TA, BK, TM, WM, WGM>(a[nxt], lds_a[s], wm, kk8 + 1, r, h);
+        read_frag<TB, BK, TN, WN, WGN>(b[nxt], lds_b[s], wn, kk8 + 1, r, h);
       }
       if (SPLIT_REFILL) {
-        // each operand's LDS stores and loads in a k-group of their own (table REFILL_SPLIT)
+        // each operand's LDS stores and loads in a k-group of their own (REFILL_A, REFILL_B above)
         if (kk8 == REFILL_A) {
           if (kt + 1 < kt_end) { if (TA) store_xc<BK, TM, NT>(fa, lds_a[s ^ 1]); else store_kc<BK, TM, NT>(fa, lds_a[s ^ 1]); }
           if (kt + 2 < kt_end) load_panel<BK, TM, NT, ALIGNED>(fa, base_a + (size_t)(kt + 2) * (TA ? BK * lda : BK), off_a);
@@ -458,7 +480,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
-  //   row = 32*i + 8*(v/4) + 4*h + v%4,  col = 32*j + r   within the wave's (32*WM) x (32*WN) tile.
+  //   row = 8*(v/4) + 4*h + v%4,  col = r   within the 32 x 32 block at (block_of(wm, i), block_of(wn, j)).
   // No load may sit between two stores: C, pre_act and dst can be the same memory as far as the
   // compiler knows, so a `beta * C[idx]` read after a store waits for that store, 64 times in a
   // row (measured: 7.5 us per workgroup, more than a 128x128x128 product itself).  Hence: first
@@ -471,10 +493,10 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
     for (int i = 0; i < WM; ++i)
 #pragma unroll
       for (int j = 0; j < WN; ++j) {
-        const size_t col = n0 + wn * 32 * WN + 32 * j + r;
+        const size_t col = n0 + block_of<WGN>(wn, j) + r;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const size_t row = m0 + wm * 32 * WM + 32 * i + 8 * (v / 4) + 4 * h + (v % 4);
+          const size_t row = m0 + block_of<WGM>(wm, i) + 8 * (v / 4) + 4 * h + (v % 4);
           if (interior || (row < g.M && col < g.N)) fn(i, j, v, row * g.N + col, col);
         }
       }
@@ -493,7 +515,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
     float bv[WN];
 #pragma unroll
     for (int j = 0; j < WN; ++j) {
-      const size_t col = n0 + wn * 32 * WN + 32 * j + r;
+      const size_t col = n0 + block_of<WGN>(wn, j) + r;
       bv[j] = col < g.N ? g.bias[col] : 0.0f;
     }
     for_each([&](int i, int j, int v, size_t, size_t) { acc[i][j][v] = acc[i][j][v] + bv[j]; });
