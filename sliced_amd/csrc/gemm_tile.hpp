@@ -260,15 +260,15 @@ __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, un
   tn = local / gsize;
 }
 
-// Where the k loop's code starts relative to a 32-byte boundary is worth up to 1.5 % of the kernel's
-// speed, repeatably: measured on 4096^3 with the start 0 / 8 / 16 / 24 bytes past a boundary
-// (TFLOP/s, launches back to back): A*B 135.4 / 136.2 / 135.4 / 134.6, A*Bt 140.0 / 141.4 / 141.2 /
-// 140.8, At*B 137.4 / 136.9 / 136.8 / 136.7; the eight-wave tile at 2048^3: A*B 126.4 / 127.7 /
-// 127.5 / 126.9, A*Bt 133.5 / 133.5 / 132.8 / 132.6, At*B 119.4 / 119.8 / 119.4 / 119.5.  (With
-// 64-bit vector address arithmetic still in the loop the spread was up to 4 %.)  Left to chance the
-// start moves whenever code earlier in the file changes, so it is pinned, per form, for the loops
-// that large products spend their time in.  The best offset is a property of the loop's code:
-// after a change to the loop or to what precedes it in gemm_tiles, measure the four offsets
+// Where the k loop's code starts relative to a 32-byte boundary used to be worth up to 4 % of the
+// kernel's speed (with vector address arithmetic in the loop); it is worth 0.5 % now, repeatably:
+// measured on 4096^3 with the start 0 / 8 / 16 / 24 bytes past a boundary (TFLOP/s, launches back to
+// back): A*B 141.9 / 142.5 / 142.9 / 142.4, A*Bt 143.4 / 143.6 / 143.8 / 143.5, At*B 141.4 / 142.2 /
+// 142.0 / 141.6; the eight-wave tile at 2048^3 within 0.5 % everywhere; the 64 x 64 tile at 1024^3:
+// 93.7 / 92.3 / 94.9 / 94.3, 94.1 / 92.7 / 94.5 / 93.2, 93.0 / 92.2 / 92.9 / 93.5.  Left to chance the
+// start moves whenever code earlier in the file changes, so it stays pinned, per form, for the
+// loops that large products spend their time in.  The best offset is a property of the loop's
+// code: after a change to the loop or to what precedes it in gemm_tiles, measure the four offsets
 // again.  P = offset in units of 8 bytes.
 template <int P>
 __device__ __forceinline__ void pin_loop_start() {
@@ -278,11 +278,11 @@ __device__ __forceinline__ void pin_loop_start() {
   if (P == 2) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
   if (P == 3) asm volatile(".p2align 5\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0\n s_nop 0");
 }
-constexpr int PIN_ONLY_FAST[2][2] = {{1, 1}, {0, 1}};  // [TA][TB]; the kernel that holds no other loop
-constexpr int PIN_FAST[2][2] = {{1, 1}, {0, 1}};       // the same loop in the kernel that holds all four
+constexpr int PIN_ONLY_FAST[2][2] = {{2, 2}, {1, 2}};  // [TA][TB]; the kernel that holds no other loop
+constexpr int PIN_FAST[2][2] = {{2, 2}, {1, 2}};       // the same loop in the kernel that holds all four
 constexpr int PIN_XCLAMP[2][2] = {{1, 2}, {1, 1}};
-constexpr int PIN_WIDE[2][2] = {{1, 1}, {1, 1}};       // the eight-wave tile
-constexpr int PIN_SMALL[2][2] = {{0, 0}, {0, 0}};      // the 64 x 64 tile's loops: no offset differs by more than 2 %
+constexpr int PIN_WIDE[2][2] = {{3, 3}, {3, 3}};       // the eight-wave tile
+constexpr int PIN_SMALL[2][2] = {{2, 2}, {2, 2}};      // the 64 x 64 tile
 
 // The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
@@ -295,16 +295,18 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;  // the workgroup's tile of C
   constexpr int NT = 64 * WGM * WGN;                      // its threads
   constexpr int KSTEPS = BK / 8;
-  constexpr int REFILL_AT = (TA && !TB) ? KSTEPS - 1 : (KSTEPS > 1 ? 1 : 0);
-  // The fast loop of the four-wave 128 x 128 tile refills the two operands in different k-groups
-  // (A's stores and loads in one, B's in another) for A*B and A*Bt: the memory instructions of a
-  // refill, issued in one run, hold the wave's MFMA issue up behind them.  Measured at 4096^3 with
-  // everything in group 1 / the split below (TFLOP/s, launches back to back): A*B 134.5 / 136.0,
-  // A*Bt 137.4 / 141.2; At*B is best with everything in the last group (137.1 against 131-134 for
-  // every split), and so is the eight-wave tile (2048^3: 127.9 / 133.5 / 120.2 unsplit).  Interleaving
-  // store A, load A, store B, load B inside ONE group is the worst order (2048^3: 114).
-  constexpr bool SPLIT_REFILL = (MODE == LOAD_FAST || MODE == LOAD_XCLAMP) && KSTEPS == 4 && WM == 2 && WN == 2 && WGM == 2 && WGN == 2 && !TA;
-  constexpr int REFILL_A = TB ? 1 : 2, REFILL_B = 3;
+  // The refill (LDS stores of tile kt+1, loads of tile kt+2) sits before the LAST k-group of a k
+  // tile, as one run: store A, store B, load A, load B.  Measured at 4096^3 for the refill before
+  // group 0 / 1 / 2 / 3 (TFLOP/s, launches back to back): A*B 133.7 / 137.1 / 136.2 / 142.8, A*Bt
+  // 135.1 / 137.3 / 137.3 / 143.8, At*B 133.0 / 135.2 / 135.0 / 141.8; the eight-wave tile at 2048^3
+  // 126 / 132.5 / 133.7 / 132.6, 129 / 133.2 / 133.4 / 132.7, 125 / 126.5 / 126.5 / 131.2; the 64 x 64
+  // tile does not care (1024^3: 92-95 everywhere).  Giving each operand a group of its own, or
+  // spreading the refill over all four groups, measured 1-5 % below the best single position, and
+  // store A, load A, store B, load B in one group 10 % below.  (While the loop still computed its
+  // load addresses and LDS row bases with vector instructions the optimum was group 1 for A*B and
+  // A*Bt: where the memory instructions sit matters because, issued in one run, they hold the
+  // wave's MFMA issue up behind them - and so did that arithmetic.)
+  constexpr int REFILL_AT = KSTEPS - 1;
   if (kt_begin >= kt_end) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave / WGN, wn = wave % WGN;
@@ -353,10 +355,8 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   //   * the registers hold tile kt+1 (its global loads were issued one iteration ago);
   //   * before k-group REFILL_AT of tile kt those registers are stored to stage s^1 and the global
   //     loads of tile kt+2 are issued, so that both the LDS stores and the load issue hide behind
-  //     the remaining MFMA groups (16 MFMAs = 1024 cycles each) instead of sitting between the
-  //     MFMA block and the barrier.  Where in the block the refill goes was measured per form on
-  //     4096^3 (TFLOP/s at group 1 / at the last group): A*B 128.9 / 125.0, A*Bt 135.7 / 135.6,
-  //     At*B 122.7 / 125.3;
+  //     the last MFMA group (16 MFMAs = 1024 cycles) instead of sitting between the MFMA block
+  //     and the barrier (see REFILL_AT above for where in the block it goes);
   //   * MFMA fragments are read from LDS one k-group ahead of the MFMAs that consume them.
   // The scheduling barriers keep the compiler from sinking the reads and stores back down.
   load_stage(kt_begin);
@@ -381,17 +381,7 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
         read_frag<!TA, BK, TM, WM, WGM>(a[nxt], lds_a[s], wm, kk8 + 1, r, h);
         read_frag<TB, BK, TN, WN, WGN>(b[nxt], lds_b[s], wn, kk8 + 1, r, h);
       }
-      if (SPLIT_REFILL) {
-        // each operand's LDS stores and loads in a k-group of their own (REFILL_A, REFILL_B above)
-        if (kk8 == REFILL_A) {
-          if (kt + 1 < kt_end) { if (TA) store_xc<BK, TM, NT>(fa, lds_a[s ^ 1]); else store_kc<BK, TM, NT>(fa, lds_a[s ^ 1]); }
-          if (kt + 2 < kt_end) load_panel<BK, TM, NT, ALIGNED>(fa, base_a + (size_t)(kt + 2) * (TA ? BK * lda : BK), off_a);
-        }
-        if (kk8 == REFILL_B) {
-          if (kt + 1 < kt_end) { if (TB) store_kc<BK, TN, NT>(fb, lds_b[s ^ 1]); else store_xc<BK, TN, NT>(fb, lds_b[s ^ 1]); }
-          if (kt + 2 < kt_end) load_panel<BK, TN, NT, ALIGNED>(fb, base_b + (size_t)(kt + 2) * (TB ? BK : BK * ldb), off_b);
-        }
-      } else if (kk8 == REFILL_AT) {
+      if (kk8 == REFILL_AT) {
         // stage s^1 was last read in the previous iteration, which ended with a barrier
         if (kt + 1 < kt_end) store_stage(s ^ 1);
         if (kt + 2 < kt_end) load_stage(kt + 2);
