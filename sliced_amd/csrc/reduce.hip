@@ -4,6 +4,8 @@
 //
 // Naming (kept from the reference): *_cols reduces along the contiguous axis (one value per
 // row); *_rows reduces along the strided axis (one value per column).
+#include <numeric>
+
 #include "common.hpp"
 
 namespace slhip {
@@ -87,16 +89,18 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
   }
 }
 
-// Contiguous-axis reduction of SHORT rows whose length is not a power of two (2, 3, 10, 100 ...):
-// with a few lanes per row every lane would start its loads at a different dword phase and the
-// wave's loads would scatter (measured 2.1-3.2 TB/s).  Here a workgroup streams a contiguous
-// chunk of whole rows into LDS with full-width vector loads, then one thread per row sums its
-// row out of LDS.  The LDS index is skewed by one word per 32 so that threads striding by an even
-// row length do not pile onto the same banks.
-constexpr int RS_CHUNK = 4096;  // floats per workgroup
+// Contiguous-axis reduction of SHORT rows (up to 64 floats, or up to 128 when the length is not a
+// power of two): with a few lanes per row every lane would start its loads at a different dword
+// phase and the wave's loads would scatter (measured 2.1-3.2 TB/s for lengths 3, 10, 100; 3.3-4.0
+// for 2, 16, 32 against 6.2-6.6 here).  Here a workgroup streams a contiguous
+// chunk of whole rows into LDS with full-width vector loads, all of them requested before the
+// first is used, then `tpr` lanes (a power of two) per row sum the row out of LDS.  The LDS index
+// is skewed by one word per 32 so that threads striding by an even row length do not pile onto the
+// same banks.  A chunk starts on a 128-byte boundary of the matrix.
+constexpr int RS_CHUNK = 4096;  // floats per workgroup at most
 __device__ __forceinline__ int rs_skew(int i) { return i + (i >> 5); }
 template <class Op>
-__global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_t cols, size_t rows_per_block,
+__global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_t cols, size_t rows_per_block, int tpr,
                                                               const float* __restrict__ x, float* __restrict__ out,
                                                               Finalize fin) {
   __shared__ float buf[RS_CHUNK + RS_CHUNK / 32 + 4];
@@ -104,25 +108,38 @@ __global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_
   const size_t nr = r0 + rows_per_block <= rows ? rows_per_block : rows - r0;
   const int len = (int)(nr * cols);  // <= RS_CHUNK
   const float* src = x + r0 * cols;
-  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
+  float4 v[RS_CHUNK / 1024];
+#pragma unroll
+  for (int j = 0; j < RS_CHUNK / 1024; ++j) {
+    const int i = 4 * threadIdx.x + 1024 * j;
+    if (i + 3 < len) v[j] = ld4s(src + i);
+  }
+#pragma unroll
+  for (int j = 0; j < RS_CHUNK / 1024; ++j) {
+    const int i = 4 * threadIdx.x + 1024 * j;
     if (i + 3 < len) {
-      const float4 v = ld4s(src + i);
-      buf[rs_skew(i)] = v.x; buf[rs_skew(i + 1)] = v.y; buf[rs_skew(i + 2)] = v.z; buf[rs_skew(i + 3)] = v.w;
+      buf[rs_skew(i)] = v[j].x; buf[rs_skew(i + 1)] = v[j].y; buf[rs_skew(i + 2)] = v[j].z; buf[rs_skew(i + 3)] = v[j].w;
     } else {
       for (int e = i; e < len; ++e) buf[rs_skew(e)] = src[e];
     }
   }
   __syncthreads();
-  for (size_t r = threadIdx.x; r < nr; r += 256) {
-    const int base = (int)(r * cols);
+  const int lane = threadIdx.x & (tpr - 1), slot = threadIdx.x / tpr, slots = 256 / tpr;
+  for (int rb = 0; rb < (int)nr; rb += slots) {  // the same trip count for every lane of the block
+    const int r = rb + slot;
     float a0 = Op::identity(), a1 = a0;
-    int c = 0;
-    for (; c + 1 < (int)cols; c += 2) {
-      a0 = Op::apply(a0, buf[rs_skew(base + c)]);
-      a1 = Op::apply(a1, buf[rs_skew(base + c + 1)]);
+    if (r < (int)nr) {
+      const int base = r * (int)cols;
+      int c = lane;
+      for (; c + tpr < (int)cols; c += 2 * tpr) {
+        a0 = Op::apply(a0, buf[rs_skew(base + c)]);
+        a1 = Op::apply(a1, buf[rs_skew(base + c + tpr)]);
+      }
+      if (c < (int)cols) a0 = Op::apply(a0, buf[rs_skew(base + c)]);
     }
-    if (c < (int)cols) a0 = Op::apply(a0, buf[rs_skew(base + c)]);
-    finalize_store(out + r0 + r, Op::apply(a0, a1), fin);
+    float s = Op::apply(a0, a1);
+    for (int off = tpr >> 1; off > 0; off >>= 1) s = Op::apply(s, __shfl_xor(s, off, WAVE));
+    if (r < (int)nr && lane == 0) finalize_store(out + r0 + r, s, fin);
   }
 }
 
@@ -158,11 +175,18 @@ template <class Op>
 static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
   // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
   if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, rows * sizeof(float));
-  if (cols <= 128 && (cols & (cols - 1)) != 0 && rows >= 1024) {  // many short rows, not a power of two long
-    const size_t rpb = RS_CHUNK / cols;
+  if (cols <= 128 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {  // many short rows
+    // whole multiples of 256 rows while they fit (every lane of the second phase busy), else as many
+    // rows as fit, rounded down so that every chunk starts on a 128-byte boundary
+    size_t rpb = RS_CHUNK / cols;
+    const size_t g32 = 32 / (size_t)std::gcd((unsigned long long)cols, 32ull);
+    if (rpb >= 256) rpb -= rpb % 256;
+    else if (rpb >= g32) rpb -= rpb % g32;
+    int tpr = 1;  // lanes per row in the second phase
+    while (tpr < 64 && rpb * (size_t)tpr * 2 <= 256 && (size_t)tpr * 2 <= cols) tpr <<= 1;
     const size_t blocks = (rows + rpb - 1) / rpb;
     SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-    hipLaunchKernelGGL((rowreduce_short_kernel<Op>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, rpb, x, out, fin);
+    hipLaunchKernelGGL((rowreduce_short_kernel<Op>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, rpb, tpr, x, out, fin);
     return post_launch();
   }
   const bool vec = cols >= 4;  // any row length: dword-aligned float4 loads plus a scalar tail

@@ -414,7 +414,9 @@ RED_SHAPES = [(1, 1), (1, 5), (5, 1), (3, 4), (7, 13), (64, 64), (33, 1000), (10
               # many short rows whose length is not a power of two (LDS-staged contiguous-axis kernel),
               # odd and even row lengths through the flat strided-axis stages, few rows of great length
               (5000, 3), (4099, 10), (2000, 100), (1025, 127), (70000, 2), (30011, 7), (9001, 33), (20000, 258),
-              (13, 300001), (9, 100002), (1500, 1001)]
+              (13, 300001), (9, 100002), (1500, 1001),
+              # short rows a power of two long (the same LDS-staged kernel, several lanes per row)
+              (3001, 64), (2100, 32), (5003, 8), (1100, 5), (1024, 4), (1029, 48)]
 
 
 def sum_bound(x, rows, cols, axis):
