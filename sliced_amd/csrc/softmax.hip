@@ -6,6 +6,8 @@
 // The reference builds the forward from five passes (max_cols, sub_cols, exp, sum_cols,
 // div_cols) and the backward from a per-sample Jacobian; the arithmetic per element is the
 // same: e = exp(x - max); out = e / sum(e);  x_grad = s * (g - <s, g>).
+#include <numeric>
+
 #include "common.hpp"
 
 namespace slhip {
@@ -295,15 +297,31 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
 constexpr int SS_CHUNK = 4096;  // floats per workgroup and tensor
 __device__ __forceinline__ int ss_skew(int i) { return i + (i >> 5); }
 
-__device__ __forceinline__ void ss_load(float* buf, const float* __restrict__ src, int len) {
-  for (int i = 4 * threadIdx.x; i < len; i += 1024) {
-    if (i + 3 < len) {
-      const float4 v = ld4s(src + i);
-      buf[ss_skew(i)] = v.x; buf[ss_skew(i + 1)] = v.y; buf[ss_skew(i + 2)] = v.z; buf[ss_skew(i + 3)] = v.w;
-    } else {
-      for (int e = i; e < len; ++e) buf[ss_skew(e)] = src[e];
+// Requests every vector of the chunk (of NB chunks at the same offsets) before the first one is
+// used, then stores them into the skewed LDS buffers.
+template <int NB>
+__device__ __forceinline__ void ss_load(float* const (&buf)[NB], const float* const (&src)[NB], int len) {
+  constexpr int NJ = SS_CHUNK / 1024;
+  float4 v[NB][NJ];
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      if (i + 3 < len) v[b][j] = ld4s(src[b] + i);
     }
-  }
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      float* d = buf[b];
+      if (i + 3 < len) {
+        d[ss_skew(i)] = v[b][j].x; d[ss_skew(i + 1)] = v[b][j].y; d[ss_skew(i + 2)] = v[b][j].z; d[ss_skew(i + 3)] = v[b][j].w;
+      } else {
+        for (int e = i; e < len; ++e) d[ss_skew(e)] = src[b][e];
+      }
+    }
 }
 
 template <int L>
@@ -313,7 +331,11 @@ __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int
   const size_t r0 = (size_t)blockIdx.x * rpb;
   const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
   const int len = nr * cols;
-  ss_load(buf, x + r0 * cols, len);
+  {
+    float* const bufs[1] = {buf};
+    const float* const srcs[1] = {x + r0 * cols};
+    ss_load<1>(bufs, srcs, len);
+  }
   __syncthreads();
   const int lane = threadIdx.x % L, group = threadIdx.x / L;
   for (int rb = 0; rb < nr; rb += 256 / L) {  // the same trip count for every thread: the shuffles need whole groups
@@ -353,8 +375,11 @@ __global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int
   const size_t r0 = (size_t)blockIdx.x * rpb;
   const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
   const int len = nr * cols;
-  ss_load(sb, out + r0 * cols, len);
-  ss_load(gb, out_grad + r0 * cols, len);
+  {
+    float* const bufs[2] = {sb, gb};
+    const float* const srcs[2] = {out + r0 * cols, out_grad + r0 * cols};
+    ss_load<2>(bufs, srcs, len);
+  }
   __syncthreads();
   const int lane = threadIdx.x % L, group = threadIdx.x / L;
   for (int rb = 0; rb < nr; rb += 256 / L) {
@@ -407,11 +432,15 @@ static SoftmaxCfg pick_cfg(size_t colsv, bool fwd) {
 template <bool FWD, bool VEC>
 static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, float* x_grad,
                                 const float* s, const float* g, float beta) {
-  // many short rows, not a power of two long (measured at 2^27 elements, forward / backward TB/s,
-  // lanes-per-row kernel -> this one: 10: 3.1 / 2.8 -> 4.8 / 3.9; 36: 2.2 / 2.9 -> 4.7 / 4.7; 100: 3.0 / 3.6 ->
-  // 4.4 / 4.3; from 200 on the lanes-per-row kernel is the faster one again)
-  if (cols >= 3 && cols <= 160 && (cols & (cols - 1)) != 0 && rows >= 1024) {
-    const int rpb = SS_CHUNK / (int)cols;
+  // many short rows (measured at 2^27 elements, forward / backward TB/s, lanes-per-row kernel -> this
+  // one: 10: 3.1 / 2.8 -> 5.8 / 6.1; 36: 2.2 / 2.9 -> 5.3 / 5.4; 100: 3.0 / 3.6 -> 4.8 / 5.2; 8: 3.3 / 4.0 ->
+  // 5.9 / 6.1; 16: 1.4 / 1.8 -> 6.2 / 6.1; 32: 1.8 / 2.5 -> 5.6 / 6.2; 64: 4.9 / 5.2 -> 5.6 / 6.2; rows of 2 only
+  // backward: 4.6 / 5.6 -> 4.0 / 6.1; at 128 and from 200 on the lanes-per-row kernel is the faster one)
+  if (cols >= (FWD ? 3 : 2) && cols <= 160 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {
+    int rpb = SS_CHUNK / (int)cols;
+    const int g32 = 32 / std::gcd((int)cols, 32);  // chunks start on 128-byte boundaries
+    if (rpb >= 256) rpb -= rpb % 256;  // every thread of the row phase busy
+    else if (rpb >= g32) rpb -= rpb % g32;
     int lanes = 1;
     while (lanes < 64 && lanes * 2 * rpb <= 256) lanes <<= 1;  // groups of `lanes` lanes, at least one per row of the chunk
     const size_t blocks = (rows + rpb - 1) / rpb;

@@ -508,7 +508,9 @@ SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (6
                   # 1025..2048 vectors per row: the forward pass runs 512 lanes there, the backward pass 1024
                   (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196),
                   # many short rows, not a power of two long: the LDS-staged kernels
-                  (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (4097, 37), (1024, 6)]
+                  (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (4097, 37), (1024, 6),
+                  # and short rows a power of two long, which take the same kernels
+                  (3000, 16), (1100, 64), (5000, 2), (2049, 32), (1030, 8), (4100, 4), (1023, 16)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=lambda s: "x".join(map(str, s)))
