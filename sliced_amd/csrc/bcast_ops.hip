@@ -1,8 +1,7 @@
 // Row / column broadcast ops with an op code, diagflat and the onehot gradient: the part of the
 // reference's op surface beside the training hot path (reference: src/ops2/row_op, src/ops2/col_op,
 // src/ops2/diagflat, src/ops2/onehot).  Plain streaming kernels; the
-// reductions of the broadcast-side gradients go through partial sums in the context workspace
-// and are combined in a fixed order.
+// reductions of the broadcast-side gradients run through the row / column reduction kernels.
 #include "common.hpp"
 
 namespace slhip {
@@ -15,25 +14,6 @@ __device__ __forceinline__ float bc_apply(int op, float a, float b) {
     default: return a / b;
   }
 }
-// d f(l, r) / d l   and   d f(l, r) / d r, as the reference's tests write them
-// (src/ops2/col_op/grad/cpu.rs:115,146: 1/rhs and lhs / -(rhs*rhs) for div)
-__device__ __forceinline__ float bc_dl(int op, float l, float r) {
-  switch (op) {
-    case SLHIP_ADD: return 1.0f;
-    case SLHIP_SUB: return 1.0f;
-    case SLHIP_MUL: return r;
-    default: return 1.0f / r;
-  }
-}
-__device__ __forceinline__ float bc_dr(int op, float l, float r) {
-  switch (op) {
-    case SLHIP_ADD: return 1.0f;
-    case SLHIP_SUB: return -1.0f;
-    case SLHIP_MUL: return l;
-    default: return l / (-(r * r));
-  }
-}
-
 // Forward and lhs gradient.  The matrix is walked as one flat run of float4 (dword-aligned, so any
 // row length and base address): a thread finds the row and column of its first element with one
 // division and steps from there.  BY_ROW_INDEX: the broadcast vector is indexed by the row
@@ -83,43 +63,6 @@ static void bc_flat_launch(slhip_ctx* ctx, int op, size_t len, size_t cols, cons
     hipLaunchKernelGGL((bc_flat_kernel<BY_ROW_INDEX, GRAD, uint32_t>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out, g);
   else
     hipLaunchKernelGGL((bc_flat_kernel<BY_ROW_INDEX, GRAD, size_t>), dim3(blocks), dim3(256), 0, ctx->stream, op, len, cols, lhs, v, out, g);
-}
-
-// col_op: v_grad[r] += sum_c dR(lhs[r,c], v[r]) * g[r,c]; one wave per row
-__global__ __launch_bounds__(256) void colop_grad_rhs_kernel(int op, size_t rows, size_t cols,
-                                                             const float* __restrict__ lhs, const float* __restrict__ v,
-                                                             float* __restrict__ v_grad, const float* __restrict__ g) {
-  const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= rows) return;
-  const int lane = threadIdx.x & 63;
-  const float vr = v[r];
-  float s = 0.0f;
-  for (size_t c = lane; c < cols; c += 64) s += bc_dr(op, lhs[r * cols + c], vr) * g[r * cols + c];
-  s = wave_reduce<SumOp>(s);
-  if (lane == 0) v_grad[r] += s;
-}
-
-// row_op: v_grad[c] += sum_r dR(lhs[r,c], v[c]) * g[r,c]; G row groups write partials, then one
-// thread per column adds them up in group order
-__global__ __launch_bounds__(256) void rowop_grad_rhs_partial_kernel(int op, size_t rows, size_t cols, size_t G,
-                                                                     const float* __restrict__ lhs,
-                                                                     const float* __restrict__ v,
-                                                                     const float* __restrict__ g, float* __restrict__ part) {
-  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= cols * G) return;
-  const size_t grp = t / cols, c = t - grp * cols;
-  const float vc = v[c];
-  float s = 0.0f;
-  for (size_t r = grp; r < rows; r += G) s += bc_dr(op, lhs[r * cols + c], vc) * g[r * cols + c];
-  part[grp * cols + c] = s;
-}
-__global__ __launch_bounds__(256) void rowop_grad_rhs_final_kernel(size_t cols, size_t G, const float* __restrict__ part,
-                                                                   float* __restrict__ v_grad) {
-  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= cols) return;
-  float s = part[c];
-  for (size_t grp = 1; grp < G; ++grp) s += part[grp * cols + c];
-  v_grad[c] += s;
 }
 
 __global__ __launch_bounds__(256) void diagflat_kernel(size_t n, const float* __restrict__ x, float* __restrict__ out) {
@@ -184,37 +127,9 @@ static int32_t bc_backward(slhip_ctx* ctx, int32_t op, size_t rows, size_t cols,
     if (rc) return rc;
   }
   if (!v_grad) return SLHIP_OK;
-  if (BY_ROW_INDEX) {
-    const size_t b = (rows + 3) / 4;
-    if (b > 0x7fffffffu) {
-      set_error("col_op grad: %zu rows exceed one launch", rows);
-      return SLHIP_EINVAL;
-    }
-    hipLaunchKernelGGL(colop_grad_rhs_kernel, dim3((unsigned)b), dim3(256), 0, ctx->stream, op, rows, cols, lhs, v, v_grad, g);
-    return post_launch();
-  }
-  // row groups: enough threads to fill the chip, never more groups than rows or than the workspace holds
-  size_t G = ((size_t)ctx->num_cu * 2048 + cols - 1) / cols;
-  if (G > rows) G = rows;
-  if (G > 1024) G = 1024;
-  const size_t fit = ctx->workspace_bytes / (cols * sizeof(float));
-  if (fit == 0) {
-    set_error("row_op grad: %zu columns exceed the workspace", cols);
-    return SLHIP_EWORKSPACE;
-  }
-  if (G > fit) G = fit;
-  if (G < 1) G = 1;
-  unsigned pb, fb;
-  if (!grid_for(cols * G, &pb) || !grid_for(cols, &fb)) {
-    set_error("row_op grad: %zu columns exceed one launch", cols);
-    return SLHIP_EINVAL;
-  }
-  float* part = (float*)ctx->workspace;
-  hipLaunchKernelGGL(rowop_grad_rhs_partial_kernel, dim3(pb), dim3(256), 0, ctx->stream, op, rows, cols, G, lhs, v, g, part);
-  int32_t rc = post_launch();
-  if (rc) return rc;
-  hipLaunchKernelGGL(rowop_grad_rhs_final_kernel, dim3(fb), dim3(256), 0, ctx->stream, cols, G, (const float*)part, v_grad);
-  return post_launch();
+  // v_grad[i] += sum over row i (col_op) or column i (row_op) of dR(lhs, v[i]) * g: the reductions'
+  // own kernels, reading the two matrices in place of one
+  return bc_grad_rhs_reduce(ctx, BY_ROW_INDEX, op, rows, cols, lhs, v, g, v_grad);
 }
 
 }  // namespace slhip

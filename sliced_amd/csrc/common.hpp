@@ -154,4 +154,28 @@ __device__ __forceinline__ void st4s(float* p, float4 v) {
 __device__ __forceinline__ float ld1s(const float* p) { return __builtin_nontemporal_load(p); }
 __device__ __forceinline__ void st1s(float* p, float v) { __builtin_nontemporal_store(v, p); }
 
+// d f(l, r) / d l   and   d f(l, r) / d r, as the reference's tests write them
+// (src/ops2/col_op/grad/cpu.rs:115,146: 1/rhs and lhs / -(rhs*rhs) for div)
+__device__ __forceinline__ float bc_dl(int op, float l, float r) {
+  switch (op) {
+    case SLHIP_ADD: return 1.0f;
+    case SLHIP_SUB: return 1.0f;
+    case SLHIP_MUL: return r;
+    default: return 1.0f / r;
+  }
+}
+__device__ __forceinline__ float bc_dr(int op, float l, float r) {
+  switch (op) {
+    case SLHIP_ADD: return 1.0f;
+    case SLHIP_SUB: return -1.0f;
+    case SLHIP_MUL: return l;
+    default: return l / (-(r * r));
+  }
+}
+
+// v_grad[i] += the rhs-gradient terms of a broadcast op summed over row i (by_row) or column i
+// (defined with the reductions, whose kernels it runs).
+int32_t bc_grad_rhs_reduce(slhip_ctx* ctx, bool by_row, int op, size_t rows, size_t cols, const float* lhs, const float* v,
+                           const float* g, float* v_grad);
+
 }  // namespace slhip

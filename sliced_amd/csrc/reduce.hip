@@ -23,13 +23,39 @@ __device__ __forceinline__ void finalize_store(float* p, float v, Finalize f) {
   *p = v;
 }
 
+// What a reduction reads.  PlainSrc: the matrix itself.  BcGradSrc: the rhs-gradient terms of a
+// broadcast op, dR(lhs[e], v) * g[e], v being the broadcast vector's entry for that element's row
+// (reductions along the contiguous axis: col_op) or column (reductions along the strided axis:
+// row_op); the kernels hand in v's entry, which they know from the row or column they work on.
+struct PlainSrc {
+  static constexpr bool HAS_V = false;
+  const float* x;
+  __device__ __forceinline__ float bvalue(size_t) const { return 0.0f; }
+  __device__ __forceinline__ float4 vec(size_t e, float, float, float, float) const { return ld4s(x + e); }
+  __device__ __forceinline__ float one(size_t e, float) const { return ld1s(x + e); }
+};
+struct BcGradSrc {
+  static constexpr bool HAS_V = true;
+  const float* l;
+  const float* g;
+  const float* v;
+  int op;
+  __device__ __forceinline__ float bvalue(size_t i) const { return v[i]; }
+  __device__ __forceinline__ float4 vec(size_t e, float v0, float v1, float v2, float v3) const {
+    const float4 a = ld4s(l + e), b = ld4s(g + e);
+    return make_float4(bc_dr(op, a.x, v0) * b.x, bc_dr(op, a.y, v1) * b.y, bc_dr(op, a.z, v2) * b.z,
+                       bc_dr(op, a.w, v3) * b.w);
+  }
+  __device__ __forceinline__ float one(size_t e, float vv) const { return bc_dr(op, ld1s(l + e), vv) * ld1s(g + e); }
+};
+
 // ---------------------------------------------------------------------------------------
 // Contiguous-axis reduction.  TPR lanes (power of two <= 64) or a whole block (TPR == 0) own one
 // row segment; gridDim.y = number of segments a row is split into (partials when > 1).
 // ---------------------------------------------------------------------------------------
-template <class Op, bool VEC, int TPR>
-__global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols, const float* __restrict__ x,
-                                                        float* __restrict__ out, Finalize fin) {
+template <class Op, bool VEC, int TPR, class Src>
+__global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols, Src src, float* __restrict__ out,
+                                                        Finalize fin) {
   __shared__ float smem[8];
   constexpr int V = VEC ? 4 : 1;
   constexpr int LANES = TPR == 0 ? 256 : TPR;
@@ -45,32 +71,33 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
 
   float a0 = Op::identity(), a1 = Op::identity(), a2 = Op::identity(), a3 = Op::identity();
   if (active) {
-    const float* xr = x + row * cols;
+    const size_t xr = row * cols;
+    const float vv = Src::HAS_V ? src.bvalue(row) : 0.0f;
     size_t c = cbeg + lane;
     if (VEC) {
       for (; c + 3 * LANES < cend; c += 4 * LANES) {
-        float4 v0 = ld4s(xr + 4 * c), v1 = ld4s(xr + 4 * (c + LANES)), v2 = ld4s(xr + 4 * (c + 2 * LANES)),
-               v3 = ld4s(xr + 4 * (c + 3 * LANES));
+        float4 v0 = src.vec(xr + 4 * c, vv, vv, vv, vv), v1 = src.vec(xr + 4 * (c + LANES), vv, vv, vv, vv),
+               v2 = src.vec(xr + 4 * (c + 2 * LANES), vv, vv, vv, vv), v3 = src.vec(xr + 4 * (c + 3 * LANES), vv, vv, vv, vv);
         a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
         a1 = Op::apply(a1, Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)));
         a2 = Op::apply(a2, Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)));
         a3 = Op::apply(a3, Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)));
       }
       for (; c < cend; c += LANES) {
-        float4 v0 = ld4s(xr + 4 * c);
+        float4 v0 = src.vec(xr + 4 * c, vv, vv, vv, vv);
         a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
       }
       // a row of odd length ends in up to 3 floats beyond its last whole vector
       if ((cols & 3) && seg == nseg - 1 && lane == 0)
-        for (size_t e = 4 * colsv; e < cols; ++e) a1 = Op::apply(a1, xr[e]);
+        for (size_t e = 4 * colsv; e < cols; ++e) a1 = Op::apply(a1, src.one(xr + e, vv));
     } else {
       for (; c + 3 * LANES < cend; c += 4 * LANES) {
-        a0 = Op::apply(a0, ld1s(xr + c));
-        a1 = Op::apply(a1, ld1s(xr + c + LANES));
-        a2 = Op::apply(a2, ld1s(xr + c + 2 * LANES));
-        a3 = Op::apply(a3, ld1s(xr + c + 3 * LANES));
+        a0 = Op::apply(a0, src.one(xr + c, vv));
+        a1 = Op::apply(a1, src.one(xr + c + LANES, vv));
+        a2 = Op::apply(a2, src.one(xr + c + 2 * LANES, vv));
+        a3 = Op::apply(a3, src.one(xr + c + 3 * LANES, vv));
       }
-      for (; c < cend; c += LANES) a0 = Op::apply(a0, ld1s(xr + c));
+      for (; c < cend; c += LANES) a0 = Op::apply(a0, src.one(xr + c, vv));
     }
   }
   float v = Op::apply(Op::apply(a0, a1), Op::apply(a2, a3));
@@ -98,29 +125,44 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
 // is skewed by one word per 32 so that threads striding by an even row length do not pile onto the
 // same banks.  A chunk starts on a 128-byte boundary of the matrix.
 constexpr int RS_CHUNK = 4096;  // floats per workgroup at most
-__device__ __forceinline__ int rs_skew(int i) { return i + (i >> 5); }
-template <class Op>
+// sh = 5 for rows of even length, 31 (no skew) for odd ones, whose stride already visits every bank
+__device__ __forceinline__ int rs_skew(int sh, int i) { return i + (i >> sh); }
+__device__ __forceinline__ int rs_skew_shift(int cols) { return (cols & 1) ? 31 : 5; }
+template <class Op, class Src>
 __global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_t cols, size_t rows_per_block, int tpr,
-                                                              const float* __restrict__ x, float* __restrict__ out,
-                                                              Finalize fin) {
+                                                              Src src, float* __restrict__ out, Finalize fin) {
   __shared__ float buf[RS_CHUNK + RS_CHUNK / 32 + 4];
+  const int sh = rs_skew_shift((int)cols);
   const size_t r0 = (size_t)blockIdx.x * rows_per_block;
   const size_t nr = r0 + rows_per_block <= rows ? rows_per_block : rows - r0;
   const int len = (int)(nr * cols);  // <= RS_CHUNK
-  const float* src = x + r0 * cols;
+  const size_t e0 = r0 * cols;
+  // the broadcast entry of local element i: the one of row r0 + i / cols
+  auto bv = [&](int i) { return src.bvalue(r0 + (size_t)(i / (int)cols)); };
   float4 v[RS_CHUNK / 1024];
 #pragma unroll
   for (int j = 0; j < RS_CHUNK / 1024; ++j) {
     const int i = 4 * threadIdx.x + 1024 * j;
-    if (i + 3 < len) v[j] = ld4s(src + i);
+    if (i + 3 < len) {
+      float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (Src::HAS_V) {
+        int rl = i / (int)cols, c = i - rl * (int)cols;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          b[q] = src.bvalue(r0 + rl);
+          if (++c == (int)cols) { c = 0; ++rl; }
+        }
+      }
+      v[j] = src.vec(e0 + i, b[0], b[1], b[2], b[3]);
+    }
   }
 #pragma unroll
   for (int j = 0; j < RS_CHUNK / 1024; ++j) {
     const int i = 4 * threadIdx.x + 1024 * j;
     if (i + 3 < len) {
-      buf[rs_skew(i)] = v[j].x; buf[rs_skew(i + 1)] = v[j].y; buf[rs_skew(i + 2)] = v[j].z; buf[rs_skew(i + 3)] = v[j].w;
+      buf[rs_skew(sh, i)] = v[j].x; buf[rs_skew(sh, i + 1)] = v[j].y; buf[rs_skew(sh, i + 2)] = v[j].z; buf[rs_skew(sh, i + 3)] = v[j].w;
     } else {
-      for (int e = i; e < len; ++e) buf[rs_skew(e)] = src[e];
+      for (int e = i; e < len; ++e) buf[rs_skew(sh, e)] = src.one(e0 + e, Src::HAS_V ? bv(e) : 0.0f);
     }
   }
   __syncthreads();
@@ -132,10 +174,10 @@ __global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_
       const int base = r * (int)cols;
       int c = lane;
       for (; c + tpr < (int)cols; c += 2 * tpr) {
-        a0 = Op::apply(a0, buf[rs_skew(base + c)]);
-        a1 = Op::apply(a1, buf[rs_skew(base + c + tpr)]);
+        a0 = Op::apply(a0, buf[rs_skew(sh, base + c)]);
+        a1 = Op::apply(a1, buf[rs_skew(sh, base + c + tpr)]);
       }
-      if (c < (int)cols) a0 = Op::apply(a0, buf[rs_skew(base + c)]);
+      if (c < (int)cols) a0 = Op::apply(a0, buf[rs_skew(sh, base + c)]);
     }
     float s = Op::apply(a0, a1);
     for (int off = tpr >> 1; off > 0; off >>= 1) s = Op::apply(s, __shfl_xor(s, off, WAVE));
@@ -143,8 +185,8 @@ __global__ __launch_bounds__(256) void rowreduce_short_kernel(size_t rows, size_
   }
 }
 
-template <class Op, bool VEC>
-static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, unsigned nseg,
+template <class Op, bool VEC, class Src>
+static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, unsigned nseg,
                                 Finalize fin) {
   const size_t colsv = cols / (VEC ? 4 : 1);
   const size_t per_seg = (colsv + nseg - 1) / nseg;
@@ -160,7 +202,7 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const 
   case T: {                                                                                                   \
     unsigned rpb = T == 0 ? 1 : 256 / (T == 0 ? 1 : T);                                                       \
     dim3 grid(ceil_div(rows, rpb), nseg);                                                                     \
-    hipLaunchKernelGGL((rowreduce_kernel<Op, VEC, T>), grid, dim3(256), 0, ctx->stream, rows, cols, x, out, fin); \
+    hipLaunchKernelGGL((rowreduce_kernel<Op, VEC, T, Src>), grid, dim3(256), 0, ctx->stream, rows, cols, x, out, fin); \
     break;                                                                                                    \
   }
   switch (tpr) {
@@ -171,10 +213,11 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, const 
 }
 
 // out[r] = reduce over the contiguous axis.
-template <class Op>
-static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
+template <class Op, class Src>
+static int32_t reduce_cols_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin) {
   // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
-  if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, rows * sizeof(float));
+  if constexpr (!Src::HAS_V)
+    if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, rows * sizeof(float));
   if (cols <= 128 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {  // many short rows
     // whole multiples of 256 rows while they fit (every lane of the second phase busy), else as many
     // rows as fit, rounded down so that every chunk starts on a 128-byte boundary
@@ -186,7 +229,7 @@ static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float
     while (tpr < 64 && rpb * (size_t)tpr * 2 <= 256 && (size_t)tpr * 2 <= cols) tpr <<= 1;
     const size_t blocks = (rows + rpb - 1) / rpb;
     SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-    hipLaunchKernelGGL((rowreduce_short_kernel<Op>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, rpb, tpr, x, out, fin);
+    hipLaunchKernelGGL((rowreduce_short_kernel<Op, Src>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, rpb, tpr, x, out, fin);
     return post_launch();
   }
   const bool vec = cols >= 4;  // any row length: dword-aligned float4 loads plus a scalar tail
@@ -202,18 +245,18 @@ static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float
     if (s > max_s) s = max_s;
     if (s > 1) nseg = (unsigned)s;
   }
-  if (nseg == 1) return vec ? rowreduce_launch<Op, true>(ctx, rows, cols, x, out, 1, fin)
-                            : rowreduce_launch<Op, false>(ctx, rows, cols, x, out, 1, fin);
+  if (nseg == 1) return vec ? rowreduce_launch<Op, true, Src>(ctx, rows, cols, x, out, 1, fin)
+                            : rowreduce_launch<Op, false, Src>(ctx, rows, cols, x, out, 1, fin);
   if (rows * nseg * sizeof(float) > ctx->workspace_bytes) {
     set_error("reduce over columns: %zu x %u partials exceed the workspace", rows, nseg);
     return SLHIP_EWORKSPACE;
   }
   float* part = (float*)ctx->workspace;
   Finalize none{1.0f, 0, 0};
-  int32_t rc = vec ? rowreduce_launch<Op, true>(ctx, rows, cols, x, part, nseg, none)
-                   : rowreduce_launch<Op, false>(ctx, rows, cols, x, part, nseg, none);
+  int32_t rc = vec ? rowreduce_launch<Op, true, Src>(ctx, rows, cols, x, part, nseg, none)
+                   : rowreduce_launch<Op, false, Src>(ctx, rows, cols, x, part, nseg, none);
   if (rc) return rc;
-  return rowreduce_launch<Op, false>(ctx, rows, nseg, part, out, 1, fin);
+  return rowreduce_launch<Op, false, PlainSrc>(ctx, rows, nseg, PlainSrc{part}, out, 1, fin);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -226,22 +269,32 @@ static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float
 // one-column-per-thread kernel with scalar loads reduced at 3.1-3.5 TB/s, stream at the same rate
 // as rows that are a multiple of 4 long; one sweep of the grid reads one contiguous span of 16T bytes.
 // ---------------------------------------------------------------------------------------
-template <class Op>
-__global__ __launch_bounds__(256) void colreduce_flat_kernel(size_t n, size_t T, const float* __restrict__ x,
+template <class Op, class Src>
+__global__ __launch_bounds__(256) void colreduce_flat_kernel(size_t n, size_t T, size_t cols, Src src,
                                                              float* __restrict__ part) {
   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (t >= T) return;
+  float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // the broadcast entries of this thread's four columns
+  if (Src::HAS_V) {
+    size_t c = (4 * t) % cols;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      b[q] = src.bvalue(c);
+      if (++c == cols) c = 0;
+    }
+  }
   const size_t nv = n >> 2;  // whole vectors of the stream
   const float id = Op::identity();
   float4 a0 = make_float4(id, id, id, id), a1 = a0, a2 = a0, a3 = a0;
 #define SL_ACC(A, Q) A.x = Op::apply(A.x, Q.x); A.y = Op::apply(A.y, Q.y); A.z = Op::apply(A.z, Q.z); A.w = Op::apply(A.w, Q.w);
   size_t i = t;
   for (; i + 3 * T < nv; i += 4 * T) {
-    float4 v0 = ld4s(x + 4 * i), v1 = ld4s(x + 4 * (i + T)), v2 = ld4s(x + 4 * (i + 2 * T)), v3 = ld4s(x + 4 * (i + 3 * T));
+    float4 v0 = src.vec(4 * i, b[0], b[1], b[2], b[3]), v1 = src.vec(4 * (i + T), b[0], b[1], b[2], b[3]),
+           v2 = src.vec(4 * (i + 2 * T), b[0], b[1], b[2], b[3]), v3 = src.vec(4 * (i + 3 * T), b[0], b[1], b[2], b[3]);
     SL_ACC(a0, v0) SL_ACC(a1, v1) SL_ACC(a2, v2) SL_ACC(a3, v3)
   }
   for (; i < nv; i += T) {
-    float4 v0 = ld4s(x + 4 * i);
+    float4 v0 = src.vec(4 * i, b[0], b[1], b[2], b[3]);
     SL_ACC(a0, v0)
   }
   SL_ACC(a0, a1) SL_ACC(a2, a3) SL_ACC(a0, a2)
@@ -250,8 +303,8 @@ __global__ __launch_bounds__(256) void colreduce_flat_kernel(size_t n, size_t T,
   for (size_t e = nv << 2; e < n; ++e) {
     const size_t pos = e % (4 * T);
     if (pos >> 2 == t) {
-      const float v = x[e];
       const int q = (int)(pos & 3);
+      const float v = src.one(e, b[q]);
       if (q == 0) a0.x = Op::apply(a0.x, v);
       else if (q == 1) a0.y = Op::apply(a0.y, v);
       else if (q == 2) a0.z = Op::apply(a0.z, v);
@@ -263,23 +316,24 @@ __global__ __launch_bounds__(256) void colreduce_flat_kernel(size_t n, size_t T,
 
 // Stage 2 (also the only stage for short matrices): a block owns CW adjacent columns, its
 // 256/CW row-lanes stride over the rows and combine through LDS.
-template <class Op, int CW>
-__global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_t cols, const float* __restrict__ x,
-                                                              float* __restrict__ out, Finalize fin) {
+template <class Op, int CW, class Src>
+__global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_t cols, Src src, float* __restrict__ out,
+                                                              Finalize fin) {
   constexpr int RL = 256 / CW;
   __shared__ float sm[256];
   const int cx = threadIdx.x % CW, ry = threadIdx.x / CW;
   const size_t c = (size_t)blockIdx.x * CW + cx;
   float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
   if (c < cols) {
+    const float vv = Src::HAS_V ? src.bvalue(c) : 0.0f;
     size_t r = ry;
     for (; r + 3 * RL < rows; r += 4 * RL) {  // four loads in flight per lane
-      a0 = Op::apply(a0, x[r * cols + c]);
-      a1 = Op::apply(a1, x[(r + RL) * cols + c]);
-      a2 = Op::apply(a2, x[(r + 2 * RL) * cols + c]);
-      a3 = Op::apply(a3, x[(r + 3 * RL) * cols + c]);
+      a0 = Op::apply(a0, src.one(r * cols + c, vv));
+      a1 = Op::apply(a1, src.one((r + RL) * cols + c, vv));
+      a2 = Op::apply(a2, src.one((r + 2 * RL) * cols + c, vv));
+      a3 = Op::apply(a3, src.one((r + 3 * RL) * cols + c, vv));
     }
-    for (; r < rows; r += RL) a0 = Op::apply(a0, x[r * cols + c]);
+    for (; r < rows; r += RL) a0 = Op::apply(a0, src.one(r * cols + c, vv));
   }
   a0 = Op::apply(a0, a2);
   a1 = Op::apply(a1, a3);
@@ -293,9 +347,49 @@ __global__ __launch_bounds__(256) void colreduce_final_kernel(size_t rows, size_
   if (ry == 0 && c < cols) finalize_store(out + c, sm[cx], fin);
 }
 
-template <class Op>
-static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out,
-                                      Finalize fin) {
+// Strided-axis reduction of a matrix of fewer than 8 rows (a single row that is added into `out`
+// included): one thread per four adjacent columns, every row's vector requested before the first
+// is used.  colreduce_final_kernel would leave three lanes in four idle on such a matrix and read
+// it with scalar loads (measured 1.4 TB/s on [1 x 2^27] into an accumulating output).
+constexpr int FEW_ROWS = 8;
+template <class Op, class Src>
+__global__ __launch_bounds__(256) void colreduce_fewrows_kernel(size_t rows, size_t cols, Src src, float* __restrict__ out,
+                                                                Finalize fin) {
+  const size_t c0 = 4 * ((size_t)blockIdx.x * 256 + threadIdx.x);
+  if (c0 >= cols) return;
+  float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (Src::HAS_V)
+    for (int q = 0; q < 4 && c0 + q < cols; ++q) b[q] = src.bvalue(c0 + q);
+  const float id = Op::identity();
+  float a[4] = {id, id, id, id};
+  if (c0 + 3 < cols) {
+    float4 v[FEW_ROWS];
+#pragma unroll
+    for (int r = 0; r < FEW_ROWS; ++r)
+      if ((size_t)r < rows) v[r] = src.vec((size_t)r * cols + c0, b[0], b[1], b[2], b[3]);
+#pragma unroll
+    for (int r = 0; r < FEW_ROWS; ++r)
+      if ((size_t)r < rows) {
+        a[0] = Op::apply(a[0], v[r].x); a[1] = Op::apply(a[1], v[r].y);
+        a[2] = Op::apply(a[2], v[r].z); a[3] = Op::apply(a[3], v[r].w);
+      }
+    float4 o = make_float4(a[0], a[1], a[2], a[3]);
+    if (fin.divide) { o.x = o.x / fin.scale; o.y = o.y / fin.scale; o.z = o.z / fin.scale; o.w = o.w / fin.scale; }
+    if (fin.accumulate) {
+      const float4 old = ld4g(out + c0);
+      o.x = old.x + o.x; o.y = old.y + o.y; o.z = old.z + o.z; o.w = old.w + o.w;
+    }
+    st4g(out + c0, o);
+  } else {
+    for (int q = 0; c0 + q < cols; ++q) {
+      for (size_t r = 0; r < rows; ++r) a[q] = Op::apply(a[q], src.one(r * cols + c0 + q, b[q]));
+      finalize_store(out + c0 + q, a[q], fin);
+    }
+  }
+}
+
+template <class Op, class Src>
+static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin) {
   // the widest column strip that still leaves every row-lane at most 16 rows
   int cw = 1;
   if (cols >= 64 && rows * 64 <= 4096) cw = 64;
@@ -304,7 +398,7 @@ static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, 
   else if (rows > 4096) cw = cols >= 16 ? 16 : cols >= 4 ? 4 : 1;  // long inputs: coalescing matters more
   SLHIP_REQUIRE(grid_fits(cols, cw), "too many columns for one launch");
 #define SL_CF(CW_)                                                                                                    \
-  hipLaunchKernelGGL((colreduce_final_kernel<Op, CW_>), dim3(ceil_div(cols, CW_)), dim3(256), 0, ctx->stream, rows, cols, \
+  hipLaunchKernelGGL((colreduce_final_kernel<Op, CW_, Src>), dim3(ceil_div(cols, CW_)), dim3(256), 0, ctx->stream, rows, cols, \
                      x, out, fin)
   if (cw == 64) SL_CF(64);
   else if (cw == 16) SL_CF(16);
@@ -317,10 +411,10 @@ static int32_t colreduce_final_launch(slhip_ctx* ctx, size_t rows, size_t cols, 
 // ---------------------------------------------------------------------------------------
 // Whole-buffer reduction: per-block partials, then one block.
 // ---------------------------------------------------------------------------------------
-template <class Op, bool VEC>
-__global__ __launch_bounds__(256) void fullreduce_kernel(size_t n, const float* __restrict__ x,
-                                                         float* __restrict__ part) {
+template <class Op, bool VEC, class Src>
+__global__ __launch_bounds__(256) void fullreduce_kernel(size_t n, Src src, float* __restrict__ part) {
   __shared__ float smem[8];
+  const float vv = Src::HAS_V ? src.bvalue(0) : 0.0f;  // a matrix of one column: one broadcast entry
   // every block streams ONE contiguous chunk (measured: 7.0-7.2 TB/s, against 5.7 TB/s when the
   // blocks interleave grid-stride fashion)
   float a0 = Op::identity(), a1 = a0, a2 = a0, a3 = a0;
@@ -331,40 +425,41 @@ __global__ __launch_bounds__(256) void fullreduce_kernel(size_t n, const float* 
     const size_t end = beg + chunk < n4 ? beg + chunk : n4;
     size_t i = beg + threadIdx.x;
     for (; i + 3 * 256 < end; i += 4 * 256) {
-      float4 v0 = ld4s(x + 4 * i), v1 = ld4s(x + 4 * (i + 256)), v2 = ld4s(x + 4 * (i + 512)),
-             v3 = ld4s(x + 4 * (i + 768));
+      float4 v0 = src.vec(4 * i, vv, vv, vv, vv), v1 = src.vec(4 * (i + 256), vv, vv, vv, vv),
+             v2 = src.vec(4 * (i + 512), vv, vv, vv, vv), v3 = src.vec(4 * (i + 768), vv, vv, vv, vv);
       a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
       a1 = Op::apply(a1, Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)));
       a2 = Op::apply(a2, Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)));
       a3 = Op::apply(a3, Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)));
     }
     for (; i < end; i += 256) {
-      float4 v0 = ld4s(x + 4 * i);
+      float4 v0 = src.vec(4 * i, vv, vv, vv, vv);
       a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
     }
-    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) a1 = Op::apply(a1, x[(n4 << 2) + threadIdx.x]);
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3)) a1 = Op::apply(a1, src.one((n4 << 2) + threadIdx.x, vv));
   } else {
     const size_t chunk = (n + gridDim.x - 1) / gridDim.x;
     const size_t beg = (size_t)blockIdx.x * chunk;
     const size_t end = beg + chunk < n ? beg + chunk : n;
-    for (size_t i = beg + threadIdx.x; i < end; i += 256) a0 = Op::apply(a0, ld1s(x + i));
+    for (size_t i = beg + threadIdx.x; i < end; i += 256) a0 = Op::apply(a0, src.one(i, vv));
   }
   float v = block_reduce<Op>(Op::apply(Op::apply(a0, a1), Op::apply(a2, a3)), smem);
   if (threadIdx.x == 0) part[blockIdx.x] = v;
 }
 
-template <class Op>
-__global__ __launch_bounds__(1024) void fullreduce_final_kernel(size_t n, const float* __restrict__ part,
-                                                                float* __restrict__ out, Finalize fin) {
+template <class Op, class Src>
+__global__ __launch_bounds__(1024) void fullreduce_final_kernel(size_t n, Src part, float* __restrict__ out,
+                                                                Finalize fin) {
   __shared__ float smem[16];
+  const float vv = Src::HAS_V ? part.bvalue(0) : 0.0f;
   float a = Op::identity();
-  for (size_t i = threadIdx.x; i < n; i += 1024) a = Op::apply(a, part[i]);
+  for (size_t i = threadIdx.x; i < n; i += 1024) a = Op::apply(a, part.one(i, vv));
   a = block_reduce<Op>(a, smem);
   if (threadIdx.x == 0) finalize_store(out, a, fin);
 }
 
-template <class Op>
-static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin, float* part) {
+template <class Op, class Src>
+static int32_t reduce_all_src(slhip_ctx* ctx, size_t n, Src x, float* out, Finalize fin, float* part) {
   const bool vec = true;
   size_t items = vec ? (n >> 2) + 1 : n;
   size_t blocks = (items + 256 * 16 - 1) / (256 * 16);
@@ -374,33 +469,36 @@ static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, 
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   if (n <= 16384) {  // short buffers: the one-block kernel reads x itself
-    hipLaunchKernelGGL((fullreduce_final_kernel<Op>), dim3(1), dim3(1024), 0, ctx->stream, n, x, out, fin);
+    hipLaunchKernelGGL((fullreduce_final_kernel<Op, Src>), dim3(1), dim3(1024), 0, ctx->stream, n, x, out, fin);
     return post_launch();
   }
   if (vec)
-    hipLaunchKernelGGL((fullreduce_kernel<Op, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
+    hipLaunchKernelGGL((fullreduce_kernel<Op, true, Src>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
   else
-    hipLaunchKernelGGL((fullreduce_kernel<Op, false>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
+    hipLaunchKernelGGL((fullreduce_kernel<Op, false, Src>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, n, x, part);
   int32_t rc = post_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL((fullreduce_final_kernel<Op>), dim3(1), dim3(1024), 0, ctx->stream, blocks, part, out, fin);
+  hipLaunchKernelGGL((fullreduce_final_kernel<Op, PlainSrc>), dim3(1), dim3(1024), 0, ctx->stream, blocks, PlainSrc{part}, out,
+                     fin);
   return post_launch();
 }
 
 // out[c] = reduce over the strided axis.  ws / ws_left: where the partial results of the streaming
 // stages go (the context workspace, or the static scratch array), in floats.
-template <class Op>
-static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin, float* ws,
+template <class Op, class Src>
+static int32_t reduce_rows_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin, float* ws,
                            size_t ws_left) {
-  if (cols == 1) return reduce_all<Op>(ctx, rows, x, out, fin, ws);  // at most 4 partials per CU
+  if (cols == 1) return reduce_all_src<Op, Src>(ctx, rows, x, out, fin, ws);  // at most 4 partials per CU
   // one row: the reduction over rows is that row itself
-  if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x, cols * sizeof(float));
+  if constexpr (!Src::HAS_V)
+    if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, cols * sizeof(float));
   // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
   // about 512 per CU (measured optimum: 7.0 TB/s at 131072 threads on [16384 x 16384]; 5.4 TB/s at
   // four times as many), at least 16 vectors each, and a multiple of cols / gcd(cols, 4) so that
   // 4T is a multiple of cols.
   const size_t unit = cols / (cols % 4 == 0 ? 4 : cols % 2 == 0 ? 2 : 1);
-  const float* cur = x;
+  PlainSrc cur{nullptr};  // the partials of the stage before, once a stage has run
+  bool first = true;
   size_t cur_rows = rows;
   // (the last stage is quick for up to 256 rows of any length - 16 rows per lane, 16 columns per
   // workgroup - and for small matrices of up to 4096 rows)
@@ -412,24 +510,45 @@ static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float
     if (T < unit) T = unit;
     if (4 * T > ws_left || 8 * T > n) break;  // no room, or nothing gained: the last stage takes it as it is
     SLHIP_REQUIRE((T + 255) / 256 <= 0x7fffffffu, "matrix too wide for one launch");
-    hipLaunchKernelGGL((colreduce_flat_kernel<Op>), dim3((unsigned)((T + 255) / 256)), dim3(256), 0, ctx->stream, n, T, cur, ws);
+    if (first)
+      hipLaunchKernelGGL((colreduce_flat_kernel<Op, Src>), dim3((unsigned)((T + 255) / 256)), dim3(256), 0, ctx->stream, n, T, cols, x, ws);
+    else
+      hipLaunchKernelGGL((colreduce_flat_kernel<Op, PlainSrc>), dim3((unsigned)((T + 255) / 256)), dim3(256), 0, ctx->stream, n, T, cols, cur, ws);
     int32_t rc = post_launch();
     if (rc) return rc;
-    cur = ws;
+    first = false;
+    cur.x = ws;
     cur_rows = 4 * T / cols;
     ws += 4 * T;
     ws_left -= 4 * T;
   }
-  return colreduce_final_launch<Op>(ctx, cur_rows, cols, cur, out, fin);
+  if (cur_rows < (size_t)FEW_ROWS && cols >= 4) {
+    const size_t blocks = ((cols + 3) / 4 + 255) / 256;
+    SLHIP_REQUIRE(blocks <= 0x7fffffffu, "matrix too wide for one launch");
+    if (first)
+      hipLaunchKernelGGL((colreduce_fewrows_kernel<Op, Src>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, cur_rows, cols, x,
+                         out, fin);
+    else
+      hipLaunchKernelGGL((colreduce_fewrows_kernel<Op, PlainSrc>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, cur_rows,
+                         cols, cur, out, fin);
+    return post_launch();
+  }
+  if (first) return colreduce_final_launch<Op, Src>(ctx, cur_rows, cols, x, out, fin);
+  return colreduce_final_launch<Op, PlainSrc>(ctx, cur_rows, cols, cur, out, fin);
 }
 
 template <class Op>
 static int32_t reduce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
-  return reduce_rows<Op>(ctx, rows, cols, x, out, fin, (float*)ctx->workspace, ctx->workspace_bytes / sizeof(float));
+  return reduce_rows_src<Op, PlainSrc>(ctx, rows, cols, PlainSrc{x}, out, fin, (float*)ctx->workspace,
+                                   ctx->workspace_bytes / sizeof(float));
+}
+template <class Op>
+static int32_t reduce_cols(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, Finalize fin) {
+  return reduce_cols_src<Op, PlainSrc>(ctx, rows, cols, PlainSrc{x}, out, fin);
 }
 template <class Op>
 static int32_t reduce_all(slhip_ctx* ctx, size_t n, const float* x, float* out, Finalize fin) {
-  return reduce_all<Op>(ctx, n, x, out, fin, (float*)ctx->workspace);
+  return reduce_all_src<Op, PlainSrc>(ctx, n, PlainSrc{x}, out, fin, (float*)ctx->workspace);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -525,6 +644,76 @@ __global__ __launch_bounds__(256) void max_cols_grad_kernel(size_t rows, size_t 
   }
 }
 
+// rhs gradient of a broadcast op: v_grad[i] += sum of dR(lhs, v[i]) * g over row i (by_row: col_op)
+// or over column i (row_op), through the same kernels as the plain sums.
+int32_t bc_grad_rhs_reduce(slhip_ctx* ctx, bool by_row, int op, size_t rows, size_t cols, const float* lhs, const float* v,
+                           const float* g, float* v_grad) {
+  const BcGradSrc src{lhs, g, v, op};
+  const Finalize add{1.0f, 0, 1};
+  if (by_row) return reduce_cols_src<SumOp, BcGradSrc>(ctx, rows, cols, src, v_grad, add);
+  return reduce_rows_src<SumOp, BcGradSrc>(ctx, rows, cols, src, v_grad, add, (float*)ctx->workspace,
+                                           ctx->workspace_bytes / sizeof(float));
+}
+
+// Few rows of great length: one workgroup per row would leave most of the chip idle (measured
+// 1.9 TB/s on [134 x 10^6], 34 ms on [1 x 2^27]).  Every row is cut into segments, each workgroup
+// scans one segment and lowers the row's slot to the smallest matching index it found, and a last
+// kernel applies the slots.  The slots (one 64-bit word per row) live in the context workspace.
+__global__ __launch_bounds__(256) void max_cols_grad_init_kernel(size_t rows, unsigned long long* __restrict__ slot) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < rows) slot[i] = ~0ull;
+}
+__global__ __launch_bounds__(256) void max_cols_grad_seg_kernel(size_t cols, size_t seg_vecs, const float* __restrict__ out,
+                                                                const float* __restrict__ x, unsigned long long* slot) {
+  __shared__ unsigned long long smin;
+  const unsigned long long NONE = ~0ull;
+  const size_t row = blockIdx.y;
+  const float m = out[row];
+  const float* xr = x + row * cols;
+  const size_t colsv = cols >> 2;
+  const size_t vbeg = (size_t)blockIdx.x * seg_vecs;
+  const size_t vend = vbeg + seg_vecs < colsv ? vbeg + seg_vecs : colsv;
+  if (threadIdx.x == 0) smin = NONE;
+  __syncthreads();
+  unsigned long long best = NONE;
+  auto hit = [&](const float4& v, size_t c4) {
+    unsigned long long h = NONE;
+    if (v.w == m) h = 4 * c4 + 3;
+    if (v.z == m) h = 4 * c4 + 2;
+    if (v.y == m) h = 4 * c4 + 1;
+    if (v.x == m) h = 4 * c4;
+    return h;
+  };
+  size_t c = vbeg + threadIdx.x;
+  for (; c + 3 * 256 < vend; c += 4 * 256) {
+    const float4 v0 = ld4s(xr + 4 * c), v1 = ld4s(xr + 4 * (c + 256)), v2 = ld4s(xr + 4 * (c + 512)),
+                 v3 = ld4s(xr + 4 * (c + 768));
+    const unsigned long long h0 = hit(v0, c), h1 = hit(v1, c + 256), h2 = hit(v2, c + 512), h3 = hit(v3, c + 768);
+    best = h0 < best ? h0 : best;
+    best = h1 < best ? h1 : best;
+    best = h2 < best ? h2 : best;
+    best = h3 < best ? h3 : best;
+  }
+  for (; c < vend; c += 256) {
+    const unsigned long long h0 = hit(ld4s(xr + 4 * c), c);
+    best = h0 < best ? h0 : best;
+  }
+  // the up to three floats behind the row's last whole vector go with the last segment
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0)
+    for (size_t e = colsv << 2; e < cols; ++e)
+      if (xr[e] == m && e < best) best = e;
+  if (best != NONE) atomicMin(&smin, best);
+  __syncthreads();
+  if (threadIdx.x == 0 && smin != NONE) atomicMin(slot + row, smin);
+}
+__global__ __launch_bounds__(256) void max_cols_grad_apply_kernel(size_t rows, size_t cols,
+                                                                  const unsigned long long* __restrict__ slot,
+                                                                  float* __restrict__ x_grad,
+                                                                  const float* __restrict__ out_grad) {
+  const size_t row = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (row < rows && slot[row] != ~0ull) x_grad[row * cols + slot[row]] += out_grad[row];
+}
+
 }  // namespace slhip
 
 using namespace slhip;
@@ -565,7 +754,8 @@ SLHIP_API int32_t slhip_sum_rows_static(slhip_ctx* ctx, size_t rows, size_t cols
     return SLHIP_EWORKSPACE;
   }
   SLHIP_REQUIRE(ctx->static_scratch, "the context has no static scratch address");
-  return reduce_rows<SumOp>(ctx, rows, cols, x, out, Finalize{1.0f, 0, 0}, ctx->static_scratch, STATIC_SCRATCH_FLOATS);
+  return reduce_rows_src<SumOp, PlainSrc>(ctx, rows, cols, PlainSrc{x}, out, Finalize{1.0f, 0, 0}, ctx->static_scratch,
+                                          STATIC_SCRATCH_FLOATS);
 }
 SLHIP_API int32_t slhip_max_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out) {
   SL_DIMS_OK();
@@ -618,6 +808,22 @@ SLHIP_API int32_t slhip_max_cols_grad(slhip_ctx* ctx, size_t rows, size_t cols, 
   size_t len;
   SLHIP_REQUIRE(ctx && out && x && x_grad && out_grad, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
+  // few long rows: several workgroups per row
+  if (rows < (size_t)ctx->num_cu * 2 && cols >= 65536 && rows <= 65535 && rows * sizeof(unsigned long long) <= ctx->workspace_bytes) {
+    const size_t colsv = cols >> 2;
+    size_t nseg = ((size_t)ctx->num_cu * 8 + rows - 1) / rows;
+    if (nseg > colsv / 4096) nseg = colsv / 4096;  // at least 4096 vectors per segment
+    if (nseg < 1) nseg = 1;
+    const size_t seg_vecs = (colsv + nseg - 1) / nseg;
+    nseg = (colsv + seg_vecs - 1) / seg_vecs;
+    unsigned long long* slot = (unsigned long long*)ctx->workspace;
+    hipLaunchKernelGGL(max_cols_grad_init_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, ctx->stream, rows, slot);
+    hipLaunchKernelGGL(max_cols_grad_seg_kernel, dim3((unsigned)nseg, (unsigned)rows), dim3(256), 0, ctx->stream, cols, seg_vecs,
+                       out, x, slot);
+    hipLaunchKernelGGL(max_cols_grad_apply_kernel, dim3(ceil_div(rows, 256)), dim3(256), 0, ctx->stream, rows, cols,
+                       (const unsigned long long*)slot, x_grad, out_grad);
+    return post_launch();
+  }
   int tpr;
   if (cols >= 4096) tpr = 0;
   else {

@@ -295,12 +295,14 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
 // streamed out again.  The LDS index is skewed by one word per 32 (rows of even length would
 // otherwise pile onto the same banks).
 constexpr int SS_CHUNK = 4096;  // floats per workgroup and tensor
-__device__ __forceinline__ int ss_skew(int i) { return i + (i >> 5); }
+// sh = 5 for rows of even length, 31 (no skew) for odd ones, whose stride already visits every bank
+__device__ __forceinline__ int ss_skew(int sh, int i) { return i + (i >> sh); }
+__device__ __forceinline__ int ss_skew_shift(int cols) { return (cols & 1) ? 31 : 5; }
 
 // Requests every vector of the chunk (of NB chunks at the same offsets) before the first one is
 // used, then stores them into the skewed LDS buffers.
 template <int NB>
-__device__ __forceinline__ void ss_load(float* const (&buf)[NB], const float* const (&src)[NB], int len) {
+__device__ __forceinline__ void ss_load(float* const (&buf)[NB], const float* const (&src)[NB], int len, int sh) {
   constexpr int NJ = SS_CHUNK / 1024;
   float4 v[NB][NJ];
 #pragma unroll
@@ -317,9 +319,9 @@ __device__ __forceinline__ void ss_load(float* const (&buf)[NB], const float* co
       const int i = 4 * threadIdx.x + 1024 * j;
       float* d = buf[b];
       if (i + 3 < len) {
-        d[ss_skew(i)] = v[b][j].x; d[ss_skew(i + 1)] = v[b][j].y; d[ss_skew(i + 2)] = v[b][j].z; d[ss_skew(i + 3)] = v[b][j].w;
+        d[ss_skew(sh, i)] = v[b][j].x; d[ss_skew(sh, i + 1)] = v[b][j].y; d[ss_skew(sh, i + 2)] = v[b][j].z; d[ss_skew(sh, i + 3)] = v[b][j].w;
       } else {
-        for (int e = i; e < len; ++e) d[ss_skew(e)] = src[b][e];
+        for (int e = i; e < len; ++e) d[ss_skew(sh, e)] = src[b][e];
       }
     }
 }
@@ -328,13 +330,14 @@ template <int L>
 __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int cols, int rpb, const float* __restrict__ x,
                                                                 float* __restrict__ out) {
   __shared__ float buf[SS_CHUNK + SS_CHUNK / 32 + 4];
+  const int sh = ss_skew_shift(cols);
   const size_t r0 = (size_t)blockIdx.x * rpb;
   const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
   const int len = nr * cols;
   {
     float* const bufs[1] = {buf};
     const float* const srcs[1] = {x + r0 * cols};
-    ss_load<1>(bufs, srcs, len);
+    ss_load<1>(bufs, srcs, len, sh);
   }
   __syncthreads();
   const int lane = threadIdx.x % L, group = threadIdx.x / L;
@@ -344,25 +347,25 @@ __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int
     const int base = r * cols;
     float m = -__builtin_huge_valf();
     if (active)
-      for (int c = lane; c < cols; c += L) m = fmaxf(m, buf[ss_skew(base + c)]);
+      for (int c = lane; c < cols; c += L) m = fmaxf(m, buf[ss_skew(sh, base + c)]);
     m = wave_reduce<MaxOp, L>(m);
     float sum = 0.0f;
     if (active)
       for (int c = lane; c < cols; c += L) {
-        const float e = expf(buf[ss_skew(base + c)] - m);
-        buf[ss_skew(base + c)] = e;
+        const float e = expf(buf[ss_skew(sh, base + c)] - m);
+        buf[ss_skew(sh, base + c)] = e;
         sum += e;
       }
     sum = wave_reduce<SumOp, L>(sum);
     if (active)
-      for (int c = lane; c < cols; c += L) buf[ss_skew(base + c)] = buf[ss_skew(base + c)] / sum;
+      for (int c = lane; c < cols; c += L) buf[ss_skew(sh, base + c)] = buf[ss_skew(sh, base + c)] / sum;
   }
   __syncthreads();
   float* dst = out + r0 * cols;
   for (int i = 4 * threadIdx.x; i < len; i += 1024) {
-    if (i + 3 < len) st4s(dst + i, make_float4(buf[ss_skew(i)], buf[ss_skew(i + 1)], buf[ss_skew(i + 2)], buf[ss_skew(i + 3)]));
+    if (i + 3 < len) st4s(dst + i, make_float4(buf[ss_skew(sh, i)], buf[ss_skew(sh, i + 1)], buf[ss_skew(sh, i + 2)], buf[ss_skew(sh, i + 3)]));
     else
-      for (int e = i; e < len; ++e) dst[e] = buf[ss_skew(e)];
+      for (int e = i; e < len; ++e) dst[e] = buf[ss_skew(sh, e)];
   }
 }
 
@@ -372,13 +375,14 @@ __global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int
                                                                 const float* __restrict__ out_grad, float beta) {
   __shared__ float sb[SS_CHUNK + SS_CHUNK / 32 + 4];
   __shared__ float gb[SS_CHUNK + SS_CHUNK / 32 + 4];
+  const int sh = ss_skew_shift(cols);
   const size_t r0 = (size_t)blockIdx.x * rpb;
   const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
   const int len = nr * cols;
   {
     float* const bufs[2] = {sb, gb};
     const float* const srcs[2] = {out + r0 * cols, out_grad + r0 * cols};
-    ss_load<2>(bufs, srcs, len);
+    ss_load<2>(bufs, srcs, len, sh);
   }
   __syncthreads();
   const int lane = threadIdx.x % L, group = threadIdx.x / L;
@@ -388,23 +392,23 @@ __global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int
     const int base = r * cols;
     float dot = 0.0f;
     if (active)
-      for (int c = lane; c < cols; c += L) dot += sb[ss_skew(base + c)] * gb[ss_skew(base + c)];
+      for (int c = lane; c < cols; c += L) dot += sb[ss_skew(sh, base + c)] * gb[ss_skew(sh, base + c)];
     dot = wave_reduce<SumOp, L>(dot);
     if (active)
-      for (int c = lane; c < cols; c += L) sb[ss_skew(base + c)] = sb[ss_skew(base + c)] * (gb[ss_skew(base + c)] - dot);
+      for (int c = lane; c < cols; c += L) sb[ss_skew(sh, base + c)] = sb[ss_skew(sh, base + c)] * (gb[ss_skew(sh, base + c)] - dot);
   }
   __syncthreads();
   float* dst = x_grad + r0 * cols;
   for (int i = 4 * threadIdx.x; i < len; i += 1024) {
     if (i + 3 < len) {
-      float4 v = make_float4(sb[ss_skew(i)], sb[ss_skew(i + 1)], sb[ss_skew(i + 2)], sb[ss_skew(i + 3)]);
+      float4 v = make_float4(sb[ss_skew(sh, i)], sb[ss_skew(sh, i + 1)], sb[ss_skew(sh, i + 2)], sb[ss_skew(sh, i + 3)]);
       if (beta != 0.0f) {
         const float4 o = ld4g(dst + i);
         v.x = beta * o.x + v.x; v.y = beta * o.y + v.y; v.z = beta * o.z + v.z; v.w = beta * o.w + v.w;
       }
       st4g(dst + i, v);
     } else {
-      for (int e = i; e < len; ++e) dst[e] = beta != 0.0f ? beta * dst[e] + sb[ss_skew(e)] : sb[ss_skew(e)];
+      for (int e = i; e < len; ++e) dst[e] = beta != 0.0f ? beta * dst[e] + sb[ss_skew(sh, e)] : sb[ss_skew(sh, e)];
     }
   }
 }

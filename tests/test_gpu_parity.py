@@ -466,7 +466,9 @@ def test_max_is_bit_exact_with_injected_ties_and_negatives(hip, orc):
 
 
 def test_max_grads_tie_rules(hip, orc):
-    for rows, cols in [(3, 4), (50, 200), (300, 40), (17, 5000), (2000, 1), (1, 2000)]:
+    # (the last three: few rows of great length, which several workgroups per row scan)
+    for rows, cols in [(3, 4), (50, 200), (300, 40), (17, 5000), (2000, 1), (1, 2000), (3, 70001), (1, 300000),
+                       (40, 65536)]:
         say("max grads", rows, cols)
         x = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED + cols)
         g_r = rng.normal(rows, 1.0, tag=1, seed=SEED)
@@ -645,7 +647,7 @@ def test_negative_base_integer_pow_is_finite(hip):
 
 def test_row_op_and_bias_grad(hip, orc):
     for rows, cols in [(3, 5), (1, 9), (9, 1), (1024, 64), (1000, 10), (8192, 10), (300, 2048), (4097, 130),
-                       (1234, 679), (7, 100003), (100003, 3), (2, 2)]:
+                       (1234, 679), (7, 100003), (100003, 3), (2, 2), (1, 100000), (5, 4096), (3, 6)]:
         say("row op", rows, cols)
         lhs = rng.uniform(rows * cols, -10, 10, tag=0, seed=SEED)
         rhs = rng.uniform(cols, -10, 10, tag=1, seed=SEED)
@@ -674,7 +676,8 @@ def test_cce_and_onehot(hip, orc):
     assert np.array_equal(hip.cce_grad(rows, cols, p, t), orc.cce_grad(rows, cols, p, t))
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 10), (257, 129), (4096, 33), (5, 70000), (2000, 2048)],
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 10), (257, 129), (4096, 33), (5, 70000), (2000, 2048),
+                                   (5000, 1), (3000, 7), (1, 5000), (20000, 2), (1500, 64), (40, 4099)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("kind", ["row_op", "col_op"])
 def test_broadcast_ops_with_op_code(hip, orc, shape, kind):
