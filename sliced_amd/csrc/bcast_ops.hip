@@ -42,14 +42,26 @@ __global__ __launch_bounds__(256) void bc_flat_kernel(int op, size_t len, size_t
       if (GRAD) { gv[q] = g[e0 + q]; o[q] = out[e0 + q]; }
     }
   }
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    if (e0 + q < len) {
-      const float vv = v[BY_ROW_INDEX ? r : c];
-      o[q] = GRAD ? o[q] + bc_dl(op, l[q], vv) * gv[q] : bc_apply(op, l[q], vv);
+  // the broadcast entries of the four elements: one load where they lie in one row
+  float vv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (whole && (size_t)c + 3 < cols) {
+    if (BY_ROW_INDEX) {
+      vv[0] = vv[1] = vv[2] = vv[3] = v[r];
+    } else {
+      const float4 t = ld4g(v + c);
+      vv[0] = t.x; vv[1] = t.y; vv[2] = t.z; vv[3] = t.w;
     }
-    if (++c == (IDX)cols) { c = 0; ++r; }
+  } else {
+    IDX rq = r, cq = c;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (e0 + q < len) vv[q] = v[BY_ROW_INDEX ? rq : cq];
+      if (++cq == (IDX)cols) { cq = 0; ++rq; }
+    }
   }
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    if (e0 + q < len) o[q] = GRAD ? o[q] + bc_dl(op, l[q], vv[q]) * gv[q] : bc_apply(op, l[q], vv[q]);
   if (whole) st4g(out + e0, make_float4(o[0], o[1], o[2], o[3]));
   else
     for (size_t q = 0; e0 + q < len; ++q) out[e0 + q] = o[q];

@@ -249,15 +249,32 @@ __global__ __launch_bounds__(EW_BLOCK) void bcast_flat_kernel(size_t len, size_t
       if (MODE != 0) o[q] = out[e0 + q];
     }
   }
+  // the broadcast entries of the four elements: one vector load where they lie in one row (a thread
+  // that gathers them one by one streams a matrix of odd row length at 4.0-4.6 TB/s)
+  float vv[4] = {0.f, 0.f, 0.f, 0.f}, gv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (MODE != 2 && whole && (size_t)c + 3 < cols) {
+    float4 t = ld4g(v + c);
+    vv[0] = t.x; vv[1] = t.y; vv[2] = t.z; vv[3] = t.w;
+    if (MODE == 3) { t = ld4g(g + c); gv[0] = t.x; gv[1] = t.y; gv[2] = t.z; gv[3] = t.w; }
+  } else {
+    IDX rq = r, cq = c;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (e0 + q < len) {
+        vv[q] = MODE == 2 ? v[rq] : v[cq];
+        if (MODE == 3) gv[q] = g[cq];
+      }
+      if (++cq == (IDX)cols) { cq = 0; ++rq; }
+    }
+  }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     if (e0 + q < len) {
-      if (MODE == 0) o[q] = av[q] + v[c];
-      else if (MODE == 1) o[q] += s * v[c];
-      else if (MODE == 2) o[q] += DIVCOLS ? v[r] / s : v[r];
-      else if (av[q] == v[c]) o[q] += g[c];
+      if (MODE == 0) o[q] = av[q] + vv[q];
+      else if (MODE == 1) o[q] += s * vv[q];
+      else if (MODE == 2) o[q] += DIVCOLS ? vv[q] / s : vv[q];
+      else if (av[q] == vv[q]) o[q] += gv[q];
     }
-    if (++c == (IDX)cols) { c = 0; ++r; }
   }
   if (whole) st4s(out + e0, make_float4(o[0], o[1], o[2], o[3]));
   else

@@ -142,34 +142,67 @@ __global__ __launch_bounds__(256) void transpose_narrow_kernel(size_t long_side,
   // LDS holds the chunk in the narrow matrix's order: element (l, s) at l*S + s.  Global memory is
   // touched with dword-aligned float4 on both sides (scalar accesses stream at a third of the rate).
   const int nr4 = nr & ~3, len4 = len & ~3;
+  // every vector of the chunk is requested before the first one is stored to LDS: a loop that loads
+  // and stores in turn keeps one request per thread in flight
+  constexpr int NJ = TS_CHUNK / 1024;
+  float4 v[NJ];
   if (NARROW_IN) {
     const float* src = x + l0 * S;
-    for (int i = 4 * threadIdx.x; i < len4; i += 1024) {
-      const float4 v = ld4s(src + i);
-      buf[ts_skew(i)] = v.x; buf[ts_skew(i + 1)] = v.y; buf[ts_skew(i + 2)] = v.z; buf[ts_skew(i + 3)] = v.w;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      if (i < len4) v[j] = ld4s(src + i);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int i = 4 * threadIdx.x + 1024 * j;
+      if (i < len4) {
+        buf[ts_skew(i)] = v[j].x; buf[ts_skew(i + 1)] = v[j].y; buf[ts_skew(i + 2)] = v[j].z; buf[ts_skew(i + 3)] = v[j].w;
+      }
     }
     for (int i = len4 + threadIdx.x; i < len; i += 256) buf[ts_skew(i)] = src[i];
   } else {
+    // the S runs of nr floats, cut into vectors and dealt out over the threads: vector j of the
+    // chunk is vector j % RV of run j / RV (R is a multiple of 4 here, so RV = R / 4 covers a run)
+    const int RV = R >> 2, nrv = nr4 >> 2;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int k = threadIdx.x + 256 * j, run = k / RV, lv = k - run * RV;
+      if (run < S && lv < nrv) v[j] = ld4s(x + (size_t)run * long_side + l0 + 4 * lv);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int k = threadIdx.x + 256 * j, run = k / RV, lv = k - run * RV;
+      if (run < S && lv < nrv) {
+        const int l = 4 * lv;
+        buf[ts_skew(l * S + run)] = v[j].x; buf[ts_skew((l + 1) * S + run)] = v[j].y;
+        buf[ts_skew((l + 2) * S + run)] = v[j].z; buf[ts_skew((l + 3) * S + run)] = v[j].w;
+      }
+    }
     for (int s = 0; s < S; ++s) {
       const float* src = x + (size_t)s * long_side + l0;
-      for (int l = 4 * threadIdx.x; l < nr4; l += 1024) {
-        const float4 v = ld4s(src + l);
-        buf[ts_skew(l * S + s)] = v.x; buf[ts_skew((l + 1) * S + s)] = v.y;
-        buf[ts_skew((l + 2) * S + s)] = v.z; buf[ts_skew((l + 3) * S + s)] = v.w;
-      }
       for (int l = nr4 + threadIdx.x; l < nr; l += 256) buf[ts_skew(l * S + s)] = src[l];
     }
   }
   __syncthreads();
   if (NARROW_IN) {
+    // the S output runs of nr floats, cut into vectors and dealt out over the threads as on the
+    // load side of the other direction
+    const int RV = R >> 2, nrv = nr4 >> 2;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int k = threadIdx.x + 256 * j, run = k / RV, lv = k - run * RV;
+      if (run < S && lv < nrv) {
+        const int l = 4 * lv;
+        float* dst = out + (size_t)run * long_side + l0 + l;
+        float4 w = make_float4(buf[ts_skew(l * S + run)], buf[ts_skew((l + 1) * S + run)], buf[ts_skew((l + 2) * S + run)],
+                               buf[ts_skew((l + 3) * S + run)]);
+        if (ACC) { const float4 o = ld4g(dst); w.x += o.x; w.y += o.y; w.z += o.z; w.w += o.w; }
+        st4g(dst, w);
+      }
+    }
     for (int s = 0; s < S; ++s) {
       float* dst = out + (size_t)s * long_side + l0;
-      for (int l = 4 * threadIdx.x; l < nr4; l += 1024) {
-        float4 v = make_float4(buf[ts_skew(l * S + s)], buf[ts_skew((l + 1) * S + s)], buf[ts_skew((l + 2) * S + s)],
-                               buf[ts_skew((l + 3) * S + s)]);
-        if (ACC) { const float4 o = ld4g(dst + l); v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
-        st4g(dst + l, v);
-      }
       for (int l = nr4 + threadIdx.x; l < nr; l += 256) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + s)] : buf[ts_skew(l * S + s)];
     }
   } else {
@@ -208,11 +241,18 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     hipLaunchKernelGGL(axpy_copy_kernel, dim3((unsigned)((len + 63) / 64)), dim3(64), 0, ctx->stream, len, x, out);
     return post_launch();
   }
-  if (cols <= 40 || rows <= 40) {  // measured: from a side of 48 on the tiled kernel is the faster one
-    const bool narrow_in = cols <= 40 && (rows > 40 || cols <= rows);  // which matrix has the short rows
+  // Which kernel (measured at 2^27 elements, TB/s, chunk kernel / tiled kernel): a narrow input
+  // [long x S]: S = 31: 4.0 / 2.4, 40: 4.1 / 3.3, 48: 3.8 / 3.5, 64: 5.3 / 5.8, 100: 3.1 / 3.4, 128: 5.4 / 5.8;
+  // a narrow output, input [S x long]: S = 48: 4.9 / 2.7, 64: 5.4 / 3.3, 100: 4.0 / 3.4, 128: 5.8 / 4.1,
+  // 160: 4.4 / 4.0, 200: 4.2 / -, 224: 3.1 / -, 257: 2.6 / 3.4.
+  const bool narrow_in = cols <= 56 && cols <= rows;
+  const bool narrow_out = !narrow_in && rows <= 200 && rows < cols;
+  if (narrow_in || narrow_out) {
     const size_t long_side = narrow_in ? rows : cols;
     const int S = (int)(narrow_in ? cols : rows);
-    const int R = TS_CHUNK / S;
+    int R = TS_CHUNK / S;
+    if (R >= 256) R &= ~31;  // runs that start on 128-byte boundaries of their rows, where that costs little
+    else if (R >= 4) R &= ~3;  // whole vectors per run
     const size_t blocks = (long_side + R - 1) / R;
     SLHIP_REQUIRE(blocks <= 0x7fffffffu, "matrix too large for one launch");
 #define SL_TN(NI, A) \

@@ -566,7 +566,10 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (2, 5), (32, 70000), (259, 66),
              # the narrow-matrix kernel: chunk boundaries, sides 2..40, both directions, tiny and ragged long sides
              (70001, 2), (2, 70001), (30000, 31), (31, 30000), (9999, 40), (40, 9999), (5000, 16), (16, 5003), (41, 3000),
-             (3000, 41), (3, 3), (40, 40), (17, 23)]
+             (3000, 41), (3, 3), (40, 40), (17, 23),
+             # the limits of the narrow kernels (56 columns in, 200 rows out) and what lies just beyond
+             (5000, 56), (5001, 57), (200, 3001), (201, 3000), (224, 3001), (100, 8193), (128, 5000), (200, 41), (56, 57), (57, 56),
+             (163, 9000), (9000, 55)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
