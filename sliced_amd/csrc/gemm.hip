@@ -320,6 +320,10 @@ static bool wave_plan(const slhip_ctx* ctx, size_t M, size_t N, size_t K, unsign
 
 static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
                         float* C, float beta, const float* bias, int relu, float* pre_act, const float* mask) {
+  // an operand that is a single row or column reads the same either way: the form measured faster
+  // (16384 x 1 x 16384: A*B 186 us, A*Bt 328; 16384 x 16384 x 1: 226 against 244)
+  if (N == 1 || K == 1) tb = false;
+  if (M == 1 || K == 1) ta = false;
   GemmArgs g;
   g.M = M; g.N = N; g.K = K; g.A = A; g.B = B; g.C = C; g.beta = beta;
   g.bias = bias; g.relu = relu; g.pre_act = pre_act; g.mask = mask;
