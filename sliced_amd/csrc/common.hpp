@@ -178,4 +178,20 @@ __device__ __forceinline__ float bc_dr(int op, float l, float r) {
 int32_t bc_grad_rhs_reduce(slhip_ctx* ctx, bool by_row, int op, size_t rows, size_t cols, const float* lhs, const float* v,
                            const float* g, float* v_grad);
 
+// loss[r] = -ln sum_c clip(p[r, c], 1e-7, 1 - 1e-7) * t[r, c], through the contiguous-axis
+// reduction kernels (defined with them).
+int32_t cce_rows_reduce(slhip_ctx* ctx, size_t rows, size_t cols, const float* p, const float* t, float* loss);
+
+// logits_grad = beta * logits_grad + (probs * sum_c targets - targets) * (upstream / rows), through
+// the softmax backward kernels (defined with them).
+int32_t softmax_cce_grad_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* probs, const float* targets,
+                              float* logits_grad, float beta, const float* upstream_dev);
+
+// probs = softmax(logits) (probs may be null), loss_rows[r] = -ln sum_c clip(probs) * targets, in
+// one pass through the softmax forward kernels; rows of more than softmax_one_pass_cols() floats
+// are refused (defined with those kernels).
+int32_t softmax_cce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* logits, const float* targets, float* probs,
+                         float* loss_rows);
+size_t softmax_one_pass_cols();
+
 }  // namespace slhip

@@ -65,10 +65,8 @@ __global__ __launch_bounds__(256) void mse_grad_kernel(size_t n, const float* __
 }
 
 // ---------------------------------------------------------------- softmax cross-entropy
-// L lanes per row (a power of two up to 64, about 8 classes per lane), 256 / L rows per workgroup;
-// the row is swept from global memory three times (the second and third sweep hit the caches: a
-// workgroup's rows are a few KiB).  With one wave per row, whatever its length, rows of 10 classes
-// used 10 of 64 lanes: [13M x 10] streamed at 0.35 TB/s.
+// The fallback for rows too long for the one-pass softmax kernels when the caller wants no
+// probabilities: L lanes per row, the row swept from global memory three times.
 template <int L>
 __global__ __launch_bounds__(256) void softmax_cce_kernel(size_t rows, size_t cols, const float* __restrict__ x,
                                                           const float* __restrict__ t, float* __restrict__ probs,
@@ -96,35 +94,6 @@ __global__ __launch_bounds__(256) void softmax_cce_kernel(size_t rows, size_t co
     }
   acc = wave_reduce<SumOp, L>(acc);
   if (active && lane == 0) loss_rows[r] = -logf(acc);
-}
-
-template <int L>
-__global__ __launch_bounds__(256) void softmax_cce_grad_kernel(size_t rows, size_t cols, const float* __restrict__ p,
-                                                               const float* __restrict__ t, float* __restrict__ lg,
-                                                               float beta, const float* __restrict__ upstream) {
-  const size_t r = (size_t)blockIdx.x * (256 / L) + threadIdx.x / L;
-  const bool active = r < rows;
-  const int lane = threadIdx.x % L;
-  const float* pr = p + (active ? r : 0) * cols;
-  const float* tr = t + (active ? r : 0) * cols;
-  float st = 0.0f;
-  if (active)
-    for (size_t c = lane; c < cols; c += L) st += tr[c];
-  st = wave_reduce<SumOp, L>(st);
-  const float scale = upstream[0] / (float)rows;
-  if (active)
-    for (size_t c = lane; c < cols; c += L) {
-      const float g = (pr[c] * st - tr[c]) * scale;
-      float* dst = lg + r * cols + c;
-      *dst = beta != 0.0f ? beta * *dst + g : g;
-    }
-}
-
-// lanes per row for the row-wise loss kernels
-static int loss_lanes(size_t cols) {
-  int lanes = 1;
-  while (lanes < 64 && (size_t)lanes * 8 < cols) lanes <<= 1;
-  return lanes;
 }
 
 }  // namespace slhip
@@ -170,22 +139,19 @@ SLHIP_API int32_t slhip_softmax_cce(slhip_ctx* ctx, size_t rows, size_t cols, co
   size_t len;
   SLHIP_REQUIRE(ctx && logits && targets && loss_rows, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  // Long rows of a large batch: the register-resident softmax kernel followed by the cce pass moves
-  // 16 B per element at 6 TB/s; the fused kernel's three sweeps with two exponentials per element
-  // move 12 B at 2.6 ([32768 x 4096]: 0.62 ms fused, 0.35 ms as two kernels).  The fused kernel stays
-  // for what it was made for, the launch-bound training step with a few classes.
-  if (probs && cols >= 256 && len >= ((size_t)1 << 22)) {
+  SLHIP_REQUIRE(rows <= 0x7fffffffu, "too many rows for one launch");
+  // rows that fit the softmax kernels' registers or LDS chunks: one pass, 12 B per element
+  if (cols <= softmax_one_pass_cols()) return softmax_cce_rows(ctx, rows, cols, logits, targets, probs, loss_rows);
+  // longer rows: the streaming softmax, then the cross-entropy as a row reduction
+  if (probs) {
     int32_t rc = slhip_softmax(ctx, rows, cols, logits, probs);
     if (rc) return rc;
     return slhip_cce(ctx, rows, cols, probs, targets, loss_rows);
   }
-  const int lanes = loss_lanes(cols);
-  const size_t blocks = (rows + 256 / lanes - 1) / (256 / lanes);
-  SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-#define SL_SC(L) \
-  case L: hipLaunchKernelGGL((softmax_cce_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, logits, targets, probs, loss_rows); break;
-  switch (lanes) { SL_SC(1) SL_SC(2) SL_SC(4) SL_SC(8) SL_SC(16) SL_SC(32) SL_SC(64) }
-#undef SL_SC
+  // ... and without a buffer for the probabilities: one wave per row, three sweeps
+  const size_t blocks = (rows + 3) / 4;
+  hipLaunchKernelGGL((softmax_cce_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, logits, targets, probs,
+                     loss_rows);
   return post_launch();
 }
 
@@ -195,12 +161,6 @@ SLHIP_API int32_t slhip_softmax_cce_grad(slhip_ctx* ctx, size_t rows, size_t col
   size_t len;
   SLHIP_REQUIRE(ctx && probs && targets && logits_grad && upstream_dev, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  const int lanes = loss_lanes(cols);
-  const size_t blocks = (rows + 256 / lanes - 1) / (256 / lanes);
-  SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many rows for one launch");
-#define SL_SG(L) \
-  case L: hipLaunchKernelGGL((softmax_cce_grad_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, probs, targets, logits_grad, beta, upstream_dev); break;
-  switch (lanes) { SL_SG(1) SL_SG(2) SL_SG(4) SL_SG(8) SL_SG(16) SL_SG(32) SL_SG(64) }
-#undef SL_SG
-  return post_launch();
+  SLHIP_REQUIRE(rows <= 0x7fffffffu, "too many rows for one launch");
+  return softmax_cce_grad_rows(ctx, rows, cols, probs, targets, logits_grad, beta, upstream_dev);
 }

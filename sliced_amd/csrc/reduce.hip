@@ -14,11 +14,12 @@ namespace slhip {
 // reference divides), optionally added to what out already holds.
 struct Finalize {
   float scale;     // divisor of the means; unused otherwise
-  int divide;      // 1: v = v / scale
+  int divide;      // 1: v = v / scale; 2: v = -ln v (the cross-entropy of a row)
   int accumulate;  // 1: out += v
 };
 __device__ __forceinline__ void finalize_store(float* p, float v, Finalize f) {
-  if (f.divide) v = v / f.scale;
+  if (f.divide == 2) v = -logf(v);
+  else if (f.divide) v = v / f.scale;
   if (f.accumulate) v = *p + v;
   *p = v;
 }
@@ -29,6 +30,7 @@ __device__ __forceinline__ void finalize_store(float* p, float v, Finalize f) {
 // row_op); the kernels hand in v's entry, which they know from the row or column they work on.
 struct PlainSrc {
   static constexpr bool HAS_V = false;
+  static constexpr bool IS_PLAIN = true;
   const float* x;
   __device__ __forceinline__ float bvalue(size_t) const { return 0.0f; }
   __device__ __forceinline__ float4 vec(size_t e, float, float, float, float) const { return ld4s(x + e); }
@@ -36,6 +38,7 @@ struct PlainSrc {
 };
 struct BcGradSrc {
   static constexpr bool HAS_V = true;
+  static constexpr bool IS_PLAIN = false;
   const float* l;
   const float* g;
   const float* v;
@@ -47,6 +50,24 @@ struct BcGradSrc {
                        bc_dr(op, a.w, v3) * b.w);
   }
   __device__ __forceinline__ float one(size_t e, float vv) const { return bc_dr(op, ld1s(l + e), vv) * ld1s(g + e); }
+};
+
+// The terms of the categorical cross-entropy of a row: clip(p, 1e-7, 1 - 1e-7) * t
+// (reference: examples/nn.rs:124-143).
+struct CceSrc {
+  static constexpr bool HAS_V = false;
+  static constexpr bool IS_PLAIN = false;
+  const float* p;
+  const float* t;
+  static __device__ __forceinline__ float term(float p, float t) {
+    return fminf(fmaxf(p, (float)1e-7), (float)(1.0 - 1e-7)) * t;
+  }
+  __device__ __forceinline__ float bvalue(size_t) const { return 0.0f; }
+  __device__ __forceinline__ float4 vec(size_t e, float, float, float, float) const {
+    const float4 a = ld4s(p + e), b = ld4s(t + e);
+    return make_float4(term(a.x, b.x), term(a.y, b.y), term(a.z, b.z), term(a.w, b.w));
+  }
+  __device__ __forceinline__ float one(size_t e, float) const { return term(ld1s(p + e), ld1s(t + e)); }
 };
 
 // ---------------------------------------------------------------------------------------
@@ -216,7 +237,7 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, Src x,
 template <class Op, class Src>
 static int32_t reduce_cols_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin) {
   // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
-  if constexpr (!Src::HAS_V)
+  if constexpr (Src::IS_PLAIN)
     if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, rows * sizeof(float));
   if (cols <= 128 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {  // many short rows
     // whole multiples of 256 rows while they fit (every lane of the second phase busy), else as many
@@ -374,7 +395,8 @@ __global__ __launch_bounds__(256) void colreduce_fewrows_kernel(size_t rows, siz
         a[2] = Op::apply(a[2], v[r].z); a[3] = Op::apply(a[3], v[r].w);
       }
     float4 o = make_float4(a[0], a[1], a[2], a[3]);
-    if (fin.divide) { o.x = o.x / fin.scale; o.y = o.y / fin.scale; o.z = o.z / fin.scale; o.w = o.w / fin.scale; }
+    if (fin.divide == 2) { o.x = -logf(o.x); o.y = -logf(o.y); o.z = -logf(o.z); o.w = -logf(o.w); }
+    else if (fin.divide) { o.x = o.x / fin.scale; o.y = o.y / fin.scale; o.z = o.z / fin.scale; o.w = o.w / fin.scale; }
     if (fin.accumulate) {
       const float4 old = ld4g(out + c0);
       o.x = old.x + o.x; o.y = old.y + o.y; o.z = old.z + o.z; o.w = old.w + o.w;
@@ -490,7 +512,7 @@ static int32_t reduce_rows_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, 
                            size_t ws_left) {
   if (cols == 1) return reduce_all_src<Op, Src>(ctx, rows, x, out, fin, ws);  // at most 4 partials per CU
   // one row: the reduction over rows is that row itself
-  if constexpr (!Src::HAS_V)
+  if constexpr (Src::IS_PLAIN)
     if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, cols * sizeof(float));
   // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
   // about 512 per CU (measured optimum: 7.0 TB/s at 131072 threads on [16384 x 16384]; 5.4 TB/s at
@@ -642,6 +664,11 @@ __global__ __launch_bounds__(256) void max_cols_grad_kernel(size_t rows, size_t 
     }
     if (row < rows && lane == 0 && best != NONE) x_grad[row * cols + best] += out_grad[row];
   }
+}
+
+// loss[r] = -ln sum_c clip(p[r, c]) * t[r, c]
+int32_t cce_rows_reduce(slhip_ctx* ctx, size_t rows, size_t cols, const float* p, const float* t, float* loss) {
+  return reduce_cols_src<SumOp, CceSrc>(ctx, rows, cols, CceSrc{p, t}, loss, Finalize{1.0f, 2, 0});
 }
 
 // rhs gradient of a broadcast op: v_grad[i] += sum of dR(lhs, v[i]) * g over row i (by_row: col_op)

@@ -32,10 +32,17 @@ __device__ __forceinline__ float row_reduce(float v, float* smem) {
 // TAIL: the row length is not a multiple of 4 (VEC only): lane 0 also takes the up to 3 floats
 // beyond the last whole vector.  A template parameter because even an untaken tail costs the
 // whole-vector rows 10-15 % of their bandwidth.
-template <bool VEC, int LANES, int ITEMS, bool TAIL>
+//
+// CCE: the categorical cross-entropy of every row against the targets tg rides along,
+// loss_rows[r] = -ln sum_c clip(p, 1e-7, 1 - 1e-7) * tg (reference: Matrix::softmax followed by cce,
+// examples/nn.rs:124-143); out may then be null (the probabilities are not stored).
+__device__ __forceinline__ float cce_term(float p, float t) { return fminf(fmaxf(p, (float)1e-7), (float)(1.0 - 1e-7)) * t; }
+template <bool VEC, int LANES, int ITEMS, bool TAIL, bool CCE>
 __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(size_t rows, size_t cols,
                                                                                 const float* __restrict__ x,
-                                                                                float* __restrict__ out) {
+                                                                                float* __restrict__ out,
+                                                                                const float* __restrict__ tg,
+                                                                                float* __restrict__ loss_rows) {
   __shared__ float smem[32];
   constexpr int V = VEC ? 4 : 1;
   constexpr int RPB = LANES <= 64 ? 256 / LANES : 1;
@@ -46,16 +53,21 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
   const float NEG_INF = -__builtin_huge_valf();
 
   float v[ITEMS][V];
+  float w[CCE ? ITEMS : 1][V];  // the targets of the same elements
   float m = NEG_INF;
   // every lane of the row holds ITEMS full vectors: unconditional loads, all in flight together
   const bool full = active && (size_t)LANES * ITEMS <= colsv;
   if (VEC && full) {
-    float4 t[ITEMS];
+    float4 t[ITEMS], u[CCE ? ITEMS : 1];
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) t[j] = ld4s(x + row * cols + 4 * ((size_t)lane + (size_t)j * LANES));
+    for (int j = 0; j < ITEMS; ++j) {
+      t[j] = ld4s(x + row * cols + 4 * ((size_t)lane + (size_t)j * LANES));
+      if (CCE) u[j] = ld4s(tg + row * cols + 4 * ((size_t)lane + (size_t)j * LANES));
+    }
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       v[j][0] = t[j].x; v[j][V > 1 ? 1 : 0] = t[j].y; v[j][V > 1 ? 2 : 0] = t[j].z; v[j][V > 1 ? 3 : 0] = t[j].w;
+      if (CCE) { w[j][0] = u[j].x; w[j][V > 1 ? 1 : 0] = u[j].y; w[j][V > 1 ? 2 : 0] = u[j].z; w[j][V > 1 ? 3 : 0] = u[j].w; }
     }
   } else {
 #pragma unroll
@@ -65,12 +77,20 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
         if (VEC) {
           float4 t = ld4s(x + row * cols + 4 * c);
           v[j][0] = t.x; v[j][V > 1 ? 1 : 0] = t.y; v[j][V > 1 ? 2 : 0] = t.z; v[j][V > 1 ? 3 : 0] = t.w;
+          if (CCE) {
+            t = ld4s(tg + row * cols + 4 * c);
+            w[j][0] = t.x; w[j][V > 1 ? 1 : 0] = t.y; w[j][V > 1 ? 2 : 0] = t.z; w[j][V > 1 ? 3 : 0] = t.w;
+          }
         } else {
           v[j][0] = x[row * cols + c];
+          if (CCE) w[j][0] = tg[row * cols + c];
         }
       } else {
 #pragma unroll
-        for (int q = 0; q < V; ++q) v[j][q] = NEG_INF;
+        for (int q = 0; q < V; ++q) {
+          v[j][q] = NEG_INF;
+          if (CCE) w[j][q] = 0.0f;
+        }
       }
     }
   }
@@ -111,6 +131,18 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
   constexpr bool RECIP = LANES > 64;
   const float inv = RECIP ? 1.0f / s : s;
   auto scale = [&](float e) { return RECIP ? e * inv : e / inv; };
+  if (CCE) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j)
+#pragma unroll
+      for (int q = 0; q < V; ++q) acc += cce_term(scale(v[j][q]), w[j][q]);  // (elements outside the row: e = 0, t = 0)
+    if (tail)
+      for (int q = 0; q < rem; ++q) acc += cce_term(scale(tv[q]), tg[row * cols + 4 * colsv + q]);
+    acc = row_reduce<SumOp, LANES>(acc, smem);  // (every lane is past its reads of the first reduction)
+    if (active && lane == 0) loss_rows[row] = -logf(acc);
+    if (!out) return;
+  }
   if (tail)
     for (int q = 0; q < rem; ++q) out[row * cols + 4 * colsv + q] = scale(tv[q]);
 
@@ -125,11 +157,29 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
   }
 }
 
-template <bool VEC, int LANES, int ITEMS, bool TAIL>
+// What the backward kernels make of a row (s, g): the softmax gradient s * (g - <s, g>), or, with
+// s = the probabilities and g = the targets, the gradient of the mean cross-entropy pushed through
+// the softmax in closed form, (p * sum_c t - t) * (upstream / rows) (reference: cce_grad followed by
+// softmax_grad, examples/nn.rs:145-152, which divides by p and yields inf * 0 when p underflows).
+struct SoftmaxGradForm {
+  __device__ __forceinline__ float term(float s, float g) const { return s * g; }
+  __device__ __forceinline__ float k() const { return 0.0f; }
+  __device__ __forceinline__ float result(float s, float g, float red, float) const { return s * (g - red); }
+};
+struct CceGradForm {
+  const float* upstream;
+  float rows;
+  __device__ __forceinline__ float term(float, float g) const { return g; }
+  __device__ __forceinline__ float k() const { return upstream[0] / rows; }
+  __device__ __forceinline__ float result(float s, float g, float red, float kk) const { return (s * red - g) * kk; }
+};
+
+template <bool VEC, int LANES, int ITEMS, bool TAIL, class RG>
 __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(size_t rows, size_t cols,
                                                                                 float* x_grad,
                                                                                 const float* __restrict__ out,
-                                                                                const float* out_grad, float beta) {
+                                                                                const float* out_grad, float beta, RG rg) {
+  const float kk = rg.k();
   __shared__ float smem[16];
   constexpr int V = VEC ? 4 : 1;
   constexpr int RPB = LANES <= 64 ? 256 / LANES : 1;
@@ -176,7 +226,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
-    for (int q = 0; q < V; ++q) dot += s[j][q] * g[j][q];
+    for (int q = 0; q < V; ++q) dot += rg.term(s[j][q], g[j][q]);
   // the up to 3 floats beyond the last whole vector of a row of odd length: lane 0 takes them
   const int rem = TAIL ? (int)(cols & 3) : 0;
   const bool tail = TAIL && rem != 0 && active && lane == 0;
@@ -185,13 +235,13 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
     for (int q = 0; q < rem; ++q) {
       ts[q] = out[row * cols + 4 * colsv + q];
       tg[q] = out_grad[row * cols + 4 * colsv + q];
-      dot += ts[q] * tg[q];
+      dot += rg.term(ts[q], tg[q]);
     }
   dot = row_reduce<SumOp, LANES>(dot, smem);
   if (tail)
     for (int q = 0; q < rem; ++q) {
       float* p = x_grad + row * cols + 4 * colsv + q;
-      const float r = ts[q] * (tg[q] - dot);
+      const float r = rg.result(ts[q], tg[q], dot, kk);
       *p = beta != 0.0f ? beta * *p + r : r;
     }
 
@@ -201,7 +251,7 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
     if (active && c < colsv) {
       float r[V];
 #pragma unroll
-      for (int q = 0; q < V; ++q) r[q] = s[j][q] * (g[j][q] - dot);
+      for (int q = 0; q < V; ++q) r[q] = rg.result(s[j][q], g[j][q], dot, kk);
       float* p = x_grad + row * cols + c * V;
       if (beta != 0.0f) {
         if (VEC) {
@@ -257,10 +307,12 @@ __global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(size_t cols, c
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) o[c] = expf(xr[c] - M) / S;
 }
 
+template <class RG>
 __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, float* x_grad,
                                                                   const float* __restrict__ out, const float* out_grad,
-                                                                  float beta) {
+                                                                  float beta, RG rg) {
   __shared__ float smem[16];
+  const float kk = rg.k();
   const size_t base = (size_t)blockIdx.x * cols;
   const float* sr = out + base;
   const float* gr = out_grad + base;
@@ -269,13 +321,14 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
   float dot = 0.0f;
   for (size_t c = threadIdx.x; c < nv; c += 1024) {
     const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
-    dot += (a.x * b.x + a.y * b.y) + (a.z * b.z + a.w * b.w);
+    dot += (rg.term(a.x, b.x) + rg.term(a.y, b.y)) + (rg.term(a.z, b.z) + rg.term(a.w, b.w));
   }
-  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) dot += sr[c] * gr[c];
+  for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) dot += rg.term(sr[c], gr[c]);
   dot = block_reduce<SumOp>(dot, smem);
   for (size_t c = threadIdx.x; c < nv; c += 1024) {
     const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
-    float4 r = make_float4(a.x * (b.x - dot), a.y * (b.y - dot), a.z * (b.z - dot), a.w * (b.w - dot));
+    float4 r = make_float4(rg.result(a.x, b.x, dot, kk), rg.result(a.y, b.y, dot, kk), rg.result(a.z, b.z, dot, kk),
+                           rg.result(a.w, b.w, dot, kk));
     if (beta != 0.0f) {
       const float4 p = ld4g(xr + 4 * c);
       r = make_float4(beta * p.x + r.x, beta * p.y + r.y, beta * p.z + r.z, beta * p.w + r.w);
@@ -283,7 +336,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
     st4s(xr + 4 * c, r);
   }
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) {
-    const float r = sr[c] * (gr[c] - dot);
+    const float r = rg.result(sr[c], gr[c], dot, kk);
     xr[c] = beta != 0.0f ? beta * xr[c] + r : r;
   }
 }
@@ -326,15 +379,21 @@ __device__ __forceinline__ void ss_load(float* const (&buf)[NB], const float* co
     }
 }
 
-template <int L>
+template <int L, bool CCE>
 __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int cols, int rpb, const float* __restrict__ x,
-                                                                float* __restrict__ out) {
+                                                                float* __restrict__ out, const float* __restrict__ tg,
+                                                                float* __restrict__ loss_rows) {
   __shared__ float buf[SS_CHUNK + SS_CHUNK / 32 + 4];
+  __shared__ float tbuf[CCE ? SS_CHUNK + SS_CHUNK / 32 + 4 : 1];  // the targets of the same rows
   const int sh = ss_skew_shift(cols);
   const size_t r0 = (size_t)blockIdx.x * rpb;
   const int nr = r0 + rpb <= rows ? rpb : (int)(rows - r0);
   const int len = nr * cols;
-  {
+  if (CCE) {
+    float* const bufs[2] = {buf, tbuf};
+    const float* const srcs[2] = {x + r0 * cols, tg + r0 * cols};
+    ss_load<2>(bufs, srcs, len, sh);
+  } else {
     float* const bufs[1] = {buf};
     const float* const srcs[1] = {x + r0 * cols};
     ss_load<1>(bufs, srcs, len, sh);
@@ -357,9 +416,19 @@ __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int
         sum += e;
       }
     sum = wave_reduce<SumOp, L>(sum);
+    float acc = 0.0f;
     if (active)
-      for (int c = lane; c < cols; c += L) buf[ss_skew(sh, base + c)] = buf[ss_skew(sh, base + c)] / sum;
+      for (int c = lane; c < cols; c += L) {
+        const float p = buf[ss_skew(sh, base + c)] / sum;
+        buf[ss_skew(sh, base + c)] = p;
+        if (CCE) acc += cce_term(p, tbuf[ss_skew(sh, base + c)]);
+      }
+    if (CCE) {
+      acc = wave_reduce<SumOp, L>(acc);
+      if (active && lane == 0) loss_rows[r0 + r] = -logf(acc);
+    }
   }
+  if (CCE && !out) return;
   __syncthreads();
   float* dst = out + r0 * cols;
   for (int i = 4 * threadIdx.x; i < len; i += 1024) {
@@ -369,10 +438,11 @@ __global__ __launch_bounds__(256) void softmax_fwd_short_kernel(size_t rows, int
   }
 }
 
-template <int L>
+template <int L, class RG>
 __global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int cols, int rpb, float* x_grad,
                                                                 const float* __restrict__ out,
-                                                                const float* __restrict__ out_grad, float beta) {
+                                                                const float* __restrict__ out_grad, float beta, RG rg) {
+  const float kk = rg.k();
   __shared__ float sb[SS_CHUNK + SS_CHUNK / 32 + 4];
   __shared__ float gb[SS_CHUNK + SS_CHUNK / 32 + 4];
   const int sh = ss_skew_shift(cols);
@@ -392,10 +462,11 @@ __global__ __launch_bounds__(256) void softmax_bwd_short_kernel(size_t rows, int
     const int base = r * cols;
     float dot = 0.0f;
     if (active)
-      for (int c = lane; c < cols; c += L) dot += sb[ss_skew(sh, base + c)] * gb[ss_skew(sh, base + c)];
+      for (int c = lane; c < cols; c += L) dot += rg.term(sb[ss_skew(sh, base + c)], gb[ss_skew(sh, base + c)]);
     dot = wave_reduce<SumOp, L>(dot);
     if (active)
-      for (int c = lane; c < cols; c += L) sb[ss_skew(sh, base + c)] = sb[ss_skew(sh, base + c)] * (gb[ss_skew(sh, base + c)] - dot);
+      for (int c = lane; c < cols; c += L)
+        sb[ss_skew(sh, base + c)] = rg.result(sb[ss_skew(sh, base + c)], gb[ss_skew(sh, base + c)], dot, kk);
   }
   __syncthreads();
   float* dst = x_grad + r0 * cols;
@@ -433,9 +504,10 @@ static SoftmaxCfg pick_cfg(size_t colsv, bool fwd) {
   return {0, 0};
 }
 
-template <bool FWD, bool VEC>
+template <bool FWD, bool VEC, class RG = SoftmaxGradForm, bool CCE = false>
 static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const float* x, float* out, float* x_grad,
-                                const float* s, const float* g, float beta) {
+                                const float* s, const float* g, float beta, RG rg = RG{}, const float* tg = nullptr,
+                                float* loss_rows = nullptr) {
   // many short rows (measured at 2^27 elements, forward / backward TB/s, lanes-per-row kernel -> this
   // one: 10: 3.1 / 2.8 -> 5.8 / 6.1; 36: 2.2 / 2.9 -> 5.3 / 5.4; 100: 3.0 / 3.6 -> 4.8 / 5.2; 8: 3.3 / 4.0 ->
   // 5.9 / 6.1; 16: 1.4 / 1.8 -> 6.2 / 6.1; 32: 1.8 / 2.5 -> 5.6 / 6.2; 64: 4.9 / 5.2 -> 5.6 / 6.2; rows of 2 only
@@ -452,11 +524,11 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
 #define SL_SS(L)                                                                                                          \
   case L:                                                                                                                 \
     if (FWD)                                                                                                              \
-      hipLaunchKernelGGL((softmax_fwd_short_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, (int)cols, \
-                         rpb, x, out);                                                                                    \
+      hipLaunchKernelGGL((softmax_fwd_short_kernel<L, CCE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows,      \
+                         (int)cols, rpb, x, out, tg, loss_rows);                                                          \
     else                                                                                                                  \
-      hipLaunchKernelGGL((softmax_bwd_short_kernel<L>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, (int)cols, \
-                         rpb, x_grad, s, g, beta);                                                                        \
+      hipLaunchKernelGGL((softmax_bwd_short_kernel<L, RG>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows,       \
+                         (int)cols, rpb, x_grad, s, g, beta, rg);                                                         \
     break;
     switch (lanes) { SL_SS(1) SL_SS(2) SL_SS(4) SL_SS(8) SL_SS(16) SL_SS(32) SL_SS(64) }
 #undef SL_SS
@@ -466,8 +538,12 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
   SoftmaxCfg cfg = pick_cfg(colsv, FWD);
   SLHIP_REQUIRE(rows <= MAX_GRID, "too many rows for one launch");
   if (cfg.lanes == 0) {
+    if (CCE) {  // rows too long for registers: the caller splits the work
+      set_error("softmax with cross-entropy: rows of %zu floats do not fit the one-pass kernels", cols);
+      return SLHIP_EINVAL;
+    }
     if (FWD) hipLaunchKernelGGL(softmax_fwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x, out);
-    else hipLaunchKernelGGL(softmax_bwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta);
+    else hipLaunchKernelGGL((softmax_bwd_stream_kernel<RG>), dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta, rg);
     return post_launch();
   }
 #define SL_SM2(L, I, T)                                                                                              \
@@ -475,11 +551,11 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
     constexpr int RPB = L <= 64 ? 256 / L : 1;                                                                       \
     constexpr int BLOCK = L <= 64 ? 256 : L;                                                                         \
     if (FWD)                                                                                                         \
-      hipLaunchKernelGGL((softmax_fwd_kernel<VEC, L, I, T>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
-                         rows, cols, x, out);                                                                        \
+      hipLaunchKernelGGL((softmax_fwd_kernel<VEC, L, I, T, CCE>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
+                         rows, cols, x, out, tg, loss_rows);                                                         \
     else                                                                                                             \
-      hipLaunchKernelGGL((softmax_bwd_kernel<VEC, L, I, T>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
-                         rows, cols, x_grad, s, g, beta);                                                            \
+      hipLaunchKernelGGL((softmax_bwd_kernel<VEC, L, I, T, RG>), dim3(ceil_div(rows, RPB)), dim3(BLOCK), 0, ctx->stream, \
+                         rows, cols, x_grad, s, g, beta, rg);                                                        \
   } while (0)
 #define SL_SM(L, I)                                  \
   case L:                                            \
@@ -492,6 +568,37 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
 #undef SL_SM
 #undef SL_SM2
   return post_launch();
+}
+
+// The longest row the one-pass forward kernels hold in registers.
+constexpr size_t SOFTMAX_ONE_PASS_COLS = 16384 + 3;
+
+// probs = softmax(logits) (probs may be null) and loss_rows[r] = the cross-entropy of row r against
+// targets, in one pass through the softmax forward kernels; rows beyond SOFTMAX_ONE_PASS_COLS are
+// the caller's business.
+int32_t softmax_cce_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* logits, const float* targets, float* probs,
+                         float* loss_rows) {
+  if (cols > SOFTMAX_ONE_PASS_COLS) {
+    set_error("softmax with cross-entropy: rows of %zu floats do not fit the one-pass kernels", cols);
+    return SLHIP_EINVAL;
+  }
+  return cols >= 4 ? softmax_dispatch<true, true, SoftmaxGradForm, true>(ctx, rows, cols, logits, probs, nullptr, nullptr,
+                                                                        nullptr, 0.0f, SoftmaxGradForm{}, targets, loss_rows)
+                   : softmax_dispatch<true, false, SoftmaxGradForm, true>(ctx, rows, cols, logits, probs, nullptr, nullptr,
+                                                                         nullptr, 0.0f, SoftmaxGradForm{}, targets, loss_rows);
+}
+
+size_t softmax_one_pass_cols() { return SOFTMAX_ONE_PASS_COLS; }
+
+// logits_grad = beta * logits_grad + (p * sum_c t - t) * (upstream / rows), row by row, through the
+// softmax backward kernels.
+int32_t softmax_cce_grad_rows(slhip_ctx* ctx, size_t rows, size_t cols, const float* probs, const float* targets,
+                              float* logits_grad, float beta, const float* upstream_dev) {
+  const CceGradForm rg{upstream_dev, (float)rows};
+  return cols >= 4 ? softmax_dispatch<false, true, CceGradForm>(ctx, rows, cols, nullptr, nullptr, logits_grad, probs, targets,
+                                                                beta, rg)
+                   : softmax_dispatch<false, false, CceGradForm>(ctx, rows, cols, nullptr, nullptr, logits_grad, probs, targets,
+                                                                 beta, rg);
 }
 
 }  // namespace slhip
