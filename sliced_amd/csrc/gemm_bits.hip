@@ -144,15 +144,38 @@ __global__ __launch_bounds__(64) void gemm_bits_small_kernel(GemmArgs g, const u
   if (in) g.C[row * g.N + col] = val;
 }
 
-// x_grad += bit * out_grad: the ReLU gradient (src/matrix.rs:190-199) from the packed mask.
+// x_grad += bit * out_grad: the ReLU gradient (src/matrix.rs:190-199) from the packed mask.  One
+// vector of four elements per thread over the flat matrix; a thread finds the row and column of
+// its first element with one division and steps from there (any row length).
+template <class IDX>
 __global__ __launch_bounds__(256) void relu_grad_bits_kernel(size_t rows, size_t cols, size_t W, const uint32_t* __restrict__ bits,
                                                              float* x_grad, const float* __restrict__ out_grad) {
   const size_t n = rows * cols;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
-    const size_t row = i / cols, col = i - row * cols;
-    const uint32_t bit = (bits[row * W + (col >> 5)] >> (col & 31)) & 1u;
-    x_grad[i] = x_grad[i] + (bit ? 1.0f : 0.0f) * out_grad[i];
+  const size_t e0 = 4 * ((size_t)blockIdx.x * 256 + threadIdx.x);
+  if (e0 >= n) return;
+  IDX r = (IDX)e0 / (IDX)cols;
+  IDX c = (IDX)e0 - r * (IDX)cols;
+  const bool whole = e0 + 3 < n;
+  float g[4] = {0.f, 0.f, 0.f, 0.f}, o[4] = {0.f, 0.f, 0.f, 0.f};
+  if (whole) {
+    float4 t = ld4s(out_grad + e0);
+    g[0] = t.x; g[1] = t.y; g[2] = t.z; g[3] = t.w;
+    t = ld4g(x_grad + e0);
+    o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+  } else {
+    for (size_t q = 0; e0 + q < n; ++q) { g[q] = out_grad[e0 + q]; o[q] = x_grad[e0 + q]; }
   }
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (e0 + q < n) {
+      const uint32_t bit = (bits[(size_t)r * W + (c >> 5)] >> (c & 31)) & 1u;
+      o[q] = o[q] + (bit ? 1.0f : 0.0f) * g[q];
+    }
+    if (++c == (IDX)cols) { c = 0; ++r; }
+  }
+  if (whole) st4g(x_grad + e0, make_float4(o[0], o[1], o[2], o[3]));
+  else
+    for (size_t q = 0; e0 + q < n; ++q) x_grad[e0 + q] = o[q];
 }
 
 static int32_t gemm_bits_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, size_t K, const float* A, const float* B,
@@ -250,10 +273,13 @@ SLHIP_API int32_t slhip_relu_grad_bits(slhip_ctx* ctx, size_t rows, size_t cols,
   size_t len;
   SLHIP_REQUIRE(ctx && bits && x_grad && out_grad, "null argument");
   SLHIP_REQUIRE(checked_len(rows, cols, &len), "bad dims");
-  size_t blocks = (len + 255) / 256;
-  const size_t cap = (size_t)ctx->num_cu * 32;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(relu_grad_bits_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols, (cols + 31) / 32, bits,
-                     x_grad, out_grad);
+  const size_t blocks = ((len + 3) / 4 + 255) / 256;
+  SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many elements for one launch");
+  if (len <= 0xffffffffu)
+    hipLaunchKernelGGL((relu_grad_bits_kernel<uint32_t>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols,
+                       (cols + 31) / 32, bits, x_grad, out_grad);
+  else
+    hipLaunchKernelGGL((relu_grad_bits_kernel<size_t>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, rows, cols,
+                       (cols + 31) / 32, bits, x_grad, out_grad);
   return post_launch();
 }
