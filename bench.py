@@ -43,7 +43,7 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
 # A counter run cannot happen inside this program; the figure is that profile's, not this run's.
-GEMM_4096_TRAFFIC_BYTES = 1208151499  # (557161.0 x 2.000 + 65536.0 x 1.000) KiB: FETCH_SIZE + WRITE_SIZE medians of the headline kernel, scaled by the 1 GiB copy
+GEMM_4096_TRAFFIC_BYTES = 1208124515  # (557147.5 x 2.000 + 65536.0 x 1.000) KiB: FETCH_SIZE + WRITE_SIZE medians of the headline kernel, scaled by the 1 GiB copy
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 MIN_ITERS, MIN_WARMUP = 20, 5
@@ -223,6 +223,43 @@ def bench_bandwidth_suite(ctx, iters):
         for name, olen in (("sum_rows", cols), ("max_rows", cols), ("sum_cols", rows)):
             add("%s [%dx%d]" % (name, rows, cols), 4 * ne + 4 * olen,
                 lambda name=name: ctx.call("slhip_" + name, rows, cols, xs.ptr, ov.ptr), iters)
+    # the other row-shaped ops on the narrow shapes (2^27 elements each): softmax and the fused loss on
+    # short rows, transposes of narrow matrices, the broadcast-side gradients, the first-tie gradient
+    # on few long rows
+    ctx.call("slhip_fill", 1, 1.0, one.ptr)
+    lrb = ctx.empty(13421772)
+    for rows, cols in [(13421772, 10), (8388608, 16)]:
+        ne = rows * cols
+        xs, g, s, xg = x.view(0, ne), x.view(ne, ne), y.view(0, ne), y.view(ne, ne)
+        lr = lrb.view(0, rows)
+        add("softmax fwd [%dx%d]" % (rows, cols), 8 * ne, lambda: ctx.call("slhip_softmax", rows, cols, xs.ptr, s.ptr), iters)
+        add("softmax bwd [%dx%d]" % (rows, cols), 12 * ne,
+            lambda: ctx.call("slhip_softmax_grad", rows, cols, xg.ptr, s.ptr, g.ptr, 0.0), iters)
+        add("softmax_cce [%dx%d]" % (rows, cols), 12 * ne + 4 * rows,
+            lambda: ctx.call("slhip_softmax_cce", rows, cols, xs.ptr, g.ptr, s.ptr, lr.ptr), iters)
+        add("softmax_cce_grad [%dx%d]" % (rows, cols), 12 * ne,
+            lambda: ctx.call("slhip_softmax_cce_grad", rows, cols, s.ptr, g.ptr, xg.ptr, 0.0, one.ptr), iters)
+    lrb.free()
+    for rows, cols in [(13421772, 10), (10, 13421772), (128, 1 << 20), (1342177, 100)]:
+        ne = rows * cols
+        add("transpose [%dx%d]" % (rows, cols), 8 * ne,
+            lambda rows=rows, cols=cols: ctx.call("slhip_transpose", rows, cols, x.ptr, y.ptr, 0.0), iters)
+    for rows, cols in [(13421772, 10), (4026, 33333)]:
+        ne = rows * cols
+        lhs, g, lg = x.view(0, ne), x.view(ne, ne), y.view(0, ne)
+        v, vg = y.view(ne, max(rows, cols)), y.view(ne + max(rows, cols), max(rows, cols))
+        ctx.call("slhip_fill", max(rows, cols), 1.5, v.ptr)
+        add("row_op_grad mul, rhs side [%dx%d]" % (rows, cols), 8 * ne + 12 * cols,
+            lambda rows=rows, cols=cols: ctx.call("slhip_row_op_grad", 2, rows, cols, lhs.ptr, v.ptr, None, vg.ptr, g.ptr), iters)
+        add("col_op_grad div, rhs side [%dx%d]" % (rows, cols), 8 * ne + 12 * rows,
+            lambda rows=rows, cols=cols: ctx.call("slhip_col_op_grad", 3, rows, cols, lhs.ptr, v.ptr, None, vg.ptr, g.ptr), iters)
+        add("add_row [%dx%d]" % (rows, cols), 8 * ne + 4 * cols,
+            lambda rows=rows, cols=cols: ctx.call("slhip_add_row", rows, cols, lhs.ptr, v.ptr, lg.ptr), iters)
+    rows, cols = 134, 1000000
+    ne = rows * cols
+    ctx.call("slhip_max_cols", rows, cols, x.ptr, vec_r.ptr)
+    add("max_cols_grad [%dx%d]" % (rows, cols), 4 * ne + 16 * rows,
+        lambda: ctx.call("slhip_max_cols_grad", rows, cols, vec_r.ptr, x.ptr, y.ptr, y.view(ne, rows).ptr), iters)
     # config 4: the elementwise chain on 2^28 elements per tensor: 4 reads + 1 write
     bb, cc, dd = ctx.uniform(n, -10, 10, 2, SEED), ctx.uniform(n, -10, 10, 3, SEED), ctx.uniform(n, -10, 10, 4, SEED)
     add("ew_chain ((a+b)*c-d)^2^2 [2^28], hand-fused kernel", 20 * n,

@@ -36,13 +36,13 @@ struct PlainSrc {
   __device__ __forceinline__ float4 vec(size_t e, float, float, float, float) const { return ld4s(x + e); }
   __device__ __forceinline__ float one(size_t e, float) const { return ld1s(x + e); }
 };
+template <int op>  // compile-time op code: the switch inside the load loops cost the two-matrix read a fifth of its rate
 struct BcGradSrc {
   static constexpr bool HAS_V = true;
   static constexpr bool IS_PLAIN = false;
   const float* l;
   const float* g;
   const float* v;
-  int op;
   __device__ __forceinline__ float bvalue(size_t i) const { return v[i]; }
   __device__ __forceinline__ float4 vec(size_t e, float v0, float v1, float v2, float v3) const {
     const float4 a = ld4s(l + e), b = ld4s(g + e);
@@ -675,11 +675,20 @@ int32_t cce_rows_reduce(slhip_ctx* ctx, size_t rows, size_t cols, const float* p
 // or over column i (row_op), through the same kernels as the plain sums.
 int32_t bc_grad_rhs_reduce(slhip_ctx* ctx, bool by_row, int op, size_t rows, size_t cols, const float* lhs, const float* v,
                            const float* g, float* v_grad) {
-  const BcGradSrc src{lhs, g, v, op};
   const Finalize add{1.0f, 0, 1};
-  if (by_row) return reduce_cols_src<SumOp, BcGradSrc>(ctx, rows, cols, src, v_grad, add);
-  return reduce_rows_src<SumOp, BcGradSrc>(ctx, rows, cols, src, v_grad, add, (float*)ctx->workspace,
-                                           ctx->workspace_bytes / sizeof(float));
+#define SL_BG(OP)                                                                                                    \
+  case OP: {                                                                                                         \
+    const BcGradSrc<OP> src{lhs, g, v};                                                                              \
+    if (by_row) return reduce_cols_src<SumOp, BcGradSrc<OP>>(ctx, rows, cols, src, v_grad, add);                     \
+    return reduce_rows_src<SumOp, BcGradSrc<OP>>(ctx, rows, cols, src, v_grad, add, (float*)ctx->workspace,          \
+                                                 ctx->workspace_bytes / sizeof(float));                              \
+  }
+  switch (op) {
+    SL_BG(SLHIP_ADD) SL_BG(SLHIP_SUB) SL_BG(SLHIP_MUL) SL_BG(SLHIP_DIV)
+  }
+#undef SL_BG
+  set_error("broadcast op grad: unknown op %d", op);
+  return SLHIP_EINVAL;
 }
 
 // Few rows of great length: one workgroup per row would leave most of the chip idle (measured
