@@ -514,12 +514,13 @@ def mse_grad(x, y, x_grad, upstream=1.0):
     return x_grad
 
 
-def softmax_cce(rows, cols, logits, targets):
-    """(probs, loss per row)"""
+def softmax_cce(rows, cols, logits, targets, want_probs=True):
+    """(probs, loss per row); probs is None when want_probs is False (the library then stores none)"""
     with _Scope() as s:
-        dl, dt, dp, do = s.up(logits), s.up(targets), s.empty(rows * cols), s.empty(rows)
-        s.c.call("slhip_softmax_cce", rows, cols, dl.ptr, dt.ptr, dp.ptr, do.ptr)
-        return dp.numpy(), do.numpy()
+        dl, dt, do = s.up(logits), s.up(targets), s.empty(rows)
+        dp = s.empty(rows * cols) if want_probs else None
+        s.c.call("slhip_softmax_cce", rows, cols, dl.ptr, dt.ptr, _ptr(dp), do.ptr)
+        return (dp.numpy() if want_probs else None), do.numpy()
 
 
 def softmax_cce_grad(rows, cols, probs, targets, logits_grad, beta=0.0, upstream=1.0):

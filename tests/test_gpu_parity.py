@@ -785,6 +785,9 @@ def test_fused_softmax_cross_entropy_against_the_op_chain(hip, orc, shape):
     L = -np.log(np.sum(np.clip(P, 1e-7, 1 - 1e-7) * t.reshape(rows, cols), 1))
     assert np.all(np.abs(loss - L) <= 2e-6 * np.maximum(np.abs(L), 1.0))
     assert np.all(np.abs(loss - loss_ref) <= 2e-6 * np.maximum(np.abs(L), 1.0) + np.abs(loss_ref - L))
+    # without a buffer for the probabilities: the same losses
+    none, loss_only = hip.softmax_cce(rows, cols, x, t, want_probs=False)
+    assert none is None and np.all(np.abs(loss_only - loss) <= 2e-6 * np.maximum(np.abs(L), 1.0))
     # gradient of mean_r loss_r wrt the logits: (p - t)/rows; the reference's chain is cce_grad
     # (unclipped p) pushed through softmax_grad
     for beta, up in ((0.0, 1.0), (1.0, 0.5)):
