@@ -309,6 +309,12 @@ __global__ __launch_bounds__(512) void gemm_rows_narrow_kernel(GemmArgs g) {
   const int N = (int)g.N;
   const size_t groups = (M + 3) / 4;
   const size_t chunks = (K + KC - 1) / KC;
+  // few long rows: gridDim.y workgroups share the chunks of a row group and leave raw partial sums
+  // (g.partial[y][M][N]) for the split-K combine, which then applies the epilogue
+  const bool raw = gridDim.y > 1;
+  const size_t per_y = (chunks + gridDim.y - 1) / gridDim.y;
+  const size_t ch_beg = (size_t)blockIdx.y * per_y;
+  const size_t ch_end = ch_beg + per_y < chunks ? ch_beg + per_y : chunks;
   for (size_t grp0 = (size_t)blockIdx.x * 8; grp0 < groups; grp0 += (size_t)gridDim.x * 8) {
     const size_t grp = grp0 + w;
     const bool have = grp < groups;
@@ -316,7 +322,7 @@ __global__ __launch_bounds__(512) void gemm_rows_narrow_kernel(GemmArgs g) {
     rn_f4 acc[G];
 #pragma unroll
     for (int gi = 0; gi < G; ++gi) acc[gi] = rn_f4{0.f, 0.f, 0.f, 0.f};
-    for (size_t ch = 0; ch < chunks; ++ch) {
+    for (size_t ch = ch_beg; ch < ch_end; ++ch) {
       const size_t k0 = ch * KC;
       const int klen = (int)(k0 + KC < K ? KC : K - k0);
       // B's chunk is staged on the first pass, and again whenever the chunk changes (K > KC), BEFORE
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(512) void gemm_rows_narrow_kernel(GemmArgs g) {
       // would not be usable before all of A has arrived.  A thread takes four whole rows of B
       // (k = thread + 512 r): N loads each, contiguous across the threads and all in flight together,
       // then 4 * G scattered LDS writes per row, which also lay down the zeros beyond N and K.
-      if (grp0 == (size_t)blockIdx.x * 8 || chunks > 1) {
+      if (grp0 == (size_t)blockIdx.x * 8 || ch_end - ch_beg > 1) {
         float f[KC / 512][4 * G];
 #pragma unroll
         for (int r = 0; r < KC / 512; ++r) {
@@ -391,6 +397,18 @@ __global__ __launch_bounds__(512) void gemm_rows_narrow_kernel(GemmArgs g) {
         acc[gi][v] = x;
       }
     if (b != 0) continue;
+    if (raw) {
+      float* part = g.partial + (size_t)blockIdx.y * M * (size_t)N;
+#pragma unroll
+      for (int gi = 0; gi < G; ++gi)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const size_t r = grp * 4 + v;
+          const int c = 4 * gi + ij;
+          if (r < M && c < N) part[r * (size_t)N + c] = acc[gi][v];
+        }
+      continue;
+    }
     // lanes 0..3 hold everything: every read (mask, C for beta) before the first store
     float val[G][4];
 #pragma unroll
@@ -464,15 +482,43 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
   const size_t M = g.M, N = g.N, K = g.K;
   // short K: the result is the large side
   if (gemm_short_k_launch(ctx, ta, tb, g, nullptr, rc)) return 1;
+  // A narrow B stored N x K (the transposed form) is first turned into K x N at the top of the
+  // workspace: it is at most 16 rows, and the kernels below want k to run down its columns
+  // (2048 x 10 x 65536 A*Bt: 328 us through the tiled kernel, whose tile is mostly empty).
+  constexpr size_t BT_RESERVE = (size_t)16 << 20;
+  const bool bt_fits = tb && N <= 16 && K * N * sizeof(float) <= BT_RESERVE && ctx->workspace_bytes >= 4 * BT_RESERVE;
+  const size_t ws_bytes = bt_fits ? ctx->workspace_bytes - BT_RESERVE : ctx->workspace_bytes;
+  auto b_as_k_by_n = [&]() -> int32_t {
+    if (!tb) return SLHIP_OK;
+    float* bt = (float*)((char*)ctx->workspace + ws_bytes);
+    const int32_t r = slhip_transpose(ctx, N, K, g.B, bt, 0.0f);
+    if (r == SLHIP_OK) g.B = bt;
+    return r;
+  };
   // narrow N, A row-major: A (M x K) is the large side, the reduction runs along its rows
-  if (!ta && !tb && N <= 16 && K % 4 == 0 && K >= 256 && M >= 32 && M * K >= (size_t(1) << 22)) {
+  if (!ta && (!tb || bt_fits) && N <= 16 && K % 4 == 0 && K >= 256 && M >= 32 && M * K >= (size_t(1) << 22)) {
+    if ((*rc = b_as_k_by_n()) != SLHIP_OK) return 1;
     const int G = (int)((N + 3) / 4);
     const size_t lds = (size_t)ROWS_NARROW_KC * 4 * G * sizeof(float);
     const size_t groups8 = ((M + 3) / 4 + 7) / 8;  // workgroups' worth of row groups
     // one workgroup per CU (its chunk of B takes 32 KiB of LDS per column group), each looping
     // over its share of the rows
     const size_t blocks = groups8 < (size_t)ctx->num_cu ? groups8 : (size_t)ctx->num_cu;
-    const dim3 grid((unsigned)blocks);
+    // few long rows (measured 2048 x 1 x 65536: 300 us with 64 workgroups): the chunks of K are
+    // dealt out over several workgroups per row group, at least two chunks each
+    size_t splits = 1;
+    const size_t chunks = (K + ROWS_NARROW_KC - 1) / ROWS_NARROW_KC;
+    if (blocks * 2 <= (size_t)ctx->num_cu && chunks >= 4) {
+      splits = (size_t)ctx->num_cu / blocks;
+      if (splits > chunks / 2) splits = chunks / 2;
+      if (splits > 64) splits = 64;
+      if (splits > ws_bytes / (M * N * sizeof(float))) splits = ws_bytes / (M * N * sizeof(float));
+      if (splits < 1) splits = 1;
+      const size_t per = (chunks + splits - 1) / splits;
+      splits = (chunks + per - 1) / per;  // no empty share
+    }
+    g.splits = (unsigned)splits;
+    const dim3 grid((unsigned)blocks, (unsigned)splits);
 #define SL_RN(G_)                                                                                                        \
   do {                                                                                                                   \
     static bool sized = false;                                                                                           \
@@ -489,10 +535,10 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
     else SL_RN(4);
 #undef SL_RN
     *rc = post_launch();
-    return 1;
+    return splits > 1 && *rc == SLHIP_OK ? 2 : 1;
   }
   // narrow N: A (K x M) is the large side
-  if (ta && !tb && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22)) {
+  if (ta && (!tb || bt_fits) && N <= 16 && M % 4 == 0 && M >= 256 && K >= 512 && M * K >= (size_t(1) << 22)) {
     const int NP = (int)((N + 3) / 4 * 4);
     const size_t gx = (M / 4 + 63) / 64;
     // K splits: one workgroup of eight waves per CU (its LDS holds seven waves' sums), every wave
@@ -504,11 +550,12 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
     if (splits < (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK) splits = (K + NARROW_K_CHUNK - 1) / NARROW_K_CHUNK;
     if (splits > 65535) splits = 65535;
     const size_t part_bytes = M * NP * sizeof(float);
-    if (splits > ctx->workspace_bytes / part_bytes) splits = ctx->workspace_bytes / part_bytes;
+    if (splits > ws_bytes / part_bytes) splits = ws_bytes / part_bytes;
     if (splits < 1) return 0;
     const size_t k_chunk = ((K + splits - 1) / splits + GRAIN - 1) / GRAIN * GRAIN;
     splits = (K + k_chunk - 1) / k_chunk;
     if (gx > 0x7fffffffu) return 0;
+    if ((*rc = b_as_k_by_n()) != SLHIP_OK) return 1;
     const dim3 grid((unsigned)gx, (unsigned)splits);
     const size_t outs = M * N;
     const dim3 cgrid((unsigned)((outs + 255) / 256));

@@ -194,7 +194,9 @@ def test_gemm_rows_narrow_kernel(hip, orc):
     of 4 or of the workgroup's 32 rows, every epilogue, and a row of A that holds an inf (it must not
     leak into other rows through the zero padding)."""
     for (m, n, k) in [(8192, 10, 2048), (2049, 1, 2048), (4099, 3, 2052), (33000, 16, 260), (1030, 13, 4100), (2048, 8, 6148),
-                      (4096, 5, 1024), (16385, 12, 256), (3001, 10, 2000), (70000, 2, 64 * 5 + 4)]:
+                      (4096, 5, 1024), (16385, 12, 256), (3001, 10, 2000), (70000, 2, 64 * 5 + 4),
+                      # few long rows: the chunks of K shared out over several workgroups per row group
+                      (2048, 1, 65536), (513, 10, 30000), (64, 16, 131072 + 4), (1000, 3, 8192)]:
         say("rows-narrow gemm", m, n, k)
         a, b = gemm_operands(0, 0, m, n, k)
         exact, bound = gemm_bound(0, 0, m, n, k, a, b)
@@ -217,6 +219,45 @@ def test_gemm_rows_narrow_kernel(hip, orc):
     a[7 * k + 999] = np.inf          # the last element of row 7: the vector after it is another lane's padding
     got = hip.sgemm(0, 0, m, n, k, a, b).reshape(m, n)
     assert np.all(np.isinf(got[7])) and np.all(np.isfinite(np.delete(got, 7, axis=0)))
+
+
+def test_gemm_narrow_b_stored_transposed(hip, orc):
+    """A narrow B handed over as N x K (A*Bt, At*Bt with N <= 16): turned into K x N in the workspace
+    and run through the narrow-N kernels; results within the GEMM bound, beta and the epilogues too."""
+    for (m, n, k, ta) in [(8192, 10, 2048, 0), (2048, 10, 65536, 0), (3001, 16, 2000, 0), (4099, 3, 2052, 0),
+                          (8192, 10, 2048, 1), (2048, 7, 8192, 1), (4096, 16, 1024, 1), (512, 2, 262144, 0)]:
+        say("narrow B transposed", m, n, k, ta)
+        a, b = gemm_operands(ta, 1, m, n, k)
+        exact, bound = gemm_bound(ta, 1, m, n, k, a, b)
+        got = hip.sgemm(ta, 1, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        bt = np.ascontiguousarray(b.reshape(n, k).T).ravel()
+        assert np.array_equal(got, hip.sgemm(ta, 0, m, n, k, a, bt))        # the same kernel, the same sums
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(ta, 1, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(ta, 1, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+
+
+def test_gemm_with_a_row_vector_runs_as_matrix_times_column(hip, orc):
+    """M = 1: the product is computed as op(B)^T * a through the narrow-N kernels; all four forms (the
+    form of A is immaterial), beta, shapes that do and do not meet those kernels' conditions, and the
+    epilogues that keep the plain route."""
+    for (n, k) in [(4096, 2048), (4100, 4096), (1000, 999), (2048, 8192), (16, 100000), (300, 64)]:
+        for ta, tb in ((0, 0), (0, 1), (1, 0), (1, 1)):
+            say("row-vector gemm", n, k, ta, tb)
+            a, b = gemm_operands(ta, tb, 1, n, k)
+            exact, bound = gemm_bound(ta, tb, 1, n, k, a, b)
+            got = hip.sgemm(ta, tb, 1, n, k, a, b)
+            assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+            c0 = rng.uniform(n, -1, 1, tag=2, seed=SEED)
+            assert np.all(np.abs(hip.sgemm(ta, tb, 1, n, k, a, b, c=c0.copy(), beta=1.0) - (exact + c0)) <= bound + 1e-6 * np.abs(c0))
+        a, b = gemm_operands(0, 0, 1, n, k)
+        exact, bound = gemm_bound(0, 0, 1, n, k, a, b)
+        bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+        out, pre_act = hip.linear_fwd(1, k, n, a, b, bias, relu=True, want_pre_act=True)
+        assert np.all(np.abs(pre_act - (exact + bias)) <= bound + 1e-6 * np.abs(bias))
+        assert np.array_equal(out, orc.unary(orc.RELU, pre_act))
 
 
 def test_gemm_small_tile(hip, orc):
