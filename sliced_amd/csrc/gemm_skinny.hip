@@ -486,7 +486,10 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
   // workspace: it is at most 16 rows, and the kernels below want k to run down its columns
   // (2048 x 10 x 65536 A*Bt: 328 us through the tiled kernel, whose tile is mostly empty).
   constexpr size_t BT_RESERVE = (size_t)16 << 20;
-  const bool bt_fits = tb && N <= 16 && K * N * sizeof(float) <= BT_RESERVE && ctx->workspace_bytes >= 4 * BT_RESERVE;
+  // (from 2^25 elements of A on: below, the extra launch costs what the better kernel gains -
+  // 8192 x 10 x 2048 A*Bt 24 us through the wave kernel, 33 this way)
+  const bool bt_fits = tb && N <= 16 && M * K >= (size_t(1) << 25) && K * N * sizeof(float) <= BT_RESERVE &&
+                       ctx->workspace_bytes >= 4 * BT_RESERVE;
   const size_t ws_bytes = bt_fits ? ctx->workspace_bytes - BT_RESERVE : ctx->workspace_bytes;
   auto b_as_k_by_n = [&]() -> int32_t {
     if (!tb) return SLHIP_OK;
