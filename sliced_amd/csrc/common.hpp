@@ -156,7 +156,7 @@ __device__ __forceinline__ void st1s(float* p, float v) { __builtin_nontemporal_
 
 // d f(l, r) / d l   and   d f(l, r) / d r, as the reference's tests write them
 // (src/ops2/col_op/grad/cpu.rs:115,146: 1/rhs and lhs / -(rhs*rhs) for div)
-__device__ __forceinline__ float bc_dl(int op, float l, float r) {
+__device__ __forceinline__ float bc_dl(int op, float /*l*/, float r) {
   switch (op) {
     case SLHIP_ADD: return 1.0f;
     case SLHIP_SUB: return 1.0f;
