@@ -98,3 +98,30 @@ def test_random_matrix_op_shapes(hip, orc):
         exact_b = S * (G - (S * G).sum(1, keepdims=True))
         bound = 1e-6 * (np.abs(S) * (np.abs(G) + (np.abs(S) * np.abs(G)).sum(1, keepdims=True))) + 1e-37
         assert np.all(np.abs(got.reshape(rows, cols) - exact_b) <= bound), (rows, cols)
+        # the losses that ride the softmax kernels, and the cross-entropy as a row reduction
+        t = np.zeros((rows, cols), np.float32)
+        t[np.arange(rows), np.asarray(r.integers(0, cols, rows))] = 1.0
+        p2, loss = hip.softmax_cce(rows, cols, x, t.ravel())
+        assert np.all(np.abs(p2.reshape(rows, cols) - P) <= 1e-6 * P + 1e-37), (rows, cols)
+        L = -np.log(np.sum(np.clip(P, 1e-7, 1 - 1e-7) * t, 1))
+        assert np.all(np.abs(loss - L) <= 2e-6 * np.maximum(np.abs(L), 1.0)), (rows, cols)
+        assert np.all(np.abs(hip.cce(rows, cols, s, t.ravel()) - L) <= 2e-6 * np.maximum(np.abs(L), 1.0)), (rows, cols)
+        lg = hip.softmax_cce_grad(rows, cols, s, t.ravel(), np.zeros(n, np.float32), 0.0, 1.0)
+        exact_l = (s.astype(np.float64) - t.ravel()) / rows
+        assert np.all(np.abs(lg - exact_l) <= 2e-6 * (np.abs(s) + t.ravel()) / rows + 1e-37), (rows, cols)
+        # broadcast-side gradients of the op-code broadcast ops (reduction kernels reading two matrices)
+        lhs = rng.uniform(n, 0.5, 2.0, tag=4, seed=SEED + case)
+        for kind, vlen, axis in (("row_op", cols, 0), ("col_op", rows, 1)):
+            vv = rng.uniform(vlen, 0.5, 2.0, tag=5, seed=SEED + case)
+            for op in (orc.MUL, orc.DIV):
+                _, vg = getattr(hip, kind + "_grad")(op, cols, lhs, vv, None, np.zeros(vlen, np.float32), g)
+                Lh, Gd = lhs.reshape(rows, cols).astype(np.float64), g.reshape(rows, cols).astype(np.float64)
+                V = vv.astype(np.float64)[None, :] if kind == "row_op" else vv.astype(np.float64)[:, None]
+                terms = (Lh if op == orc.MUL else -Lh / (V * V)) * Gd
+                assert np.all(np.abs(vg - terms.sum(axis)) <= 2e-6 * np.abs(terms).sum(axis) + 1e-30), (kind, op, rows, cols)
+        # first-tie gradient of the row maximum, bit-exact
+        xt = rng.inject_row_max_ties(x.copy(), rows, cols, 0.05)
+        mx = orc.max_cols(cols, xt)
+        base = rng.normal(n, 1.0, tag=6, seed=SEED + case)
+        assert np.array_equal(hip.max_cols_grad(cols, mx, xt, base.copy(), gr), orc.max_cols_grad(cols, mx, xt, base.copy(), gr))
+
