@@ -273,6 +273,11 @@ def bench_bandwidth_suite(ctx, iters):
         a_, b_, c_ = x.view(0, m_ * k_), x.view(m_ * k_, k_ * n_), y.view(0, m_ * n_)
         add("gemm %s [%dx%dx%d]" % (what, m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_),
             lambda: ctx.call("slhip_sgemm", ta, tb, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), iters, sweep=sweep)
+    # a head of 16 classes on a 1 GiB activation matrix: the tall-A kernel on the 32 x 32 x 2 instruction
+    m_, n_, k_ = 16384, 16, 16384
+    a_, b_, c_ = x.view(0, m_ * k_), y.view(0, k_ * n_), y.view(k_ * n_, m_ * n_)
+    add("gemm A*B [%dx%dx%d]" % (m_, n_, k_), 4 * (m_ * k_ + k_ * n_ + m_ * n_),
+        lambda: ctx.call("slhip_sgemm", 0, 0, m_, n_, k_, a_.ptr, b_.ptr, c_.ptr, 0.0), iters)
     # what a launch costs in this way of timing, and what a plain streaming kernel reaches on operands
     # of the head products' size (64 MiB) timed the same way: the lines those three stand against
     add("fill of one element (the launch floor of a per-launch event pair)", 4, lambda: ctx.call("slhip_fill", 1, 1.0, one.ptr), iters)

@@ -342,7 +342,8 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // HBM-bound skinny products with float4-friendly shapes: vector-ALU kernels of their own
   {
     int32_t rc = SLHIP_OK;
-    const int took = gemm_skinny_launch(ctx, ta, tb, g, &rc);
+    int took = gemm_tall_launch(ctx, ta, tb, g, &rc);
+    if (took == 0) took = gemm_skinny_launch(ctx, ta, tb, g, &rc);
     if (took == 1 || rc) return rc;
     if (took == 2) return splitk_combine(ctx, g, g.splits);
   }

@@ -1,0 +1,196 @@
+// C = A * B for a tall A (stored M x K, K a multiple of 4, the large side: read once) and a B of
+// at most 32 columns, on the 32 x 32 x 2 matrix instruction.
+//
+// A wave owns 32 rows of A and the whole 32 x 32 block of C.  Per step it takes 64 k: its 32 x 64
+// block of A comes in with eight loads per lane that each read 256 contiguous bytes of four rows,
+// goes through a wave-private LDS block and comes back as the instruction's A operand; B waits in
+// the workspace as Bt[32][K'] (column-major, zero beyond N and K) and its 32 x 64 block takes
+// the same route through a block of LDS that the workgroup's four waves fill and read together
+// (a lane that fetched its 128 bytes of Bt itself touched 64 cache lines per load instruction:
+// 3.4-3.9 TB/s).  The instruction's k index is
+// ours to assign, as long as both operands agree: lane (r, h) feeds k = 32 h + 4 j + t at issue
+// (j, t), which makes both operands whole float4.  The next step's loads are requested before
+// the current step's 32 instructions run.  Few rows: workgroups split K and the split-K combine
+// finishes.
+//
+// Measured on 1 GiB of A (16384 x N x 16384, pack and combine launches included): 213-240 us for
+// any N up to 32 (4.5-5.0 TB/s of A); the matrix pipes are busy 61 % of the time a CU holds the
+// kernel and a CU holds it 77 % of the kernel's time (every workgroup is resident at once, and they
+// do not finish together).
+#include "gemm_tile.hpp"
+
+namespace slhip {
+
+constexpr int TALL_KC = 64;             // k per wave and step
+constexpr int TALL_PITCH = TALL_KC + 4; // floats per LDS row: rows 8 apart share banks, which a b128 read of 32 lanes needs anyway
+constexpr int TALL_ROWS = 128;          // rows of A per workgroup (four waves)
+
+// Bt[c][k] = B[k][c] (or B[c][k] for a B stored N x K), zero for c >= N and k >= K.
+__global__ __launch_bounds__(256) void tall_pack_b_kernel(size_t K, size_t Kp, int N, int tb, const float* __restrict__ B,
+                                                          float* __restrict__ Bt) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= 32 * Kp) return;
+  const size_t c = i / Kp, k = i - c * Kp;
+  float v = 0.0f;
+  if (c < (size_t)N && k < K) v = tb ? B[c * K + k] : B[k * (size_t)N + c];
+  Bt[i] = v;
+}
+
+__global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float* __restrict__ Bt, size_t Kp) {
+  // [4 waves][32][TALL_PITCH] of A, wave-private, then [2][32][TALL_PITCH] of Bt, shared by the four waves
+  extern __shared__ __attribute__((aligned(16))) float tall_lds[];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  float* blk = tall_lds + w * 32 * TALL_PITCH;
+  float* bblk = tall_lds + 4 * 32 * TALL_PITCH;
+  const size_t M = g.M, K = g.K;
+  const int N = (int)g.N;
+  const size_t m0 = ((size_t)blockIdx.x * 4 + w) * 32;  // (a wave wholly past the edge works on copies of the last row)
+  const size_t chunks = (K + TALL_KC - 1) / TALL_KC;
+  const size_t per_y = (chunks + gridDim.y - 1) / gridDim.y;
+  const size_t cbeg = (size_t)blockIdx.y * per_y;
+  const size_t cend = cbeg + per_y < chunks ? cbeg + per_y : chunks;
+
+  // load side: lane l takes the float4 at column 4 * (l % 16) of rows 4 p + l / 16 (p = 0..7) of
+  // the wave's block of A, and of rows 8 w + 4 q + l / 16 (q = 0, 1) of the 32 x 64 block of Bt
+  const int lrow = lane >> 4, lcol = 4 * (lane & 15);
+  const float* arow[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const size_t row = m0 + 4 * p + lrow;
+    arow[p] = g.A + (row < M ? row : M - 1) * K;  // rows past the edge: copies that are never stored
+  }
+  const float* brow[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) brow[q] = Bt + (size_t)(8 * w + 4 * q + lrow) * Kp + lcol;
+
+  floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+  // two steps' loads are in flight at any time: set u holds the steps cbeg + u, cbeg + u + 2, ...
+  float4 a[2][8], b[2][2];
+  auto request = [&](size_t ch, float4 (&as)[8], float4 (&bs)[2]) {
+    const size_t k0 = ch * TALL_KC;
+    const size_t k = k0 + lcol;
+    // K is a multiple of 4: a vector lies inside the row or wholly beyond it (then it is zeroed below)
+    const size_t kc = k < K ? k : K - 4;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) as[p] = ld4s(arow[p] + kc);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) bs[q] = ld4g(brow[q] + k0);
+  };
+  if (cbeg < cend) request(cbeg, a[0], b[0]);
+  if (cbeg + 1 < cend) request(cbeg + 1, a[1], b[1]);
+  for (size_t ch0 = cbeg; ch0 < cend; ch0 += 2) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const size_t ch = ch0 + u;
+      if (ch >= cend) break;  // the same for every wave of the workgroup
+      const bool beyond = ch * TALL_KC + lcol >= K;
+      float* bb = bblk + u * 32 * TALL_PITCH;
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const float4 v = beyond ? make_float4(0.f, 0.f, 0.f, 0.f) : a[u][p];
+        st4(blk + (4 * p + lrow) * TALL_PITCH + lcol, v);
+      }
+#pragma unroll
+      for (int q = 0; q < 2; ++q) st4(bb + (8 * w + 4 * q + lrow) * TALL_PITCH + lcol, b[u][q]);
+      // one barrier per step: the other half of the Bt buffer is written in the next step, which a
+      // wave enters only after every wave has passed this barrier and so has read that half
+      __syncthreads();
+      if (ch + 2 < cend) request(ch + 2, a[u], b[u]);
+      float4 av[8], bv[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        av[j] = ld4(blk + r * TALL_PITCH + 32 * h + 4 * j);
+        bv[j] = ld4(bb + r * TALL_PITCH + 32 * h + 4 * j);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].x, bv[j].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].y, bv[j].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].z, bv[j].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].w, bv[j].w, acc, 0, 0, 0);
+      }
+    }
+  }
+  if (m0 >= M) return;
+
+  // register v of lane (r, h): row 8 * (v / 4) + 4 * h + v % 4 of the wave's block, column r
+  if (r >= N) return;
+  const bool raw = gridDim.y > 1;
+  float* dst = raw ? g.partial + (size_t)blockIdx.y * M * (size_t)N : g.C;
+  float val[16], old[16], msk[16];
+  const bool with_mask = !raw && g.mask != nullptr, with_c = !raw && g.beta != 0.0f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const size_t row = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+    const size_t at = row * (size_t)N + r;
+    msk[v] = with_mask && row < M ? g.mask[at] : 0.0f;
+    old[v] = with_c && row < M ? g.C[at] : 0.0f;
+  }
+  const float bias = !raw && g.bias ? g.bias[r] : 0.0f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    float x = acc[v];
+    if (with_mask) x = (msk[v] >= 0.0f ? 1.0f : 0.0f) * x;
+    if (with_c) x = g.beta * old[v] + x;
+    if (!raw && g.bias) x = x + bias;
+    val[v] = x;
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const size_t row = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+    if (row >= M) continue;
+    const size_t at = row * (size_t)N + r;
+    float x = val[v];
+    if (!raw) {
+      if (g.pre_act) g.pre_act[at] = x;
+      if (g.relu) x = (x >= 0.0f ? 1.0f : 0.0f) * x;
+    }
+    dst[at] = x;
+  }
+}
+
+// Returns 0 if the product is not this kernel's, 1 if it ran to completion (*rc = status), 2 if
+// partials of g.splits k ranges wait in the workspace for the split-K combine.
+int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
+  const size_t M = g.M, N = g.N, K = g.K;
+  // From 13 columns on the sixteen-block kernel is bound by the matrix pipes (16384 x 16 x 16384:
+  // 396 us against 240 here); from 8 on this kernel is the faster one once A is 512 MiB or more
+  // (16384 x 8 / 10 / 12 x 16384: 265 / 231 / 246 -> 224 / 215 / 213 us), while at 64-256 MiB the
+  // two are level or the other ahead (8192 x 10 x 2048: 26.8 against 29.1 us).
+  if (ta || N > 32 || N < 8 || K % 4 != 0 || K < 256 || M < 512) return 0;
+  if (M * K < (N >= 13 ? (size_t(1) << 24) : (size_t(1) << 27))) return 0;
+  const size_t Kp = (K + TALL_KC - 1) / TALL_KC * TALL_KC;
+  const size_t bt_bytes = 32 * Kp * sizeof(float);
+  if (bt_bytes > ((size_t)32 << 20) || ctx->workspace_bytes < 4 * bt_bytes + ((size_t)64 << 20)) return 0;
+  // Bt at the top of the workspace, partials from its start
+  float* bt = (float*)((char*)ctx->workspace + ctx->workspace_bytes - bt_bytes);
+  const size_t ws_bytes = ctx->workspace_bytes - bt_bytes;
+  const size_t gx = (M + TALL_ROWS - 1) / TALL_ROWS;
+  if (gx > 0x7fffffffu) return 0;
+  const size_t chunks = Kp / TALL_KC;
+  size_t splits = 1;
+  // one round of three workgroups per CU (two, three, four and eight rounds measured 3-15 % slower)
+  const size_t want = (size_t)ctx->num_cu * 3;
+  if (gx < want) {
+    splits = (want + gx - 1) / gx;
+    if (splits > chunks / 8) splits = chunks / 8;  // at least eight steps each
+    if (splits > 64) splits = 64;
+    if (splits > ws_bytes / (M * N * sizeof(float))) splits = ws_bytes / (M * N * sizeof(float));
+    if (splits < 1) splits = 1;
+    const size_t per = (chunks + splits - 1) / splits;
+    splits = (chunks + per - 1) / per;
+  }
+  g.splits = (unsigned)splits;
+  const size_t pack_blocks = (32 * Kp + 255) / 256;
+  hipLaunchKernelGGL(tall_pack_b_kernel, dim3((unsigned)pack_blocks), dim3(256), 0, ctx->stream, K, Kp, (int)N, tb ? 1 : 0, g.B, bt);
+  const size_t lds = (size_t)6 * 32 * TALL_PITCH * sizeof(float);
+  hipLaunchKernelGGL(gemm_tall_kernel, dim3((unsigned)gx, (unsigned)splits), dim3(256), lds, ctx->stream, g, (const float*)bt, Kp);
+  *rc = post_launch();
+  return splits > 1 && *rc == SLHIP_OK ? 2 : 1;
+}
+
+}  // namespace slhip

@@ -569,6 +569,8 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 // gemm_skinny.hip: K <= 12, or A^T * B with N <= 16.  Returns 0 (not taken), 1 (done, *rc holds the
 // result) or 2 (partials of g.splits k ranges are in the workspace: the caller combines them).
 int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc);
+// The tall-A, at most 32 columns kernel (gemm_tall.hip), same convention.
+int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc);
 // The K <= 12 kernel alone, with the mask of the product given as bits (row-major, 32 columns to a
 // word) or NULL.  Returns 1 if it took the product (*rc = launch status), else 0.
 int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, const uint32_t* bits, int32_t* rc);

@@ -221,6 +221,37 @@ def test_gemm_rows_narrow_kernel(hip, orc):
     assert np.all(np.isinf(got[7])) and np.all(np.isfinite(np.delete(got, 7, axis=0)))
 
 
+def test_gemm_tall_kernel(hip, orc):
+    """A * B and A * Bt with a tall row-major A and 13..32 columns (8..12 from 2^27 elements of A on):
+    the 32 x 32 x 2 kernel whose waves own 32 rows each.  M off the multiples of 32 and 128, K a
+    multiple of 4 that is not one of 64, few rows with K split among workgroups and many rows without a
+    split, every epilogue."""
+    for (m, n, k, tb) in [(16384, 16, 1024, 0), (4100, 13, 4100, 0), (100000, 32, 260, 0), (513, 20, 40000, 0),
+                          (8192, 31, 2048, 1), (1000, 17, 16388, 1), (65536, 10, 2048, 0), (131072 + 5, 8, 1024, 1)]:
+        say("tall gemm", m, n, k, tb)
+        a, b = gemm_operands(0, tb, m, n, k)
+        exact, bound = gemm_bound(0, tb, m, n, k, a, b)
+        got = hip.sgemm(0, tb, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        assert np.array_equal(got, hip.sgemm(0, tb, m, n, k, a, b))         # same order of sums on every run
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(0, tb, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(0, tb, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+        if not tb:
+            bias = rng.uniform(n, -1, 1, tag=3, seed=SEED)
+            out, pre_act = hip.linear_fwd(m, k, n, a, b, bias, relu=True, want_pre_act=True)
+            pre_ref = orc.add_row(m, n, got, bias)
+            assert np.array_equal(pre_act, pre_ref)
+            assert np.array_equal(out, orc.unary(orc.RELU, pre_ref))
+    m, n, k = 4100, 16, 4100
+    a, b = gemm_operands(0, 0, m, n, k)
+    a = a.copy()
+    a[7 * k + k - 1] = np.inf            # the last element of row 7: it must stay in row 7
+    got = hip.sgemm(0, 0, m, n, k, a, b).reshape(m, n)
+    assert np.all(np.isinf(got[7])) and np.all(np.isfinite(np.delete(got, 7, axis=0)))
+
+
 def test_gemm_narrow_b_stored_transposed(hip, orc):
     """A narrow B handed over as N x K (A*Bt, At*Bt with N <= 16): turned into K x N in the workspace
     and run through the narrow-N kernels; results within the GEMM bound, beta and the epilogues too."""
