@@ -7,18 +7,22 @@ Headline (the JSON line's `value`): f32 GEMM TFLOP/s at M=N=K=4096, C = A·B, op
 U(-1,1) and resident in HBM before the timed region.  One step = one pass of the kernel; W untimed
 launches, then exactly K launches between two stream synchronisations.
 
-The same line carries
+stdout carries exactly one line, a JSON object of a few KB (a reader that keeps only the tail of the
+output still gets all of it):
   roofline     - the GEMM kernel against the fp32 matrix peak: `achieved` is the flop count divided
                  by the average launch duration of those K launches, from HIP events on the stream they
-                 run on.  Beside it: the median of per-launch event pairs (`achieved_median`), the same
-                 with the caches swept before every launch, the other two forms, the GEMM sweep, every
-                 bandwidth-bound op of the metric as GB/s of ALGORITHMIC bytes against 8 TB/s
-                 (`ops`, and flat `GBps: <op>` / `frac: <op>` keys), and the MLP training loops in
-                 steps/s (`mlp`, flat `steps/s: <loop>` keys);
+                 run on.  Beside it, flat: the median of per-launch event pairs (`achieved_median`),
+                 the three forms at the headline size, the slowest form of each size of the GEMM sweep,
+                 one GB/s figure of ALGORITHMIC bytes (against 8 TB/s) per bandwidth-bound op of the
+                 metric, the slowest op of a GiB or more, and the two MLP training loops in steps/s;
   cpu_baseline - the CPU side on this host's cores: the oracle's sgemm (a restatement of the
                  reference's loops; `kind: port`) on one pass of the same 4096^3 product, the same
                  product through numpy's bundled OpenBLAS (the reference's CPU GEMM is a CBLAS sgemm),
-                 the streaming ops and the two training loops.
+                 and the two training loops in steps/s.
+The full tables (every sweep entry, every op of the bandwidth suite with its times, the training
+loops' variants, the CPU streaming ops) go to stderr as they are measured and, as JSON, to the file
+named by --detail.  An untimed second of matrix-core load (`config.spin_up_s`) precedes the W
+declared warm-up launches of the headline.
 Bandwidth ops and sweep entries are timed as the median of per-launch HIP-event pairs over at least
 20 launches after at least 5 warm-ups; operands below 512 MiB have the caches swept (a read of a
 1 GiB scratch) between launches, outside the event pair.  A per-launch pair contains the launch gap
@@ -47,6 +51,22 @@ GEMM_4096_TRAFFIC_BYTES = 1208124539  # (557147.5 x 2.000 + 65536.0 x 1.000) KiB
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 MIN_ITERS, MIN_WARMUP = 20, 5
+SPIN_UP_SECONDS = 1.0             # untimed load before the headline's declared warm-up launches
+MAX_LINE_BYTES = 4096             # the result line stays well below what a log tail keeps
+DETAIL_DEFAULT = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+# the ops the metric names, as they appear in the one-line summary: (short key, entry of the suite)
+COMPACT_OPS = [
+    ("sum_rows 16384^2", "sum_rows [16384x16384]"), ("sum_cols 16384^2", "sum_cols [16384x16384]"),
+    ("max_rows 16384^2", "max_rows [16384x16384]"), ("max_cols 16384^2", "max_cols [16384x16384]"),
+    ("mean 2^28", "mean [2^28]"), ("transpose 16384^2", "transpose [16384x16384]"),
+    ("sum_cols 1x2^28", "sum_cols [1x268435456] -> 1"), ("max_rows 2^28x1", "max_rows [268435456x1] -> 1"),
+    ("softmax fwd 32768x4096", "softmax fwd [32768x4096]"), ("softmax bwd 32768x4096", "softmax bwd [32768x4096]"),
+    ("softmax fwd 8192x16384", "softmax fwd [8192x16384]"), ("softmax bwd 8192x16384", "softmax bwd [8192x16384]"),
+    ("softmax fwd 2^20x128", "softmax fwd [1048576x128]"), ("max_rows 32768x4096", "max_rows [32768x4096]"),
+    ("sum_rows 32768x4096", "sum_rows [32768x4096]"), ("transpose 32768x4096", "transpose [32768x4096]"),
+    ("ew chain 2^28", "ew_chain ((a+b)*c-d)^2^2 [2^28], hand-fused kernel"),
+    ("copy 1 GiB", "device copy [1 GiB] (achievable line)"),
+]
 
 
 def log(*a):
@@ -103,7 +123,23 @@ def median_ms(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
     return statistics.median(pair_times(ctx, fn, iters, warmup, sweep))
 
 
-def spin_up(ctx, a, b, c, n, seconds=1.0):
+def write_detail(path, detail):
+    """The full tables (GEMM sweep, every op of the bandwidth suite, the training loops, the CPU side)
+    as one JSON file; the directory is created if it is missing.  Returns the path, or None when it
+    cannot be written (the tables have gone to stderr as they were measured either way)."""
+    if not path:
+        return None
+    try:
+        os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(detail, f, indent=1)
+        return path
+    except OSError as e:
+        log("detail not written:", e)
+        return None
+
+
+def spin_up(ctx, a, b, c, n, seconds=SPIN_UP_SECONDS):
     """Untimed: keep the matrix cores under the headline's own load until clocks and power state have
     settled (the first launches after an idle period run at about 2.0 instead of 2.4 GHz, and a lighter
     spin-up kernel, or operand set-up between spin-up and timing, left the first timed block 2-4 % slow
@@ -209,6 +245,8 @@ def bench_bandwidth_suite(ctx, iters):
         add("softmax bwd [%dx%d]" % (rows, cols), 12 * ne,
             lambda: ctx.call("slhip_softmax_grad", rows, cols, xg.ptr, s.ptr, g.ptr, 0.0), iters)
         if cols == 4096:
+            add("transpose [%dx%d]" % (rows, cols), 8 * ne,
+                lambda: ctx.call("slhip_transpose", rows, cols, xs.ptr, s.ptr, 0.0), iters)
             for name, o1, olen in (("max_rows", vec_c.view(0, cols), cols), ("sum_rows", vec_c.view(0, cols), cols),
                                    ("max_cols", vec_r.view(0, R), rows), ("sum_cols", vec_r.view(0, R), rows)):
                 if olen > o1.n:
@@ -433,6 +471,8 @@ def main():
                     help="leave out the MLP variants that replay a recorded step (for runs under a kernel tracer, "
                          "which has crashed inside hipGraphLaunch; the kernels of a step are the same either way)")
     ap.add_argument("--size", type=int, default=4096)
+    ap.add_argument("--detail", default=os.environ.get("SLICED_BENCH_DETAIL", DETAIL_DEFAULT),
+                    help="file that receives the full tables as JSON ('' for none); stdout carries one short line")
     ap.add_argument("--only", default="", help="comma list of suite parts to run: gemm,sweep,bandwidth,chain,mlp")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -445,39 +485,43 @@ def main():
     log("device:", ctx.name())
     M = N = K = args.size
 
+    detail = {}
     head = bench_gemm(ctx, M, N, K, 0, 0, args.steps, args.warmup, headline=True)
     log("gemm A*B", head)
+    detail["headline"] = head
     roof = {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": head["frac_of_peak"], "traffic": GEMM_4096_TRAFFIC_BYTES if M == 4096 else None,
-            "traffic_source": "profiles/hbm_traffic_gemm_and_bandwidth_suite.md (rocprofv3 --pmc of this program, not this run)",
-            "achieved_median": head["tflops_median"], "frac_median": head["frac_median"],
-            "timing": "achieved: average over the timed launches; *_median and every op below: median of per-launch "
-                      "HIP-event pairs, >= %d launches after >= %d warm-ups" % (MIN_ITERS, MIN_WARMUP)}
+            "achieved_median": round(head["tflops_median"], 2)}
+    detail["notes"] = {
+        "traffic_source": "profiles/hbm_traffic_gemm_and_bandwidth_suite.md (rocprofv3 --pmc of this program, not this run)",
+        "timing": "achieved: average over the timed launches; *_median and every op: median of per-launch "
+                  "HIP-event pairs, >= %d launches after >= %d warm-ups" % (MIN_ITERS, MIN_WARMUP)}
     # the clock while the matrix cores are busy: queue 0.3 s of launches, sample, then wait
     a, b, c = ctx.uniform(M * K, -1, 1, 0, SEED), ctx.uniform(K * N, -1, 1, 1, SEED), ctx.zeros(M * N)
     for _ in range(min(200, int(300 / max(head["ms_kernel"], 0.01)) + 1)):
         ctx.call("slhip_sgemm", 0, 0, M, N, K, a.ptr, b.ptr, c.ptr, 0.0)
     time.sleep(0.15)
-    roof["shader_clock_mhz_under_gemm_load"] = shader_clock_mhz()
+    roof["sclk_mhz"] = shader_clock_mhz()
     ctx.sync()
+    kernel_name = ctx.last_gemm_plan()
     for x in (a, b, c):
         x.free()
-    log("sclk under load:", roof["shader_clock_mhz_under_gemm_load"])
+    log("sclk under load:", roof["sclk_mhz"], " plan:", kernel_name)
     parts = set(args.only.split(",")) if args.only else {"gemm", "sweep", "bandwidth", "chain", "mlp"}
     if args.no_suite:
         parts = set()
     iters = max(MIN_ITERS, args.steps)
+    r1 = lambda v: round(v, 1)
     if "gemm" in parts:
         sweep_buf = ctx.empty(1 << 28)
         forms = {}
         for form, (ta, tb) in {"A*B": (0, 0), "A*Bt": (0, 1), "At*B": (1, 0)}.items():
             r = bench_gemm(ctx, M, N, K, ta, tb, iters, MIN_WARMUP, sweep=sweep_buf)
             forms[form] = r
-            roof["TFLOPs: %d^3 %s" % (M, form)] = r["tflops_median"]
-            roof["TFLOPs: %d^3 %s, caches swept" % (M, form)] = r["tflops_median_caches_swept"]
+            roof["TFLOPs %s" % form] = r1(r["tflops_median"])
             log(form, r)
-        roof["achieved_caches_swept"] = forms["A*B"]["tflops_median_caches_swept"]
-        roof["gemm_forms"] = forms
+        roof["TFLOPs A*B caches swept"] = r1(forms["A*B"]["tflops_median_caches_swept"])
+        detail["gemm_forms"] = forms
         sweep_buf.free()
     if "sweep" in parts:
         sweep = {}
@@ -488,35 +532,56 @@ def main():
                 key = "%dx%dx%d %s" % (m, n, k, form)
                 sweep[key] = {"tflops": r["tflops_median"], "frac": r["frac_median"], "ms": r["ms_median"],
                               "tflops_back_to_back": r["tflops_back_to_back"], "ms_back_to_back": r["ms_back_to_back"]}
-                roof["TFLOPs: " + key] = round(r["tflops_median"], 2)
-                roof["TFLOPs, launches back to back: " + key] = round(r["tflops_back_to_back"], 2)
                 log(key, sweep[key])
-        roof["gemm_sweep"] = sweep
+        detail["gemm_sweep"] = sweep
+        # per size: the slowest of the three forms, per launch (median of event pairs)
+        for size, label in (("512x512x512", "512^3"), ("1024x1024x1024", "1024^3"), ("2048x2048x2048", "2048^3"),
+                            ("8192x8192x8192", "8192^3"), ("8192x2048x784", "8192x2048x784"), ("784x2048x8192", "784x2048x8192")):
+            roof["TFLOPs %s min of forms" % label] = r1(min(v["tflops"] for kk, v in sweep.items() if kk.startswith(size + " ")))
     if "bandwidth" in parts:
         ops = bench_bandwidth_suite(ctx, iters)
-        roof["ops"] = ops
-        for e in ops:
-            roof["GBps: " + e["op"]] = round(e["GBps"], 1)
+        detail["ops"] = ops
+        by_name = {e["op"]: e["GBps"] for e in ops}
+        for short, name in COMPACT_OPS:
+            if name in by_name:
+                roof["GBps " + short] = int(round(by_name[name]))
+        metric_ops = [e for e in ops if e["algorithmic_bytes"] >= (1 << 30) and not e["op"].startswith(("device copy", "gemm"))]
+        worst = min(metric_ops, key=lambda e: e["GBps"])
+        roof["GBps min over %d ops >= 1 GiB" % len(metric_ops)] = int(round(worst["GBps"]))
+        roof["min op"] = worst["op"]
     ctx.close()
     if "chain" in parts:
         ch = bench_tape_chain(None, iters)
         log("tape chain", ch)
-        roof["tape_chain"] = ch
-        for key in ("GBps_fused_tape", "GBps_op_by_op_tape"):
-            if key in ch:
-                roof["GBps: ew chain [2^28], " + key[5:].replace("_", " ")] = round(ch[key], 1)
+        detail["tape_chain"] = ch
+        if "GBps_fused_tape" in ch:
+            roof["GBps chain on the tape, fused"] = int(round(ch["GBps_fused_tape"]))
     if "mlp" in parts:
         mlp = bench_mlp(50, 200, graph=not args.no_graph)
         log(mlp)
-        roof["mlp"] = mlp
-        for loop, row in mlp.items():
-            if isinstance(row, dict) and "steps_per_s" in row:
-                roof["steps/s: " + loop] = round(row["steps_per_s"], 1)
+        detail["mlp"] = mlp
+        for cfg in ("C1", "C5"):
+            rows = {loop: row["steps_per_s"] for loop, row in mlp.items()
+                    if loop.startswith(cfg) and isinstance(row, dict) and "steps_per_s" in row}
+            if rows:
+                best = max(rows, key=rows.get)
+                roof["steps/s %s" % cfg] = r1(rows[best])
+                roof["steps/s %s variant" % cfg] = best[best.index("(") + 1:-1]
 
     cpu = None
     if not args.no_cpu:
-        cpu = cpu_baseline(M, N, K)
-        log("cpu", cpu)
+        full = cpu_baseline(M, N, K)
+        log("cpu", full)
+        detail["cpu_baseline"] = full
+        cpu = {key: full[key] for key in ("value", "unit", "cores", "kind", "sample", "cblas_TFLOPs", "cblas_threads") if key in full}
+        for key, v in full.items():
+            if key.startswith(("C1 steps_per_s", "C5 steps_per_s")):
+                cpu[key] = round(v, 2)
+        if isinstance(full.get("ops"), dict):
+            for op in ("sum_rows", "max_cols", "transpose", "softmax fwd"):
+                row = full["ops"].get(op)
+                if isinstance(row, dict):
+                    cpu["GBps " + op] = {kk.replace("GBps_", ""): round(v, 1) for kk, v in row.items()}
 
     line = {
         "metric": "f32 GEMM TFLOP/s @4096^3",
@@ -532,11 +597,19 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
-                   "kernel": "gemm_kernel<false,false,32,true,2,2>: 128x128 tiles, BK=32, v_mfma_f32_32x32x2_f32"},
+                   "kernel": kernel_name, "spin_up_s": SPIN_UP_SECONDS},
         "roofline": roof,
         "cpu_baseline": cpu,
     }
-    print(json.dumps(line))
+    detail["line"] = line
+    path = write_detail(args.detail, detail)
+    if path:
+        log("detail written to", path)
+    text = json.dumps(line)
+    if len(text) > MAX_LINE_BYTES:
+        raise SystemExit("bench.py: the result line is %d bytes, above the %d that a reader of the last line can rely on"
+                         % (len(text), MAX_LINE_BYTES))
+    print(text, flush=True)
 
 
 if __name__ == "__main__":

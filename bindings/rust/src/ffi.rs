@@ -137,6 +137,7 @@ extern "C" {
     ) -> i32;
     pub fn slhip_gemm_tail_policy(ctx: *mut SlhipCtx, policy: i32) -> i32;
     pub fn slhip_gemm_tile_policy(ctx: *mut SlhipCtx, policy: i32) -> i32;
+    pub fn slhip_gemm_plan_describe(ctx: *mut SlhipCtx, buf: *mut c_char, len: usize) -> i32;
     pub fn slhip_gemm(
         ctx: *mut SlhipCtx,
         m: usize,

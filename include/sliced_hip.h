@@ -150,6 +150,10 @@ int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy);
  * testing knob with no counterpart in the reference. */
 enum { SLHIP_TILE_AUTO = 0, SLHIP_TILE_128X128 = 1, SLHIP_TILE_64X64 = 3, SLHIP_TILE_128X128_WIDE = 4 };
 int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy);
+/* Writes into buf (len bytes, NUL-terminated) which kernel and plan the last product issued on this
+ * context ran as: kernel template, tile, waves per workgroup, k splits.  For logs and benchmark
+ * records; no counterpart in the reference. */
+int32_t slhip_gemm_plan_describe(slhip_ctx* ctx, char* buf, size_t len);
 
 /* Gemm::gemm (src/ops2/gemm/mod.rs:21-32), trait argument order (m, k, n). */
 int32_t slhip_gemm(slhip_ctx* ctx, size_t m, size_t k, size_t n, const float* lhs, const float* rhs,

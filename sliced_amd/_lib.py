@@ -44,6 +44,7 @@ PROTOTYPES = {
     "slhip_sgemm": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_gemm_tail_policy": [c_vp, c_i32],
     "slhip_gemm_tile_policy": [c_vp, c_i32],
+    "slhip_gemm_plan_describe": [c_vp, C.c_char_p, c_sz],
     "slhip_sgemm_relu_mask": [c_vp, c_i32, c_i32, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, C.c_float],
     "slhip_gemm": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_gemm_grad": [c_vp, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp, C.c_float],

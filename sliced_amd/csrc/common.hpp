@@ -23,6 +23,12 @@ struct slhip_ctx {
   int gemm_tail = 0;             // SLHIP_TAIL_*: how the tiled GEMM treats a partly filled last round
   int gemm_tile = 0;             // SLHIP_TILE_*: tile of C per workgroup of the tiled GEMM
   float* static_scratch = nullptr;  // this device's copy of the file-scope scratch array of reduce.hip
+  // what the last product on this context ran as (slhip_gemm_plan_describe); set by gemm_run
+  struct GemmPlan {
+    int kind = 0;  // 0 none, 1 wave-per-tile, 2 tiled four waves, 3 tiled eight waves, 4 spread tail, 5 tall A, 6 skinny
+    bool ta = false, tb = false, only_fast = false, small_tile = false;
+    unsigned splits = 1, waves = 4;
+  } last_gemm;
 };
 
 struct slhip_event {

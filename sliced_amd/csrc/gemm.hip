@@ -343,7 +343,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   {
     int32_t rc = SLHIP_OK;
     int took = gemm_tall_launch(ctx, ta, tb, g, &rc);
-    if (took == 0) took = gemm_skinny_launch(ctx, ta, tb, g, &rc);
+    ctx->last_gemm.kind = 5;
+    if (took == 0) {
+      took = gemm_skinny_launch(ctx, ta, tb, g, &rc);
+      ctx->last_gemm.kind = 6;
+    }
+    ctx->last_gemm.ta = ta; ctx->last_gemm.tb = tb; ctx->last_gemm.splits = took == 2 ? g.splits : 1;
     if (took == 1 || rc) return rc;
     if (took == 2) return splitk_combine(ctx, g, g.splits);
   }
@@ -385,6 +390,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     else SL_WGEMM(true, true);
 #undef SL_WGEMM
 #undef SL_WGEMM2
+    ctx->last_gemm = {1, ta, tb, full, false, (unsigned)splits, nw};
     int32_t rc = post_launch();
     if (rc || splits == 1) return rc;
     return splitk_combine(ctx, g, splits);
@@ -532,12 +538,15 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // every k tile of every workgroup complete, inside and 16-byte aligned: the kernel without the
   // clamped loops (k_chunk is a multiple of BK, so only the end of K can leave a partial tile)
   const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % tile_m == 0 && N % tile_n == 0 && K % BK == 0;
+  ctx->last_gemm = {spread_workers ? 4 : 2, ta, tb, only_fast, small_tile, (unsigned)splits, 4};
   if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tiles - sp.first);
 
   // One workgroup per CU at most (and the 128 x 128 tile): the eight-wave kernel
   const bool wide_fits = !small_tile && !(ta && tb);
   if (wide_fits && (ctx->gemm_tile == SLHIP_TILE_128X128_WIDE ||
                     (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && tiles * splits <= (size_t)ctx->num_cu))) {
+    ctx->last_gemm.kind = 3;
+    ctx->last_gemm.waves = 8;
     int32_t rc = gemm_wide_launch(ctx, ta, tb, only_fast, g);
     if (rc || splits == 1) return rc;
     return splitk_combine(ctx, g, splits);
@@ -611,6 +620,37 @@ SLHIP_API int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy) {
                     policy == SLHIP_TILE_128X128_WIDE,
                 "unknown policy");
   ctx->gemm_tile = policy;
+  return SLHIP_OK;
+}
+
+SLHIP_API int32_t slhip_gemm_plan_describe(slhip_ctx* ctx, char* buf, size_t len) {
+  SLHIP_REQUIRE(ctx && buf && len > 0, "null argument");
+  const slhip_ctx::GemmPlan& p = ctx->last_gemm;
+  const char* tf[2] = {"false", "true"};
+  switch (p.kind) {
+    case 1:
+      snprintf(buf, len, "gemm_wave_kernel<%s,%s,...,%s>: one wave per 32x32 tile, %u waves per workgroup, %u k splits, v_mfma_f32_32x32x2_f32",
+               tf[p.ta], tf[p.tb], tf[p.only_fast], p.waves, p.splits);
+      break;
+    case 2:
+    case 4:
+      snprintf(buf, len, "%s<%s,%s,%d,%s,%s>: %s tiles on 4 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32",
+               p.kind == 4 ? "gemm_spread_kernel" : "gemm_kernel", tf[p.ta], tf[p.tb], GEMM_BK, tf[p.only_fast],
+               p.small_tile ? "1,1" : "2,2", p.small_tile ? "64x64" : "128x128", GEMM_BK, p.splits);
+      break;
+    case 3:
+      snprintf(buf, len, "gemm_wide_kernel<%s,%s,%s>: 128x128 tiles on 8 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32", tf[p.ta],
+               tf[p.tb], tf[p.only_fast], GEMM_BK, p.splits);
+      break;
+    case 5:
+      snprintf(buf, len, "tall-A kernel (at most 32 columns), form %s,%s", tf[p.ta], tf[p.tb]);
+      break;
+    case 6:
+      snprintf(buf, len, "skinny kernel (short K or narrow N), form %s,%s, %u k splits", tf[p.ta], tf[p.tb], p.splits);
+      break;
+    default:
+      snprintf(buf, len, "no product has run on this context");
+  }
   return SLHIP_OK;
 }
 

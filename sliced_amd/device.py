@@ -60,6 +60,12 @@ class Context:
         self.call("slhip_device_name", b, 128)
         return b.value.decode()
 
+    def last_gemm_plan(self):
+        """Kernel and plan of the last product issued on this context, as text."""
+        b = C.create_string_buffer(256)
+        self.call("slhip_gemm_plan_describe", b, 256)
+        return b.value.decode()
+
     def empty(self, n):
         p = C.c_void_p()
         self.call("slhip_malloc", int(n) * 4, C.byref(p))
