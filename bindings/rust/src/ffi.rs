@@ -84,6 +84,7 @@ extern "C" {
     pub fn slhip_device_name(ctx: *mut SlhipCtx, buf: *mut c_char, buflen: usize) -> i32;
     pub fn slhip_stream(ctx: *mut SlhipCtx, hip_stream: *mut *mut c_void) -> i32;
     pub fn slhip_workspace_bytes(ctx: *mut SlhipCtx) -> usize;
+    pub fn slhip_workspace(ctx: *mut SlhipCtx, dptr: *mut *mut c_void) -> i32;
     pub fn slhip_malloc(ctx: *mut SlhipCtx, bytes: usize, dptr: *mut *mut c_void) -> i32;
     pub fn slhip_free(ctx: *mut SlhipCtx, dptr: *mut c_void) -> i32;
     pub fn slhip_memcpy_h2d(ctx: *mut SlhipCtx, dst_dev: *mut c_void, src_host: *const c_void, bytes: usize) -> i32;

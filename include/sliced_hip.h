@@ -76,6 +76,11 @@ const char* slhip_last_error_string(void);
 int32_t slhip_device_name(slhip_ctx* ctx, char* buf, size_t buflen);
 int32_t slhip_stream(slhip_ctx* ctx, void** hip_stream);
 size_t slhip_workspace_bytes(slhip_ctx* ctx);
+/* The device address of the context's workspace (slhip_workspace_bytes long), where two-stage
+ * reductions and split products keep their partial results between launches.  Its contents mean
+ * nothing between calls; a caller may use it as scratch of its own while no op of this context is
+ * in flight.  No counterpart in the reference, whose devices hand out scratch through retrieve(). */
+int32_t slhip_workspace(slhip_ctx* ctx, void** dptr);
 
 int32_t slhip_malloc(slhip_ctx* ctx, size_t bytes, void** dptr);
 int32_t slhip_free(slhip_ctx* ctx, void* dptr);

@@ -23,6 +23,7 @@ PROTOTYPES = {
     "slhip_device_name": [c_vp, C.c_char_p, c_sz],
     "slhip_stream": [c_vp, C.POINTER(c_vp)],
     "slhip_workspace_bytes": [c_vp],
+    "slhip_workspace": [c_vp, C.POINTER(c_vp)],
     "slhip_malloc": [c_vp, c_sz, C.POINTER(c_vp)],
     "slhip_free": [c_vp, c_vp],
     "slhip_memcpy_h2d": [c_vp, c_vp, c_vp, c_sz],

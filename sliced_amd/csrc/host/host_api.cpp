@@ -102,6 +102,14 @@ SLH_API int slh_matrix_chain(void* dev, int which, size_t rows, size_t cols, uin
     }
   });
 }
+// Matrix::rand (src/matrix.rs:266-271) on a rows x cols view of the buffer
+SLH_API int slh_matrix_rand(void* dev, uint64_t id, size_t rows, size_t cols, float lo, float hi, uint64_t seed, uint64_t tag) {
+  return guard([&] {
+    HIP* dv = (HIP*)dev;
+    Matrix m(dv->lookup(id), rows, cols);
+    m.rand(lo, hi, seed, tag);
+  });
+}
 SLH_API int slh_buffer_from(void* dev, const float* host, size_t len, uint64_t* id) {
   return guard([&] { *id = ((HIP*)dev)->from(host, len).id; });
 }

@@ -175,6 +175,14 @@ class HIP {
   }
   void release(uint64_t id) {
     if (pending_.count(id) || !pending_order_.empty()) run();
+    // intermediates that a fused chain kept in registers and that are computed from this buffer
+    // get their values now, while it still holds what they were computed from
+    if (!virtual_.empty()) {
+      std::vector<uint64_t> readers;
+      for (auto& kv : virtual_)
+        if (kv.second.a == id || (!kv.second.unary && kv.second.b == id)) readers.push_back(kv.first);
+      for (uint64_t r : readers) materialise(r);
+    }
     virtual_.erase(id);
     auto it = allocs_.find(id);
     if (it == allocs_.end()) return;
@@ -220,9 +228,10 @@ class HIP {
       size_t i;
       size_t operator*() const { return i; }
       bool operator!=(const It& o) const { return i != o.i; }
-      It& operator++() { ++i; dev->cursor_ = 0; return *this; }
+      // what one iteration deferred runs before the next hands the same buffers out again
+      It& operator++() { ++i; dev->run(); dev->cursor_ = 0; return *this; }
     };
-    It begin() { dev->cursor_ = 0; return {dev, 0}; }
+    It begin() { dev->run(); dev->cursor_ = 0; return {dev, 0}; }
     It end() { return {dev, n}; }
   };
   Range range(size_t n) { return Range{this, n}; }
@@ -295,8 +304,10 @@ class HIP {
       for (uint64_t id : order)
         if (pending_.count(id)) emit_group(id);
     } catch (...) {
+      // the ops that did not launch have left placeholder closures on the tape: a backward pass over
+      // it would silently skip them, so the tape goes with them
       flushing_ = false;
-      pending_.clear();
+      clear_tape();
       throw;
     }
     pending_.clear();
@@ -367,6 +378,8 @@ class HIP {
   }
   // After a backward pass, finished or failed, the device holds no tape: a closure that throws
   // (a released buffer, a refused launch) must not leave the rest behind for the next pass to replay.
+  // (virtual_ stays: an intermediate that a chain kept in registers can still be asked for after
+  // the backward pass, and is computed then)
   void clear_tape() {
     tape_.clear();
     relu_pre_.clear();
@@ -743,6 +756,13 @@ class HIP {
     check(slhip_memcpy_d2d(ctx_, dst.ptr + dst_off, src.ptr + src_off, n * sizeof(float)), "slhip_memcpy_d2d");
   }
 
+  // RandOp::rand (src/rawops/cpu/rand.rs:7-12) on the device: x[i] = lo + (hi - lo) * u_i
+  void rand(const Buffer& x, float lo, float hi, uint64_t seed, uint64_t tag) {
+    ready(x);
+    drop_pending_zero(x);
+    check(slhip_rand_uniform(ctx_, seed, tag, lo, hi, x.len, x.ptr), "slhip_rand_uniform");
+  }
+
   // SGD of the examples (examples/sine_net.rs:105-116): value -= grad * lr, on the device
   void sgd_step(const Buffer& p, float lr) {
     ready(p);
@@ -905,7 +925,8 @@ class HIP {
       in.op = (uint8_t)(n.unary ? (SLHIP_EW_UNARY | n.op) : n.op);
       in.src0 = reg_of(n.a);
       in.src1 = n.unary ? in.src0 : reg_of(n.b);
-      in.flags = n.with_grad ? 0 : SLHIP_EW_NOGRAD;
+      // an op issued while the tape was off has no gradient step, as on the op-by-op tape
+      in.flags = n.with_grad && n.tape_slot != SIZE_MAX ? 0 : SLHIP_EW_NOGRAD;
       in.p = n.p;
       in.q = n.q;
       prog.push_back(in);
@@ -915,7 +936,22 @@ class HIP {
     check(slhip_ew_program(ctx_, last.len, in_ptrs.size(), in_ptrs.data(), prog.size(), prog.data(), lookup(last.out).ptr),
           "slhip_ew_program");
     for (size_t i = 0; i + 1 < group.size(); ++i) virtual_[group[i].out] = group[i];
-    if (last.tape_slot == SIZE_MAX) return;
+    if (last.tape_slot == SIZE_MAX) {
+      // The root carries no gradient (exp, clip, or issued with the tape off), so nothing flows into
+      // the chain from above; a later reader of an intermediate may still leave a gradient for it.
+      // Each intermediate keeps its own gradient step at its own place on the tape, as issued op by
+      // op: it computes what it reads (a fused-away intermediate) first.
+      for (size_t i = 0; i + 1 < group.size(); ++i) {
+        const EwNode n = group[i];
+        if (n.tape_slot == SIZE_MAX) continue;
+        tape_[n.tape_slot] = [this, n] {
+          materialise(n.a);
+          if (!n.unary) materialise(n.b);
+          single_grad(n);
+        };
+      }
+      return;
+    }
     tape_[last.tape_slot] = [this, group, leaves, prog] {
       const EwNode& root_node = group.back();
       // Another op has read an intermediate after all and left a gradient for it: that term has to
@@ -925,7 +961,7 @@ class HIP {
       if (touched) {
         for (size_t i = 0; i + 1 < group.size(); ++i) materialise(group[i].out);
         for (size_t i = group.size(); i-- > 0;)
-          if (group[i].with_grad && has_grad(group[i].out)) single_grad(group[i]);
+          if (group[i].with_grad && group[i].tape_slot != SIZE_MAX && has_grad(group[i].out)) single_grad(group[i]);
         return;
       }
       std::vector<const float*> ins;
@@ -1065,6 +1101,11 @@ class Matrix {
   Matrix grad() const { return Matrix(data.grad(), rows, cols); }
   void backward() const { data.backward(); }
   void backward_with(const Matrix& g) const { data.backward_with(g.data); }
+
+  // Matrix::rand (src/matrix.rs:266-271 -> RandOp::rand, src/rawops/cpu/rand.rs:7-12): every element
+  // uniform in [lo, hi).  The reference draws from an unseeded generator; here the stream is
+  // counter-based and named by (seed, tag), so a run can be repeated and checked on the host.
+  void rand(float lo, float hi, uint64_t seed = 0x51CED, uint64_t tag = 0) { device().rand(data, lo, hi, seed, tag); }
 
   Matrix T() const { return Matrix(device().transpose(rows, cols, data), cols, rows); }                         // :98-107
   Matrix gemm(const Matrix& rhs) const { return Matrix(device().gemm(rows, cols, rhs.cols, data, rhs.data), rows, rhs.cols); }  // :111-122

@@ -4,6 +4,7 @@
 //
 // Naming (kept from the reference): *_cols reduces along the contiguous axis (one value per
 // row); *_rows reduces along the strided axis (one value per column).
+#include <mutex>
 #include <numeric>
 
 #include "common.hpp"
@@ -585,12 +586,14 @@ constexpr size_t STATIC_SCRATCH_FLOATS = size_t(1) << 20;  // 4 MiB per GPU, hel
 static __device__ __align__(256) float static_scratch[STATIC_SCRATCH_FLOATS];
 constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
 static float* g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];  // device address per ordinal, 0 = not asked yet
+static std::mutex g_static_scratch_lock;                    // contexts may be created from several threads
 
 int32_t static_scratch_resolve(int device, float** ptr) {
   if (device < 0 || device >= STATIC_SCRATCH_MAX_DEVICES) {
     set_error("device ordinal %d beyond the %d this library keeps scratch addresses for", device, STATIC_SCRATCH_MAX_DEVICES);
     return SLHIP_EINVAL;
   }
+  std::lock_guard<std::mutex> hold(g_static_scratch_lock);
   if (!g_static_scratch[device]) {
     void* p = nullptr;
     SLHIP_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)));

@@ -158,6 +158,11 @@ SLHIP_API int32_t slhip_stream(slhip_ctx* ctx, void** s) {
 }
 
 SLHIP_API size_t slhip_workspace_bytes(slhip_ctx* ctx) { return ctx ? ctx->workspace_bytes : 0; }
+SLHIP_API int32_t slhip_workspace(slhip_ctx* ctx, void** dptr) {
+  SLHIP_REQUIRE(ctx && dptr, "null argument");
+  *dptr = ctx->workspace;
+  return SLHIP_OK;
+}
 
 SLHIP_API int32_t slhip_malloc(slhip_ctx* ctx, size_t bytes, void** dptr) {
   SLHIP_REQUIRE(ctx && dptr, "null argument");

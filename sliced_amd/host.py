@@ -158,6 +158,10 @@ class HIP:
         c, d = c or a, d or a
         return self._out(lib().slh_matrix_chain, int(which), _sz(rows), _sz(cols), _u64(a.id), _u64(b.id), _u64(c.id), _u64(d.id))
 
+    def matrix_rand(self, buf, rows, cols, lo, hi, seed=rng.DEFAULT_SEED, tag=0):
+        """Matrix::rand(lo, hi) on a rows x cols view of buf (src/matrix.rs:266-271), seeded."""
+        _ck(lib().slh_matrix_rand(self.h, _u64(buf.id), _sz(rows), _sz(cols), _f(lo), _f(hi), _u64(seed), _u64(tag)))
+
     def buffer(self, data):
         a = np.ascontiguousarray(data, dtype=np.float32).ravel()
         return self._out(lib().slh_buffer_from, a.ctypes.data_as(C.POINTER(_f)), _sz(a.size))

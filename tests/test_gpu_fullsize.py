@@ -50,13 +50,11 @@ def test_reductions_16384_squared_against_oracle(big, orc, deviations):
     exact = X.sum(1, dtype=np.float64)
     got, ref = out_r.numpy(), orc.sum_cols(C, x)
     assert np.all(np.abs(got - exact) <= 1e-6 * abs_r)
-    assert np.all(np.abs(got - ref) <= 1e-6 * abs_r + np.abs(ref - exact))
     deviations("sum_cols [16384x16384]", "max |gpu-oracle| / sum|x|", np.max(np.abs(got.astype(np.float64) - ref) / abs_r), 1e-6)
     c.call("slhip_sum_rows", R, C, d.ptr, out_c.ptr)
     exact = X.sum(0, dtype=np.float64)
     got, ref = out_c.numpy(), orc.sum_rows(C, x)
     assert np.all(np.abs(got - exact) <= 1e-6 * abs_c)
-    assert np.all(np.abs(got - ref) <= 1e-6 * abs_c + np.abs(ref - exact))
     deviations("sum_rows [16384x16384]", "max |gpu-oracle| / sum|x|", np.max(np.abs(got.astype(np.float64) - ref) / abs_c), 1e-6)
     say("mean over 2^28")
     one = c.empty(1)
@@ -156,7 +154,6 @@ def test_softmax_full_size(hip, orc, deviations, shape):
     e = np.exp(shifted)
     exact = (e / e.sum(1, keepdims=True)).ravel()
     assert np.max(np.abs(s - exact) / np.maximum(exact, 1e-300)) <= 1e-6
-    assert np.all(np.abs(s - ref) <= 1e-6 * exact + np.abs(ref - exact))
     assert np.max(np.abs(s.reshape(rows, cols).sum(1, dtype=np.float64) - 1.0)) <= 1e-6
     # the direct deviation from the reference's five-pass f32 result: what remains beyond 1e-6 for long
     # rows is the rounding of the reference's own sequential sum of `cols` exponentials
@@ -172,7 +169,6 @@ def test_softmax_full_size(hip, orc, deviations, shape):
     bound = 1e-6 * (np.abs(S) * (np.abs(G) + (np.abs(S) * np.abs(G)).sum(1, keepdims=True))).ravel() + 1e-37
     assert np.all(np.abs(got - exact_b) <= bound)
     ob = orc.softmax_grad(rows, cols, s, g)
-    assert np.all(np.abs(got - ob) <= bound + np.abs(ob - exact_b))
     # (the oracle's closed form sums <s, g> sequentially in f32 over `cols` terms: again its own rounding)
     deviations(cfg + " grad", "max |gpu-oracle| / (|s|(|g|+sum|s||g|))", np.max(np.abs(got.astype(np.float64) - ob) / (bound * 1e6)), SOFTMAX_GRAD_DIRECT[cols])
     deviations(cfg + " grad", "max |oracle-f64| / same scale (the reference's own)", np.max(np.abs(ob - exact_b) / (bound * 1e6)), SOFTMAX_GRAD_DIRECT[cols])
@@ -204,9 +200,12 @@ def test_gemm_4096_cubed_against_oracle(hip, orc, form):
     rows = rng.integers(64, n, tag=5, seed=SEED)
     scale = (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
     exact = A[rows].astype(np.float64) @ B.astype(np.float64)
-    tol = 1e-5 * np.sqrt(n) * scale
+    # the contract's bar is 1e-5 * sqrt(K) = 6.4e-4 of |A||B|; asserted: 3e-6, a hundredth of what one
+    # product dropped from a dot product would cost
+    tol = 3e-6 * scale
     assert np.all(np.abs(got.reshape(n, n)[rows] - exact) <= tol)
-    assert np.all(np.abs(got - ref) <= 1e-5 * np.sqrt(n) * (n / 4.0) * 0.5)
+    assert np.all(np.abs(got.reshape(n, n)[rows] - ref.reshape(n, n)[rows]) <= tol)
+    assert np.all(np.abs(got - ref) <= 3e-6 * (n / 4.0) * 1.5)
     # linearity: (2A)·B == 2·(A·B) exactly (scaling by two commutes with every rounding)
     c.call("slhip_ew_unary", 6, 2.0, 0.0, n * n, da.ptr, da.ptr)
     c.call("slhip_sgemm", int(ta), int(tb), n, n, n, da.ptr, db.ptr, dc.ptr, 0.0)

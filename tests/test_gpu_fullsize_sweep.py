@@ -47,8 +47,12 @@ def test_gemm_sweep_against_oracle(hip, orc, deviations, form, shape):
     A = a.reshape(k, m).T if ta else a.reshape(m, k)
     B = b.reshape(n, k).T if tb else b.reshape(k, n)
     scale = (np.abs(A) @ np.abs(B)).ravel().astype(np.float64)      # f32 BLAS is plenty for a scale
-    tol = 1e-5 * np.sqrt(k)
-    deviations(name, "max |gpu-oracle| / (|A||B|), bar 1e-5*sqrt(K)", np.max(np.abs(got.astype(np.float64) - ref) / scale), tol)
+    # The contract's bar is 1e-5 * sqrt(K) (3e-4 .. 9e-4 here).  What is asserted is fifty to a
+    # hundred times tighter: f32 accumulation on both sides leaves a few 1e-7 of |A||B|, while one
+    # product dropped from one dot product is worth about 4/K of it (5e-4 .. 5e-3) - a lost k tail
+    # or a missing chunk of a split cannot hide under this ceiling.
+    tol = min(1e-5 * np.sqrt(k), 3e-6)
+    deviations(name, "max |gpu-oracle| / (|A||B|), bar 1e-5*sqrt(K), asserted 3e-6", np.max(np.abs(got.astype(np.float64) - ref) / scale), tol)
     rows = np.unique(np.concatenate([rng.integers(48, m, tag=5, seed=SEED), [0, m - 1]]))
     exact = A[rows].astype(np.float64) @ B.astype(np.float64)
     srow = np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64)

@@ -295,6 +295,56 @@ def test_intermediate_needed_after_its_chain_ran(device):
     device.set_fuse_elementwise(False)
 
 
+@pytest.mark.parametrize("root", ["exp", "clip", "tape off at the root"])
+def test_chain_under_a_root_without_gradient_keeps_the_intermediates_gradient_steps(device, root):
+    """t = a * b feeds u = exp(t) (or clip, or an op issued with the tape off): u carries no gradient,
+    so the fused chain has no closure of its own.  A later reader of t (a product with W) leaves a
+    gradient for t, and t's own gradient step must still carry it on to a and b, as it does op by op."""
+    m, k, n = 24, 16, 8
+    av, bv = rng.uniform(m * k, -1, 1, tag=0, seed=SEED), rng.uniform(m * k, -1, 1, tag=1, seed=SEED)
+    wv = rng.uniform(k * n, -1, 1, tag=2, seed=SEED)
+    res = {}
+    for fuse in (False, True):
+        device.set_fuse_elementwise(fuse)
+        a, b, w = (device.buffer(x) for x in (av, bv, wv))
+        t = device.mul(a, b)
+        if root == "exp":
+            u = device.exp(t)
+        elif root == "clip":
+            u = device.clip(t, -0.5, 0.5)
+        else:
+            device.enable_tape(False)
+            u = device.square(t)
+            device.enable_tape(True)
+        us = u.read()                            # flushes the chain: with fusion on, t stays in registers
+        v = device.gemm(m, k, n, t, w)           # the later reader of t
+        v.backward()
+        res[fuse] = [us, v.read(), t.grad().read(), a.grad().read(), b.grad().read(), w.grad().read()]
+    device.set_fuse_elementwise(False)
+    for got, want in zip(res[True], res[False]):
+        assert np.array_equal(got, want)
+    tg = np.ones((m, n), np.float32) @ wv.reshape(k, n).T
+    assert np.allclose(res[True][3].reshape(m, k), tg * bv.reshape(m, k), rtol=1e-5, atol=1e-6)
+    assert np.abs(res[True][3]).max() > 0
+
+
+def test_release_of_a_chains_input_computes_the_intermediates_that_read_it(device):
+    """t = a + b is kept in registers by the chain t * c; releasing a afterwards must not leave t
+    uncomputable: it is given its value at the release."""
+    n = 300
+    av, bv, cv = (rng.uniform(n, -2, 2, tag=j, seed=SEED) for j in range(3))
+    device.set_fuse_elementwise(True)
+    a, b, c = (device.buffer(x) for x in (av, bv, cv))
+    t = device.add(a, b)
+    u = device.mul(t, c)
+    assert np.array_equal(u.read(), (av + bv) * cv)
+    device.release(a)
+    junk = device.buffer(np.full(n, 99.0, np.float32))   # may take a's memory
+    assert np.array_equal(t.read(), av + bv)
+    assert junk.read()[0] == 99.0
+    device.set_fuse_elementwise(False)
+
+
 def test_fusion_in_a_cached_loop_with_inplace_updates():
     """The sine fit's loss chain (sub, square, sum, scale) in a cached loop with SGD updates in
     between: deferred ops see every update, and the cache hands the same buffers out again."""

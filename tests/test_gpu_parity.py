@@ -506,12 +506,22 @@ def test_reductions(hip, orc, shape):
     assert np.array_equal(hip.max_cols(cols, x), orc.max_cols(cols, x))
     assert np.array_equal(hip.max_rows(cols, x), orc.max_rows(cols, x))
     # sums
+    # sums of small integers have one right answer in f32 whatever the order: the oracle's bits
+    xi = (rng.integers(rows * cols, 17, tag=9, seed=SEED + rows) - 8).astype(np.float32)
+    for name in ("sum_cols", "sum_rows", "mean_cols", "mean_rows"):
+        assert np.array_equal(getattr(hip, name)(cols, xi), getattr(orc, name)(cols, xi)), name
+    # sums of the U(-10, 10) data: within 1e-6 of sum|x| of the exact sum, and of the oracle's
+    # sequential f32 sum directly where that sum is short enough to be that accurate itself
     got, ref = hip.sum_cols(cols, x), orc.sum_cols(cols, x)
     b = sum_bound(x, rows, cols, 1)
-    assert np.all(np.abs(got - x64.sum(1)) <= b) and np.all(np.abs(got - ref) <= 2 * b + np.abs(ref - x64.sum(1)))
+    assert np.all(np.abs(got - x64.sum(1)) <= b)
+    if cols <= 64:
+        assert np.all(np.abs(got - ref) <= b)
     got, ref = hip.sum_rows(cols, x), orc.sum_rows(cols, x)
     b = sum_bound(x, rows, cols, 0)
-    assert np.all(np.abs(got - x64.sum(0)) <= b) and np.all(np.abs(got - ref) <= 2 * b + np.abs(ref - x64.sum(0)))
+    assert np.all(np.abs(got - x64.sum(0)) <= b)
+    if rows <= 64:
+        assert np.all(np.abs(got - ref) <= b)
     # means
     got = hip.mean_cols(cols, x)
     assert np.all(np.abs(got - x64.mean(1)) <= sum_bound(x, rows, cols, 1) / cols + 1e-7 * np.abs(x64.mean(1)))
@@ -604,8 +614,8 @@ def test_softmax_forward_backward(hip, orc, shape):
     got, ref = hip.softmax(rows, cols, x), orc.softmax(rows, cols, x)
     rel = np.abs(got - exact) / np.maximum(np.abs(exact), 1e-30)
     assert rel.max() <= 1e-6, rel.max()
-    ref_off = np.abs(ref - exact)
-    assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(exact) + ref_off + 1e-37)
+    if cols <= 64:     # the oracle's sequential sum of a short row is itself accurate: the direct bar
+        assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + 1e-37), np.max(np.abs(got - ref) / np.maximum(ref, 1e-37))
     assert np.all(np.abs(got.reshape(rows, cols).astype(np.float64).sum(1) - 1.0) <= 1e-6)
     # backward on the device's own forward output, SET and accumulate
     s64 = got.reshape(rows, cols).astype(np.float64)
@@ -617,7 +627,8 @@ def test_softmax_forward_backward(hip, orc, shape):
     gb = hip.softmax_grad(rows, cols, got, g)
     ob = orc.softmax_grad(rows, cols, got, g)
     assert np.all(np.abs(gb - exact_b) <= bound), np.max(np.abs(gb - exact_b) / bound)
-    assert np.all(np.abs(gb - ob) <= bound + np.abs(ob - exact_b))
+    if cols <= 64:
+        assert np.all(np.abs(gb - ob) <= bound), np.max(np.abs(gb - ob) / bound)
     base = rng.normal(rows * cols, 1.0, tag=2, seed=SEED)
     gacc = hip.softmax_grad(rows, cols, got, g, x_grad=base.copy(), beta=1.0)
     assert np.all(np.abs(gacc - (base + exact_b)) <= bound + 1e-6 * np.abs(base))
@@ -780,7 +791,8 @@ def test_broadcast_ops_with_op_code(hip, orc, shape, kind):
         bound = 1e-6 * (np.abs(dr).sum(axis) + np.abs(vg0)) + 1e-30
         exact = vg0 + dr.sum(axis)
         assert np.all(np.abs(vg_h - exact) <= bound + 1e-6 * np.abs(exact))
-        assert np.all(np.abs(vg_h - vg_o) <= bound + np.abs(vg_o - exact))
+        if (cols if kind == "col_op" else rows) <= 64:      # short sums: the oracle's own rounding is below the bar
+            assert np.all(np.abs(vg_h - vg_o) <= bound + 1e-6 * np.abs(exact))
         # one side only
         lg1, _ = getattr(hip, kind + "_grad")(op, cols, lhs, v, lg0.copy(), None, g)
         assert np.array_equal(lg1, lg_o)
@@ -794,7 +806,7 @@ def test_tanh_sigmoid_diagflat_onehot_grad(hip, orc):
                       (orc.SIGMOID, lambda v: 1 / (1 + np.exp(-v)), lambda v: np.exp(-v) / (1 + np.exp(-v)) ** 2)]:
         got, ref = hip.unary(op, x), orc.unary(op, x)
         assert np.all(np.abs(got - f(x64)) <= 1e-6 * np.abs(f(x64)) + 1e-37)
-        assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + np.abs(ref - f(x64)) + 1e-37)
+        assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + 1e-37), np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-37))
         xg0 = rng.uniform(x.size, -1, 1, tag=2, seed=SEED)
         gg, gr = hip.unary_grad(op, x, xg0.copy(), g), orc.unary_grad(op, x, xg0.copy(), g)
         exact = xg0 + df(x64) * g
@@ -802,7 +814,7 @@ def test_tanh_sigmoid_diagflat_onehot_grad(hip, orc):
         # error of a few ulp(1) there, whoever evaluates it
         bound = (3e-7 + 2e-6 * np.abs(df(x64))) * np.abs(g) + 2e-6 * np.abs(xg0) + 1e-37
         assert np.all(np.abs(gg - exact) <= bound)
-        assert np.all(np.abs(gg - gr) <= bound + np.abs(gr - exact))
+        assert np.all(np.abs(gg - gr) <= bound), np.max(np.abs(gg - gr) / bound)
     v = rng.uniform(300, -1, 1, tag=3, seed=SEED)
     assert np.array_equal(hip.diagflat(v), orc.diagflat(v))
     og = rng.normal(300 * 300, 1.0, tag=4, seed=SEED)
@@ -826,7 +838,8 @@ def test_fused_mse_against_the_op_chain(hip, orc, n):
     exact = np.sum(d.astype(np.float64) ** 2) / n
     got = hip.mse(x, y)
     assert abs(got - exact) <= 1e-6 * exact + 1e-37
-    assert abs(got - ref) <= 1e-6 * exact + abs(ref - exact)
+    if n <= 4099:      # the oracle's sequential sum of a few thousand squares is within the bar itself
+        assert abs(got - ref) <= 1e-6 * exact + 1e-37, abs(got - ref) / exact
     xg0 = rng.uniform(n, -1, 1, tag=2, seed=SEED)
     for up in (1.0, -0.25):
         gs, _ = orc.binary_ew_grad(orc.MUL, np.zeros(1, np.float32), c, np.zeros(1, np.float32), np.zeros(1, np.float32),
@@ -857,7 +870,8 @@ def test_fused_softmax_cross_entropy_against_the_op_chain(hip, orc, shape):
     assert np.all(np.abs(p.reshape(rows, cols) - P) <= 1e-6 * P + 1e-37)
     L = -np.log(np.sum(np.clip(P, 1e-7, 1 - 1e-7) * t.reshape(rows, cols), 1))
     assert np.all(np.abs(loss - L) <= 2e-6 * np.maximum(np.abs(L), 1.0))
-    assert np.all(np.abs(loss - loss_ref) <= 2e-6 * np.maximum(np.abs(L), 1.0) + np.abs(loss_ref - L))
+    if cols <= 64:     # the oracle's probabilities come from short sequential sums: the direct bar
+        assert np.all(np.abs(loss - loss_ref) <= 2e-6 * np.maximum(np.abs(L), 1.0)), np.max(np.abs(loss - loss_ref))
     # without a buffer for the probabilities: the same losses
     none, loss_only = hip.softmax_cce(rows, cols, x, t, want_probs=False)
     assert none is None and np.all(np.abs(loss_only - loss) <= 2e-6 * np.maximum(np.abs(L), 1.0))
@@ -875,7 +889,8 @@ def test_fused_softmax_cross_entropy_against_the_op_chain(hip, orc, shape):
         got = hip.softmax_cce_grad(rows, cols, p, t, np.zeros(n, np.float32))
         exact = (P - t.reshape(rows, cols)).ravel() / rows
         scale = (np.abs(P) + 1.0).ravel() / rows
-        assert np.all(np.abs(got - chain) <= 4e-6 * scale + np.abs(chain - exact))
+        if cols <= 64:
+            assert np.all(np.abs(got - chain) <= 4e-6 * scale), np.max(np.abs(got - chain) / scale)
 
 
 def test_sgd_step_for_a_parameter_list_is_bit_exact(hip, orc):

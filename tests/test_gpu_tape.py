@@ -493,6 +493,46 @@ def test_failed_backward_leaves_no_tape_behind(device):
     eq(d.grad(), [1, 2, 3])
 
 
+def test_repeated_backward_with_manual_descent(device, orc):
+    """tests/test_combination.rs:5-23: a hundred times square(x) -> backward -> x.grad *= 0.1 ->
+    x -= x.grad -> clear the gradient.  Every step against the oracle's unary op and gradient, bit
+    for bit; the sum of squares falls by 0.8^2 a step."""
+    xv = np.array([10, -10, 10, -5, 6, 3, 1], np.float32)
+    x = device.buffer(xv)
+    ref = xv.copy()
+    sums = []
+    for i in range(100):
+        squared = device.square(x)
+        sq_ref = orc.unary(orc.SQUARE, ref)
+        assert np.array_equal(squared.read(), sq_ref), i
+        sums.append(float(sq_ref.sum()))
+        squared.backward()
+        g_ref = orc.unary_grad(orc.SQUARE, ref, np.zeros_like(ref), np.ones_like(ref))
+        assert np.array_equal(x.grad().read(), g_ref), i
+        device.sgd_step(x, 0.1)                  # x -= x.grad * 0.1: the two assign loops of the test
+        ref = orc.sgd_step(ref, g_ref, 0.1)
+        assert np.array_equal(x.read(), ref), i
+        device.zero_grad()                       # x_grad.clear()
+        eq(x.grad(), np.zeros(7))
+        assert device.tape_len() == 0
+    assert all(b < a for a, b in zip(sums, sums[1:]))
+    assert abs(sums[-1] / sums[0] - 0.64 ** 99) < 1e-5 * 0.64 ** 99 * 100
+
+
+def test_matrix_rand_fills_from_the_seeded_stream(device):
+    """Matrix::rand(lo, hi) (src/matrix.rs:266-271): in range, and the very numbers the host-side
+    generator gives for the same seed and tag."""
+    from sliced_amd import host
+    rows, cols = 37, 53
+    b = device.zeros(rows * cols)
+    device.matrix_rand(b, rows, cols, -0.25, 0.75, tag=5)
+    got = b.read()
+    assert got.min() >= -0.25 and got.max() < 0.75 and len(np.unique(got)) > rows * cols // 2
+    assert np.array_equal(got, rng.uniform(rows * cols, -0.25, 0.75, tag=5))
+    with pytest.raises(host.HostError):
+        device.matrix_rand(b, rows, cols + 1, 0.0, 1.0)   # the view's length assert (src/matrix/impl_from.rs:7-10)
+
+
 # --------------------------------------------------------------------------- training loops
 def loss_parity(got, ref, tol):
     rel = np.abs(got - ref) / np.maximum(np.abs(ref), 1e-30)

@@ -52,6 +52,65 @@ def test_two_calls_in_a_row_second_smaller(hip):
         b.free()
 
 
+def test_static_variant_neither_uses_the_workspace_nor_allocates(hip):
+    """The context workspace, where slhip_sum_rows keeps its partials, is filled with NaN before the
+    call: a result that still has the bits of slhip_sum_rows did not pass through it.  Free device
+    memory is the same before and after the calls."""
+    import torch
+    c = hip.ctx()
+    rows, cols = 16384, 2049                    # two streaming stages: partials must live somewhere
+    x = rng.uniform(rows * cols, -10, 10, tag=30, seed=SEED)
+    want = hip.sum_rows(cols, x)
+    dx, out = c.array(x), c.empty(cols)
+    ws = C.c_void_p()
+    c.call("slhip_workspace", C.byref(ws))
+    ws_floats = c.lib.slhip_workspace_bytes(c.h) // 4
+    assert ws.value and ws_floats >= (1 << 20)
+    c.call("slhip_fill", ws_floats, float("nan"), ws.value)
+    c.sync()
+    torch.cuda.mem_get_info(0)                  # the first query sets the runtime's own bookkeeping up
+    free0 = torch.cuda.mem_get_info(0)[0]
+    for _ in range(3):
+        c.call("slhip_sum_rows_static", rows, cols, dx.ptr, out.ptr)
+    c.sync()
+    assert torch.cuda.mem_get_info(0)[0] == free0
+    got = out.numpy()
+    assert not np.isnan(got).any() and np.array_equal(got, want)
+    # the control: the workspace variant does read what the poisoned workspace holds only after
+    # writing it, so it is still right - and leaves the NaNs overwritten
+    assert np.array_equal(hip.sum_rows(cols, x), want)
+    dx.free()
+    out.free()
+
+
+def test_static_variant_inside_a_recorded_sequence(hip):
+    """The setting the entry point is for: between slhip_graph_begin and slhip_graph_end nothing may
+    allocate.  The recording is replayed three times with eager work and waits in between; every
+    replay gives the bits of the eager call."""
+    c = hip.ctx()
+    rows, cols = 8192, 1000
+    x = rng.uniform(rows * cols, -10, 10, tag=31, seed=SEED)
+    want = hip.sum_rows(cols, x)
+    dx, out = c.array(x), c.empty(cols)
+    c.call("slhip_graph_begin")
+    try:
+        c.call("slhip_sum_rows_static", rows, cols, dx.ptr, out.ptr)
+    finally:
+        g = C.c_void_p()
+        c.call("slhip_graph_end", C.byref(g))
+    for replay in range(3):
+        say("replay", replay)
+        c.call("slhip_fill", cols, -1.0, out.ptr)
+        c.sync()
+        c.call("slhip_graph_launch", g)
+        assert np.array_equal(out.numpy(), want), replay
+        other = rng.uniform(64 * 300, -1, 1, tag=40 + replay, seed=SEED)
+        hip.sum_rows_static(300, other)              # an eager call shares the array between replays
+    c.lib.slhip_graph_destroy(g)
+    dx.free()
+    out.free()
+
+
 def test_static_variant_rejects_what_does_not_fit(hip):
     c = hip.ctx()
     x = c.zeros(2 * 131076)
