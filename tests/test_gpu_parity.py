@@ -838,7 +838,7 @@ def test_fused_mse_against_the_op_chain(hip, orc, n):
     exact = np.sum(d.astype(np.float64) ** 2) / n
     got = hip.mse(x, y)
     assert abs(got - exact) <= 1e-6 * exact + 1e-37
-    if n <= 4099:      # the oracle's sequential sum of a few thousand squares is within the bar itself
+    if n <= 1024:      # the oracle's sequential sum of a thousand squares is within the bar itself (of 4099: 1.3e-6 off)
         assert abs(got - ref) <= 1e-6 * exact + 1e-37, abs(got - ref) / exact
     xg0 = rng.uniform(n, -1, 1, tag=2, seed=SEED)
     for up in (1.0, -0.25):
