@@ -653,7 +653,11 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (3000, 41), (3, 3), (40, 40), (17, 23),
              # the limits of the narrow kernels (56 columns in, 200 rows out) and what lies just beyond
              (5000, 56), (5001, 57), (200, 3001), (201, 3000), (224, 3001), (100, 8193), (128, 5000), (200, 41), (56, 57), (57, 56),
-             (163, 9000), (9000, 55)]
+             (163, 9000), (9000, 55),
+             # the 64 x 256 tile: tall matrices of 256 columns and more, whole tiles and ragged edges, and wide
+             # ones of 64 / 128 / 192 rows; 128 KiB chunks: inputs of 57..128 columns off the 64-grid
+             (2048, 512), (1100, 260), (4100, 257), (8200, 1023), (1025, 256), (64, 5000), (128, 1024), (192, 777), (64, 256),
+             (128, 513), (2000, 100), (1700, 65), (3000, 127), (1600, 100), (2049, 128), (1919, 119), (330, 100)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
