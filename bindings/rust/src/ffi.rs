@@ -373,6 +373,9 @@ extern "C" {
         out_grad: *const f32,
     ) -> i32;
     pub fn slhip_sgd_step(ctx: *mut SlhipCtx, n: usize, p: *mut f32, g: *const f32, lr: f32) -> i32;
+    pub fn slhip_mlp3_mse_step(ctx: *mut SlhipCtx, batch: usize, d_in: usize, d_h: usize, d_out: usize, x: *const f32,
+                               target: *const f32, w1: *mut f32, b1: *mut f32, w2: *mut f32, b2: *mut f32, w3: *mut f32, b3: *mut f32,
+                               grads: *const *mut f32, lr: f32, loss_dev: *mut f32) -> i32;
     pub fn slhip_sgd_step_multi(
         ctx: *mut SlhipCtx,
         count: usize,

@@ -375,6 +375,19 @@ int32_t slhip_softmax_cce(slhip_ctx* ctx, size_t rows, size_t cols, const float*
                           float* probs, float* loss_rows /*rows*/);
 int32_t slhip_softmax_cce_grad(slhip_ctx* ctx, size_t rows, size_t cols, const float* probs, const float* targets,
                                float* logits_grad, float beta, const float* upstream_dev /*1*/);
+/* One whole training step of the sine-fit loop (examples/sine_net.rs:119-166) in two launches:
+ * x[batch×d_in] → Linear(d_in,d_h) → ReLU → Linear(d_h,d_h) → ReLU → Linear(d_h,d_out) (Linear = gemm +
+ * add_row_mut, :32-40; Matrix::relu, src/matrix.rs:169-190), loss_dev[0] = (Σ (out − target)²)·1/(batch·d_out)
+ * (the loss tape sub, squared, sum, scale of :150-156), backward with seed one, and SGD
+ * `value -= grad * lr` (:105-116) on all six parameter tensors in place.  grads (may be NULL) names
+ * six device arrays W1,b1,W2,b2,W3,b3-shaped that receive the step's gradients (SET), for callers
+ * that keep gradient buffers.  d_h ≤ 64, d_in ≤ 8 and d_out ≤ 8 (larger layers: the ops one by one);
+ * the per-row intermediates live in the context workspace (272 floats per row).  Same values as the
+ * op sequence up to rounding (fused multiply-adds, tree sums over the hidden units); every sum has
+ * a fixed order, so a step is reproducible bit for bit. */
+int32_t slhip_mlp3_mse_step(slhip_ctx* ctx, size_t batch, size_t d_in, size_t d_h, size_t d_out, const float* x,
+                            const float* target, float* w1, float* b1, float* w2, float* b2, float* w3, float* b3,
+                            float* const* grads, float lr, float* loss_dev /*1*/);
 /* onehot_grad (src/ops2/onehot/grad/cpu.rs:3-12): cls_grad[r] += out_grad[r*classes + cls[r]]. */
 int32_t slhip_onehot_grad(slhip_ctx* ctx, size_t n, size_t classes, const float* cls, float* cls_grad,
                           const float* out_grad);

@@ -95,6 +95,7 @@ PROTOTYPES = {
     "slhip_mse_grad": [c_vp, c_sz, c_vp, c_vp, c_vp, c_vp],
     "slhip_softmax_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp],
     "slhip_softmax_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp, C.c_float, c_vp],
+    "slhip_mlp3_mse_step": [c_vp, c_sz, c_sz, c_sz, c_sz, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, C.c_float, c_vp],
     "slhip_sgd_step_multi": [c_vp, c_sz, c_vp, c_vp, c_vp, C.c_float],
     "slhip_cce": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],
     "slhip_cce_grad": [c_vp, c_sz, c_sz, c_vp, c_vp, c_vp],

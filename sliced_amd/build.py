@@ -20,7 +20,7 @@ LIB_HIP = os.path.join(HERE, "libsliced_hip.so")
 LIB_HOST = os.path.join(HERE, "libsliced_host.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-KERNEL_SOURCES = ["runtime.hip", "elementwise.hip", "ew_program.hip", "reduce.hip", "softmax.hip", "transpose.hip", "gemm.hip", "gemm_spread.hip", "gemm_wide.hip", "gemm_skinny.hip", "gemm_tall.hip", "gemm_bits.hip", "bcast_ops.hip", "loss.hip"]
+KERNEL_SOURCES = ["runtime.hip", "elementwise.hip", "ew_program.hip", "reduce.hip", "softmax.hip", "transpose.hip", "gemm.hip", "gemm_spread.hip", "gemm_wide.hip", "gemm_skinny.hip", "gemm_tall.hip", "gemm_bits.hip", "bcast_ops.hip", "loss.hip", "mlp_step.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",

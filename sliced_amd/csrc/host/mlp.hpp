@@ -58,7 +58,8 @@ struct MlpResult {
 enum MlpMode {
   MLP_FUSED = 1,  // Linear (+ReLU) forward as one kernel, ReLU gradient inside the next layer's input-gradient GEMM
   MLP_GRAPH = 2,  // step 0 runs eagerly, step 1 is recorded, every later step replays the recording
-  MLP_FUSED_LOSS = 4  // the loss chain (MSE, or softmax + cross-entropy) as one forward and one backward kernel
+  MLP_FUSED_LOSS = 4,  // the loss chain (MSE, or softmax + cross-entropy) as one forward and one backward kernel
+  MLP_WHOLE_STEP = 8   // kind 0 with at most 64 hidden units: the whole step as two launches (HIP::mlp3_mse_step)
 };
 
 // kind 0: MSE on the tape (sub, square, sum_cols, mul by 1/n; seed 1).
@@ -143,6 +144,30 @@ inline MlpResult mlp_train(HIP& dev, int kind, size_t batch, size_t d_in, size_t
   MlpResult res;
   Graph recorded;
   std::chrono::steady_clock::time_point t0;
+  if (mode & MLP_WHOLE_STEP) {
+    if (kind != 0) throw Error("the whole-step kernels serve the MSE loop only");
+    const std::vector<Buffer> ps{lin1.weights.data, lin1.bias.data, lin2.weights.data, lin2.bias.data, lin3.weights.data, lin3.bias.data};
+    Buffer log = dev.alloc(warmup + steps, true);
+    for (size_t it = 0; it < warmup + steps; ++it) {
+      if (it == warmup) {
+        dev.sync();
+        t0 = std::chrono::steady_clock::now();
+      }
+      dev.mlp3_mse_step(batch, d_in, d_h, d_out, x.data, y.data, ps, lr, log, it);  // the loss of step `it` lands in log[it]
+    }
+    dev.sync();
+    res.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    res.graph_nodes = 2;
+    std::vector<float> all = log.read();
+    for (size_t i = 0; i < steps; ++i) losses[i] = all[warmup + i];
+    const Linear* ls[3] = {&lin1, &lin2, &lin3};
+    for (int i = 0; i < 3; ++i) {
+      std::vector<float> w = ls[i]->weights.read(), b = ls[i]->bias.read();
+      for (size_t j = 0; j < w.size(); ++j) params[2 * i][j] = w[j];
+      for (size_t j = 0; j < b.size(); ++j) params[2 * i + 1][j] = b[j];
+    }
+    return res;
+  }
   for (size_t it : dev.range(warmup + steps)) {
     if (it == warmup) {
       dev.sync();

@@ -756,6 +756,30 @@ class HIP {
     check(slhip_memcpy_d2d(ctx_, dst.ptr + dst_off, src.ptr + src_off, n * sizeof(float)), "slhip_memcpy_d2d");
   }
 
+  // One whole training step of the sine-fit loop (examples/sine_net.rs:119-166) as two launches:
+  // forward through three Linear layers with ReLU between them, the MSE loss into loss[loss_at],
+  // backward, and SGD on the six parameter buffers (W1, b1, W2, b2, W3, b3) in place.  Nothing goes
+  // on the tape; the parameters' gradient buffers receive this step's gradients (overwritten), so
+  // `.grad()` reads what the op-by-op step would have left there.
+  void mlp3_mse_step(size_t batch, size_t d_in, size_t d_h, size_t d_out, const Buffer& x, const Buffer& y,
+                     const std::vector<Buffer>& params, float lr, const Buffer& loss, size_t loss_at = 0) {
+    if (params.size() != 6) throw Error("mlp3_mse_step: six parameter buffers expected");
+    expect(x, batch * d_in, "mlp3_mse_step x"); expect(y, batch * d_out, "mlp3_mse_step y");
+    const size_t lens[6] = {d_in * d_h, d_h, d_h * d_h, d_h, d_h * d_out, d_out};
+    if (loss_at >= loss.len) throw Error("mlp3_mse_step: loss slot outside the buffer");
+    run();
+    ready(x); ready(y); ready(loss);
+    float* g[6];
+    for (int i = 0; i < 6; ++i) {
+      expect(params[i], lens[i], "mlp3_mse_step parameter");
+      ready(params[i]);
+      g[i] = grad_out(params[i], true).ptr;
+    }
+    check(slhip_mlp3_mse_step(ctx_, batch, d_in, d_h, d_out, x.ptr, y.ptr, params[0].ptr, params[1].ptr, params[2].ptr,
+                              params[3].ptr, params[4].ptr, params[5].ptr, g, lr, loss.ptr + loss_at),
+          "slhip_mlp3_mse_step");
+  }
+
   // RandOp::rand (src/rawops/cpu/rand.rs:7-12) on the device: x[i] = lo + (hi - lo) * u_i
   void rand(const Buffer& x, float lo, float hi, uint64_t seed, uint64_t tag) {
     ready(x);

@@ -321,9 +321,10 @@ def mlp_data(kind, batch, d_in, d_out, seed=rng.DEFAULT_SEED):
 
 
 def mlp_train(kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmup=0, fused=False, ordinal=0,
-              graph=False, info=None, fused_loss=False):
+              graph=False, info=None, fused_loss=False, whole_step=False):
     """Runs the C++ training loop on the GPU.  params (six float32 arrays) are updated in place.
     graph=True records one step as a HIP graph and replays it (losses are read once at the end).
+    whole_step=True (the MSE loop with at most 64 hidden units) runs every step as two launches.
     Returns (losses[steps], seconds for the timed steps); info, a dict, receives graph_nodes."""
     losses = np.zeros(steps, np.float32)
     secs = C.c_double()
@@ -332,7 +333,7 @@ def mlp_train(kind, batch, d_in, d_h, d_out, x, target, params, lr, steps, warmu
     x = np.ascontiguousarray(x, np.float32)
     target = np.ascontiguousarray(target, np.float32)
     _ck(lib().slh_mlp_train(ordinal, int(kind), _sz(batch), _sz(d_in), _sz(d_h), _sz(d_out), p(x), p(target),
-                            *[p(a) for a in params], _f(lr), _sz(steps), _sz(warmup), int(bool(fused)) | (2 if graph else 0) | (4 if fused_loss else 0),
+                            *[p(a) for a in params], _f(lr), _sz(steps), _sz(warmup), int(bool(fused)) | (2 if graph else 0) | (4 if fused_loss else 0) | (8 if whole_step else 0),
                             p(losses), C.byref(secs), C.byref(nodes)))
     if info is not None:
         info["graph_nodes"] = nodes.value
@@ -402,12 +403,12 @@ C1 = dict(kind=0, batch=1024, d_in=1, d_h=64, d_out=1, lr=0.01, steps=200)
 C5 = dict(kind=1, batch=8192, d_in=784, d_h=2048, d_out=10, lr=0.05, steps=50)
 
 
-def run_config(cfg, fused, warmup=0, steps=None, graph=False, info=None, fused_loss=False):
+def run_config(cfg, fused, warmup=0, steps=None, graph=False, info=None, fused_loss=False, whole_step=False):
     steps = steps or cfg["steps"]
     x, t = mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
     params = mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
     losses, secs = mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, params,
-                             cfg["lr"], steps, warmup, fused, graph=graph, info=info, fused_loss=fused_loss)
+                             cfg["lr"], steps, warmup, fused, graph=graph, info=info, fused_loss=fused_loss, whole_step=whole_step)
     return losses, secs, params
 
 
@@ -429,6 +430,11 @@ def bench_mlp(steps_c5=50, steps_c1=200, graph=True):
                 "first_loss": float(losses[0]), "last_loss": float(losses[-1])}
             if graph_variant:
                 out["%s (%s)" % (name, label)]["kernels_per_step"] = info["graph_nodes"]
+    info = {}
+    losses, secs, _ = run_config(C1, True, warmup=5, steps=steps_c1, info=info, whole_step=True)
+    out["C1 sine fit 1-64-64-1 batch 1024 (whole step in two launches)"] = {
+        "steps_per_s": steps_c1 / secs, "ms_per_step": 1e3 * secs / steps_c1, "first_loss": float(losses[0]),
+        "last_loss": float(losses[-1]), "kernels_per_step": info["graph_nodes"]}
     flop_c5 = 259.8e9
     k = "C5 classifier 784-2048-2048-10 batch 8192 (fused linear)"
     out["C5_fused_TFLOPs"] = flop_c5 * out[k]["steps_per_s"] / 1e12

@@ -3,6 +3,8 @@ trait method (same names and argument meaning as the CPU oracle's front-end), so
 parity test is the same call on both sides.  Every call uploads its operands, runs the HIP
 kernels and downloads the result; nothing is computed on the host.
 """
+import ctypes as C
+
 import numpy as np
 
 from .device import Context
@@ -495,6 +497,20 @@ def diagflat_grad(x_grad, out_grad):
         s.c.call("slhip_diagflat_grad", x_grad.size, dx.ptr, dg.ptr)
         x_grad[:] = dx.numpy()
     return x_grad
+
+
+def mlp3_mse_step(batch, d_in, d_h, d_out, x, target, params, lr, with_grads=True):
+    """slhip_mlp3_mse_step on host arrays: params (W1, b1, W2, b2, W3, b3) are updated in place;
+    returns (loss, the six gradients or None)."""
+    with _Scope() as s:
+        dx, dt, dl = s.up(x), s.up(target), s.empty(1)
+        dp = [s.up(p) for p in params]
+        dg = [s.empty(p.size) for p in params] if with_grads else None
+        garr = (C.c_void_p * 6)(*[g.ptr for g in dg]) if with_grads else None
+        s.c.call("slhip_mlp3_mse_step", batch, d_in, d_h, d_out, dx.ptr, dt.ptr, *[p.ptr for p in dp], garr, float(lr), dl.ptr)
+        for host, dev in zip(params, dp):
+            host[:] = dev.numpy().reshape(host.shape)
+        return dl.numpy()[0], ([g.numpy() for g in dg] if with_grads else None)
 
 
 def mse(x, y):

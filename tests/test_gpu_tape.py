@@ -539,6 +539,76 @@ def loss_parity(got, ref, tol):
     return rel.max()
 
 
+def test_whole_step_kernels_train_the_sine_fit_like_the_oracle(orc):
+    """Config 1 with every step as two launches (slhip_mlp3_mse_step): per-step loss within 1e-4
+    relative of the oracle's loop over all 200 steps, the trained parameters beside the oracle's, and
+    a second run bit-identical to the first."""
+    from sliced_amd import host
+    cfg = host.C1
+    x, t = host.mlp_data(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_out"])
+    p_ref = host.mlp_init(cfg["kind"], cfg["d_in"], cfg["d_h"], cfg["d_out"])
+    runs = []
+    for _ in range(2):
+        p_gpu = [a.copy() for a in p_ref]
+        got, _ = host.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_gpu, cfg["lr"],
+                                cfg["steps"], 0, True, whole_step=True)
+        runs.append((got, p_gpu))
+    ref = orc.mlp_train(cfg["kind"], cfg["batch"], cfg["d_in"], cfg["d_h"], cfg["d_out"], x, t, p_ref, cfg["lr"], cfg["steps"])
+    got, p_gpu = runs[0]
+    worst = loss_parity(got, ref, 1e-4)
+    say("C1 whole-step worst relative loss deviation", worst, "loss", ref[0], "->", ref[-1], "gpu", got[0], "->", got[-1])
+    assert worst <= 1e-4
+    for a, b in zip(p_gpu, p_ref):
+        assert np.max(np.abs(a - b)) <= 1e-4 * max(1.0, np.max(np.abs(b)))
+    assert np.array_equal(runs[0][0], runs[1][0])
+    for a, b in zip(runs[0][1], runs[1][1]):
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dims", [(1024, 1, 64, 1), (37, 3, 50, 2), (1, 8, 64, 8), (4099, 2, 7, 3), (256, 1, 1, 1), (9, 5, 33, 1)],
+                         ids=lambda d: "-".join(map(str, d)))
+def test_whole_step_against_the_oracles_step(hip, orc, dims):
+    """One and three steps of slhip_mlp3_mse_step on odd sizes (fewer hidden units than lanes, several
+    inputs and outputs, batches that are no multiple of 4 or 8) against the oracle's training loop:
+    the loss, the updated parameters, and the gradients as (old - new) / lr says they must be."""
+    batch, d_in, d_h, d_out = dims
+    x = rng.uniform(batch * d_in, -2, 2, tag=0)
+    t = rng.uniform(batch * d_out, -1, 1, tag=1)
+    shapes = [d_in * d_h, d_h, d_h * d_h, d_h, d_h * d_out, d_out]
+    p0 = [rng.uniform(n, -0.25, 0.25, tag=10 + i) for i, n in enumerate(shapes)]
+    lr = 0.02
+    p_ref = [a.copy() for a in p0]
+    ref_losses = orc.mlp_train(0, batch, d_in, d_h, d_out, x, t, p_ref, lr, 3)
+    p_gpu = [a.copy() for a in p0]
+    for step in range(3):
+        before = [a.copy() for a in p_gpu]
+        loss, grads = hip.mlp3_mse_step(batch, d_in, d_h, d_out, x, t, p_gpu, lr)
+        # (the first step sees identical parameters; later ones the two sides' own, a rounding apart)
+        assert abs(loss - ref_losses[step]) <= (2e-6 if step == 0 else 1e-5) * abs(ref_losses[step]) + 1e-30, (step, loss, ref_losses[step])
+        for b, a, g in zip(before, p_gpu, grads):
+            assert np.array_equal(a, b - g * np.float32(lr))       # value -= grad * lr, the gradient handed out
+    for a, b, n in zip(p_gpu, p_ref, ("W1", "b1", "W2", "b2", "W3", "b3")):
+        assert np.max(np.abs(a - b)) <= 5e-6 * max(1.0, np.max(np.abs(b))), n
+    # without gradient buffers: the same parameters
+    p_again = [a.copy() for a in p0]
+    for step in range(3):
+        hip.mlp3_mse_step(batch, d_in, d_h, d_out, x, t, p_again, lr, with_grads=False)
+    for a, b in zip(p_again, p_gpu):
+        assert np.array_equal(a, b)
+
+
+def test_whole_step_refuses_layers_it_does_not_serve(hip):
+    c = hip.ctx()
+    z = c.zeros(1 << 16)
+    args = lambda d_in, d_h, d_out: (4, d_in, d_h, d_out, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, None, 0.1, z.ptr)
+    assert c.lib.slhip_mlp3_mse_step(c.h, *args(1, 65, 1)) == -1
+    assert b"64 hidden units" in c.lib.slhip_last_error_string()
+    assert c.lib.slhip_mlp3_mse_step(c.h, *args(9, 64, 1)) == -1
+    assert c.lib.slhip_mlp3_mse_step(c.h, *args(1, 64, 9)) == -1
+    assert c.lib.slhip_mlp3_mse_step(c.h, 0, 1, 64, 1, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, z.ptr, None, 0.1, z.ptr) == -1
+    z.free()
+
+
 @pytest.mark.parametrize("fused", [False, True], ids=["op-by-op", "fused-linear"])
 def test_sine_mlp_loss_curve_matches_oracle(orc, fused):
     """Config 1: batch 1024, 1-64-64-1, MSE, SGD lr 0.01, 200 steps; per-step loss within 1e-4 rel."""
