@@ -92,6 +92,12 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
   if (VEC_ST) {
     constexpr int LPR = TR / 4, RPP = 256 / LPR, NP = TC / RPP;  // float4 per output row of the tile, output rows per pass
     const int lx = t % LPR, ly = t / LPR;
+    // Sixteen lanes cover an output row of the 64-row tile, so a wave reads four columns of the tile at
+    // a time.  Side by side they share LDS banks four ways; sixteen apart they do not, which pays when
+    // the output rows are short and lie close together anyway ([128 x 2^20] 5.74 -> 5.95 TB/s) and costs
+    // when they are long: the wave's four stores then land 16 output rows apart ([32768 x 4096],
+    // output rows of 128 KiB: 5.63 -> 5.40)
+    const bool spread = TR == 64 && rows <= 512;
     const size_t orow0 = r0 + 4 * lx;
     // `+=`: all reads of the old output before the first store (a read after a store to what may be
     // the same memory waits for that store)
@@ -99,13 +105,13 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
     if (ACC) {
 #pragma unroll
       for (int p = 0; p < NP; ++p) {
-        const size_t oc = c0 + ly + RPP * p;
+        const size_t oc = c0 + (spread ? ly * NP + p : ly + RPP * p);
         old[p] = (oc < cols && orow0 + 3 < rows) ? ld4s(out + oc * rows + orow0) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-      const int cc = ly + RPP * p;  // input column = output row
+      const int cc = spread ? ly * NP + p : ly + RPP * p;  // input column = output row
       const size_t oc = c0 + cc;
       if (oc < cols && orow0 < rows) {
         float4 v = make_float4(tile(4 * lx + 0, cc), tile(4 * lx + 1, cc), tile(4 * lx + 2, cc), tile(4 * lx + 3, cc));
