@@ -150,93 +150,132 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 // CHUNK floats per workgroup of NTH threads.  64 KiB chunks on 512 threads serve narrow inputs up
 // to 56 columns and narrow outputs up to 200 rows (against 32 KiB the runs on the wide side are twice
 // as long: narrow inputs of 10..56 columns gain 5-11 %, narrow outputs of 100..200 rows 5-11 %);
-// 128 KiB chunks on 1024 threads, one workgroup to a CU, serve inputs of 57..128 columns that are not
-// a multiple of 64 wide, where runs of 160 floats on the wide side are too short:
-// [1342177 x 100] 3.7 -> 4.3 TB/s, and 3.4 for the tiled kernel, whose second tile column is mostly empty.
+// 128 KiB chunks on 1024 threads, one workgroup to a CU, serve tall inputs of 41..256 columns that are
+// not a multiple of 64 wide, where the runs of a 64 KiB chunk on the wide side are too short:
+// [1342177 x 100] 3.7 -> 4.7 TB/s, and 3.4 for the tiled kernel, whose last tile column is mostly empty.
 // Stores are streaming (non-temporal): 4-20 % over plain stores on every shape measured
 // ([100 x 1342177] 4.3 -> 5.2 TB/s, [13421772 x 10] 5.0 -> 5.2, [33 x 4067000] 5.5 -> 5.9).
 __device__ __forceinline__ int ts_skew(int i) { return i + (i >> 5); }
 template <bool NARROW_IN, bool ACC, int CHUNK, int NTH>
 __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side, int S, int R, const float* __restrict__ x,
-                                                               float* out) {
+                                                               float* out, unsigned chunks) {
   __shared__ float buf[CHUNK + CHUNK / 32 + 4];
-  const size_t l0 = (size_t)blockIdx.x * R;
-  const int nr = l0 + R <= long_side ? R : (int)(long_side - l0);
-  const int len = nr * S;
   // LDS holds the chunk in the narrow matrix's order: element (l, s) at l*S + s.  Global memory is
   // touched with dword-aligned float4 on both sides (scalar accesses stream at a third of the rate).
-  const int nr4 = nr & ~3, len4 = len & ~3;
-  // every vector of the chunk is requested before the first one is stored to LDS: a loop that loads
-  // and stores in turn keeps one request per thread in flight
+  // Every vector of a chunk is requested before the first one is stored to LDS: a loop that loads
+  // and stores in turn keeps one request per thread in flight.
+  // A workgroup takes chunks blockIdx.x, blockIdx.x + gridDim.x, ...: the vectors of its next chunk
+  // are requested before the current one is written out, so a CU that holds a single workgroup
+  // (128 KiB chunks) still has loads in flight while it stores.
   constexpr int NJ = CHUNK / (4 * NTH);
+  const int RV = R >> 2;  // vectors per run on the wide side (R is a multiple of 4 whenever a run has vectors)
   float4 v[NJ];
-  if (NARROW_IN) {
-    const float* src = x + l0 * S;
+  auto rows_of = [&](unsigned c) { const size_t l0 = (size_t)c * R; return l0 + R <= long_side ? R : (int)(long_side - l0); };
+  auto request = [&](unsigned c) {
+    const size_t l0 = (size_t)c * R;
+    const int nr = rows_of(c);
+    if (NARROW_IN) {
+      const float* src = x + l0 * S;
+      const int len4 = (nr * S) & ~3;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int i = 4 * threadIdx.x + 4 * NTH * j;
-      if (i < len4) v[j] = ld4s(src + i);
-    }
+      for (int j = 0; j < NJ; ++j) {
+        const int i = 4 * threadIdx.x + 4 * NTH * j;
+        if (i < len4) v[j] = ld4s(src + i);
+      }
+    } else {
+      // the S runs of nr floats, cut into vectors and dealt out over the threads: vector k of the
+      // chunk is vector k % RV of run k / RV
+      const int nrv = nr >> 2;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int i = 4 * threadIdx.x + 4 * NTH * j;
-      if (i < len4) {
-        buf[ts_skew(i)] = v[j].x; buf[ts_skew(i + 1)] = v[j].y; buf[ts_skew(i + 2)] = v[j].z; buf[ts_skew(i + 3)] = v[j].w;
+      for (int j = 0; j < NJ; ++j) {
+        const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
+        if (run < S && lv < nrv) v[j] = ld4s(x + (size_t)run * long_side + l0 + 4 * lv);
       }
     }
-    for (int i = len4 + threadIdx.x; i < len; i += NTH) buf[ts_skew(i)] = src[i];
-  } else {
-    // the S runs of nr floats, cut into vectors and dealt out over the threads: vector j of the
-    // chunk is vector j % RV of run j / RV (R is a multiple of 4 here, so RV = R / 4 covers a run)
-    const int RV = R >> 2, nrv = nr4 >> 2;
+  };
+  auto stage = [&](unsigned c) {  // v, and the few floats beside the vectors, into LDS
+    const size_t l0 = (size_t)c * R;
+    const int nr = rows_of(c), len = nr * S, nr4 = nr & ~3, len4 = len & ~3;
+    if (NARROW_IN) {
+      const float* src = x + l0 * S;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
-      if (run < S && lv < nrv) v[j] = ld4s(x + (size_t)run * long_side + l0 + 4 * lv);
-    }
+      for (int j = 0; j < NJ; ++j) {
+        const int i = 4 * threadIdx.x + 4 * NTH * j;
+        if (i < len4) {
+          buf[ts_skew(i)] = v[j].x; buf[ts_skew(i + 1)] = v[j].y; buf[ts_skew(i + 2)] = v[j].z; buf[ts_skew(i + 3)] = v[j].w;
+        }
+      }
+      for (int i = len4 + threadIdx.x; i < len; i += NTH) buf[ts_skew(i)] = src[i];
+    } else {
+      const int nrv = nr4 >> 2;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
-      if (run < S && lv < nrv) {
-        const int l = 4 * lv;
-        buf[ts_skew(l * S + run)] = v[j].x; buf[ts_skew((l + 1) * S + run)] = v[j].y;
-        buf[ts_skew((l + 2) * S + run)] = v[j].z; buf[ts_skew((l + 3) * S + run)] = v[j].w;
+      for (int j = 0; j < NJ; ++j) {
+        const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
+        if (run < S && lv < nrv) {
+          const int l = 4 * lv;
+          buf[ts_skew(l * S + run)] = v[j].x; buf[ts_skew((l + 1) * S + run)] = v[j].y;
+          buf[ts_skew((l + 2) * S + run)] = v[j].z; buf[ts_skew((l + 3) * S + run)] = v[j].w;
+        }
+      }
+      for (int s = 0; s < S; ++s) {
+        const float* src = x + (size_t)s * long_side + l0;
+        for (int l = nr4 + threadIdx.x; l < nr; l += NTH) buf[ts_skew(l * S + s)] = src[l];
       }
     }
-    for (int s = 0; s < S; ++s) {
-      const float* src = x + (size_t)s * long_side + l0;
-      for (int l = nr4 + threadIdx.x; l < nr; l += NTH) buf[ts_skew(l * S + s)] = src[l];
-    }
-  }
-  __syncthreads();
-  if (NARROW_IN) {
-    // the S output runs of nr floats, cut into vectors and dealt out over the threads as on the
-    // load side of the other direction
-    const int RV = R >> 2, nrv = nr4 >> 2;
+  };
+  auto drain = [&](unsigned c) {  // LDS to the output
+    const size_t l0 = (size_t)c * R;
+    const int nr = rows_of(c), len = nr * S, nr4 = nr & ~3, len4 = len & ~3;
+    if (NARROW_IN) {
+      // The S output runs of nr floats, cut into vectors and dealt out over the threads as on the
+      // load side of the other direction.  Run s starts at float s * long_side + l0 of the output,
+      // which is 16-byte aligned only by chance when the long side is odd: its first `lead` floats
+      // and what is left behind its last whole vector go one by one, so that every vector store is
+      // aligned ([1342177 x 100]: 4.2 -> 4.7 TB/s).
+      const size_t obase = (reinterpret_cast<uintptr_t>(out) >> 2) + l0;
+      auto lead_of = [&](int run) { return (int)((4 - ((obase + (size_t)run * long_side) & 3)) & 3); };
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
-      if (run < S && lv < nrv) {
-        const int l = 4 * lv;
-        float* dst = out + (size_t)run * long_side + l0 + l;
-        float4 w = make_float4(buf[ts_skew(l * S + run)], buf[ts_skew((l + 1) * S + run)], buf[ts_skew((l + 2) * S + run)],
-                               buf[ts_skew((l + 3) * S + run)]);
-        if (ACC) { const float4 o = ld4g(dst); w.x += o.x; w.y += o.y; w.z += o.z; w.w += o.w; }
-        st4s(dst, w);
+      for (int j = 0; j < NJ; ++j) {
+        const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
+        if (run < S) {
+          const int l = lead_of(run) + 4 * lv;
+          if (l + 3 < nr) {
+            float* dst = out + (size_t)run * long_side + l0 + l;
+            float4 w = make_float4(buf[ts_skew(l * S + run)], buf[ts_skew((l + 1) * S + run)], buf[ts_skew((l + 2) * S + run)],
+                                   buf[ts_skew((l + 3) * S + run)]);
+            if (ACC) { const float4 o = ld4(dst); w.x += o.x; w.y += o.y; w.z += o.z; w.w += o.w; }
+            st4s(dst, w);
+          }
+        }
       }
+      // at most three floats before and three behind the vectors of a run (more when a run holds no
+      // whole vector): thread s sees to run s
+      for (int run = threadIdx.x; run < S; run += NTH) {
+        const int lead = lead_of(run) < nr ? lead_of(run) : nr;
+        const int tail = lead + ((nr - lead) & ~3);
+        float* dst = out + (size_t)run * long_side + l0;
+        for (int l = 0; l < lead; ++l) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + run)] : buf[ts_skew(l * S + run)];
+        for (int l = tail; l < nr; ++l) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + run)] : buf[ts_skew(l * S + run)];
+      }
+    } else {
+      float* dst = out + l0 * S;
+      for (int i = 4 * threadIdx.x; i < len4; i += 4 * NTH) {
+        float4 w = make_float4(buf[ts_skew(i)], buf[ts_skew(i + 1)], buf[ts_skew(i + 2)], buf[ts_skew(i + 3)]);
+        if (ACC) { const float4 o = ld4g(dst + i); w.x += o.x; w.y += o.y; w.z += o.z; w.w += o.w; }
+        st4s(dst + i, w);
+      }
+      for (int i = len4 + threadIdx.x; i < len; i += NTH) dst[i] = ACC ? dst[i] + buf[ts_skew(i)] : buf[ts_skew(i)];
     }
-    for (int s = 0; s < S; ++s) {
-      float* dst = out + (size_t)s * long_side + l0;
-      for (int l = nr4 + threadIdx.x; l < nr; l += NTH) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + s)] : buf[ts_skew(l * S + s)];
-    }
-  } else {
-    float* dst = out + l0 * S;
-    for (int i = 4 * threadIdx.x; i < len4; i += 4 * NTH) {
-      float4 v = make_float4(buf[ts_skew(i)], buf[ts_skew(i + 1)], buf[ts_skew(i + 2)], buf[ts_skew(i + 3)]);
-      if (ACC) { const float4 o = ld4g(dst + i); v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
-      st4s(dst + i, v);
-    }
-    for (int i = len4 + threadIdx.x; i < len; i += NTH) dst[i] = ACC ? dst[i] + buf[ts_skew(i)] : buf[ts_skew(i)];
+  };
+  unsigned c = blockIdx.x;
+  if (c >= chunks) return;
+  request(c);
+  for (; c < chunks; c += gridDim.x) {
+    stage(c);
+    __syncthreads();
+    if (c + gridDim.x < chunks) request(c + gridDim.x);
+    drain(c);
+    __syncthreads();  // the next chunk's stage overwrites what this drain reads
   }
 }
 
@@ -266,12 +305,12 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     return post_launch();
   }
   // Which kernel (measured at 2^27 elements, TB/s, chunk kernel / 256 x 64 tiles): a narrow input
-  // [long x S]: S = 31: 4.0 / 2.4, 40: 4.1 / 3.3, 48: 3.8 / 3.5, 64: 5.3 / 5.8, 100: 4.3 (128 KiB chunks) / 3.4,
-  // 128: 5.4 / 5.8; a narrow output, input [S x long]: S = 48: 4.9 / 2.7, 64: 5.4 / 3.3, 100: 5.2 / 3.4,
+  // [long x S]: S = 33: 5.2 / 2.4, 56: 4.9 (128 KiB chunks; 4.2 with 64 KiB) / 3.5, 64: 5.3 / 5.8, 72: 4.9 / -,
+  // 100: 4.7 / 3.4, 128: 5.4 / 5.8, 140: 4.4 / -, 180: 4.2 / -, 200: 5.1 / 3.8; a narrow output, input [S x long]: S = 48: 4.9 / 2.7, 64: 5.4 / 3.3, 100: 5.2 / 3.4,
   // 128: 5.8 / 4.1 (64 x 256 tiles: 5.9), 160: 4.4 / 4.0, 200: 4.9 / -, 224: 3.1 / -, 257: 2.6 / 3.4.
   const bool mirrored_rows = rows % 64 == 0 && rows >= 64 && rows <= 192 && cols >= 4 * rows;  // the 64 x 256 tile below
-  const bool narrow_in = cols <= 56 && cols <= rows;
-  const bool narrow_in_big = !narrow_in && cols <= 128 && cols % 64 != 0 && rows >= 16 * cols;
+  const bool narrow_in_big = cols > 40 && cols <= 256 && cols % 64 != 0 && rows >= 16 * cols;
+  const bool narrow_in = !narrow_in_big && cols <= 56 && cols <= rows;
   const bool narrow_out = !narrow_in && !narrow_in_big && !mirrored_rows && rows <= 200 && rows < cols;
   if (narrow_in || narrow_in_big || narrow_out) {
     const bool in = !narrow_out;
@@ -283,8 +322,11 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     else if (R >= 4) R &= ~3;  // whole vectors per run
     const size_t blocks = (long_side + R - 1) / R;
     SLHIP_REQUIRE(blocks <= 0x7fffffffu, "matrix too large for one launch");
+    // 128 KiB chunks: one workgroup per CU, each walking its share of the chunks; 64 KiB chunks: one
+    // workgroup per chunk
+    const size_t wgs = narrow_in_big && blocks > (size_t)ctx->num_cu ? (size_t)ctx->num_cu : blocks;
 #define SL_TN(NI, A, CH, NT_) \
-  hipLaunchKernelGGL((transpose_narrow_kernel<NI, A, CH, NT_>), dim3((unsigned)blocks), dim3(NT_), 0, ctx->stream, long_side, S, R, x, out)
+  hipLaunchKernelGGL((transpose_narrow_kernel<NI, A, CH, NT_>), dim3((unsigned)wgs), dim3(NT_), 0, ctx->stream, long_side, S, R, x, out, (unsigned)blocks)
     if (narrow_in_big) { if (acc) SL_TN(true, true, 32768, 1024); else SL_TN(true, false, 32768, 1024); }
     else if (in) { if (acc) SL_TN(true, true, 16384, 512); else SL_TN(true, false, 16384, 512); }
     else { if (acc) SL_TN(false, true, 16384, 512); else SL_TN(false, false, 16384, 512); }

@@ -657,7 +657,8 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              # the 64 x 256 tile: tall matrices of 256 columns and more, whole tiles and ragged edges, and wide
              # ones of 64 / 128 / 192 rows; 128 KiB chunks: inputs of 57..128 columns off the 64-grid
              (2048, 512), (1100, 260), (4100, 257), (8200, 1023), (1025, 256), (64, 5000), (128, 1024), (192, 777), (64, 256),
-             (128, 513), (2000, 100), (1700, 65), (3000, 127), (1600, 100), (2049, 128), (1919, 119), (330, 100)]
+             (128, 513), (2000, 100), (1700, 65), (3000, 127), (1600, 100), (2049, 128), (1919, 119), (330, 100),
+             (4000, 200), (4200, 255), (700, 41), (9001, 140), (3300, 193), (5000, 256), (4095, 250)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
