@@ -113,6 +113,43 @@ impl<Mods> HIP<Mods> {
     }
 }
 
+impl<Mods> HIP<Mods> {
+    /// One whole training step of the sine-fit loop (examples/sine_net.rs:119-166) as two launches:
+    /// forward through three Linear layers with ReLU between them, the MSE loss into `loss[0]`,
+    /// backward and SGD on the six parameter buffers in place; their gradient buffers receive the
+    /// step's gradients.  Layers of more than 64 hidden units or 8 inputs / outputs come back as
+    /// `Err` (status `SLHIP_EINVAL`): run the op traits one by one then.
+    #[allow(clippy::too_many_arguments)]
+    pub fn mlp3_mse_step<S: Shape>(
+        &self,
+        batch: usize,
+        d_in: usize,
+        d_h: usize,
+        d_out: usize,
+        x: &Buffer<f32, Self, S>,
+        target: &Buffer<f32, Self, S>,
+        params: &mut [&mut Buffer<f32, Self, S>; 6],
+        lr: f32,
+        loss: &mut Buffer<f32, Self, S>,
+    ) -> Result<(), HipError>
+    where
+        Self: Device,
+    {
+        let grads: Vec<*mut f32> = params.iter_mut().map(|p| p.grad_mut().ptr_mut()).collect();
+        let p: Vec<*mut f32> = params.iter_mut().map(|p| p.ptr_mut()).collect();
+        check(unsafe {
+            ffi::slhip_mlp3_mse_step(self.ctx, batch, d_in, d_h, d_out, x.ptr(), target.ptr(), p[0], p[1], p[2], p[3], p[4], p[5],
+                                     grads.as_ptr(), lr, loss.ptr_mut())
+        })
+    }
+    /// Which kernel and plan the last product on this device ran as (for logs).
+    pub fn last_gemm_plan(&self) -> String {
+        let mut buf = [0 as std::os::raw::c_char; 256];
+        unsafe { ffi::slhip_gemm_plan_describe(self.ctx, buf.as_mut_ptr(), buf.len()) };
+        unsafe { std::ffi::CStr::from_ptr(buf.as_ptr()) }.to_string_lossy().into_owned()
+    }
+}
+
 impl<Mods> Drop for HIP<Mods> {
     fn drop(&mut self) {
         unsafe { ffi::slhip_destroy(self.ctx) };
