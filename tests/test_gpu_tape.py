@@ -519,6 +519,33 @@ def test_repeated_backward_with_manual_descent(device, orc):
     assert abs(sums[-1] / sums[0] - 0.64 ** 99) < 1e-5 * 0.64 ** 99 * 100
 
 
+def test_repeated_backward_with_manual_descent_through_pow(device, orc):
+    """tests/matrix/min_fn.rs:3-23: the same loop with `x.pow(2.)` in place of `square`; powf is not
+    pinned to the last ulp between libm and the device (1e-6 relative per step), the descent is."""
+    xv = np.array([10, -10, 10, -5, 6, 3, 1], np.float32)
+    x = device.buffer(xv)
+    ref = xv.copy()
+    first = last = None
+    for i in range(100):
+        p2 = device.pow(x, 2.0)
+        want = orc.unary(orc.POW, ref, 2.0)
+        got = p2.read()
+        assert np.all(np.abs(got - want) <= 1e-6 * np.abs(want) + 1e-37), i
+        first = float(want.sum()) if first is None else first
+        last = float(want.sum())
+        p2.backward()
+        g_ref = orc.unary_grad(orc.POW, ref, np.zeros_like(ref), np.ones_like(ref), 2.0)
+        g = x.grad().read()
+        assert np.all(np.abs(g - g_ref) <= 1e-6 * np.abs(g_ref) + 1e-37), i
+        device.sgd_step(x, 0.1)
+        ref = orc.sgd_step(ref, g_ref, 0.1)
+        assert np.all(np.abs(x.read() - ref) <= 2e-6 * np.abs(ref) + 1e-37), i
+        # the next step starts from the device's own x on both sides, so roundings do not pile up
+        ref = x.read().copy()
+        device.zero_grad()
+    assert last < first * 1e-15
+
+
 def test_matrix_rand_fills_from_the_seeded_stream(device):
     """Matrix::rand(lo, hi) (src/matrix.rs:266-271): in range, and the very numbers the host-side
     generator gives for the same seed and tag."""
