@@ -53,7 +53,7 @@ SEED = 0x51CED
 MIN_ITERS, MIN_WARMUP = 20, 5
 SPIN_UP_SECONDS = 1.0             # untimed load before the headline's declared warm-up launches
 MAX_LINE_BYTES = 4096             # the result line stays well below what a log tail keeps
-DETAIL_DEFAULT = os.path.join(ROOT, "gpurun_out", "bench_detail.json")
+DETAIL_DEFAULT = os.path.join(ROOT, "bench_detail.json")
 # the ops the metric names, as they appear in the one-line summary: (short key, entry of the suite)
 COMPACT_OPS = [
     ("sum_rows 16384^2", "sum_rows [16384x16384]"), ("sum_cols 16384^2", "sum_cols [16384x16384]"),
