@@ -225,7 +225,7 @@ __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side,
   };
   auto drain = [&](unsigned c) {  // LDS to the output
     const size_t l0 = (size_t)c * R;
-    const int nr = rows_of(c), len = nr * S, nr4 = nr & ~3, len4 = len & ~3;
+    const int nr = rows_of(c), len = nr * S, len4 = len & ~3;
     if (NARROW_IN) {
       // The S output runs of nr floats, cut into vectors and dealt out over the threads as on the
       // load side of the other direction.  Run s starts at float s * long_side + l0 of the output,
