@@ -529,7 +529,16 @@ static int32_t reduce_rows_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, 
     const size_t n = cur_rows * cols, nv = n >> 2;
     size_t T = (size_t)ctx->num_cu * 512;
     if (T > nv / 16) T = nv / 16;
-    T = T / unit * unit;
+    // A multiple of `unit`: the one below for a single stream (rows of 33333 floats: 3 x 33333 threads
+    // 6.2 TB/s, 4 x 33333 - more than 512 per CU - 5.5), the nearest one for the two-matrix sources
+    // of the first stage, which want more loads in flight (5.1 -> 6.1 TB/s on the same shape,
+    // 3.8 -> 6.0 on rows of 66667)
+    if (first && !Src::IS_PLAIN) {
+      T = (T + unit / 2) / unit * unit;
+      if (T > nv / 8 && T > unit) T -= unit;
+    } else {
+      T = T / unit * unit;
+    }
     if (T < unit) T = unit;
     if (4 * T > ws_left || 8 * T > n) break;  // no room, or nothing gained: the last stage takes it as it is
     SLHIP_REQUIRE((T + 255) / 256 <= 0x7fffffffu, "matrix too wide for one launch");
