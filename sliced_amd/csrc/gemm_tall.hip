@@ -13,10 +13,11 @@
 // the current step's 32 instructions run.  Few rows: workgroups split K and the split-K combine
 // finishes.
 //
-// Measured on 1 GiB of A (16384 x N x 16384, pack and combine launches included): 213-240 us for
-// any N up to 32 (4.5-5.0 TB/s of A); the matrix pipes are busy 61 % of the time a CU holds the
-// kernel and a CU holds it 77 % of the kernel's time (every workgroup is resident at once, and they
-// do not finish together).
+// Measured on 1 GiB of A (16384 x N x 16384, pack and combine launches included): 180-183 us for
+// N up to 16 (5.9-6.0 TB/s of A) on the 16 x 16 x 4 instruction, 213-240 us for 17..32 columns
+// (4.5-5.0 TB/s) on the 32 x 32 x 2 one, where the matrix pipes are busy 61 % of the time a CU holds
+// the kernel and a CU holds it 77 % of the kernel's time (every workgroup is resident at once, and
+// they do not finish together).
 #include "gemm_tile.hpp"
 
 namespace slhip {
@@ -36,11 +37,20 @@ __global__ __launch_bounds__(256) void tall_pack_b_kernel(size_t K, size_t Kp, i
   Bt[i] = v;
 }
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// N16: B has at most 16 columns.  The wave's 32 rows are then two blocks of 16 rows on the
+// 16 x 16 x 4 instruction (half the matrix-pipe time per byte of A: a 32-column instruction with 16
+// columns of zeros in it is the bound from 13 columns on), lane (r, q) = (lane % 16, lane / 16)
+// feeds k = 16 q + 4 j + t at issue (j, t), and only 16 rows of Bt are staged.
+template <bool N16>
 __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float* __restrict__ Bt, size_t Kp) {
   // [4 waves][32][TALL_PITCH] of A, wave-private, then [2][32][TALL_PITCH] of Bt, shared by the four waves
   extern __shared__ __attribute__((aligned(16))) float tall_lds[];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int r = lane & 31, h = lane >> 5;
+  const int r = N16 ? lane & 15 : lane & 31, h = N16 ? lane >> 4 : lane >> 5;
+  constexpr int KL = N16 ? 16 : 32;  // k per lane group and step
+  constexpr int NJ = KL / 4;         // float4 per operand row, lane and step
   float* blk = tall_lds + w * 32 * TALL_PITCH;
   float* bblk = tall_lds + 4 * 32 * TALL_PITCH;
   const size_t M = g.M, K = g.K;
@@ -52,7 +62,9 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
   const size_t cend = cbeg + per_y < chunks ? cbeg + per_y : chunks;
 
   // load side: lane l takes the float4 at column 4 * (l % 16) of rows 4 p + l / 16 (p = 0..7) of
-  // the wave's block of A, and of rows 8 w + 4 q + l / 16 (q = 0, 1) of the 32 x 64 block of Bt
+  // the wave's block of A, and of rows 8 w + 4 q + l / 16 (q = 0, 1; N16: rows 4 w + l / 16) of the
+  // block of Bt
+  constexpr int NB = N16 ? 1 : 2;
   const int lrow = lane >> 4, lcol = 4 * (lane & 15);
   const float* arow[8];
 #pragma unroll
@@ -60,17 +72,24 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
     const size_t row = m0 + 4 * p + lrow;
     arow[p] = g.A + (row < M ? row : M - 1) * K;  // rows past the edge: copies that are never stored
   }
-  const float* brow[2];
+  int bstage[NB];
+  const float* brow[NB];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) brow[q] = Bt + (size_t)(8 * w + 4 * q + lrow) * Kp + lcol;
+  for (int q = 0; q < NB; ++q) {
+    bstage[q] = N16 ? 4 * w + lrow : 8 * w + 4 * q + lrow;
+    brow[q] = Bt + (size_t)bstage[q] * Kp + lcol;
+  }
 
   floatx16 acc;
+  floatx4 acc4[2];
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) acc4[0][v] = acc4[1][v] = 0.0f;
 
   // two steps' loads are in flight at any time: set u holds the steps cbeg + u, cbeg + u + 2, ...
-  float4 a[2][8], b[2][2];
-  auto request = [&](size_t ch, float4 (&as)[8], float4 (&bs)[2]) {
+  float4 a[2][8], b[2][NB];
+  auto request = [&](size_t ch, float4 (&as)[8], float4 (&bs)[NB]) {
     const size_t k0 = ch * TALL_KC;
     const size_t k = k0 + lcol;
     // K is a multiple of 4: a vector lies inside the row or wholly beyond it (then it is zeroed below)
@@ -78,7 +97,7 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
 #pragma unroll
     for (int p = 0; p < 8; ++p) as[p] = ld4s(arow[p] + kc);
 #pragma unroll
-    for (int q = 0; q < 2; ++q) bs[q] = ld4g(brow[q] + k0);
+    for (int q = 0; q < NB; ++q) bs[q] = ld4g(brow[q] + k0);
   };
   if (cbeg < cend) request(cbeg, a[0], b[0]);
   if (cbeg + 1 < cend) request(cbeg + 1, a[1], b[1]);
@@ -95,53 +114,79 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
         st4(blk + (4 * p + lrow) * TALL_PITCH + lcol, v);
       }
 #pragma unroll
-      for (int q = 0; q < 2; ++q) st4(bb + (8 * w + 4 * q + lrow) * TALL_PITCH + lcol, b[u][q]);
+      for (int q = 0; q < NB; ++q) st4(bb + bstage[q] * TALL_PITCH + lcol, b[u][q]);
       // one barrier per step: the other half of the Bt buffer is written in the next step, which a
       // wave enters only after every wave has passed this barrier and so has read that half
       __syncthreads();
       if (ch + 2 < cend) request(ch + 2, a[u], b[u]);
-      float4 av[8], bv[8];
+      if constexpr (N16) {
+        float4 av[2][NJ], bv[NJ];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        av[j] = ld4(blk + r * TALL_PITCH + 32 * h + 4 * j);
-        bv[j] = ld4(bb + r * TALL_PITCH + 32 * h + 4 * j);
-      }
+        for (int j = 0; j < NJ; ++j) {
+          av[0][j] = ld4(blk + r * TALL_PITCH + KL * h + 4 * j);
+          av[1][j] = ld4(blk + (16 + r) * TALL_PITCH + KL * h + 4 * j);
+          bv[j] = ld4(bb + r * TALL_PITCH + KL * h + 4 * j);
+        }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].x, bv[j].x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].y, bv[j].y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].z, bv[j].z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].w, bv[j].w, acc, 0, 0, 0);
+        for (int j = 0; j < NJ; ++j) {
+          acc4[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j].x, bv[j].x, acc4[0], 0, 0, 0);
+          acc4[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[1][j].x, bv[j].x, acc4[1], 0, 0, 0);
+          acc4[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j].y, bv[j].y, acc4[0], 0, 0, 0);
+          acc4[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[1][j].y, bv[j].y, acc4[1], 0, 0, 0);
+          acc4[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j].z, bv[j].z, acc4[0], 0, 0, 0);
+          acc4[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[1][j].z, bv[j].z, acc4[1], 0, 0, 0);
+          acc4[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j].w, bv[j].w, acc4[0], 0, 0, 0);
+          acc4[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[1][j].w, bv[j].w, acc4[1], 0, 0, 0);
+        }
+      } else {
+        float4 av[NJ], bv[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          av[j] = ld4(blk + r * TALL_PITCH + KL * h + 4 * j);
+          bv[j] = ld4(bb + r * TALL_PITCH + KL * h + 4 * j);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].x, bv[j].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].y, bv[j].y, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].z, bv[j].z, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].w, bv[j].w, acc, 0, 0, 0);
+        }
       }
     }
   }
   if (m0 >= M) return;
 
-  // register v of lane (r, h): row 8 * (v / 4) + 4 * h + v % 4 of the wave's block, column r
+  // 32 columns: register v of lane (r, h) is row 8 * (v / 4) + 4 * h + v % 4 of the wave's block,
+  // column r; 16 columns: register v of block hh is row 16 * hh + 4 * h + v, column r
   if (r >= N) return;
+  constexpr int NV = N16 ? 8 : 16;
+  auto row_of = [&](int v) -> size_t { return m0 + (N16 ? 16 * (v / 4) + 4 * h + (v % 4) : 8 * (v / 4) + 4 * h + (v % 4)); };
   const bool raw = gridDim.y > 1;
   float* dst = raw ? g.partial + (size_t)blockIdx.y * M * (size_t)N : g.C;
-  float val[16], old[16], msk[16];
+  float val[NV], old[NV], msk[NV];
   const bool with_mask = !raw && g.mask != nullptr, with_c = !raw && g.beta != 0.0f;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const size_t row = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+  for (int v = 0; v < NV; ++v) {
+    const size_t row = row_of(v);
     const size_t at = row * (size_t)N + r;
     msk[v] = with_mask && row < M ? g.mask[at] : 0.0f;
     old[v] = with_c && row < M ? g.C[at] : 0.0f;
   }
   const float bias = !raw && g.bias ? g.bias[r] : 0.0f;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    float x = acc[v];
+  for (int v = 0; v < NV; ++v) {
+    float x;
+    if constexpr (N16) x = acc4[(v / 4) & 1][v % 4];
+    else x = acc[v];
     if (with_mask) x = (msk[v] >= 0.0f ? 1.0f : 0.0f) * x;
     if (with_c) x = g.beta * old[v] + x;
     if (!raw && g.bias) x = x + bias;
     val[v] = x;
   }
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const size_t row = m0 + 8 * (v / 4) + 4 * h + (v % 4);
+  for (int v = 0; v < NV; ++v) {
+    const size_t row = row_of(v);
     if (row >= M) continue;
     const size_t at = row * (size_t)N + r;
     float x = val[v];
@@ -157,12 +202,15 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
 // partials of g.splits k ranges wait in the workspace for the split-K combine.
 int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
   const size_t M = g.M, N = g.N, K = g.K;
-  // From 13 columns on the sixteen-block kernel is bound by the matrix pipes (16384 x 16 x 16384:
-  // 396 us against 240 here); from 8 on this kernel is the faster one once A is 512 MiB or more
-  // (16384 x 8 / 10 / 12 x 16384: 265 / 231 / 246 -> 224 / 215 / 213 us), while at 64-256 MiB the
-  // two are level or the other ahead (8192 x 10 x 2048: 26.8 against 29.1 us).
+  // Against the sixteen-block kernel (which is bound by the matrix pipes from 13 columns on:
+  // 16384 x 16 x 16384 takes it 377 us, this one 182): ahead at 8 columns and more wherever K is
+  // long enough to amortise the pack and the combine (16384 x 8 / 10 / 12 x 16384: 253 / 223 / 242
+  // -> 180 us; 8192 x 10 x 2048: 27.0 -> 24.8; 2048 x 10 x 8192: 33.4 -> 27.6), level at 2^23
+  // elements of A, behind with K = 1024 (65536 x 8 / 12 x 1024: 50 / 64 us there, 71 here) and below 8
+  // columns except on 1 GiB (16384 x 2 / 4 / 6 x 16384: 192 / 184 / 192 there, 183 / 182 / 180 here,
+  // but 16384 x 2 x 8192 93 there and 101 here).
   if (ta || N > 32 || N < 8 || K % 4 != 0 || K < 256 || M < 512) return 0;
-  if (M * K < (N >= 13 ? (size_t(1) << 24) : (size_t(1) << 27))) return 0;
+  if (N >= 13 ? M * K < (size_t(1) << 22) : (K < 2048 || M * K < (size_t(1) << 24))) return 0;
   const size_t Kp = (K + TALL_KC - 1) / TALL_KC * TALL_KC;
   const size_t bt_bytes = 32 * Kp * sizeof(float);
   if (bt_bytes > ((size_t)32 << 20) || ctx->workspace_bytes < 4 * bt_bytes + ((size_t)64 << 20)) return 0;
@@ -188,7 +236,8 @@ int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc)
   const size_t pack_blocks = (32 * Kp + 255) / 256;
   hipLaunchKernelGGL(tall_pack_b_kernel, dim3((unsigned)pack_blocks), dim3(256), 0, ctx->stream, K, Kp, (int)N, tb ? 1 : 0, g.B, bt);
   const size_t lds = (size_t)6 * 32 * TALL_PITCH * sizeof(float);
-  hipLaunchKernelGGL(gemm_tall_kernel, dim3((unsigned)gx, (unsigned)splits), dim3(256), lds, ctx->stream, g, (const float*)bt, Kp);
+  if (N <= 16) hipLaunchKernelGGL(gemm_tall_kernel<true>, dim3((unsigned)gx, (unsigned)splits), dim3(256), lds, ctx->stream, g, (const float*)bt, Kp);
+  else hipLaunchKernelGGL(gemm_tall_kernel<false>, dim3((unsigned)gx, (unsigned)splits), dim3(256), lds, ctx->stream, g, (const float*)bt, Kp);
   *rc = post_launch();
   return splits > 1 && *rc == SLHIP_OK ? 2 : 1;
 }

@@ -222,12 +222,14 @@ def test_gemm_rows_narrow_kernel(hip, orc):
 
 
 def test_gemm_tall_kernel(hip, orc):
-    """A * B and A * Bt with a tall row-major A and 13..32 columns (8..12 from 2^27 elements of A on):
-    the 32 x 32 x 2 kernel whose waves own 32 rows each.  M off the multiples of 32 and 128, K a
-    multiple of 4 that is not one of 64, few rows with K split among workgroups and many rows without a
-    split, every epilogue."""
+    """A * B and A * Bt with a tall row-major A and 13..32 columns (8..12 with K >= 2048 and 2^24
+    elements of A): the kernel whose waves own 32 rows each, on the 16 x 16 x 4 instruction up to 16
+    columns and on the 32 x 32 x 2 one above.  M off the multiples of 32 and 128, K a multiple of 4 that
+    is not one of 64, few rows with K split among workgroups and many rows without a split, every
+    epilogue."""
     for (m, n, k, tb) in [(16384, 16, 1024, 0), (4100, 13, 4100, 0), (100000, 32, 260, 0), (513, 20, 40000, 0),
-                          (8192, 31, 2048, 1), (1000, 17, 16388, 1), (65536, 10, 2048, 0), (131072 + 5, 8, 1024, 1)]:
+                          (8192, 31, 2048, 1), (1000, 17, 16388, 1), (65536, 10, 2048, 0), (131072 + 5, 8, 1024, 1),
+                          (8200, 9, 4100, 1), (2049, 14, 2052, 0), (530, 12, 32772, 0)]:
         say("tall gemm", m, n, k, tb)
         a, b = gemm_operands(0, tb, m, n, k)
         exact, bound = gemm_bound(0, tb, m, n, k, a, b)
