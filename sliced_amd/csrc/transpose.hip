@@ -150,15 +150,24 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 // CHUNK floats per workgroup of NTH threads.  64 KiB chunks on 512 threads serve narrow inputs up
 // to 56 columns and narrow outputs up to 200 rows (against 32 KiB the runs on the wide side are twice
 // as long: narrow inputs of 10..56 columns gain 5-11 %, narrow outputs of 100..200 rows 5-11 %);
-// 128 KiB chunks on 1024 threads, one workgroup to a CU, serve tall inputs of 41..256 columns that are
-// not a multiple of 64 wide, where the runs of a 64 KiB chunk on the wide side are too short:
-// [1342177 x 100] 3.7 -> 4.7 TB/s, and 3.4 for the tiled kernel, whose last tile column is mostly empty.
+// 128 KiB chunks on 1024 threads, one workgroup to a CU, serve tall inputs of 57..256 columns that are
+// not a multiple of 64 wide, where the runs of a 64 KiB chunk on the wide side are too short
+// ([1342177 x 100]: 3.7 TB/s with 64 KiB chunks, 3.4 for the tiled kernel, whose last tile column is
+// mostly empty) - unless the output runs start on 64-byte boundaries by themselves, where 64 KiB
+// chunks are ahead up to 200 columns ([1342176 x 100] 5.5 against 5.3).
+// What a chunk writes of an output run is a piece that starts on a 64- or 128-byte boundary of the
+// output and is a multiple of that long: a piece that ends inside such a block leaves the block to
+// two workgroups on two L2s, and the memory sees two partial writes ([1342176 x 100], whose runs
+// start on 128-byte boundaries: 5.4 TB/s; [1342180 x 100]: 4.0-4.4 with the same code).  With an odd
+// long side the boundaries lie elsewhere in every run, so the chunk shifts its piece of run s by
+// d_s floats and stages 16 or 32 more rows of the input than it writes ([1342177 x 100] 4.7 -> 5.05
+// TB/s, [13421772 x 10] 5.2 -> 5.7, [4067000 x 33] 5.0 -> 5.5, [958698 x 140] 4.4 -> 5.0).
 // Stores are streaming (non-temporal): 4-20 % over plain stores on every shape measured
 // ([100 x 1342177] 4.3 -> 5.2 TB/s, [13421772 x 10] 5.0 -> 5.2, [33 x 4067000] 5.5 -> 5.9).
 __device__ __forceinline__ int ts_skew(int i) { return i + (i >> 5); }
 template <bool NARROW_IN, bool ACC, int CHUNK, int NTH>
 __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side, int S, int R, const float* __restrict__ x,
-                                                               float* out, unsigned chunks) {
+                                                               float* out, unsigned chunks, int halo, int align) {
   __shared__ float buf[CHUNK + CHUNK / 32 + 4];
   // LDS holds the chunk in the narrow matrix's order: element (l, s) at l*S + s.  Global memory is
   // touched with dword-aligned float4 on both sides (scalar accesses stream at a third of the rate).
@@ -170,9 +179,20 @@ __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side,
   constexpr int NJ = CHUNK / (4 * NTH);
   const int RV = R >> 2;  // vectors per run on the wide side (R is a multiple of 4 whenever a run has vectors)
   float4 v[NJ];
-  auto rows_of = [&](unsigned c) { const size_t l0 = (size_t)c * R; return l0 + R <= long_side ? R : (int)(long_side - l0); };
+  // NARROW_IN with halo = align (16 or 32 floats; the runs of the output do not all start on
+  // boundaries of that many floats): chunk c writes, of output run s, the floats
+  // [c R - d_s, c R + R - d_s) (cut to the run), where d_s < align is what puts that piece on such a
+  // boundary of the output; it stages the rows [c R - halo, c R + R) of the input, `halo` rows of
+  // which its neighbour stages too.
+  // Otherwise (halo = 0): chunk c is the floats [c R, c R + R) of every run.
+  auto first_row = [&](unsigned c) { const size_t l0 = (size_t)c * R; return NARROW_IN && c ? l0 - halo : l0; };
+  auto rows_of = [&](unsigned c) {
+    const size_t l0 = (size_t)c * R, lb = first_row(c);
+    if (lb >= long_side) return 0;
+    return l0 + R <= long_side ? (int)(l0 + R - lb) : (int)(long_side - lb);
+  };
   auto request = [&](unsigned c) {
-    const size_t l0 = (size_t)c * R;
+    const size_t l0 = first_row(c);
     const int nr = rows_of(c);
     if (NARROW_IN) {
       const float* src = x + l0 * S;
@@ -194,7 +214,7 @@ __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side,
     }
   };
   auto stage = [&](unsigned c) {  // v, and the few floats beside the vectors, into LDS
-    const size_t l0 = (size_t)c * R;
+    const size_t l0 = first_row(c);
     const int nr = rows_of(c), len = nr * S, nr4 = nr & ~3, len4 = len & ~3;
     if (NARROW_IN) {
       const float* src = x + l0 * S;
@@ -227,35 +247,51 @@ __global__ __launch_bounds__(NTH) void transpose_narrow_kernel(size_t long_side,
     const size_t l0 = (size_t)c * R;
     const int nr = rows_of(c), len = nr * S, len4 = len & ~3;
     if (NARROW_IN) {
-      // The S output runs of nr floats, cut into vectors and dealt out over the threads as on the
-      // load side of the other direction.  Run s starts at float s * long_side + l0 of the output,
-      // which is 16-byte aligned only by chance when the long side is odd: its first `lead` floats
-      // and what is left behind its last whole vector go one by one, so that every vector store is
-      // aligned ([1342177 x 100]: 4.2 -> 4.7 TB/s).
-      const size_t obase = (reinterpret_cast<uintptr_t>(out) >> 2) + l0;
-      auto lead_of = [&](int run) { return (int)((4 - ((obase + (size_t)run * long_side) & 3)) & 3); };
+      // The S output runs, cut into vectors and dealt out over the threads as on the load side of
+      // the other direction.  Run s starts at float s * long_side of the output, which is aligned
+      // only by chance when the long side is odd; shifted by d_s, this chunk's piece of it starts
+      // on a 64-byte boundary and is R floats long, so it is written as whole 64-byte blocks
+      // (pieces that end inside a block leave it to two workgroups, which costs a sixth of the rate:
+      // [1342177 x 100] 4.7 -> 5.2 TB/s).  The pieces at the two ends of a run are cut there: what
+      // lies before the first aligned vector and behind the last whole one goes float by float.
+      // (all of it in row numbers relative to the first staged row, in 32 bits)
+      const size_t lb = first_row(c);
+      const int off = (int)(l0 - lb);  // halo, or 0 for the first chunk
+      const int ob = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & (align - 1)), lm = (int)(long_side & (align - 1));
+      // the piece of `run`: rows [lo, hi) of the staged ones; returns the floats before its first aligned vector
+      auto piece = [&](int run, int& lo, int& hi) {
+        const int d = (ob + run * lm) & (align - 1);
+        lo = off > d ? off - d : 0;
+        hi = off + R - d < nr ? off + R - d : nr;
+        return lo ? 0 : (4 - (d & 3)) & 3;  // lo > 0: the piece starts on a boundary
+      };
+      float* const obeg = out + lb;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const int k = threadIdx.x + NTH * j, run = k / RV, lv = k - run * RV;
         if (run < S) {
-          const int l = lead_of(run) + 4 * lv;
-          if (l + 3 < nr) {
-            float* dst = out + (size_t)run * long_side + l0 + l;
-            float4 w = make_float4(buf[ts_skew(l * S + run)], buf[ts_skew((l + 1) * S + run)], buf[ts_skew((l + 2) * S + run)],
-                                   buf[ts_skew((l + 3) * S + run)]);
+          int lo, hi;
+          const int l = piece(run, lo, hi) + lo + 4 * lv;
+          if (l + 3 < hi) {
+            float* dst = obeg + (size_t)run * long_side + l;
+            const int at = l * S + run;
+            float4 w = make_float4(buf[ts_skew(at)], buf[ts_skew(at + S)], buf[ts_skew(at + 2 * S)], buf[ts_skew(at + 3 * S)]);
             if (ACC) { const float4 o = ld4(dst); w.x += o.x; w.y += o.y; w.z += o.z; w.w += o.w; }
             st4s(dst, w);
           }
         }
       }
-      // at most three floats before and three behind the vectors of a run (more when a run holds no
+      // at most three floats before and three behind the vectors of a piece (more when it holds no
       // whole vector): thread s sees to run s
       for (int run = threadIdx.x; run < S; run += NTH) {
-        const int lead = lead_of(run) < nr ? lead_of(run) : nr;
-        const int tail = lead + ((nr - lead) & ~3);
-        float* dst = out + (size_t)run * long_side + l0;
-        for (int l = 0; l < lead; ++l) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + run)] : buf[ts_skew(l * S + run)];
-        for (int l = tail; l < nr; ++l) dst[l] = ACC ? dst[l] + buf[ts_skew(l * S + run)] : buf[ts_skew(l * S + run)];
+        int lo, hi;
+        int lead = piece(run, lo, hi) + lo;
+        if (lo >= hi) continue;
+        if (lead > hi) lead = hi;
+        const int tail = lead + ((hi - lead) & ~3);
+        float* dst = obeg + (size_t)run * long_side;
+        for (int l = lo; l < lead; ++l) { const float t = buf[ts_skew(l * S + run)]; dst[l] = ACC ? dst[l] + t : t; }
+        for (int l = tail; l < hi; ++l) { const float t = buf[ts_skew(l * S + run)]; dst[l] = ACC ? dst[l] + t : t; }
       }
     } else {
       float* dst = out + l0 * S;
@@ -305,28 +341,39 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     return post_launch();
   }
   // Which kernel (measured at 2^27 elements, TB/s, chunk kernel / 256 x 64 tiles): a narrow input
-  // [long x S]: S = 33: 5.2 / 2.4, 56: 4.9 (128 KiB chunks; 4.2 with 64 KiB) / 3.5, 64: 5.3 / 5.8, 72: 4.9 / -,
-  // 100: 4.7 / 3.4, 128: 5.4 / 5.8, 140: 4.4 / -, 180: 4.2 / -, 200: 5.1 / 3.8; a narrow output, input [S x long]: S = 48: 4.9 / 2.7, 64: 5.4 / 3.3, 100: 5.2 / 3.4,
+  // [long x S] with an odd long side: S = 33: 5.5 / 2.4, 56: 5.5 / 3.5, 64: 5.3 / 5.8, 72: 5.4 / -,
+  // 100: 5.05 / 3.4, 128: 5.4 / 5.8, 140: 5.0 / -, 180: 4.9 / -, 200: 4.8 / 3.8, 250: 4.75 / -; a narrow output, input [S x long]: S = 48: 4.9 / 2.7, 64: 5.4 / 3.3, 100: 5.2 / 3.4,
   // 128: 5.8 / 4.1 (64 x 256 tiles: 5.9), 160: 4.4 / 4.0, 200: 4.9 / -, 224: 3.1 / -, 257: 2.6 / 3.4.
   const bool mirrored_rows = rows % 64 == 0 && rows >= 64 && rows <= 192 && cols >= 4 * rows;  // the 64 x 256 tile below
-  const bool narrow_in_big = cols > 40 && cols <= 256 && cols % 64 != 0 && rows >= 16 * cols;
-  const bool narrow_in = !narrow_in_big && cols <= 56 && cols <= rows;
+  // The pieces of the output runs that a narrow input's chunks write start on boundaries of `unit`
+  // floats: 64 bytes, which is what the rate depends on ([1342176 / 1342160 / 1342168 / 1342180 x 100]:
+  // runs that start on multiples of 128 / 64 / 32 / 16 bytes, 5.4 / 5.25 / 4.4 / 4.0 TB/s), or 128 where
+  // that is free (the runs start there by themselves) or cheap (chunks of 256 rows and more: 1-5 %
+  // faster again).  Odd long sides get there with a halo of that many rows.
+  const int unit = cols <= 64 || (rows % 32 == 0 && (reinterpret_cast<uintptr_t>(out) & 127) == 0) ? 32 : 16;
+  const bool runs_aligned = rows % unit == 0 && (reinterpret_cast<uintptr_t>(out) & (4 * unit - 1)) == 0;
+  const bool narrow_in_wide = cols > 56 && cols <= 256 && cols % 64 != 0 && rows >= 16 * cols;
+  const bool narrow_in_big = narrow_in_wide && !(runs_aligned && cols <= 200);
+  const bool narrow_in = !narrow_in_big && (narrow_in_wide || (cols <= 56 && cols <= rows));
   const bool narrow_out = !narrow_in && !narrow_in_big && !mirrored_rows && rows <= 200 && rows < cols;
   if (narrow_in || narrow_in_big || narrow_out) {
     const bool in = !narrow_out;
     const size_t long_side = in ? rows : cols;
     const int S = (int)(in ? cols : rows);
+    const int halo = in && !runs_aligned ? unit : 0;
     const int chunk = narrow_in_big ? 32768 : 16384;
     int R = chunk / S;
-    if (R >= 256) R &= ~31;  // runs that start on 128-byte boundaries of their rows, where that costs little
+    if (in) R = (R - halo) & ~(unit - 1);  // the chunk holds `halo` rows more than it writes of every run
+    else if (R >= 256) R &= ~31;  // runs that start on 128-byte boundaries of their rows, where that costs little
     else if (R >= 4) R &= ~3;  // whole vectors per run
-    const size_t blocks = (long_side + R - 1) / R;
+    // (with a halo the last chunk ends unit - 1 floats or more behind the runs: every shifted piece ends inside it)
+    const size_t blocks = (long_side + (halo ? halo - 1 : 0) + R - 1) / R;
     SLHIP_REQUIRE(blocks <= 0x7fffffffu, "matrix too large for one launch");
     // 128 KiB chunks: one workgroup per CU, each walking its share of the chunks; 64 KiB chunks: one
     // workgroup per chunk
     const size_t wgs = narrow_in_big && blocks > (size_t)ctx->num_cu ? (size_t)ctx->num_cu : blocks;
 #define SL_TN(NI, A, CH, NT_) \
-  hipLaunchKernelGGL((transpose_narrow_kernel<NI, A, CH, NT_>), dim3((unsigned)wgs), dim3(NT_), 0, ctx->stream, long_side, S, R, x, out, (unsigned)blocks)
+  hipLaunchKernelGGL((transpose_narrow_kernel<NI, A, CH, NT_>), dim3((unsigned)wgs), dim3(NT_), 0, ctx->stream, long_side, S, R, x, out, (unsigned)blocks, halo, unit)
     if (narrow_in_big) { if (acc) SL_TN(true, true, 32768, 1024); else SL_TN(true, false, 32768, 1024); }
     else if (in) { if (acc) SL_TN(true, true, 16384, 512); else SL_TN(true, false, 16384, 512); }
     else { if (acc) SL_TN(false, true, 16384, 512); else SL_TN(false, false, 16384, 512); }

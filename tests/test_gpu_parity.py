@@ -660,7 +660,11 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              # ones of 64 / 128 / 192 rows; 128 KiB chunks: inputs of 57..128 columns off the 64-grid
              (2048, 512), (1100, 260), (4100, 257), (8200, 1023), (1025, 256), (64, 5000), (128, 1024), (192, 777), (64, 256),
              (128, 513), (2000, 100), (1700, 65), (3000, 127), (1600, 100), (2049, 128), (1919, 119), (330, 100),
-             (4000, 200), (4200, 255), (700, 41), (9001, 140), (3300, 193), (5000, 256), (4095, 250)]
+             (4000, 200), (4200, 255), (700, 41), (9001, 140), (3300, 193), (5000, 256), (4095, 250),
+             # narrow inputs whose output runs start off / on 64- and 128-byte boundaries (long sides odd, multiples
+             # of 16 and of 32): shifted pieces with a halo, first and last chunks, pieces cut at both ends
+             (50001, 100), (50016, 100), (50048, 100), (20001, 250), (20000, 250), (100003, 56), (100000, 33), (99984, 33),
+             (17, 3), (31, 10), (33, 10), (8209, 10), (1647, 10), (1648, 10), (1649, 10), (3301, 10), (40007, 72), (5000001, 3)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -675,6 +679,32 @@ def test_transpose_bit_exact(hip, orc, shape):
     base = rng.uniform(rows * cols, -1, 1, tag=1, seed=SEED)
     acc = hip.transpose(rows, cols, x, out=base.copy(), assign=True)   # `Assign` (+=)
     assert np.array_equal(acc, orc.transpose(rows, cols, x, out=base.copy(), assign=True))
+
+
+@pytest.mark.parametrize("shape", [(50001, 100), (50016, 100), (8209, 10), (100003, 56), (64, 5000), (100, 8193), (1234, 679)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_transpose_between_views_off_the_allocation_grid(hip, orc, shape):
+    """Input and output that start 1, 5, 16 and 17 floats into their allocations: no kernel may rely on
+    the 256-byte alignment of a fresh buffer, and what lies around the output stays as it was."""
+    rows, cols = shape
+    n = rows * cols
+    c = hip.ctx()
+    x = rng.uniform(n, -10, 10, tag=0, seed=SEED)
+    want = orc.transpose(rows, cols, x)
+    pad = 64
+    src, dst = c.empty(n + pad), c.empty(n + 2 * pad)
+    for off in (1, 5, 16, 17):
+        say("transpose into a view", rows, cols, off)
+        src.view(off, n).upload(x)
+        c.call("slhip_fill", n + 2 * pad, -3.0, dst.ptr)
+        c.call("slhip_transpose", rows, cols, src.view(off, n).ptr, dst.view(pad + off, n).ptr, 0.0)
+        got = dst.numpy()
+        assert np.array_equal(got[pad + off:pad + off + n], want), off
+        assert np.all(got[:pad + off] == -3.0) and np.all(got[pad + off + n:] == -3.0), off
+        c.call("slhip_transpose", rows, cols, src.view(off, n).ptr, dst.view(pad + off, n).ptr, 1.0)
+        assert np.array_equal(dst.numpy()[pad + off:pad + off + n], want + want), off
+    src.free()
+    dst.free()
 
 
 # --------------------------------------------------------------------------- elementwise / row op
