@@ -92,7 +92,7 @@ struct EwpLane {
 #define EWP_EACH_ROLLED(expr)            \
   _Pragma("unroll 1") for (int c = 0; c < W; ++c) { expr; }
 
-// Runs the program; on return v holds the last instruction's result (which is also in its slot).
+// Runs the program; on return v holds the last instruction's result (which has no slot).
 template <int W>
 __device__ __forceinline__ void ewp_forward(const EwProgArgs& a, const EwpLane<W>& r, float (&v)[W]) {
   EwpInsn next = a.insn[0];
@@ -121,7 +121,7 @@ __device__ __forceinline__ void ewp_forward(const EwProgArgs& a, const EwpLane<W
     else if (op == (U_ | SLHIP_TANH)) { EWP_EACH_ROLLED(v[c] = tanhf(x[c])) }
     else if (op == (U_ | SLHIP_SIGMOID)) { EWP_EACH_ROLLED(v[c] = 1.0f / (1.0f + expf(-x[c]))) }
     else { EWP_EACH_ROLLED(v[c] = -logf(x[c])) }  // SLHIP_NEG_LN
-    r.put(in.dst, v);
+    if (i + 1 < a.n_ops) r.put(in.dst, v);  // the last result stays in v
   }
 }
 
@@ -287,39 +287,58 @@ static int32_t ewp_prepare(const char* who, size_t n, size_t n_inputs, const flo
   return SLHIP_OK;
 }
 
-// Forward only: renumbers the intermediates onto as few registers as their lifetimes allow - a
-// value's register is free again after the last instruction that reads it, and an instruction may
-// write the register of an operand that dies there.  (The gradient pass reads every intermediate
-// again on its way back and keeps the ABI's numbering.)
-static void ewp_pack_registers(EwProgArgs* a) {
+// Renumbers the values onto as few registers as their lifetimes allow: a value's register is free
+// again after the last instruction that reads it (an input's too), and an instruction may write
+// the register of an operand that dies there.  The last instruction's result stays in VGPRs and
+// gets no register.  For the gradient pass (`grad`) a value that a backward step reads - the
+// operands of mul and div, the operand of every unary op but scale - keeps its register to the
+// end; what add, sub and scale read on the way back is not used, so it may be anything.
+// Waves per CU follow from the KiB of LDS per wave: the gradient pass of ((a+b)*c-d) -> pow 2 ->
+// square went from 15 KiB and 5.3 TB/s to 10 KiB; 5, 10 and 20 KiB more measured 4.5, 3.6, 2.6 TB/s.
+static void ewp_pack_registers(EwProgArgs* a, bool grad) {
   int last_use[EWP_REGS];
-  for (int k = 0; k < EWP_REGS; ++k) last_use[k] = -1;
+  bool keep[EWP_REGS];
+  for (int k = 0; k < EWP_REGS; ++k) {
+    last_use[k] = -1;
+    keep[k] = false;
+  }
   for (int i = 0; i < a->n_ops; ++i) {
-    last_use[a->insn[i].src0] = i;
-    last_use[a->insn[i].src1] = i;
+    const EwpInsn& in = a->insn[i];
+    last_use[in.src0] = i;
+    last_use[in.src1] = i;
+    if (!grad || ((a->nograd >> i) & 1u)) continue;
+    if (in.op & SLHIP_EW_UNARY) {
+      if ((in.op & 0xf) != SLHIP_SCALE) keep[in.src0] = true;
+    } else if (in.op == SLHIP_MUL || in.op == SLHIP_DIV) {
+      keep[in.src0] = keep[in.src1] = true;
+    }
   }
   int phys[EWP_REGS];
   bool busy[EWP_REGS];
   for (int k = 0; k < EWP_REGS; ++k) {
     phys[k] = k;
-    busy[k] = k < EWP_IN;
+    busy[k] = k < a->n_in;  // the kernel puts input j into register j
   }
-  int top = EWP_IN;
+  int top = a->n_in;
   for (int i = 0; i < a->n_ops; ++i) {
     EwpInsn& in = a->insn[i];
     const int s0 = in.src0, s1 = in.src1;
     in.src0 = (uint8_t)phys[s0];
     in.src1 = (uint8_t)phys[s1];
-    if (s0 >= EWP_IN && last_use[s0] == i) busy[phys[s0]] = false;
-    if (s1 >= EWP_IN && last_use[s1] == i) busy[phys[s1]] = false;
-    int d = EWP_IN;
-    while (busy[d]) ++d;  // at most 8 intermediates: one of 4..11 is free
+    if (last_use[s0] == i && !keep[s0]) busy[phys[s0]] = false;
+    if (last_use[s1] == i && !keep[s1]) busy[phys[s1]] = false;
+    if (i + 1 == a->n_ops) {  // never stored
+      in.dst = 0;
+      break;
+    }
+    int d = 0;
+    while (busy[d]) ++d;  // at most 4 inputs and 7 stored intermediates: one of 0..11 is free
     busy[d] = last_use[EWP_IN + i] >= 0;  // a result nobody reads does not hold its register
     phys[EWP_IN + i] = d;
     in.dst = (uint8_t)d;
     if (d + 1 > top) top = d + 1;
   }
-  a->n_regs = top;
+  a->n_regs = top > 0 ? top : 1;
 }
 
 // Gradient pass: gives every intermediate's adjoint a slot for as long as it lives - from the
@@ -348,7 +367,7 @@ static void ewp_plan_adjoints(EwProgArgs* a) {
   a->seed_slot = ((a->nograd >> (a->n_ops - 1)) & 1u) ? -1 : slot[last];
   for (int i = a->n_ops - 1; i >= 0; --i) {
     const int dst = EWP_IN + i;
-    const int s0 = a->insn[i].src0, s1 = a->insn[i].src1;  // the gradient pass keeps the ABI's numbering
+    const int s0 = a->insn[i].src0, s1 = a->insn[i].src1;  // (still the ABI's numbering)
     int fl = 0;
     if ((a->nograd >> i) & 1u) {
       if (slot[dst] >= EWP_IN) busy[slot[dst]] = false;
@@ -382,11 +401,12 @@ static int32_t ewp_launch(slhip_ctx* ctx, size_t n, EwProgArgs a, bool grad) {
   }
   const dim3 grid(ceil_div(threads, 64));
   if (grad) {
-    ewp_plan_adjoints(&a);
+    ewp_plan_adjoints(&a);  // on the ABI's numbering, which the packing below replaces
+    ewp_pack_registers(&a, true);
     const size_t lds = (size_t)(a.n_regs + a.n_adj) * 1024;
     hipLaunchKernelGGL(ew_program_kernel<true>, grid, dim3(64), lds, ctx->stream, n, a);
   } else {
-    ewp_pack_registers(&a);
+    ewp_pack_registers(&a, false);
     hipLaunchKernelGGL(ew_program_kernel<false>, grid, dim3(64), (size_t)a.n_regs * 1024, ctx->stream, n, a);
   }
   return post_launch();

@@ -105,6 +105,47 @@ def test_program_equals_the_ops_one_by_one(hip, orc, name):
         assert np.all(out == np.float32(9.336999))        # examples/chained_perf.rs:91
 
 
+def random_program(r):
+    """A well-formed program of 2..8 instructions over 1..4 inputs: any earlier value may be read any
+    number of times (or never), exp and clip carry NOGRAD, now and then so does another op."""
+    n_in = int(r.integers(1, 5))
+    n_ops = int(r.integers(2, 9))
+    prog = []
+    for i in range(n_ops):
+        avail = list(range(n_in)) + [4 + k for k in range(i)]
+        # the newest value most of the time, so that chains form, but not always
+        pick = lambda: int(avail[-1] if i and r.random() < 0.5 else avail[int(r.integers(0, len(avail)))])
+        if r.random() < 0.5:
+            op = int(r.integers(0, 4))
+            prog.append((op, pick(), pick(), NOGRAD if r.random() < 0.1 else 0))
+        else:
+            op = int(r.choice([SQUARE, POW, RELU, EXP, CLIP, SCALE, TANH, SIGMOID]))
+            s = pick()
+            flags = NOGRAD if op in (EXP, CLIP) or r.random() < 0.1 else 0
+            p, q = {POW: (3.0, 0.0), CLIP: (-0.5, 0.75), SCALE: (-1.75, 0.0)}.get(op, (0.0, 0.0))
+            prog.append((U | op, s, s, flags, p, q))
+    return n_in, prog
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_programs_equal_the_ops_one_by_one(hip, seed):
+    """Values die, share registers and are needed again on the way back in every pattern a random
+    program produces: result and every input gradient bit for bit the ops run one by one."""
+    r = np.random.default_rng(1000 + seed)
+    n_in, prog = random_program(r)
+    n = 4099
+    say("random program", seed, n_in, prog)
+    inputs = [rng.uniform(n, -1.5, 1.5, tag=j, seed=SEED + seed) for j in range(n_in)]
+    want = run_one_by_one(hip, inputs, prog)[4 + len(prog) - 1]
+    assert np.array_equal(hip.ew_program(inputs, prog), want, equal_nan=True)
+    g = rng.normal(n, 1.0, tag=9, seed=SEED)
+    grads0 = [rng.uniform(n, -1, 1, tag=20 + j, seed=SEED) for j in range(n_in)]
+    want_g = grads_one_by_one(hip, inputs, grads0, prog, g)
+    got_g = hip.ew_program_grad(inputs, grads0, prog, g)
+    for j in range(n_in):
+        assert np.array_equal(got_g[j], want_g[j], equal_nan=True), j
+
+
 def test_program_skips_null_gradients_and_validates(hip):
     n = 1000
     a, b = rng.uniform(n, -1, 1, tag=0), rng.uniform(n, -1, 1, tag=1)
