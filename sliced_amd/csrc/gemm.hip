@@ -251,8 +251,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
         s.x = beta * c.x + s.x; s.y = beta * c.y + s.y; s.z = beta * c.z + s.z; s.w = beta * c.w + s.w;
       }
       if (bias) {
-        float4 b = ld4g(bias + (4 * i) % N);
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        if (N % 4 == 0) {
+          float4 b = ld4g(bias + (4 * i) % N);
+          s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        } else {  // the vector runs over a row end
+          const size_t c = (4 * i) % N;
+          s.x += bias[c]; s.y += bias[(c + 1) % N]; s.z += bias[(c + 2) % N]; s.w += bias[(c + 3) % N];
+        }
       }
       if (pre_act) st4g(pre_act + 4 * i, s);
       if (relu) {
@@ -277,7 +282,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
 
 static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) {
   const size_t mn = g.M * g.N;
-  const int vec = (mn % 4 == 0) && (g.N % 4 == 0);
+  const int vec = mn % 4 == 0;  // the flat M x N array in whole vectors (each may run over a row end)
   size_t blocks = ((vec ? mn / 4 : mn) + 255) / 256;
   const size_t cap = (size_t)ctx->num_cu * 16;
   if (blocks > cap) blocks = cap;

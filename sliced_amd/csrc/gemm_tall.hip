@@ -1,7 +1,8 @@
-// C = A * B for a tall A (stored M x K, K a multiple of 4, the large side: read once) and a B of
-// at most 32 columns, on the 32 x 32 x 2 matrix instruction.
+// Products of one large operand that is read once and a B of at most 32 columns, on the matrix
+// instructions: C = A * B and A * Bt for a tall A stored M x K (K a multiple of 4), and - second
+// kernel, further down - At * B for an A stored K x M.
 //
-// A wave owns 32 rows of A and the whole 32 x 32 block of C.  Per step it takes 64 k: its 32 x 64
+// Tall A: a wave owns 32 rows of A and the whole 32 x 32 block of C.  Per step it takes 64 k: its 32 x 64
 // block of A comes in with eight loads per lane that each read 256 contiguous bytes of four rows,
 // goes through a wave-private LDS block and comes back as the instruction's A operand; B waits in
 // the workspace as Bt[32][K'] (column-major, zero beyond N and K) and its 32 x 64 block takes
@@ -17,7 +18,8 @@
 // N up to 16 (5.9-6.0 TB/s of A) on the 16 x 16 x 4 instruction, 213-240 us for 17..32 columns
 // (4.5-5.0 TB/s) on the 32 x 32 x 2 one, where the matrix pipes are busy 61 % of the time a CU holds
 // the kernel and a CU holds it 77 % of the kernel's time (every workgroup is resident at once, and
-// they do not finish together).
+// they do not finish together).  Loading B as it is stored instead of packing it first (four scalar
+// loads per lane and step) saved the pack launch and cost more than that: 32 columns 225 -> 261 us.
 #include "gemm_tile.hpp"
 
 namespace slhip {
@@ -198,10 +200,132 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
   }
 }
 
+// C = At * B for an A stored K x M (the large operand: read once) and a B of at most 16 columns, stored
+// K x N or N x K: the weight gradient of a narrow layer.  Both operands go from global memory straight into
+// the 16 x 16 x 4 instruction, no LDS on the way: lane (i, kk) = (lane % 16, lane / 16) loads the
+// float4 A[k0 + kk][m0 + 4 i .. + 3] - a wave's load instruction reads 256 contiguous bytes of four
+// k rows - and component t of it is the A operand of the t-th of four instructions, whose block of C
+// is therefore the rows m0 + 4 i + t, i = 0..15; the B operand of all four is B[k0 + kk][lane % 16].
+// A workgroup owns 64 columns of A (rows of C) and one share of K; its four waves take the steps of
+// four k in turn and add up through LDS, wave 0 first; shares of K combine in the split-K kernel.
+// (Combining in the same launch - the workgroup that draws a row block's last ticket adds the
+// shares up - was built and measured: the device-scope release it needs costs more than the second
+// launch, 2048 x 10 x 8192 19 -> 29 us with one fence per workgroup over write-through stores, 81 us
+// with one per wave.)
+constexpr int TT_STEPS = 8;  // loads in flight per wave: 8 KiB of A
+
+__global__ __launch_bounds__(256) void gemm_tall_t_kernel(GemmArgs g, size_t k_share, int tb) {
+  __shared__ __attribute__((aligned(16))) float part[3][64][17];  // waves 1..3: [lane][16 accumulators], padded
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int i = lane & 15, kk = lane >> 4;
+  const size_t M = g.M, K = g.K;
+  const int N = (int)g.N;
+  const size_t m0 = (size_t)blockIdx.x * 64;
+  const size_t kbeg = (size_t)blockIdx.y * k_share;
+  const size_t kend = kbeg + k_share < K ? kbeg + k_share : K;
+  const size_t m = m0 + 4 * i;
+  const bool m_ok = m < M;  // M is a multiple of 4: the vector lies inside the row or beyond it
+  const bool c_ok = i < N;
+  const float* ap = g.A + (m_ok ? m : 0);
+  // B stored K x N, or (tb) N x K: element (k, c) at k * bk + c * bc
+  const size_t bk = tb ? 1 : (size_t)N, bc = tb ? K : 1;
+  const float* bp = g.B + (c_ok ? i * bc : 0);
+
+  floatx4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[t][v] = 0.0f;
+
+  // wave w takes the steps w, w + 4, ... of its share; step s covers the rows kbeg + 4 s .. + 3
+  const size_t steps = (kend - kbeg + 3) / 4;
+  // One set of loads at a time: with a second set requested before the first is multiplied the
+  // kernel needs 112 VGPRs instead of 74, holds half the waves and measured 3-20 % slower.
+  float4 a[TT_STEPS];
+  float b[TT_STEPS];
+  for (size_t s0 = w; s0 < steps; s0 += 4 * TT_STEPS) {
+#pragma unroll
+    for (int u = 0; u < TT_STEPS; ++u) {
+      const size_t k = kbeg + 4 * (s0 + 4 * (size_t)u) + kk;
+      const bool k_ok = s0 + 4 * (size_t)u < steps && k < kend;
+      const size_t kc = k_ok ? k : kbeg;
+      a[u] = ld4s(ap + kc * M);
+      b[u] = bp[kc * bk];
+      if (!k_ok || !m_ok) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!k_ok || !c_ok) b[u] = 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < TT_STEPS; ++u) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].x, b[u], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].y, b[u], acc[1], 0, 0, 0);
+      acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].z, b[u], acc[2], 0, 0, 0);
+      acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].w, b[u], acc[3], 0, 0, 0);
+    }
+  }
+  if (w) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) part[w - 1][lane][4 * t + v] = acc[t][v];
+  }
+  __syncthreads();
+  const bool raw = gridDim.y > 1;
+  if (w == 0) {
+#pragma unroll
+    for (int o = 0; o < 3; ++o)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[t][v] += part[o][lane][4 * t + v];
+
+    // register v of block t in lane (i, kk): row m0 + 4 * (4 kk + v) + t of C, column i
+    if (c_ok) {
+      float* dst = raw ? g.partial + (size_t)blockIdx.y * M * (size_t)N : g.C;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const size_t row = m0 + 4 * (4 * kk + v) + t;
+          if (row >= M) continue;
+          const size_t at = row * (size_t)N + i;
+          float x = acc[t][v];
+          if (!raw) {
+            if (g.mask) x = (g.mask[at] >= 0.0f ? 1.0f : 0.0f) * x;
+            if (g.beta != 0.0f) x = g.beta * g.C[at] + x;
+            if (g.bias) x = x + g.bias[i];
+            if (g.pre_act) g.pre_act[at] = x;
+            if (g.relu) x = (x >= 0.0f ? 1.0f : 0.0f) * x;
+          }
+          dst[at] = x;
+        }
+    }
+  }
+}
+
 // Returns 0 if the product is not this kernel's, 1 if it ran to completion (*rc = status), 2 if
 // partials of g.splits k ranges wait in the workspace for the split-K combine.
 int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc) {
   const size_t M = g.M, N = g.N, K = g.K;
+  // At * B with 8..16 columns, A in whole 128-byte lines per row piece.  Against the narrow-N kernel:
+  // 2048 x 10 x 8192 24.5 -> 19.1 us, 16384 x 10 / 16 x 16384 220 / 234 -> 172 / 177 (6.3 / 6.1 TB/s),
+  // 2048 x 16 x 2048 16.6 -> 10.1, 256 x 16 x 262144 94 -> 65, 65536 x 10 x 1024 60 -> 46; with 4..7
+  // columns the two are level (ahead on some shapes, behind on others) and the other one stays.
+  if (ta && N <= 16 && N >= 8 && M % 32 == 0 && M >= 64 && K >= 64 && M * K >= (size_t(1) << 22)) {
+    const size_t gx = (M + 63) / 64;
+    if (gx > 0x7fffffffu) return 0;
+    // two workgroups per CU; every wave of a share gets at least 8 steps of four k
+    size_t splits = ((size_t)ctx->num_cu * 2 + gx - 1) / gx;
+    if (splits > K / 128) splits = K / 128;
+    if (splits > 64) splits = 64;
+    if (splits > ctx->workspace_bytes / (M * N * sizeof(float))) splits = ctx->workspace_bytes / (M * N * sizeof(float));
+    if (splits < 1) splits = 1;
+    const size_t share = ((K + splits - 1) / splits + 3) / 4 * 4;
+    splits = (K + share - 1) / share;
+    g.splits = (unsigned)splits;
+    hipLaunchKernelGGL(gemm_tall_t_kernel, dim3((unsigned)gx, (unsigned)splits), dim3(256), 0, ctx->stream, g, share, tb ? 1 : 0);
+    *rc = post_launch();
+    return splits > 1 && *rc == SLHIP_OK ? 2 : 1;
+  }
   // Against the sixteen-block kernel (which is bound by the matrix pipes from 13 columns on:
   // 16384 x 16 x 16384 takes it 377 us, this one 182): ahead at 8 columns and more wherever K is
   // long enough to amortise the pack and the combine (16384 x 8 / 10 / 12 x 16384: 253 / 223 / 242

@@ -254,6 +254,33 @@ def test_gemm_tall_kernel(hip, orc):
     assert np.all(np.isinf(got[7])) and np.all(np.isfinite(np.delete(got, 7, axis=0)))
 
 
+def test_gemm_transposed_tall_operand_with_narrow_b(hip, orc):
+    """At * B and At * Bt with A stored K x M and 8..16 columns of B (the weight gradient of a narrow
+    layer): the kernel that feeds both operands from global memory into the 16 x 16 x 4 instruction.
+    M on and off the multiples of 64, K off the multiples of 4 and of a share, one share and many,
+    beta and the mask epilogue; the same sums whichever way B is stored and on every run."""
+    for (m, n, k) in [(2048, 10, 8192), (96, 16, 70001), (4096, 8, 1030), (64, 13, 65536), (65536, 9, 65), (8192, 12, 2048),
+                      (1056, 11, 4099)]:
+        a, b = gemm_operands(1, 0, m, n, k)
+        exact, bound = gemm_bound(1, 0, m, n, k, a, b)
+        say("At*B, narrow B", m, n, k)
+        got = hip.sgemm(1, 0, m, n, k, a, b)
+        assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+        assert np.array_equal(got, hip.sgemm(1, 0, m, n, k, a, b))
+        bt = np.ascontiguousarray(b.reshape(k, n).T).ravel()
+        assert np.array_equal(got, hip.sgemm(1, 1, m, n, k, a, bt))
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        assert np.array_equal(hip.sgemm(1, 0, m, n, k, a, b, c=c0.copy(), beta=1.0), got + c0)
+        pre = rng.uniform(m * n, -1, 1, tag=4, seed=SEED)
+        assert np.array_equal(hip.sgemm_relu_mask(1, 0, m, n, k, a, b, pre), np.where(pre >= 0, got, 0 * got))
+    m, n, k = 128, 16, 40000
+    a, b = gemm_operands(1, 0, m, n, k)
+    a = a.copy()
+    a[(k - 1) * m + 77] = np.inf          # the last k of output row 77: it must stay in row 77
+    got = hip.sgemm(1, 0, m, n, k, a, b).reshape(m, n)
+    assert np.all(np.isinf(got[77])) and np.all(np.isfinite(np.delete(got, 77, axis=0)))
+
+
 def test_gemm_narrow_b_stored_transposed(hip, orc):
     """A narrow B handed over as N x K (A*Bt, At*Bt with N <= 16): turned into K x N in the workspace
     and run through the narrow-N kernels; results within the GEMM bound, beta and the epilogues too."""
