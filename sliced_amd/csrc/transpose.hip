@@ -10,11 +10,13 @@
 // (rows >= 16 cols) walk the tiles in groups of 8 tile rows instead, so that the workgroups in
 // flight also spread over the columns: [131072 x 1024] 4.5 -> 5.6 TB/s, [65536 x 2048] 4.7 -> 5.3;
 // squarer and wide shapes measured up to 10 % slower that way and keep the plain order.
-// Tall matrices of 256 columns and more (4 cols <= rows < 64 cols) and wide ones of 64, 128 or 192 rows take
-// the mirrored tile, 64 input rows x 256 input columns (1 KiB read pieces, 256-byte write bursts),
-// walked along the input rows' direction in groups of 8 tile columns: measured at 2^27 elements,
-// [32768 x 4096] 5.1 -> 5.6 TB/s, [65536 x 2048] 5.35 -> 5.65, [128 x 2^20] 4.7 (chunk kernel) -> 5.9;
-// squarer and wide shapes are 5-10 % slower with it ([16384 x 16384] 5.7 against 6.2).
+// Tall matrices of 2048, 3072 or 4096 columns (4 cols <= rows < 64 cols, output rows on 64-byte
+// boundaries) and wide ones of 64, 128 or 192 rows take the mirrored tile, 64 input rows x 256 input
+// columns (1 KiB read pieces, 256-byte write bursts), walked along the input rows' direction in
+// groups of 8 tile columns: measured at 2^27 elements, [32768 x 4096] 4.85 -> 5.6 TB/s, [65536 x 2048]
+// 5.25 -> 5.65, [128 x 2^20] 4.7 (chunk kernel) -> 5.9.  It pays where the input pitch is 8 or 16 KiB;
+// other widths, squarer and wide shapes are 5-25 % slower with it ([16384 x 16384] 5.7 against 6.2,
+// [30000 x 4000] 4.3 against 5.4).
 // 8 B/element of HBM traffic, the algorithmic minimum.  beta selects `=` (0) or `+=` (1).
 #include "common.hpp"
 
@@ -380,8 +382,15 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
 #undef SL_TN
     return post_launch();
   }
-  // The mirrored tile for tall matrices and for wide ones of 64, 128 or 192 rows (see the header)
-  if (mirrored_rows || (rows >= 4 * cols && rows < 64 * cols && cols >= 256)) {  // (taller still: the 256 x 64 tile in groups of 8 tile rows measures 2-3 % faster)
+  // The mirrored tile for wide matrices of 64, 128 or 192 rows and for tall ones of 2048, 3072 or 4096
+  // columns whose output rows start on 64-byte boundaries (see the header).  It is a remedy for
+  // input pitches of 8 and 16 KiB, where the 256 x 64 tile reads 256 pieces of 256 bytes that far
+  // apart ([32768 x 4096] 4.85 -> 5.64 TB/s, [65536 x 2048] 5.23 -> 5.68, [16384 x 2048] 4.6 -> 5.2);
+  // at any other width, and with output rows of odd length, the 256 x 64 tile with its 1 KiB write
+  // bursts is ahead ([30000 x 4000] 4.27 -> 5.38, [32768 x 4000] 4.66 -> 5.59, [30000 x 3840] 4.8 -> 5.7,
+  // [50000 x 5120] 4.9 -> 5.6, [32768 x 8192] 5.4 -> 6.0, [65521 x 2048] 3.3 -> 4.5, [50001 x 2001] 2.6 -> 4.1).
+  const bool mirrored_cols = rows >= 4 * cols && rows < 64 * cols && cols % 1024 == 0 && cols >= 2048 && cols <= 4096 && rows % 16 == 0;
+  if (mirrored_rows || mirrored_cols) {  // (taller still: the 256 x 64 tile in groups of 8 tile rows measures 2-3 % faster)
     const size_t tiles_r = (rows + 63) / 64, tiles_c = (cols + 255) / 256;
     SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
     const unsigned group = tiles_c < 8 ? (unsigned)tiles_c : 8u;

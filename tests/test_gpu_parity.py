@@ -691,7 +691,9 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              # narrow inputs whose output runs start off / on 64- and 128-byte boundaries (long sides odd, multiples
              # of 16 and of 32): shifted pieces with a halo, first and last chunks, pieces cut at both ends
              (50001, 100), (50016, 100), (50048, 100), (20001, 250), (20000, 250), (100003, 56), (100000, 33), (99984, 33),
-             (17, 3), (31, 10), (33, 10), (8209, 10), (1647, 10), (1648, 10), (1649, 10), (3301, 10), (40007, 72), (5000001, 3)]
+             (17, 3), (31, 10), (33, 10), (8209, 10), (1647, 10), (1648, 10), (1649, 10), (3301, 10), (40007, 72), (5000001, 3),
+             # tall matrices of 2048 columns: the mirrored tile (rows a multiple of 16) and the plain one beside it
+             (8192, 2048), (8208, 2048), (8200, 2048), (8193, 2048)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
