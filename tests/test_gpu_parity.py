@@ -621,6 +621,8 @@ SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (6
                   (6, 7), (5, 5), (300, 1001), (3, 4099), (3, 16387), (2, 40003), (4, 100001), (700, 6789),
                   # 1025..2048 vectors per row: the forward pass runs 512 lanes there, the backward pass 1024
                   (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196),
+                  # 257..448 vectors per row: the forward pass runs one wave per row with eight vectors a lane
+                  (9, 1028), (9, 1030), (6, 1500), (5, 1792), (5, 1795), (5, 1796), (7, 1281),
                   # many short rows, not a power of two long: the LDS-staged kernels
                   (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (4097, 37), (1024, 6),
                   # and short rows a power of two long, which take the same kernels
