@@ -287,22 +287,37 @@ __global__ __launch_bounds__(1024) void softmax_fwd_stream_kernel(size_t cols, c
   float* o = out + (size_t)blockIdx.x * cols;
   const size_t nv = cols >> 2;
   float m = -__builtin_huge_valf(), s = 0.0f;
-  for (size_t c = threadIdx.x; c < nv; c += 1024) {
-    const float4 t = ld4g(xr + 4 * c);
-    const float m4 = fmaxf(fmaxf(t.x, t.y), fmaxf(t.z, t.w));
-    if (m4 > m) {
-      s = s * expf(m - m4);
-      m = m4;
+  // four vectors of a thread in flight per trip (one at a time left the sweep at 4.0-4.4 TB/s)
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 t[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) t[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c0 + 1024 * u >= nv) break;
+      const float m4 = fmaxf(fmaxf(t[u].x, t[u].y), fmaxf(t[u].z, t[u].w));
+      if (m4 > m) {
+        s = s * expf(m - m4);
+        m = m4;
+      }
+      s += (expf(t[u].x - m) + expf(t[u].y - m)) + (expf(t[u].z - m) + expf(t[u].w - m));
     }
-    s += (expf(t.x - m) + expf(t.y - m)) + (expf(t.z - m) + expf(t.w - m));
   }
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) online_add(m, s, xr[c]);
   const float M = block_reduce<MaxOp>(m, smem);
   // threads that saw no element hold (m, s) = (-inf, 0): their term is 0, not exp(-inf + inf)
   const float S = block_reduce<SumOp>(s > 0.0f ? s * expf(m - M) : 0.0f, smem);
-  for (size_t c = threadIdx.x; c < nv; c += 1024) {
-    const float4 t = ld4g(xr + 4 * c);
-    st4s(o + 4 * c, make_float4(expf(t.x - M) / S, expf(t.y - M) / S, expf(t.z - M) / S, expf(t.w - M) / S));
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 t[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) t[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv)
+        st4s(o + 4 * (c0 + 1024 * u),
+             make_float4(expf(t[u].x - M) / S, expf(t[u].y - M) / S, expf(t[u].z - M) / S, expf(t[u].w - M) / S));
   }
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) o[c] = expf(xr[c] - M) / S;
 }
@@ -319,23 +334,174 @@ __global__ __launch_bounds__(1024) void softmax_bwd_stream_kernel(size_t cols, f
   float* xr = x_grad + base;
   const size_t nv = cols >> 2;
   float dot = 0.0f;
-  for (size_t c = threadIdx.x; c < nv; c += 1024) {
-    const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
-    dot += (rg.term(a.x, b.x) + rg.term(a.y, b.y)) + (rg.term(a.z, b.z) + rg.term(a.w, b.w));
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {  // four vectors of each tensor in flight per trip
+    float4 a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        a[u] = ld4g(sr + 4 * (c0 + 1024 * u));
+        b[u] = ld4g(gr + 4 * (c0 + 1024 * u));
+      }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv)
+        dot += (rg.term(a[u].x, b[u].x) + rg.term(a[u].y, b[u].y)) + (rg.term(a[u].z, b[u].z) + rg.term(a[u].w, b[u].w));
   }
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) dot += rg.term(sr[c], gr[c]);
   dot = block_reduce<SumOp>(dot, smem);
-  for (size_t c = threadIdx.x; c < nv; c += 1024) {
-    const float4 a = ld4g(sr + 4 * c), b = ld4g(gr + 4 * c);
-    float4 r = make_float4(rg.result(a.x, b.x, dot, kk), rg.result(a.y, b.y, dot, kk), rg.result(a.z, b.z, dot, kk),
-                           rg.result(a.w, b.w, dot, kk));
-    if (beta != 0.0f) {
-      const float4 p = ld4g(xr + 4 * c);
-      r = make_float4(beta * p.x + r.x, beta * p.y + r.y, beta * p.z + r.z, beta * p.w + r.w);
-    }
-    st4s(xr + 4 * c, r);
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 a[4], b[4], p[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        a[u] = ld4g(sr + 4 * (c0 + 1024 * u));
+        b[u] = ld4g(gr + 4 * (c0 + 1024 * u));
+        if (beta != 0.0f) p[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+      }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        float4 r = make_float4(rg.result(a[u].x, b[u].x, dot, kk), rg.result(a[u].y, b[u].y, dot, kk),
+                               rg.result(a[u].z, b[u].z, dot, kk), rg.result(a[u].w, b[u].w, dot, kk));
+        if (beta != 0.0f) r = make_float4(beta * p[u].x + r.x, beta * p[u].y + r.y, beta * p[u].z + r.z, beta * p[u].w + r.w);
+        st4s(xr + 4 * (c0 + 1024 * u), r);
+      }
   }
   for (size_t c = 4 * nv + threadIdx.x; c < cols; c += 1024) {
+    const float r = rg.result(sr[c], gr[c], dot, kk);
+    xr[c] = beta != 0.0f ? beta * xr[c] + r : r;
+  }
+}
+
+// Few rows, each far too long for a block (a softmax over one vector of 2^23 floats ran on one CU:
+// 0.4 TB/s): the row is cut into segments of `seg` floats (a multiple of 4), one block each.  The
+// first launch leaves every segment's running maximum and its sum of exponentials relative to it
+// (backward: its share of <s, g>) in `stats`; the second combines the row's segments - every block
+// for itself, all in the same order - and writes its own segment.
+__global__ __launch_bounds__(1024) void softmax_fwd_seg_stats_kernel(size_t cols, size_t seg, const float* __restrict__ x,
+                                                                     float* __restrict__ stats) {
+  __shared__ float smem[16];
+  const size_t beg = (size_t)blockIdx.x * seg, len = beg + seg <= cols ? seg : cols - beg;
+  const float* xr = x + (size_t)blockIdx.y * cols + beg;
+  const size_t nv = len >> 2;
+  float m = -__builtin_huge_valf(), s = 0.0f;
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 t[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) t[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (c0 + 1024 * u >= nv) break;
+      const float m4 = fmaxf(fmaxf(t[u].x, t[u].y), fmaxf(t[u].z, t[u].w));
+      if (m4 > m) {
+        s = s * expf(m - m4);
+        m = m4;
+      }
+      s += (expf(t[u].x - m) + expf(t[u].y - m)) + (expf(t[u].z - m) + expf(t[u].w - m));
+    }
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < len; c += 1024) online_add(m, s, xr[c]);
+  const float M = block_reduce<MaxOp>(m, smem);
+  const float S = block_reduce<SumOp>(s > 0.0f ? s * expf(m - M) : 0.0f, smem);
+  if (threadIdx.x == 0) {
+    float* st = stats + 2 * ((size_t)blockIdx.y * gridDim.x + blockIdx.x);
+    st[0] = M;
+    st[1] = S;
+  }
+}
+
+__global__ __launch_bounds__(1024) void softmax_fwd_seg_write_kernel(size_t cols, size_t seg, const float* __restrict__ x,
+                                                                     float* __restrict__ out, const float* __restrict__ stats) {
+  __shared__ float smem[16];
+  const float* st = stats + 2 * (size_t)blockIdx.y * gridDim.x;
+  float m = -__builtin_huge_valf();
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += 1024) m = fmaxf(m, st[2 * i]);
+  const float M = block_reduce<MaxOp>(m, smem);
+  float sum = 0.0f;
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += 1024) sum += st[2 * i + 1] > 0.0f ? st[2 * i + 1] * expf(st[2 * i] - M) : 0.0f;
+  const float S = block_reduce<SumOp>(sum, smem);
+  const size_t beg = (size_t)blockIdx.x * seg, len = beg + seg <= cols ? seg : cols - beg;
+  const float* xr = x + (size_t)blockIdx.y * cols + beg;
+  float* o = out + (size_t)blockIdx.y * cols + beg;
+  const size_t nv = len >> 2;
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 t[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) t[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv)
+        st4s(o + 4 * (c0 + 1024 * u),
+             make_float4(expf(t[u].x - M) / S, expf(t[u].y - M) / S, expf(t[u].z - M) / S, expf(t[u].w - M) / S));
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < len; c += 1024) o[c] = expf(xr[c] - M) / S;
+}
+
+template <class RG>
+__global__ __launch_bounds__(1024) void softmax_bwd_seg_stats_kernel(size_t cols, size_t seg, const float* __restrict__ out,
+                                                                     const float* __restrict__ out_grad,
+                                                                     float* __restrict__ stats, RG rg) {
+  __shared__ float smem[16];
+  const size_t beg = (size_t)blockIdx.x * seg, len = beg + seg <= cols ? seg : cols - beg;
+  const size_t base = (size_t)blockIdx.y * cols + beg;
+  const float* sr = out + base;
+  const float* gr = out_grad + base;
+  const size_t nv = len >> 2;
+  float dot = 0.0f;
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        a[u] = ld4g(sr + 4 * (c0 + 1024 * u));
+        b[u] = ld4g(gr + 4 * (c0 + 1024 * u));
+      }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv)
+        dot += (rg.term(a[u].x, b[u].x) + rg.term(a[u].y, b[u].y)) + (rg.term(a[u].z, b[u].z) + rg.term(a[u].w, b[u].w));
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < len; c += 1024) dot += rg.term(sr[c], gr[c]);
+  dot = block_reduce<SumOp>(dot, smem);
+  if (threadIdx.x == 0) stats[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = dot;
+}
+
+template <class RG>
+__global__ __launch_bounds__(1024) void softmax_bwd_seg_write_kernel(size_t cols, size_t seg, float* x_grad,
+                                                                     const float* __restrict__ out, const float* out_grad,
+                                                                     float beta, const float* __restrict__ stats, RG rg) {
+  __shared__ float smem[16];
+  const float kk = rg.k();
+  float part = 0.0f;
+  for (unsigned i = threadIdx.x; i < gridDim.x; i += 1024) part += stats[(size_t)blockIdx.y * gridDim.x + i];
+  const float dot = block_reduce<SumOp>(part, smem);
+  const size_t beg = (size_t)blockIdx.x * seg, len = beg + seg <= cols ? seg : cols - beg;
+  const size_t base = (size_t)blockIdx.y * cols + beg;
+  const float* sr = out + base;
+  const float* gr = out_grad + base;
+  float* xr = x_grad + base;
+  const size_t nv = len >> 2;
+  for (size_t c0 = threadIdx.x; c0 < nv; c0 += 4096) {
+    float4 a[4], b[4], p[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        a[u] = ld4g(sr + 4 * (c0 + 1024 * u));
+        b[u] = ld4g(gr + 4 * (c0 + 1024 * u));
+        if (beta != 0.0f) p[u] = ld4g(xr + 4 * (c0 + 1024 * u));
+      }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (c0 + 1024 * u < nv) {
+        float4 r = make_float4(rg.result(a[u].x, b[u].x, dot, kk), rg.result(a[u].y, b[u].y, dot, kk),
+                               rg.result(a[u].z, b[u].z, dot, kk), rg.result(a[u].w, b[u].w, dot, kk));
+        if (beta != 0.0f) r = make_float4(beta * p[u].x + r.x, beta * p[u].y + r.y, beta * p[u].z + r.z, beta * p[u].w + r.w);
+        st4s(xr + 4 * (c0 + 1024 * u), r);
+      }
+  }
+  for (size_t c = 4 * nv + threadIdx.x; c < len; c += 1024) {
     const float r = rg.result(sr[c], gr[c], dot, kk);
     xr[c] = beta != 0.0f ? beta * xr[c] + r : r;
   }
@@ -489,7 +655,7 @@ struct SoftmaxCfg {
   int items;
 };
 
-static SoftmaxCfg pick_cfg(size_t colsv, bool fwd) {
+static SoftmaxCfg pick_cfg(size_t colsv, bool fwd, bool long_rows) {
   if (colsv <= 256) {
     int lanes = 1;
     while ((size_t)lanes * 4 < colsv) lanes <<= 1;
@@ -506,6 +672,17 @@ static SoftmaxCfg pick_cfg(size_t colsv, bool fwd) {
   // measured the other way round (6.1-6.3 against 5.7-5.8)
   if (fwd && colsv <= 2048) return {512, 4};
   if (colsv <= 4096) return {1024, 4};
+  // Rows of 16388..32768 floats still fit the registers of a block: 512 lanes with sixteen vectors each
+  // forward (two rows a CU), 1024 lanes with eight vectors of each tensor backward.  Against the
+  // two-sweep kernels below: rows of 20000 floats 4.5 -> 5.7 TB/s forward, 4.3 -> 6.0 backward; 32768:
+  // 4.5 -> 5.8, 4.2 -> 6.0.  Forward rows of 40000..65536 floats take 1024 lanes with sixteen vectors,
+  // one row a CU, which gains less (50257: 4.3 -> 4.55, 65536: 4.4 -> 4.8) and loses just above 32768,
+  // where half the lanes idle (33333: 4.4 -> 4.1).
+  if (long_rows) {
+    if (fwd && colsv <= 8192) return {512, 16};
+    if (fwd && colsv > 10000 && colsv <= 16384) return {1024, 16};
+    if (!fwd && colsv <= 8192) return {1024, 8};
+  }
   return {0, 0};
 }
 
@@ -540,12 +717,33 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
     return post_launch();
   }
   const size_t colsv = cols / (VEC ? 4 : 1);
-  SoftmaxCfg cfg = pick_cfg(colsv, FWD);
+  SoftmaxCfg cfg = pick_cfg(colsv, FWD, VEC && !CCE);
   SLHIP_REQUIRE(rows <= MAX_GRID, "too many rows for one launch");
   if (cfg.lanes == 0) {
     if (CCE) {  // rows too long for registers: the caller splits the work
       set_error("softmax with cross-entropy: rows of %zu floats do not fit the one-pass kernels", cols);
       return SLHIP_EINVAL;
+    }
+    // fewer rows than would fill the chip: segments of 64 Ki floats and more, four blocks per CU in all
+    if (rows < (size_t)ctx->num_cu * 2 && cols >= (size_t(1) << 17)) {
+      size_t nseg = ((size_t)ctx->num_cu * 4 + rows - 1) / rows;
+      if (nseg > cols >> 16) nseg = cols >> 16;
+      if (nseg > 65535) nseg = 65535;
+      const size_t seg = ((cols + nseg - 1) / nseg + 3) & ~(size_t)3;
+      nseg = (cols + seg - 1) / seg;
+      if (nseg > 1 && rows * nseg * 2 * sizeof(float) <= ctx->workspace_bytes) {
+        float* stats = (float*)ctx->workspace;
+        const dim3 grid((unsigned)nseg, (unsigned)rows);
+        if (FWD) {
+          hipLaunchKernelGGL(softmax_fwd_seg_stats_kernel, grid, dim3(1024), 0, ctx->stream, cols, seg, x, stats);
+          hipLaunchKernelGGL(softmax_fwd_seg_write_kernel, grid, dim3(1024), 0, ctx->stream, cols, seg, x, out, (const float*)stats);
+        } else {
+          hipLaunchKernelGGL((softmax_bwd_seg_stats_kernel<RG>), grid, dim3(1024), 0, ctx->stream, cols, seg, s, g, stats, rg);
+          hipLaunchKernelGGL((softmax_bwd_seg_write_kernel<RG>), grid, dim3(1024), 0, ctx->stream, cols, seg, x_grad, s, g, beta,
+                             (const float*)stats, rg);
+        }
+        return post_launch();
+      }
     }
     if (FWD) hipLaunchKernelGGL(softmax_fwd_stream_kernel, dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x, out);
     else hipLaunchKernelGGL((softmax_bwd_stream_kernel<RG>), dim3((unsigned)rows), dim3(1024), 0, ctx->stream, cols, x_grad, s, g, beta, rg);
@@ -563,17 +761,23 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
                          rows, cols, x_grad, s, g, beta, rg);                                                        \
   } while (0)
 #define SL_SM(L, I)                                  \
-  case L:                                            \
+  case (L) * 32 + (I):                               \
     if (VEC && (cols & 3)) SL_SM2(L, I, true);       \
     else SL_SM2(L, I, false);                        \
     break;
-  switch (cfg.lanes) {
-    SL_SM(1, 4) SL_SM(2, 4) SL_SM(4, 4) SL_SM(8, 4) SL_SM(16, 4) SL_SM(32, 4) SL_SM(256, 4) SL_SM(512, 4) SL_SM(1024, 4)
-    case 64:
-      if (cfg.items == 8) { if (VEC && (cols & 3)) SL_SM2(64, 8, true); else SL_SM2(64, 8, false); }
-      else { if (VEC && (cols & 3)) SL_SM2(64, 4, true); else SL_SM2(64, 4, false); }
-      break;
+  // (the long-row forms hold 64 floats of the row per lane: not compiled for the scalar and the cross-entropy forms)
+#define SL_SML(L, I)                                 \
+  case (L) * 32 + (I):                               \
+    if constexpr (VEC && !CCE) {                     \
+      if (cols & 3) SL_SM2(L, I, true);              \
+      else SL_SM2(L, I, false);                      \
+    }                                                \
+    break;
+  switch (cfg.lanes * 32 + cfg.items) {
+    SL_SM(1, 4) SL_SM(2, 4) SL_SM(4, 4) SL_SM(8, 4) SL_SM(16, 4) SL_SM(32, 4) SL_SM(64, 4) SL_SM(64, 8) SL_SM(256, 4) SL_SM(512, 4)
+    SL_SM(1024, 4) SL_SML(512, 16) SL_SML(1024, 16) SL_SML(1024, 8)
   }
+#undef SL_SML
 #undef SL_SM
 #undef SL_SM2
   return post_launch();
