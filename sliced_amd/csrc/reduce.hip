@@ -95,24 +95,32 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
   if (active) {
     const size_t xr = row * cols;
     const float vv = Src::HAS_V ? src.bvalue(row) : 0.0f;
-    size_t c = cbeg + lane;
     if (VEC) {
-      for (; c + 3 * LANES < cend; c += 4 * LANES) {
-        float4 v0 = src.vec(xr + 4 * c, vv, vv, vv, vv), v1 = src.vec(xr + 4 * (c + LANES), vv, vv, vv, vv),
-               v2 = src.vec(xr + 4 * (c + 2 * LANES), vv, vv, vv, vv), v3 = src.vec(xr + 4 * (c + 3 * LANES), vv, vv, vv, vv);
+      // Four vectors a lane and trip, requested together, in one loop without a branch in it: a lane
+      // whose trip holds fewer than four loads the row's last vector again instead and drops it.  (A
+      // loop of whole trips with a tail that took the leftovers one by one waited for each of them,
+      // and lanes of one wave that split between loop and tail ran both in turn: rows of 255 floats
+      // 4.1 TB/s against 6.2 for rows of 257, whose 64 vectors are one whole trip for every lane;
+      // tests around the loads instead of selects behind them cost max_cols 15-30 % on rows of 129,
+      // 257, 513 and 1025.  Now 161: 4.2 -> 5.6, 200: 4.6 -> 6.7, 255: 5.2, 300: 5.2 -> 6.9, 500: 5.4 ->
+      // 6.7, 1000: 5.5 -> 6.4, 16384: 6.8 -> 7.0.)
+      const float id = Op::identity();
+      const size_t last = cend - 1;
+      for (size_t c = cbeg + lane; c < cend; c += 4 * LANES) {
+        const size_t c1 = c + LANES, c2 = c + 2 * LANES, c3 = c + 3 * LANES;
+        const bool h1 = c1 < cend, h2 = c2 < cend, h3 = c3 < cend;
+        const float4 v0 = src.vec(xr + 4 * c, vv, vv, vv, vv), v1 = src.vec(xr + 4 * (h1 ? c1 : last), vv, vv, vv, vv),
+                     v2 = src.vec(xr + 4 * (h2 ? c2 : last), vv, vv, vv, vv), v3 = src.vec(xr + 4 * (h3 ? c3 : last), vv, vv, vv, vv);
         a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
-        a1 = Op::apply(a1, Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)));
-        a2 = Op::apply(a2, Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)));
-        a3 = Op::apply(a3, Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)));
-      }
-      for (; c < cend; c += LANES) {
-        float4 v0 = src.vec(xr + 4 * c, vv, vv, vv, vv);
-        a0 = Op::apply(a0, Op::apply(Op::apply(v0.x, v0.y), Op::apply(v0.z, v0.w)));
+        a1 = Op::apply(a1, h1 ? Op::apply(Op::apply(v1.x, v1.y), Op::apply(v1.z, v1.w)) : id);
+        a2 = Op::apply(a2, h2 ? Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)) : id);
+        a3 = Op::apply(a3, h3 ? Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)) : id);
       }
       // a row of odd length ends in up to 3 floats beyond its last whole vector
       if ((cols & 3) && seg == nseg - 1 && lane == 0)
         for (size_t e = 4 * colsv; e < cols; ++e) a1 = Op::apply(a1, src.one(xr + e, vv));
     } else {
+      size_t c = cbeg + lane;
       for (; c + 3 * LANES < cend; c += 4 * LANES) {
         a0 = Op::apply(a0, src.one(xr + c, vv));
         a1 = Op::apply(a1, src.one(xr + c + LANES, vv));

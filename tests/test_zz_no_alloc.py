@@ -56,8 +56,18 @@ def test_static_variant_neither_uses_the_workspace_nor_allocates(hip):
     """The context workspace, where slhip_sum_rows keeps its partials, is filled with NaN before the
     call: a result that still has the bits of slhip_sum_rows did not pass through it.  Free device
     memory is the same before and after the calls."""
-    import torch
     c = hip.ctx()
+    # free device memory as the HIP runtime the library itself runs on sees it (the library has loaded it:
+    # this is the same instance, not a second runtime in the process)
+    rt = C.CDLL("libamdhip64.so.7", mode=C.RTLD_GLOBAL)
+    rt.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    rt.hipMemGetInfo.restype = C.c_int
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert rt.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
     rows, cols = 16384, 2049                    # two streaming stages: partials must live somewhere
     x = rng.uniform(rows * cols, -10, 10, tag=30, seed=SEED)
     want = hip.sum_rows(cols, x)
@@ -68,12 +78,12 @@ def test_static_variant_neither_uses_the_workspace_nor_allocates(hip):
     assert ws.value and ws_floats >= (1 << 20)
     c.call("slhip_fill", ws_floats, float("nan"), ws.value)
     c.sync()
-    torch.cuda.mem_get_info(0)                  # the first query sets the runtime's own bookkeeping up
-    free0 = torch.cuda.mem_get_info(0)[0]
+    free_bytes()                                # the first query sets the runtime's own bookkeeping up
+    free0 = free_bytes()
     for _ in range(3):
         c.call("slhip_sum_rows_static", rows, cols, dx.ptr, out.ptr)
     c.sync()
-    assert torch.cuda.mem_get_info(0)[0] == free0
+    assert free_bytes() == free0
     got = out.numpy()
     assert not np.isnan(got).any() and np.array_equal(got, want)
     # the control: the workspace variant does read what the poisoned workspace holds only after
