@@ -693,12 +693,17 @@ static int32_t softmax_dispatch(slhip_ctx* ctx, size_t rows, size_t cols, const 
   // many short rows (measured at 2^27 elements, forward / backward TB/s, lanes-per-row kernel -> this
   // one: 10: 3.1 / 2.8 -> 5.8 / 6.1; 36: 2.2 / 2.9 -> 5.3 / 5.4; 100: 3.0 / 3.6 -> 4.8 / 5.2; 8: 3.3 / 4.0 ->
   // 5.9 / 6.1; 16: 1.4 / 1.8 -> 6.2 / 6.1; 32: 1.8 / 2.5 -> 5.6 / 6.2; 64: 4.9 / 5.2 -> 5.6 / 6.2; rows of 2 only
-  // backward: 4.6 / 5.6 -> 4.0 / 6.1; at 128 and from 200 on the lanes-per-row kernel is the faster one)
-  if (cols >= (FWD ? 3 : 2) && cols <= 160 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {
+  // backward: 4.6 / 5.6 -> 4.0 / 6.1; 161: 4.5 / 4.35 -> 4.7 / 5.6; 200: 4.7 / 5.05 -> 4.8 / 5.8; 255: 4.1 / 4.2 -> 5.2 /
+  // 5.0; at 128, 256 and from 257 on the lanes-per-row kernel is the faster one)
+  if (cols >= (FWD ? 3 : 2) && cols <= 256 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {
     int rpb = SS_CHUNK / (int)cols;
-    const int g32 = 32 / std::gcd((int)cols, 32);  // chunks start on 128-byte boundaries
+    // chunks start on 128-byte boundaries of the tensors, or on 64-byte ones where a chunk holds too few
+    // rows for that (rows of 129..255 floats of odd length: 16 of them); a 64-byte block that two
+    // workgroups each write a part of costs the write side a sixth of its rate and more
+    const int g32 = 32 / std::gcd((int)cols, 32), g16 = 16 / std::gcd((int)cols, 16);
     if (rpb >= 256) rpb -= rpb % 256;  // every thread of the row phase busy
     else if (rpb >= g32) rpb -= rpb % g32;
+    else if (rpb >= g16) rpb -= rpb % g16;
     int lanes = 1;
     while (lanes < 64 && lanes * 2 * rpb <= 256) lanes <<= 1;  // groups of `lanes` lanes, at least one per row of the chunk
     const size_t blocks = (rows + rpb - 1) / rpb;

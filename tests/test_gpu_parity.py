@@ -627,7 +627,7 @@ SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (6
                   # 257..448 vectors per row: the forward pass runs one wave per row with eight vectors a lane
                   (9, 1028), (9, 1030), (6, 1500), (5, 1792), (5, 1795), (5, 1796), (7, 1281),
                   # many short rows, not a power of two long: the LDS-staged kernels
-                  (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (4097, 37), (1024, 6),
+                  (5000, 10), (1025, 100), (3000, 3), (1500, 159), (2000, 160), (1100, 161), (1030, 255), (1024, 129), (1500, 200), (1040, 254), (1027, 131), (4097, 37), (1024, 6),
                   # and short rows a power of two long, which take the same kernels
                   (3000, 16), (1100, 64), (5000, 2), (2049, 32), (1030, 8), (4100, 4), (1023, 16)]
 
