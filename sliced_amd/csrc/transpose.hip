@@ -143,6 +143,118 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
   }
 }
 
+// The 256 x 64 tile for large matrices whose output rows do not start on 64-byte boundaries (rows
+// not a multiple of 16, or an output that starts off the grid).  What a tile writes of output row c
+// is then not the floats [r0, r0 + 256) but the piece [r0 - d_c, r0 + 256 - d_c), d_c < 16 chosen per
+// output row so that the piece starts and ends on 64-byte boundaries of the output: a 64-byte block
+// that two tiles each write a part of reaches the memory as two partial writes (see the chunk kernel
+// below, which does the same), and every vector store is aligned.  The tile stages 16 rows more than
+// it writes, which the tile above it stages too.  The pieces at the two ends of an output row are
+// cut there; what lies before a piece's first aligned vector and behind its last whole one goes
+// float by float, thread c for output row c.  Same LDS layout as above: lane l of a wave fetches
+// the rows s + 4 l .. s + 4 l + 3 of one column, whatever s, and meets no bank twice.
+// [13421 x 10000] 3.9 -> 4.7 TB/s, [65521 x 2048] 4.45 -> 5.15, [134217 x 1000] 4.1 -> 4.6, [16383 x 16385]
+// 4.1 -> 4.5, [12345 x 6789] 3.95 -> 4.2; matrices of a few million elements lose (3001 x 3003: 28 -> 32 us)
+// and keep the plain tile.  (Without the unconditional loads of a whole tile - the `full` path - the
+// same kernel measured 3-12 % behind the plain tile on every shape.)
+template <bool ACC>
+__global__ __launch_bounds__(256) void transpose_shift_kernel(size_t rows, size_t cols, const float* __restrict__ x,
+                                                              float* out, unsigned tiles_r, unsigned group) {
+  constexpr int TR = 256, TC = 64, H = 16, LR = TR + H;
+  __shared__ float tile_mem[LR * (TC + 1) + 52];
+  auto tile = [&](int r, int c) -> float& { return tile_mem[((r & 3) * (LR / 4) + (r >> 2)) * (TC + 1) + c + 17 * (r & 3)]; };
+  const unsigned tiles_c = gridDim.x / tiles_r;
+  const unsigned in_group = group * tiles_c;
+  const unsigned first = blockIdx.x / in_group * group;
+  const unsigned gsize = tiles_r - first < group ? tiles_r - first : group;
+  const unsigned local = blockIdx.x % in_group;
+  const size_t tr = first + local % gsize, tc = local / gsize;
+  const size_t r0 = tr * TR, c0 = tc * TC;
+  const size_t rb = r0 >= H ? r0 - H : 0;  // the first staged row: the first tile row has nothing above it
+  const int staged = (int)(r0 - rb) + TR;  // rows rb .. rb + staged - 1, as far as the matrix goes
+  const int t = threadIdx.x;
+  {
+    constexpr int LPR = TC / 4, RPP = 256 / LPR, NP = LR / RPP;  // float4 per tile row, rows per pass, passes
+    const int lx = t % LPR, ly = t / LPR;
+    float4 v[NP];
+    const bool full = staged == LR && rb + LR <= rows && c0 + TC <= cols;
+    if (full) {
+#pragma unroll
+      for (int p = 0; p < NP; ++p) v[p] = ld4s(x + (rb + ly + RPP * p) * cols + c0 + 4 * lx);
+    } else {
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        const int rr = ly + RPP * p;
+        const size_t r = rb + rr, c = c0 + 4 * lx;
+        if (rr >= staged || r >= rows || c >= cols) {
+          v[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else if (c + 3 < cols) {
+          v[p] = ld4s(x + r * cols + c);
+        } else {
+          const float* xr = x + r * cols;
+          v[p] = make_float4(xr[c], c + 1 < cols ? xr[c + 1] : 0.f, c + 2 < cols ? xr[c + 2] : 0.f, 0.f);
+        }
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int rr = ly + RPP * p;
+      tile(rr, 4 * lx + 0) = v[p].x;
+      tile(rr, 4 * lx + 1) = v[p].y;
+      tile(rr, 4 * lx + 2) = v[p].z;
+      tile(rr, 4 * lx + 3) = v[p].w;
+    }
+  }
+  __syncthreads();
+  constexpr int NP = TC / 4;  // four output rows per pass, 64 lanes each
+  const int lx = t & 63, ly = t >> 6;
+  // everything in rows relative to the first staged one, in 32 bits
+  const int off = (int)(r0 - rb);  // H, or 0 in the first tile row
+  const int nst = rows - rb < (size_t)staged ? (int)(rows - rb) : staged;
+  const int ob = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & (H - 1)), lm = (int)(rows & (H - 1));
+  // the piece of output row c0 + cc: staged rows [lo, hi); returns the floats before its first aligned vector
+  auto piece = [&](int cc, int& lo, int& hi) {
+    const int d = (ob + (int)((c0 + cc) & (H - 1)) * lm) & (H - 1);  // (r0 is a multiple of 256)
+    lo = off > d ? off - d : 0;
+    hi = off + TR - d < nst ? off + TR - d : nst;
+    return lo ? 0 : (4 - (d & 3)) & 3;  // lo > 0: the piece starts on a 64-byte boundary
+  };
+  float* const obeg = out + rb;
+  float4 old[NP];
+  if (ACC) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int cc = ly + 4 * p;
+      int lo, hi;
+      const int l = piece(cc, lo, hi) + lo + 4 * lx;
+      old[p] = (c0 + cc < cols && l + 3 < hi) ? ld4s(obeg + (c0 + cc) * rows + l) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int cc = ly + 4 * p;
+    int lo, hi;
+    const int l = piece(cc, lo, hi) + lo + 4 * lx;
+    if (c0 + cc < cols && l + 3 < hi) {
+      float4 v = make_float4(tile(l, cc), tile(l + 1, cc), tile(l + 2, cc), tile(l + 3, cc));
+      if (ACC) { v.x += old[p].x; v.y += old[p].y; v.z += old[p].z; v.w += old[p].w; }
+      st4s(obeg + (c0 + cc) * rows + l, v);
+    }
+  }
+  // at most three floats before and three behind the vectors of a piece: thread c sees to output row c
+  if (t < TC && c0 + t < cols) {
+    int lo, hi;
+    int lead = piece(t, lo, hi) + lo;
+    if (lo < hi) {
+      if (lead > hi) lead = hi;
+      const int tail = lead + ((hi - lead) & ~3);
+      float* orow = obeg + (c0 + t) * rows;
+      for (int l = lo; l < lead; ++l) orow[l] = ACC ? orow[l] + tile(l, t) : tile(l, t);
+      for (int l = tail; l < hi; ++l) orow[l] = ACC ? orow[l] + tile(l, t) : tile(l, t);
+    }
+  }
+}
+
 // Matrices with few columns (or few rows): the tile above would be mostly empty.  A chunk of R whole
 // rows of the narrow matrix is one contiguous run of R*S floats (S = the short side) on the narrow
 // side and S runs of R floats on the other.  A workgroup moves one such chunk through LDS: both
@@ -399,6 +511,15 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     return post_launch();
   }
   constexpr int TR = 256, TC = 64;
+  // output rows that start off the 64-byte grid, 2^24 elements and more: pieces shifted per output row
+  if (cols >= 64 && rows >= 512 && len >= (size_t(1) << 24) && (rows % 16 != 0 || (reinterpret_cast<uintptr_t>(out) & 63) != 0)) {
+    const size_t tiles_r = (rows + 15 + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;  // the last piece of every output row ends inside the last tile row
+    SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
+    const unsigned group = rows >= 16 * cols ? (tiles_r < 8 ? (unsigned)tiles_r : 8u) : (unsigned)tiles_r;
+    if (acc) hipLaunchKernelGGL(transpose_shift_kernel<true>, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+    else hipLaunchKernelGGL(transpose_shift_kernel<false>, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+    return post_launch();
+  }
   const size_t tiles_r = (rows + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;
   SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
   const unsigned grid = (unsigned)(tiles_r * tiles_c);

@@ -698,7 +698,10 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (50001, 100), (50016, 100), (50048, 100), (20001, 250), (20000, 250), (100003, 56), (100000, 33), (99984, 33),
              (17, 3), (31, 10), (33, 10), (8209, 10), (1647, 10), (1648, 10), (1649, 10), (3301, 10), (40007, 72), (5000001, 3),
              # tall matrices of 2048 columns: the mirrored tile (rows a multiple of 16) and the plain one beside it
-             (8192, 2048), (8208, 2048), (8200, 2048), (8193, 2048)]
+             (8192, 2048), (8208, 2048), (8200, 2048), (8193, 2048),
+             # 2^24 elements and more with output rows off the 64-byte grid: the 256 x 64 tile with pieces shifted
+             # per output row (first and last tile rows, ragged tile columns, rows of odd length on both sides)
+             (4100, 4099), (16385, 1031), (1031, 16390), (65521, 257), (520, 32771)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
