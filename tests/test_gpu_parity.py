@@ -701,7 +701,7 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (8192, 2048), (8208, 2048), (8200, 2048), (8193, 2048),
              # 2^24 elements and more with output rows off the 64-byte grid: the 256 x 64 tile with pieces shifted
              # per output row (first and last tile rows, ragged tile columns, rows of odd length on both sides)
-             (4100, 4099), (16385, 1031), (1031, 16390), (65521, 257), (520, 32771)]
+             (8200, 2049), (16385, 1031), (8209, 2100), (65521, 257), (8193, 2050)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
