@@ -37,8 +37,11 @@ __device__ __forceinline__ float row_reduce(float v, float* smem) {
 // loss_rows[r] = -ln sum_c clip(p, 1e-7, 1 - 1e-7) * tg (reference: Matrix::softmax followed by cce,
 // examples/nn.rs:124-143); out may then be null (the probabilities are not stored).
 __device__ __forceinline__ float cce_term(float p, float t) { return fminf(fmaxf(p, (float)1e-7), (float)(1.0 - 1e-7)) * t; }
+// (512 lanes with sixteen vectors each: two rows a CU need four waves a SIMD, i.e. at most 128 VGPRs;
+// the form with a tail came out at 3 waves otherwise - rows of 20001 floats 3.8 TB/s against 5.6 for
+// rows of 20000)
 template <bool VEC, int LANES, int ITEMS, bool TAIL, bool CCE>
-__global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(size_t rows, size_t cols,
+__global__ __launch_bounds__(LANES <= 64 ? 256 : LANES, (LANES == 512 && ITEMS == 16) ? 4 : 1) void softmax_fwd_kernel(size_t rows, size_t cols,
                                                                                 const float* __restrict__ x,
                                                                                 float* __restrict__ out,
                                                                                 const float* __restrict__ tg,
@@ -94,12 +97,15 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
       }
     }
   }
-  // a row of odd length ends in up to 3 floats beyond its last whole vector: lane 0 takes them
+  // a row of odd length ends in up to 3 floats beyond its last whole vector
   const int rem = TAIL ? (int)(cols & 3) : 0;
-  const bool tail = TAIL && rem != 0 && active && lane == 0;
+  // (from four lanes a row on, lane q takes the q-th of them: one float each, no loop)
+  constexpr bool SPREAD = LANES >= 4;
+  const bool tail = TAIL && active && (SPREAD ? lane < rem : (rem != 0 && lane == 0));
+  const int tq0 = SPREAD ? lane : 0, tq1 = SPREAD ? lane + 1 : rem;  // this lane's share of the tail
   float tv[3] = {NEG_INF, NEG_INF, NEG_INF};
   if (tail)
-    for (int q = 0; q < rem; ++q) tv[q] = x[row * cols + 4 * colsv + q];
+    for (int q = tq0; q < tq1; ++q) tv[q - tq0] = x[row * cols + 4 * colsv + q];
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
@@ -120,9 +126,9 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
     }
   }
   if (tail)
-    for (int q = 0; q < rem; ++q) {
-      tv[q] = expf(tv[q] - m);
-      s += tv[q];
+    for (int q = tq0; q < tq1; ++q) {
+      tv[q - tq0] = expf(tv[q - tq0] - m);
+      s += tv[q - tq0];
     }
   s = row_reduce<SumOp, LANES>(s, smem + 16);
   // e * (1 / sum) where the reference divides by the sum: at most 1.5 ulp from the quotient.  The
@@ -137,13 +143,13 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_fwd_kernel(
 #pragma unroll
       for (int q = 0; q < V; ++q) acc += cce_term(scale(v[j][q]), w[j][q]);  // (elements outside the row: e = 0, t = 0)
     if (tail)
-      for (int q = 0; q < rem; ++q) acc += cce_term(scale(tv[q]), tg[row * cols + 4 * colsv + q]);
+      for (int q = tq0; q < tq1; ++q) acc += cce_term(scale(tv[q - tq0]), tg[row * cols + 4 * colsv + q]);
     acc = row_reduce<SumOp, LANES>(acc, smem);  // (every lane is past its reads of the first reduction)
     if (active && lane == 0) loss_rows[row] = -logf(acc);
     if (!out) return;
   }
   if (tail)
-    for (int q = 0; q < rem; ++q) out[row * cols + 4 * colsv + q] = scale(tv[q]);
+    for (int q = tq0; q < tq1; ++q) out[row * cols + 4 * colsv + q] = scale(tv[q - tq0]);
 
 #pragma unroll
   for (int j = 0; j < ITEMS; ++j) {
@@ -226,21 +232,24 @@ __global__ __launch_bounds__(LANES <= 64 ? 256 : LANES) void softmax_bwd_kernel(
   for (int j = 0; j < ITEMS; ++j)
 #pragma unroll
     for (int q = 0; q < V; ++q) dot += rg.term(s[j][q], g[j][q]);
-  // the up to 3 floats beyond the last whole vector of a row of odd length: lane 0 takes them
+  // the up to 3 floats beyond the last whole vector of a row of odd length: lane q takes the q-th
+  // (lane 0 all of them where a row has fewer than four lanes)
   const int rem = TAIL ? (int)(cols & 3) : 0;
-  const bool tail = TAIL && rem != 0 && active && lane == 0;
+  constexpr bool SPREAD = LANES >= 4;
+  const bool tail = TAIL && active && (SPREAD ? lane < rem : (rem != 0 && lane == 0));
+  const int tq0 = SPREAD ? lane : 0, tq1 = SPREAD ? lane + 1 : rem;
   float ts[3] = {0.f, 0.f, 0.f}, tg[3] = {0.f, 0.f, 0.f};
   if (tail)
-    for (int q = 0; q < rem; ++q) {
-      ts[q] = out[row * cols + 4 * colsv + q];
-      tg[q] = out_grad[row * cols + 4 * colsv + q];
-      dot += rg.term(ts[q], tg[q]);
+    for (int q = tq0; q < tq1; ++q) {
+      ts[q - tq0] = out[row * cols + 4 * colsv + q];
+      tg[q - tq0] = out_grad[row * cols + 4 * colsv + q];
+      dot += rg.term(ts[q - tq0], tg[q - tq0]);
     }
   dot = row_reduce<SumOp, LANES>(dot, smem);
   if (tail)
-    for (int q = 0; q < rem; ++q) {
+    for (int q = tq0; q < tq1; ++q) {
       float* p = x_grad + row * cols + 4 * colsv + q;
-      const float r = rg.result(ts[q], tg[q], dot, kk);
+      const float r = rg.result(ts[q - tq0], tg[q - tq0], dot, kk);
       *p = beta != 0.0f ? beta * *p + r : r;
     }
 

@@ -622,7 +622,7 @@ SOFTMAX_SHAPES = [(2, 3), (1, 1), (7, 10), (8192, 10), (100, 128), (33, 130), (6
                   # 1025..2048 vectors per row: the forward pass runs 512 lanes there, the backward pass 1024
                   (5, 8192), (4, 4104), (3, 6000), (3, 8190), (3, 8196),
                   # rows of 16388..65536 floats held in registers, and few rows far longer than that, cut into segments
-                  (3, 16388), (2, 20000), (2, 32768), (2, 32771), (2, 32772), (2, 50257), (2, 65536), (2, 65539),
+                  (3, 16388), (2, 16389), (2, 20000), (2, 20001), (2, 24577), (2, 32768), (2, 32771), (2, 32772), (2, 50257), (2, 65536), (2, 65539),
                   (1, 1048576), (3, 300001), (2, 262147), (7, 131072), (1, 131073),
                   # 257..448 vectors per row: the forward pass runs one wave per row with eight vectors a lane
                   (9, 1028), (9, 1030), (6, 1500), (5, 1792), (5, 1795), (5, 1796), (7, 1281),
