@@ -116,9 +116,15 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(size_t rows, size_t cols
         a2 = Op::apply(a2, h2 ? Op::apply(Op::apply(v2.x, v2.y), Op::apply(v2.z, v2.w)) : id);
         a3 = Op::apply(a3, h3 ? Op::apply(Op::apply(v3.x, v3.y), Op::apply(v3.z, v3.w)) : id);
       }
-      // a row of odd length ends in up to 3 floats beyond its last whole vector
-      if ((cols & 3) && seg == nseg - 1 && lane == 0)
-        for (size_t e = 4 * colsv; e < cols; ++e) a1 = Op::apply(a1, src.one(xr + e, vv));
+      // a row of odd length ends in up to 3 floats beyond its last whole vector: lane q takes the q-th
+      // (lane 0 all of them where a row has fewer than four lanes)
+      if ((cols & 3) && seg == nseg - 1) {
+        if (LANES >= 4) {
+          if (lane < (int)(cols & 3)) a1 = Op::apply(a1, src.one(xr + 4 * colsv + lane, vv));
+        } else if (lane == 0) {
+          for (size_t e = 4 * colsv; e < cols; ++e) a1 = Op::apply(a1, src.one(xr + e, vv));
+        }
+      }
     } else {
       size_t c = cbeg + lane;
       for (; c + 3 * LANES < cend; c += 4 * LANES) {
@@ -668,9 +674,15 @@ __global__ __launch_bounds__(256) void max_cols_grad_kernel(size_t rows, size_t 
       const unsigned long long h0 = hit(ld4s(xr + 4 * c), c);
       best = h0 < best ? h0 : best;
     }
-    if (lane == 0)
+    // the up to 3 floats behind the last whole vector: lane q takes the q-th (lane 0 all of them
+    // where a row has fewer than four lanes)
+    if (LANES >= 4) {
+      const size_t e = (colsv << 2) + lane;
+      if (e < cols && xr[e] == m && e < best) best = e;
+    } else if (lane == 0) {
       for (size_t e = colsv << 2; e < cols; ++e)
         if (xr[e] == m && e < best) best = e;
+    }
   }
   if (TPR == 0) {
     if (best != NONE) atomicMin(&smin, best);
