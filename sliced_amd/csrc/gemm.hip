@@ -40,8 +40,9 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs g) {
 // NG = groups of 8 k whose loads are issued together: 8 for small problems (latency is all that
 // matters: [1024x64]x[64x64] 7.2 -> 5.9 us), 1 for large skinny ones, which have waves enough to
 // hide latency and measured 15-20 % slower with 2, 4 or 8 (8192x10x2048: 41 us against 48).
-// FULL = every k range is a whole number of groups and the k-contiguous operands are float4
-// loadable: no bounds checks, and a k-contiguous operand comes in as one float4 per group.
+// FULL = the whole groups of a k range run without bounds checks and a k-contiguous operand comes
+// in as one (dword-aligned) float4 per group; a last, partial group is checked.  (Checked element by
+// element, 257 x 17 x 33333 took 78 us as A*Bt - 0.5 TB/s - and 1000 x 17 x 33333 250 us.)
 // COLSUM (the At*B form only): the workgroups of tile row 0 also add the column sums of B over
 // this launch's k range to colsum[N] - the bias gradient of a Linear layer, whose weight gradient
 // xT*g reads the very same g.  `nw` = waves that share this tile's k range; a workgroup may hold
@@ -92,13 +93,14 @@ __device__ __forceinline__ void wave_tile(const GemmArgs& g, float* red, const u
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
   float cs = 0.0f;  // COLSUM: this lane's share of column n0 + r (its half of every group of 8 k)
   // NG groups of 8 k at a time: all 8*NG loads are issued before the first MFMA needs one
-  auto run_groups = [&](size_t gi, auto ng_tag) {
+  auto run_groups = [&](size_t gi, auto ng_tag, auto checked_tag) {
     constexpr int N = decltype(ng_tag)::value;
+    constexpr bool CHECKED = decltype(checked_tag)::value;
     float a[N][4], b[N][4];
 #pragma unroll
     for (int u = 0; u < N; ++u) {
       const size_t k = kbeg + (gi + u) * 8 + 4 * h;
-      if (FULL) {
+      if (FULL && !CHECKED) {
         if (!TA) {
           const float4 v = ld4g(ap + k);
           a[u][0] = v.x; a[u][1] = v.y; a[u][2] = v.z; a[u][3] = v.w;
@@ -135,11 +137,25 @@ __device__ __forceinline__ void wave_tile(const GemmArgs& g, float* red, const u
         for (int t = 0; t < 4; ++t) cs += b[u][t];
     }
   };
+  // FULL: the whole groups of the k range without a check; a range that ends in a partial group (a
+  // K that is not a multiple of 8: only the last range has one) finishes with that group, checked
+  const size_t whole = FULL ? (kend - kbeg) / 8 : 0;
+  const size_t gfast = FULL ? (gend < whole ? gend : whole) : gbeg;
   size_t gi = gbeg;
-  for (; gi + NG <= gend; gi += NG) run_groups(gi, std::integral_constant<int, NG>());
-  if (NG > 4)
-    for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>());
-  for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>());
+  if (FULL) {
+    using U = std::false_type;
+    for (; gi + NG <= gfast; gi += NG) run_groups(gi, std::integral_constant<int, NG>(), U());
+    if (NG > 4)
+      for (; gi + 4 <= gfast; gi += 4) run_groups(gi, std::integral_constant<int, 4>(), U());
+    for (; gi < gfast; ++gi) run_groups(gi, std::integral_constant<int, 1>(), U());
+    for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>(), std::true_type());
+  } else {
+    using C = std::true_type;
+    for (; gi + NG <= gend; gi += NG) run_groups(gi, std::integral_constant<int, NG>(), C());
+    if (NG > 4)
+      for (; gi + 4 <= gend; gi += 4) run_groups(gi, std::integral_constant<int, 4>(), C());
+    for (; gi < gend; ++gi) run_groups(gi, std::integral_constant<int, 1>(), C());
+  }
 
   const bool sums = COLSUM && colsum != nullptr && tm == 0;
   if (sums) cs += __shfl_xor(cs, 32);  // the two halves of every group of 8 k
@@ -362,8 +378,13 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // <= 6e8 flop when the kernel can use its unchecked vector-load form (it then beats the tiled
   // kernel up to about 700^3: 512^3 takes 7.2 us against 17.4), <= 2^25 flop otherwise.
   const double flop = 2.0 * (double)M * (double)N * (double)K;
-  const bool wave_full = K % 8 == 0 && (ta || g.a_vec) && (!tb || g.b_vec);
-  if (flop <= (wave_full ? 6.0e8 : 33554432.0) || M <= 32 || N <= 32 || K <= 16) {
+  // (the vector loads of a k-contiguous operand need dword alignment only; a K that is not a multiple
+  // of 8 ends in one checked group)
+  const bool wave_full = K >= 8;
+  // products whose K or bases are off the 8-float grid go to the tiled kernels from a lower size on: the
+  // staged tiles absorb the misalignment that the wave kernel's direct loads pay for
+  const bool wave_aligned = K % 8 == 0 && (ta || g.a_vec) && (!tb || g.b_vec);
+  if (flop <= (wave_aligned ? 6.0e8 : 33554432.0) || M <= 32 || N <= 32 || K <= 16) {
     const size_t wt_m = (M + 31) / 32, wt_n = (N + 31) / 32;
     if (wt_m * wt_n > 0x7fffffffu) {
       set_error("sgemm: %zu x %zu tiles exceed one launch", wt_m, wt_n);
@@ -718,9 +739,8 @@ static bool linear_grad_pair(slhip_ctx* ctx, size_t m, size_t k, size_t n, const
   gw.splits = 1; gw.k_chunk = k_chunk;
   gw.tiles_m = (unsigned)((k + 31) / 32); gw.tiles_n = (unsigned)((n + 31) / 32);
   const size_t tiles_w = (size_t)gw.tiles_m * gw.tiles_n;
-  // the unchecked form of each product, as gemm_run decides it: whole groups of 8 k and float4
-  // loads of the k-contiguous operands (g and w rows for x.grad; none for w.grad)
-  const bool fullx = n % 8 == 0 && gx.a_vec && gx.b_vec, fullw = m % 8 == 0;
+  // the unchecked form of each product, as gemm_run decides it: at least one whole group of 8 k
+  const bool fullx = n >= 8, fullw = m >= 8;
   const unsigned nw = nwx > nww ? nwx : nww;
   const size_t lds = nw > 1 ? ((size_t)nw * 16 * 64 + (size_t)nw * 32) * sizeof(float) : 0;
   const dim3 grid((unsigned)(tiles_x + tiles_w));

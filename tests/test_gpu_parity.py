@@ -57,6 +57,8 @@ GEMM_SHAPES = [
     (1, 64, 1024), (64, 1, 1024), (384, 256, 784), (200, 136, 1000), (512, 512, 512),
     # one wave per 32x32 tile: k split over waves and over the grid, skinny sides, ragged edges
     (32, 32, 100003), (2000, 10, 1000), (40, 1000, 10), (16, 3000, 500), (31, 33, 4099), (96, 64, 64),
+    # K off the multiples of 8 on that kernel: whole groups of 8 k, then one checked group of 1..7
+    (257, 17, 3333), (17, 257, 3335), (100, 100, 1001), (48, 48, 9), (40, 72, 15), (70, 30, 8),
 ]
 
 
@@ -1042,7 +1044,7 @@ def test_operands_that_are_only_float_aligned(hip, orc, off):
     bound = 2e-6 * (np.abs(S) * (np.abs(G) + (np.abs(S) * np.abs(G)).sum(1, keepdims=True))).ravel() + 1e-37
     assert np.all(np.abs(got - ob) <= bound)
     # GEMM, all forms, tiled and wave-per-tile sizes
-    for (m, nn, k) in [(300, 256, 512), (96, 40, 64)]:
+    for (m, nn, k) in [(300, 256, 512), (96, 40, 64), (96, 40, 67), (300, 17, 1001)]:
         a = rng.uniform(m * k, -1, 1, tag=3, seed=SEED)
         b = rng.uniform(k * nn, -1, 1, tag=4, seed=SEED)
         da, db, dc = pool_x.view(off, m * k), pool_g.view(off, k * nn), pool_o.view(oo, m * nn)
