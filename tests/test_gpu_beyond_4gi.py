@@ -374,3 +374,19 @@ def test_elementwise_chain_and_gradients(big):
         h = host_range(start, m + 2, 0)
         assert np.array_equal(y.view(start, m).numpy(), h[1:m + 1] * h[2:m + 2]), start
         assert np.array_equal(z.view(start, m).numpy(), h[:m] * h[2:m + 2]), start
+
+
+@pytest.mark.parametrize("k", [32, 8, 1], ids=lambda k: "k%d" % k)
+def test_product_with_a_result_beyond_2_32_elements(big, k):
+    ctx, x, y, z, small = big
+    m = nn = 65552
+    say("A * B, A * Bt with", m * nn, "results, k =", k)
+    a, b = host_range(0, m * k, 0), host_range(m * k, k * nn, 0)
+    A = a.reshape(m, k).astype(np.float64)
+    for tb in (0, 1):
+        B = (b.reshape(nn, k).T if tb else b.reshape(k, nn)).astype(np.float64)
+        ctx.call("slhip_sgemm", 0, tb, m, nn, k, x.ptr, x.view(m * k, k * nn).ptr, y.ptr, 0.0)
+        for r in (0, 1, 65535, 65536, m - 1):           # row 65535 ends just short of element 2^32 of C
+            got = y.view(r * nn, nn).numpy()
+            want, scale = A[r] @ B, np.abs(A[r]) @ np.abs(B)
+            assert np.all(np.abs(got - want) <= 3e-6 * scale), (k, tb, r)
