@@ -143,9 +143,9 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
   }
 }
 
-// The 256 x 64 tile for large matrices whose output rows do not start on 64-byte boundaries (rows
-// not a multiple of 16, or an output that starts off the grid).  What a tile writes of output row c
-// is then not the floats [r0, r0 + 256) but the piece [r0 - d_c, r0 + 256 - d_c), d_c < 16 chosen per
+// The tile (TR x TC = 256 x 64 or 128 x 128) for matrices whose output rows do not start on 64-byte
+// boundaries (rows not a multiple of 16, or an output that starts off the grid).  What a tile writes of
+// output row c is then not the floats [r0, r0 + TR) but the piece [r0 - d_c, r0 + TR - d_c), d_c < 16 chosen per
 // output row so that the piece starts and ends on 64-byte boundaries of the output: a 64-byte block
 // that two tiles each write a part of reaches the memory as two partial writes (see the chunk kernel
 // below, which does the same), and every vector store is aligned.  The tile stages 16 rows more than
@@ -154,13 +154,14 @@ __global__ __launch_bounds__(256) void transpose_kernel(size_t rows, size_t cols
 // float by float, thread c for output row c.  Same LDS layout as above: lane l of a wave fetches
 // the rows s + 4 l .. s + 4 l + 3 of one column, whatever s, and meets no bank twice.
 // [13421 x 10000] 3.9 -> 4.7 TB/s, [65521 x 2048] 4.45 -> 5.15, [134217 x 1000] 4.1 -> 4.6, [16383 x 16385]
-// 4.1 -> 4.5, [12345 x 6789] 3.95 -> 4.2; matrices of a few million elements lose (3001 x 3003: 28 -> 32 us)
-// and keep the plain tile.  (Without the unconditional loads of a whole tile - the `full` path - the
-// same kernel measured 3-12 % behind the plain tile on every shape.)
-template <bool ACC>
+// 4.1 -> 4.5, [12345 x 6789] 3.95 -> 4.2 with the 256 x 64 tile (the host's choice between the two tiles and the
+// plain one is described where it is made).  (Without the unconditional loads of a whole tile - the
+// `full` path - the same kernel measured 3-12 % behind the plain tile on every shape.)
+template <bool ACC, int TR, int TC>
 __global__ __launch_bounds__(256) void transpose_shift_kernel(size_t rows, size_t cols, const float* __restrict__ x,
                                                               float* out, unsigned tiles_r, unsigned group) {
-  constexpr int TR = 256, TC = 64, H = 16, LR = TR + H;
+  constexpr int H = 16, LR = TR + H;
+  static_assert(TR % 64 == 0 && TC % 64 == 0 && LR % (1024 / TC) == 0 && TC <= 256, "tile shape");
   __shared__ float tile_mem[LR * (TC + 1) + 52];
   auto tile = [&](int r, int c) -> float& { return tile_mem[((r & 3) * (LR / 4) + (r >> 2)) * (TC + 1) + c + 17 * (r & 3)]; };
   const unsigned tiles_c = gridDim.x / tiles_r;
@@ -196,25 +197,44 @@ __global__ __launch_bounds__(256) void transpose_shift_kernel(size_t rows, size_
         }
       }
     }
+    // a row of more than 16 vectors per wave instruction: lanes 8 apart would meet on a bank with the
+    // same component, so lane lx stores component (j + lx / 8) % 4 in the j-th instruction
+    const int rot = LPR > 16 ? (lx >> 3) & 3 : 0;
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       const int rr = ly + RPP * p;
-      tile(rr, 4 * lx + 0) = v[p].x;
-      tile(rr, 4 * lx + 1) = v[p].y;
-      tile(rr, 4 * lx + 2) = v[p].z;
-      tile(rr, 4 * lx + 3) = v[p].w;
+      if (LPR > 16) {
+        const float e[4] = {v[p].x, v[p].y, v[p].z, v[p].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int q = (j + rot) & 3;
+          tile(rr, 4 * lx + q) = q == 0 ? e[0] : q == 1 ? e[1] : q == 2 ? e[2] : e[3];
+        }
+      } else {
+        tile(rr, 4 * lx + 0) = v[p].x;
+        tile(rr, 4 * lx + 1) = v[p].y;
+        tile(rr, 4 * lx + 2) = v[p].z;
+        tile(rr, 4 * lx + 3) = v[p].w;
+      }
     }
   }
   __syncthreads();
-  constexpr int NP = TC / 4;  // four output rows per pass, 64 lanes each
-  const int lx = t & 63, ly = t >> 6;
+  constexpr int LPO = TR / 4, OPP = 256 / LPO, NP = TC / OPP;  // lanes per output row, output rows per pass, passes
+  const int lx = t % LPO, ly = t / LPO;
+  // the output row of pass p: with 16 lanes per output row a wave takes the rows {j, j + 16, j + 1, j + 17} of
+  // a block of 32 (lane l reads LDS bank l + the row's number: two rows 16 apart fill the 32 banks)
+  auto out_row = [&](int p) {
+    if (LPO >= 32) return ly + OPP * p;
+    const int q = p * 4 + (t >> 6), g = (t >> 4) & 3;
+    return (q >> 3) * 32 + 2 * (q & 7) + (g >> 1) + 16 * (g & 1);
+  };
   // everything in rows relative to the first staged one, in 32 bits
   const int off = (int)(r0 - rb);  // H, or 0 in the first tile row
   const int nst = rows - rb < (size_t)staged ? (int)(rows - rb) : staged;
   const int ob = (int)((reinterpret_cast<uintptr_t>(out) >> 2) & (H - 1)), lm = (int)(rows & (H - 1));
   // the piece of output row c0 + cc: staged rows [lo, hi); returns the floats before its first aligned vector
   auto piece = [&](int cc, int& lo, int& hi) {
-    const int d = (ob + (int)((c0 + cc) & (H - 1)) * lm) & (H - 1);  // (r0 is a multiple of 256)
+    const int d = (ob + (int)((c0 + cc) & (H - 1)) * lm) & (H - 1);  // (r0 is a multiple of 64)
     lo = off > d ? off - d : 0;
     hi = off + TR - d < nst ? off + TR - d : nst;
     return lo ? 0 : (4 - (d & 3)) & 3;  // lo > 0: the piece starts on a 64-byte boundary
@@ -224,7 +244,7 @@ __global__ __launch_bounds__(256) void transpose_shift_kernel(size_t rows, size_
   if (ACC) {
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-      const int cc = ly + 4 * p;
+      const int cc = out_row(p);
       int lo, hi;
       const int l = piece(cc, lo, hi) + lo + 4 * lx;
       old[p] = (c0 + cc < cols && l + 3 < hi) ? ld4s(obeg + (c0 + cc) * rows + l) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -232,7 +252,7 @@ __global__ __launch_bounds__(256) void transpose_shift_kernel(size_t rows, size_
   }
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
-    const int cc = ly + 4 * p;
+    const int cc = out_row(p);
     int lo, hi;
     const int l = piece(cc, lo, hi) + lo + 4 * lx;
     if (c0 + cc < cols && l + 3 < hi) {
@@ -511,16 +531,38 @@ SLHIP_API int32_t slhip_transpose(slhip_ctx* ctx, size_t rows, size_t cols, cons
     return post_launch();
   }
   constexpr int TR = 256, TC = 64;
-  // output rows of 8192 floats and more that start off the 64-byte grid, 2^24 elements and more: pieces
-  // shifted per output row (shorter output rows have too few whole pieces between their cut ends:
-  // [4026 x 33333] 4.12 -> 3.67 TB/s, [520 x 250001] 4.12 -> 3.77)
-  if (cols >= 64 && rows >= 8192 && len >= (size_t(1) << 24) && (rows % 16 != 0 || (reinterpret_cast<uintptr_t>(out) & 63) != 0)) {
-    const size_t tiles_r = (rows + 15 + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;  // the last piece of every output row ends inside the last tile row
-    SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
-    const unsigned group = rows >= 16 * cols ? (tiles_r < 8 ? (unsigned)tiles_r : 8u) : (unsigned)tiles_r;
-    if (acc) hipLaunchKernelGGL(transpose_shift_kernel<true>, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
-    else hipLaunchKernelGGL(transpose_shift_kernel<false>, dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
-    return post_launch();
+  // Output rows that start off the 64-byte grid: pieces shifted per output row.  The 256 x 64 tile for
+  // output rows of 8192 floats and more, 2^24 elements and more and an input pitch that is a multiple of
+  // 64 bytes ([65521 x 2048] 5.1 TB/s against 5.0 for the square tile, [16385 x 16384] 5.45 against 5.1);
+  // the 128 x 128 tile for every other pitch and for shorter output rows (from 256 floats): its 512-byte
+  // input pieces straddle one 128-byte line in four where 256-byte pieces straddle one in two, and its
+  // output pieces leave short output rows more whole pieces between their cut ends (the 256 x 64 tile lost
+  // to the plain one there).  Against the 256 x 64 tile, shifted: [12345 x 6789] 4.17 -> 4.46, [9001 x 50001]
+  // 4.05 -> 4.51, [23171 x 23169] 4.34 -> 4.63; against the plain tile: [8191 x 16385] 3.8 -> 4.75, [1001 x 100003]
+  // 3.4 -> 4.55, [300 x 400001] 3.4 -> 4.2, [6001 x 20000] 4.6 -> 5.2, [4026 x 32768] 4.2 -> 4.7, [5000 x 3001] 36 ->
+  // 32 us.  With fewer than 256 square tiles (or fewer than 2^24 elements below 1024 columns) the plain
+  // tile stays ([1025 x 1025] 8 against 12 us, [8193 x 1000] 23 against 25, [100001 x 257] 48 against 55).
+  if (cols >= 64 && (rows % 16 != 0 || (reinterpret_cast<uintptr_t>(out) & 63) != 0)) {
+    const bool big = len >= (size_t(1) << 24);
+    // (below 1024 columns also where the last column of 128-wide tiles would be emptier than that of 64-wide
+    // ones: [100001 x 257] 48 against 56 us)
+    const bool narrower = cols < 1024 && (cols + 63) / 64 * 64 < (cols + 127) / 128 * 128;
+    if (rows >= 8192 && big && (cols % 16 == 0 || narrower)) {
+      const size_t tiles_r = (rows + 15 + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;  // the last piece of every output row ends inside the last tile row
+      SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
+      const unsigned group = rows >= 16 * cols ? (tiles_r < 8 ? (unsigned)tiles_r : 8u) : (unsigned)tiles_r;
+      if (acc) hipLaunchKernelGGL((transpose_shift_kernel<true, 256, 64>), dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+      else hipLaunchKernelGGL((transpose_shift_kernel<false, 256, 64>), dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+      return post_launch();
+    }
+    const size_t tiles_r = (rows + 15 + 127) / 128, tiles_c = (cols + 127) / 128;
+    if (rows >= 256 && (cols >= 1024 ? tiles_r * tiles_c >= 256 : big)) {
+      SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");
+      const unsigned group = rows >= 16 * cols ? (tiles_r < 8 ? (unsigned)tiles_r : 8u) : (unsigned)tiles_r;
+      if (acc) hipLaunchKernelGGL((transpose_shift_kernel<true, 128, 128>), dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+      else hipLaunchKernelGGL((transpose_shift_kernel<false, 128, 128>), dim3((unsigned)(tiles_r * tiles_c)), dim3(256), 0, ctx->stream, rows, cols, x, out, (unsigned)tiles_r, group);
+      return post_launch();
+    }
   }
   const size_t tiles_r = (rows + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;
   SLHIP_REQUIRE(tiles_r * tiles_c <= 0x7fffffffu, "matrix too large for one launch");

@@ -703,7 +703,10 @@ TR_SHAPES = [(2, 3), (1, 7), (7, 1), (64, 64), (65, 63), (128, 256), (100, 300),
              (8192, 2048), (8208, 2048), (8200, 2048), (8193, 2048),
              # 2^24 elements and more with output rows off the 64-byte grid: the 256 x 64 tile with pieces shifted
              # per output row (first and last tile rows, ragged tile columns, rows of odd length on both sides)
-             (8200, 2049), (16385, 1031), (8209, 2100), (65521, 257), (8193, 2050)]
+             (8200, 2049), (16385, 1031), (8209, 2100), (65521, 257), (8193, 2050), (8193, 2048), (16385, 1040),
+             # the 128 x 128 tile with shifted pieces: shorter output rows and input pitches off the 64-byte grid
+             (300, 140001), (4026, 4099), (1001, 20001), (257, 131073), (2050, 2051), (5000, 3001), (383, 16400),
+             (16385, 1025)]
 
 
 @pytest.mark.parametrize("shape", TR_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -720,7 +723,8 @@ def test_transpose_bit_exact(hip, orc, shape):
     assert np.array_equal(acc, orc.transpose(rows, cols, x, out=base.copy(), assign=True))
 
 
-@pytest.mark.parametrize("shape", [(50001, 100), (50016, 100), (8209, 10), (100003, 56), (64, 5000), (100, 8193), (1234, 679)],
+@pytest.mark.parametrize("shape", [(50001, 100), (50016, 100), (8209, 10), (100003, 56), (64, 5000), (100, 8193), (1234, 679),
+                                   (4096, 4100), (8208, 2048), (2048, 2049)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_transpose_between_views_off_the_allocation_grid(hip, orc, shape):
     """Input and output that start 1, 5, 16 and 17 floats into their allocations: no kernel may rely on
