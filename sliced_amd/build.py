@@ -64,11 +64,28 @@ def build_host(verbose=False):
     return LIB_HOST
 
 
+CONSUMER_SRC = os.path.join(HERE, "..", "tests", "abi_consumer", "consumer.c")
+CONSUMER = os.path.join(OBJ, "abi_consumer")
+
+
+def build_consumer(verbose=False):
+    """The plain-C caller of the ABI that the tests run (C99, -pedantic -Werror: the header has to be C)."""
+    if not os.path.exists(CONSUMER_SRC):
+        return None
+    os.makedirs(OBJ, exist_ok=True)
+    out = _run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-O1", "-I", os.path.join(HERE, "..", "include"),
+                CONSUMER_SRC, "-o", CONSUMER, "-L", HERE, "-lsliced_hip", "-lm", "-Wl,-rpath,$ORIGIN/.."])
+    if verbose and out:
+        print(out)
+    return CONSUMER
+
+
 def build_all(verbose=False):
     libs = [build_kernels(verbose)]
     h = build_host(verbose)
     if h:
         libs.append(h)
+    build_consumer(verbose)
     return libs
 
 

@@ -60,3 +60,42 @@ def test_argument_validation_needs_no_gpu():
     assert lib.slhip_softmax(None, 2, 3, None, None) == -1
     assert lib.slhip_transpose(None, 2, 3, None, None, 0.0) == -1
     assert b"null" in lib.slhip_last_error_string().lower()
+
+
+# ---- the header and the library from plain C (tests/abi_consumer/consumer.c)
+CONSUMER_SRC = os.path.join(ROOT, "tests", "abi_consumer", "consumer.c")
+
+
+def consumer_binary():
+    from sliced_amd import build
+    if not os.path.exists(build.CONSUMER):
+        build.build_consumer()
+    return build.CONSUMER
+
+
+def test_header_is_c99():
+    import subprocess
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I",
+                        os.path.join(ROOT, "include"), CONSUMER_SRC], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+
+
+def test_c_consumer_links_and_fails_loudly_without_a_gpu():
+    import subprocess
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    r = subprocess.run([consumer_binary()], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert r.returncode == 2, (r.returncode, r.stdout, r.stderr)
+    assert "device" in r.stderr.lower() and "PASS" not in r.stdout
+
+
+@pytest.mark.gpu
+def test_c_consumer_runs_a_layer_through_the_abi():
+    """The C99 program calls init, malloc, h2d, sgemm, add_row, relu, softmax, Tgemm, sum_rows, transpose, d2h
+    and compares with its own loops: no Python between the caller and the library."""
+    import subprocess
+    r = subprocess.run([consumer_binary()], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
+    assert r.stdout.strip().splitlines()[-1] == "PASS"
