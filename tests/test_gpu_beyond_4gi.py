@@ -34,17 +34,7 @@ def say(*a):
     sys.stdout.flush()
 
 
-def host_values(idx, tag):
-    """The generator's value at the given element indices (any order), as the device computes it."""
-    idx = np.asarray(idx, dtype=np.uint64)
-    base = np.uint64((int(SEED) ^ (int(tag) << 40)) & 0xFFFFFFFFFFFFFFFF)
-    with np.errstate(over="ignore"):
-        u = (rng._splitmix64(base + idx) >> np.uint64(40)).astype(np.uint32).astype(np.float32) * np.float32(2.0 ** -24)
-    return (np.float32(LO) + (np.float32(HI) - np.float32(LO)) * u).astype(np.float32)
-
-
-def host_range(start, n, tag):
-    return host_values(np.arange(start, start + n, dtype=np.uint64), tag)
+from devgen import host_values, host_range  # noqa: E402  (the generator's values at any index)
 
 
 WINDOWS = [(0, 8192), (TWO32 - 4096, 8192), (N - 8192, 8192)]

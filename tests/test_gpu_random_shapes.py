@@ -125,3 +125,176 @@ def test_random_matrix_op_shapes(hip, orc):
         base = rng.normal(n, 1.0, tag=6, seed=SEED + case)
         assert np.array_equal(hip.max_cols_grad(cols, mx, xt, base.copy(), gr), orc.max_cols_grad(cols, mx, xt, base.copy(), gr))
 
+
+
+# --------------------------------------------------------------------------- large random shapes
+# Up to 2^27 elements per operand, where the host's choice between kernels changes with the size (the
+# shifted-piece and chunk transposes, the tall and skinny GEMM kernels, long-row softmax, the two-stage
+# reductions).  The operands come from the device generator and are checked against its values
+# recomputed on the host (devgen.py) on windows, sampled rows and columns, and through the transpose of
+# the transpose; views start 0..33 floats into their allocations.
+BIG_CAP = (1 << 27) + 4096
+SUB_OP, SCALE_OP = 1, 6   # SLHIP_SUB, SLHIP_SCALE
+
+
+@pytest.fixture(scope="module")
+def pool():
+    from sliced_amd.device import Context
+    ctx = Context(0)
+    x = ctx.uniform(BIG_CAP + 64, -1, 1, 0, SEED)
+    y, z = ctx.empty(BIG_CAP + 64), ctx.empty(BIG_CAP + 64)
+    small = ctx.zeros(1 << 22)
+    yield ctx, x, y, z, small
+    for b in (x, y, z, small):
+        b.free()
+    ctx.close()
+
+
+def near(r, base, spread=2):
+    return max(1, int(base + r.integers(-spread, spread + 1)))
+
+
+def pick_side(r, hi):
+    k = r.integers(0, 7)
+    if k == 0:
+        return int(r.integers(1, 65))
+    if k == 1:
+        return near(r, int(r.choice([16, 32, 56, 57, 64, 128, 200, 201, 256, 512, 1024, 2048, 4096, 8192, 16384])))
+    if k == 2:
+        return near(r, 64 * int(r.integers(1, 400)))
+    if k == 3:
+        return near(r, 256 * int(r.integers(1, 200)), 17)
+    if k == 4:
+        return int(r.integers(1, 4000))
+    if k == 5:
+        return int(2 ** r.uniform(6, np.log2(hi)))
+    return near(r, 1024 * int(r.integers(1, 64)), 1)
+
+
+def test_random_large_transposes(pool):
+    from devgen import host_values
+    ctx, x, y, z, small = pool
+    r = np.random.default_rng(4242)
+    done = 0
+    while done < 60:
+        rows, cols = pick_side(r, 1 << 22), pick_side(r, 1 << 22)
+        if r.integers(0, 3) == 0:
+            cols = max(1, min(cols, BIG_CAP // max(rows, 1)))
+            rows = max(1, min(int(2 ** r.uniform(20, 27)) // cols, 1 << 24))
+        n = rows * cols
+        if n > BIG_CAP:
+            continue
+        done += 1
+        ox, oy = int(r.choice([0, 0, 1, 4, 5, 16, 17, 32])), int(r.choice([0, 0, 1, 3, 16, 17, 33]))
+        xs, ys, zs = x.view(ox, n), y.view(oy, n), z.view(ox, n)
+        say("large transpose", rows, cols, ox, oy)
+
+        def want(start, m):
+            o = np.arange(start, start + m, dtype=np.uint64)
+            c, rr = o // np.uint64(rows), o % np.uint64(rows)
+            return host_values(rr * np.uint64(cols) + c + np.uint64(ox), 0)
+
+        ctx.call("slhip_transpose", rows, cols, xs.ptr, ys.ptr, 0.0)
+        w = min(n, 4096)
+        for start in (0, max(0, n // 2 - 1000), n - w):
+            m = min(w, n - start)
+            assert np.array_equal(ys.view(start, m).numpy(), want(start, m)), (rows, cols, ox, oy, start)
+        ctx.call("slhip_transpose", cols, rows, ys.ptr, zs.ptr, 0.0)          # and back: every element
+        ctx.call("slhip_ew_binary", SUB_OP, n, zs.ptr, xs.ptr, zs.ptr)
+        ctx.call("slhip_max", n, zs.ptr, small.view(0, 1).ptr)
+        ctx.call("slhip_ew_unary", SCALE_OP, -1.0, 0.0, n, zs.ptr, zs.ptr)
+        ctx.call("slhip_max", n, zs.ptr, small.view(1, 1).ptr)
+        assert np.all(small.view(0, 2).numpy() == 0.0), (rows, cols, ox, oy)
+        ctx.call("slhip_transpose", rows, cols, xs.ptr, ys.ptr, 1.0)           # `Assign`: y = 2 x^T now
+        for start in (0, n - w):
+            assert np.array_equal(ys.view(start, w).numpy(), want(start, w) + want(start, w)), (rows, cols, ox, oy, start)
+
+
+def test_random_large_products(pool):
+    from devgen import host_values, host_range
+    ctx, x, y, z, small = pool
+    r = np.random.default_rng(777)
+    ctx.call("slhip_rand_uniform", SEED, 1, -1.0, 1.0, 1 << 26, z.ptr)   # B comes from tag 1
+    done = 0
+    while done < 60:
+        kind = r.integers(0, 4)
+        if kind == 0:      # a tall A and a narrow B
+            nn, k = int(r.integers(1, 40)), near(r, 4 * int(r.integers(16, 5000)), int(r.integers(0, 2)))
+            m = max(1, min(int(2 ** r.uniform(18, 26)) // k, 1 << 21))
+        elif kind == 1:    # few outputs, long k
+            m, nn, k = int(r.integers(1, 300)), int(r.integers(1, 300)), int(2 ** r.uniform(8, 19))
+        elif kind == 2:    # sides up to 5000 near the tile and vector boundaries
+            m, nn, k = (min(pick_side(r, 4096), 5000) for _ in range(3))
+        else:              # short k
+            k, m, nn = int(r.integers(1, 20)), int(2 ** r.uniform(8, 20)), int(r.integers(1, 600))
+        ta, tb = [(0, 0), (0, 1), (1, 0), (1, 1)][int(r.integers(0, 4))]
+        if m * k > BIG_CAP or k * nn > (1 << 26) or m * nn > BIG_CAP:
+            continue
+        done += 1
+        beta = float(r.integers(0, 2))
+        say("large gemm", m, nn, k, ta, tb, beta)
+        ctx.call("slhip_fill", m * nn, 0.25, y.ptr)
+        ctx.call("slhip_sgemm", ta, tb, m, nn, k, x.ptr, z.ptr, y.ptr, beta)
+        b = host_range(0, k * nn, 1)
+        B = (b.reshape(nn, k).T if tb else b.reshape(k, nn)).astype(np.float64)
+        for i in sorted(set([0, m - 1, m // 2] + [int(v) for v in r.integers(0, m, 5)])):
+            if ta:
+                a_row = host_values(np.arange(k, dtype=np.uint64) * np.uint64(m) + np.uint64(i), 0).astype(np.float64)
+            else:
+                a_row = host_range(i * k, k, 0).astype(np.float64)
+            exact, scale = a_row @ B + beta * 0.25, np.abs(a_row) @ np.abs(B) + 0.25
+            got = y.view(i * nn, nn).numpy()
+            assert np.all(np.abs(got - exact) <= 3e-6 * scale + 1e-30), (m, nn, k, ta, tb, beta, i, ctx.last_gemm_plan())
+
+
+def test_random_large_reductions_and_softmax(pool):
+    from devgen import host_values, host_range
+    ctx, x, y, z, small = pool
+    r = np.random.default_rng(31337)
+    done = 0
+    while done < 50:
+        rows, cols = pick_side(r, 1 << 22), pick_side(r, 1 << 22)
+        if r.integers(0, 2) == 0:
+            cols = max(1, min(cols, 1 << 20))
+            rows = max(1, min(int(2 ** r.uniform(18, 27)) // cols, 1 << 24))
+        n = rows * cols
+        if n > BIG_CAP:
+            continue
+        done += 1
+        ox = int(r.choice([0, 0, 1, 3, 4, 16]))
+        xs = x.view(ox, n)
+        say("large reductions / softmax", rows, cols, ox)
+        pick_r = sorted(set([0, rows - 1, rows // 2] + [int(v) for v in r.integers(0, rows, 3)]))
+        if rows <= (1 << 21):
+            vr = small.view(0, rows)
+            ctx.call("slhip_sum_cols", rows, cols, xs.ptr, vr.ptr)
+            s = vr.numpy()
+            ctx.call("slhip_max_cols", rows, cols, xs.ptr, vr.ptr)
+            mx = vr.numpy()
+            for i in pick_r:
+                h = host_range(ox + i * cols, cols, 0)
+                assert mx[i] == h.max(), (rows, cols, ox, i)
+                assert abs(float(s[i]) - h.sum(dtype=np.float64)) <= 1e-6 * np.abs(h).sum(dtype=np.float64) + 1e-30, (rows, cols, ox, i)
+        if cols <= (1 << 21):
+            vc = small.view(1 << 21, cols)
+            ctx.call("slhip_sum_rows", rows, cols, xs.ptr, vc.ptr)
+            s = vc.numpy()
+            ctx.call("slhip_max_rows", rows, cols, xs.ptr, vc.ptr)
+            mx = vc.numpy()
+            for c in sorted(set([0, cols - 1, cols // 2] + [int(v) for v in r.integers(0, cols, 3)])):
+                h = host_values(np.arange(rows, dtype=np.uint64) * np.uint64(cols) + np.uint64(c + ox), 0)
+                assert mx[c] == h.max(), (rows, cols, ox, c)
+                assert abs(float(s[c]) - h.sum(dtype=np.float64)) <= 1e-6 * np.abs(h).sum(dtype=np.float64) + 1e-30, (rows, cols, ox, c)
+        if cols >= 2:
+            ys = y.view(int(r.choice([0, 1, 4])), n)
+            ctx.call("slhip_softmax", rows, cols, xs.ptr, ys.ptr)
+            ctx.call("slhip_softmax_grad", rows, cols, z.view(0, n).ptr, ys.ptr, x.view(ox + 1, n).ptr, 0.0)
+            for i in pick_r:
+                h = host_range(ox + i * cols, cols, 0).astype(np.float64)
+                e = np.exp(h - h.max())
+                ref = e / e.sum()
+                got = ys.view(i * cols, cols).numpy()
+                assert np.all(np.abs(got - ref) <= 2e-6 * ref + 1e-37), (rows, cols, ox, i)
+                g, sg = host_range(ox + 1 + i * cols, cols, 0).astype(np.float64), got.astype(np.float64)
+                bound = 2e-6 * (np.abs(sg) * (np.abs(g) + np.dot(np.abs(sg), np.abs(g)))) + 1e-37
+                assert np.all(np.abs(z.view(i * cols, cols).numpy() - sg * (g - np.dot(sg, g))) <= bound), (rows, cols, ox, i)
