@@ -540,6 +540,34 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
     for_each([&](int i, int j, int v, size_t idx, size_t) { dst[idx] = acc[i][j][v]; });
     return;
   }
+  // A tile inside the matrix with nothing to read back but the bias (a Linear forward with its ReLU): one
+  // wave-uniform row pointer per accumulator register and one 32-bit lane offset for all of them
+  // (8192 x 2048 x 2048 with bias and ReLU, launches back to back: 499 -> 486 us, the plain product's time).
+  if (interior && g.beta == 0.0f && !g.mask && g.N < (size_t(1) << 28)) {
+    const int uw = __builtin_amdgcn_readfirstlane(wave);
+    const int uwm = uw / WGN, uwn = uw % WGN;
+    const unsigned lane_off = (unsigned)(4 * h) * (unsigned)g.N + (unsigned)r;
+    const bool relu = g.relu != 0;
+    float bv[WN];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) bv[j] = g.bias ? g.bias[n0 + block_of<WGN>(wn, j) + r] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        const size_t first = (m0 + block_of<WGM>(uwm, i)) * g.N + n0 + block_of<WGN>(uwn, j);  // wave-uniform
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const size_t at = first + (size_t)(8 * (v / 4) + v % 4) * g.N;
+          float val = acc[i][j][v];
+          if (g.bias) val = val + bv[j];
+          if (g.pre_act) (g.pre_act + at)[lane_off] = val;
+          const float rl = (val >= 0.0f ? 1.0f : 0.0f) * val;
+          (dst + at)[lane_off] = relu ? rl : val;
+        }
+      }
+    return;
+  }
   if (g.mask)
     for_each([&](int i, int j, int v, size_t idx, size_t) {
       acc[i][j][v] = (g.mask[idx] >= 0.0f ? 1.0f : 0.0f) * acc[i][j][v];
