@@ -1,7 +1,8 @@
 """The Rust binding crate (bindings/rust) cannot be compiled here (no rustc, no custos), so what CAN
 be checked is checked mechanically: its `extern "C"` block declares exactly the functions of
-include/sliced_hip.h with the same number of arguments, its constants carry the header's values,
-and every op trait of the hot path has an impl in src/ops.rs."""
+include/sliced_hip.h with the same number of arguments and, argument by argument, the Rust type
+that the C type maps to (pointer depth and constness included), its constants carry the header's
+values, and every op trait of the hot path has an impl in src/ops.rs."""
 import os
 import re
 
@@ -63,3 +64,76 @@ def test_every_hot_path_trait_has_an_impl():
     assert "never been compiled" in readme
     for f in ("Cargo.toml", "build.rs", "src/lib.rs", "src/device.rs", "src/probe.rs", "src/graph.rs"):
         assert os.path.exists(os.path.join(CRATE, f)), f
+
+
+# ---- argument and return TYPES, one by one
+def c_type_to_rust(t):
+    """The Rust FFI type that a C parameter type of the header has to be declared as."""
+    t = re.sub(r"\s+", " ", t.strip())
+    t = t.replace(" *", "*").replace("* ", "*")
+    base = {"int32_t": "i32", "uint32_t": "u32", "uint64_t": "u64", "size_t": "usize", "float": "f32", "char": "c_char",
+            "void": "c_void", "slhip_ctx": "SlhipCtx", "slhip_graph": "SlhipGraph", "slhip_event": "SlhipEvent",
+            "slhip_ew_insn": "SlhipEwInsn"}
+    m = re.fullmatch(r"(const )?(struct )?(\w+)((?:\*(?: ?const)?)*)", t)
+    assert m, t
+    const_base, name, stars = bool(m.group(1)), m.group(3), m.group(4)
+    assert name in base, t
+    out = base[name]
+    # pointer levels from the innermost outwards: `const T*` is *const T; `T* const*` is *const *mut T
+    levels = re.findall(r"\*( ?const)?", stars)
+    pointee_const = const_base
+    for lv in levels:
+        out = ("*const " if pointee_const else "*mut ") + out
+        pointee_const = bool(lv)
+    return out
+
+
+def split_c_params(args):
+    args = args.strip()
+    if args in ("", "void"):
+        return []
+    out = []
+    for a in args.split(","):
+        a = re.sub(r"/\*.*?\*/", "", a).strip()
+        a = re.sub(r"\s+", " ", a)
+        m = re.fullmatch(r"(.*?[\*\s])(\w+)", a)     # type, then the parameter's name
+        assert m, a
+        out.append(m.group(1).strip())
+    return out
+
+
+def header_signatures():
+    src = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    sigs = {}
+    for ret, name, args in re.findall(r"\n([\w \*]+?)\s*\b(slhip_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", src, flags=re.S):
+        sigs[name] = (ret.strip(), split_c_params(args))
+    return sigs
+
+
+def rust_signatures():
+    src = open(os.path.join(CRATE, "src", "ffi.rs")).read()
+    block = src[src.index('extern "C" {'):]
+    block = re.sub(r"//[^\n]*", "", block)
+    sigs = {}
+    for name, args, ret in re.findall(r"pub fn (slhip_[a-z0-9_]+)\s*\((.*?)\)\s*->\s*([^;]+);", block, flags=re.S):
+        types = []
+        for a in [x for x in args.split(",") if x.strip()]:
+            t = a.split(":", 1)[1]
+            t = re.sub(r"\s+", " ", t.strip())
+            t = re.sub(r"\b(?:std::os::raw::|std::ffi::|core::ffi::)", "", t)
+            types.append(t)
+        sigs[name] = (re.sub(r"\s+", " ", re.sub(r"\b(?:std::os::raw::|std::ffi::|core::ffi::)", "", ret.strip())), types)
+    return sigs
+
+
+def test_ffi_argument_and_return_types_match_the_header():
+    h, r = header_signatures(), rust_signatures()
+    assert sorted(h) == sorted(r)
+    wrong = []
+    for name, (ret, params) in h.items():
+        want_ret = c_type_to_rust(ret)
+        want = [c_type_to_rust(p) for p in params]
+        got_ret, got = r[name]
+        if want_ret != got_ret or want != got:
+            wrong.append((name, want_ret, want, got_ret, got))
+    assert not wrong, wrong[:5]
