@@ -99,3 +99,36 @@ def test_c_consumer_runs_a_layer_through_the_abi():
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0, (r.returncode, r.stdout, r.stderr)
     assert r.stdout.strip().splitlines()[-1] == "PASS"
+
+
+def test_ctypes_prototypes_match_the_header_type_by_type():
+    """Every argument of sliced_amd/_lib.py's table against the C type the header declares: a pointer where the
+    header has a pointer (of whatever kind: the table passes addresses), size_t, int32_t, uint64_t and float where it
+    has those, and the return types."""
+    from test_rust_binding import header_signatures
+    # (size_t and uint64_t are one ctypes class on this ABI, 64 bits both: one kind)
+    kinds = {"int32_t": "i32", "uint32_t": "u32", "uint64_t": "u64", "size_t": "u64", "float": "f32"}
+    assert C.sizeof(C.c_size_t) == 8
+
+    def c_kind(t):
+        t = t.strip()
+        if "*" in t:
+            return "ptr"
+        return kinds[t.replace("const ", "")]
+
+    def ct_kind(t):
+        if t in (C.c_void_p, C.c_char_p) or (isinstance(t, type) and issubclass(t, C._Pointer)):
+            return "ptr"
+        return {C.c_int32: "i32", C.c_uint32: "u32", C.c_uint64: "u64", C.c_size_t: "u64", C.c_float: "f32"}[t]
+
+    sigs = header_signatures()
+    assert sorted(sigs) == sorted(_lib.PROTOTYPES)
+    wrong = []
+    for name, (ret, params) in sigs.items():
+        want = [c_kind(p) for p in params]
+        got = [ct_kind(t) for t in _lib.PROTOTYPES[name]]
+        want_ret = "ptr" if "*" in ret else kinds[ret]
+        got_ret = ct_kind(_lib._RESTYPE.get(name, C.c_int32))
+        if want != got or want_ret != got_ret:
+            wrong.append((name, want, got, want_ret, got_ret))
+    assert not wrong, wrong[:5]
