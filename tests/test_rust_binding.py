@@ -137,3 +137,22 @@ def test_ffi_argument_and_return_types_match_the_header():
         if want_ret != got_ret or want != got:
             wrong.append((name, want_ret, want, got_ret, got))
     assert not wrong, wrong[:5]
+
+
+def test_the_declarations_shown_in_the_integration_guide_match_the_header():
+    """INTEGRATION.md shows a part of the FFI block; what it shows has to be what the header declares."""
+    md = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```rust\n(.*?)```", md, flags=re.S)
+    shown = {}
+    for b in blocks:
+        if 'extern "C"' not in b:
+            continue
+        b = re.sub(r"//[^\n]*", "", b)
+        for name, args, ret in re.findall(r"pub fn (slhip_[a-z0-9_]+)\s*\((.*?)\)\s*->\s*([^;]+);", b, flags=re.S):
+            strip = lambda t: re.sub(r"\s+", " ", re.sub(r"\b(?:std::os::raw::|std::ffi::|core::ffi::)", "", t.strip()))
+            shown[name] = (strip(ret), [strip(a.split(":", 1)[1]) for a in args.split(",") if a.strip()])
+    assert len(shown) >= 30
+    h = header_signatures()
+    wrong = [(n, shown[n], (c_type_to_rust(h[n][0]), [c_type_to_rust(p) for p in h[n][1]])) for n in shown
+             if n not in h or shown[n] != (c_type_to_rust(h[n][0]), [c_type_to_rust(p) for p in h[n][1]])]
+    assert not wrong, wrong[:3]
