@@ -156,3 +156,38 @@ def test_the_declarations_shown_in_the_integration_guide_match_the_header():
     wrong = [(n, shown[n], (c_type_to_rust(h[n][0]), [c_type_to_rust(p) for p in h[n][1]])) for n in shown
              if n not in h or shown[n] != (c_type_to_rust(h[n][0]), [c_type_to_rust(p) for p in h[n][1]])]
     assert not wrong, wrong[:3]
+
+
+def test_every_call_into_the_library_passes_as_many_arguments_as_the_header_declares():
+    """The crate's sources cannot be type-checked here; the number of arguments of every ffi call can."""
+    arity = header_functions()
+    calls = 0
+    for f in ("ops.rs", "device.rs", "graph.rs", "probe.rs"):
+        src = open(os.path.join(CRATE, "src", f)).read()
+        src = re.sub(r"//[^\n]*", "", src)
+        for m in re.finditer(r"\b(slhip_[a-z0-9_]+)\s*\(", src):
+            name = m.group(1)
+            if name not in arity:
+                continue
+            i, depth, args, cur = m.end(), 1, [], ""
+            while depth:
+                ch = src[i]
+                if ch in "([{":
+                    depth += 1
+                elif ch in ")]}":
+                    depth -= 1
+                    if depth == 0:
+                        break
+                if ch == "," and depth == 1:
+                    args.append(cur)
+                    cur = ""
+                else:
+                    cur += ch
+                i += 1
+            if cur.strip():
+                args.append(cur)
+            if re.search(r"\bfn\s*$", src[max(0, m.start() - 12):m.start()]):
+                continue                      # a wrapper's own definition, not a call
+            calls += 1
+            assert len(args) == arity[name], (f, name, len(args), arity[name], src[m.start():i + 1][:200])
+    assert calls >= 50
