@@ -281,8 +281,8 @@ __device__ __forceinline__ void pin_loop_start() {
 constexpr int PIN_ONLY_FAST[2][2] = {{2, 2}, {1, 2}};  // [TA][TB]; the kernel that holds no other loop
 constexpr int PIN_FAST[2][2] = {{2, 2}, {1, 2}};       // the same loop in the kernel that holds all four
 constexpr int PIN_XCLAMP[2][2] = {{1, 2}, {1, 1}};
-constexpr int PIN_WIDE[2][2] = {{3, 3}, {3, 3}};       // the eight-wave tile
-constexpr int PIN_SMALL[2][2] = {{2, 2}, {2, 2}};      // the 64 x 64 tile
+constexpr int PIN_WIDE[2][2] = {{0, 0}, {0, 0}};       // the eight-wave tile (2048^3: 135.7 / 136.2 / 134.4 against 134.7 / 135.9 / 133.5 at 3)
+constexpr int PIN_SMALL[2][2] = {{1, 0}, {0, 0}};      // the 64 x 64 tile (1024^3: 97.1 / 97.2 / 95.7 against 96.3 / 96.8 / 94.1 at 2)
 
 // The k loop over tiles [kt_begin, kt_end) of one workgroup, fetching with load mode MODE.  The
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
