@@ -323,6 +323,27 @@ def test_gemm_with_a_row_vector_runs_as_matrix_times_column(hip, orc):
         assert np.array_equal(out, orc.unary(orc.RELU, pre_act))
 
 
+def test_gemm_few_rows_times_a_large_matrix(hip, orc):
+    """2..32 rows times a matrix of 2^24 elements and more (a small batch through a wide layer): computed as
+    C^T = op(B)^T * op(A)^T through the tall and narrow kernels and transposed into C.  All three forms and
+    A^T * B^T, beta 0 and 1 (applied by the transpose), N and K off the vector and tile grids, the row
+    counts either side of the limits (16 against a B stored K x N, 32 against one stored N x K), and what
+    lies just outside the route (33 rows, a B just below 2^24 elements, another beta)."""
+    cases = [(16, 4096, 4096, 0, 0), (10, 4099, 4100, 0, 0), (2, 8192, 4096, 0, 0), (7, 5000, 7001, 1, 0), (16, 2048, 8200, 1, 0),
+             (3, 4096, 8192, 0, 1), (8, 4096, 4096, 0, 1), (17, 4099, 4101, 0, 1), (32, 2050, 8190, 0, 1), (5, 6000, 3000, 1, 1),
+             (17, 4096, 4096, 0, 0), (33, 4096, 4096, 0, 1), (16, 4000, 4000, 0, 0), (2, 4096, 4096, 0, 1), (12, 16384, 1024, 0, 0)]
+    for (m, n, k, ta, tb) in cases:
+        a, b = gemm_operands(ta, tb, m, n, k)
+        exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
+        bound = bound * (3e-6 / (1e-5 * np.sqrt(k)))           # 3e-6 |A||B|, far inside the contract's bar
+        c0 = rng.uniform(m * n, -1, 1, tag=2, seed=SEED)
+        for beta in (0.0, 1.0, 0.5):
+            say("few rows", m, n, k, ta, tb, beta)
+            got = hip.sgemm(ta, tb, m, n, k, a, b, c=c0.copy(), beta=beta)
+            want = exact + beta * c0
+            assert np.all(np.abs(got - want) <= bound + 1e-6 * np.abs(c0) + 1e-30), (m, n, k, ta, tb, beta, float(np.max(np.abs(got - want) / (bound + 1e-30))))
+
+
 def test_gemm_small_tile(hip, orc):
     # 64 x 64 tiles (chosen by the cost model for products of a few hundred such tiles), forced here
     # so that edge tiles, rows of odd length, k remainders and the fused epilogues all run on them
