@@ -563,6 +563,20 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       small_tile = t64 < 0.92 * best;
       spread64 = small_tile && t_spread < t_whole;
     }
+    // More small tiles than the chip holds at once, short K: the large tile's workgroups spend more time
+    // on their first loads and their 64 KiB of results than on their few k tiles, and a last round of them
+    // that is partly empty cannot be spread (too few k tiles to deal out).  The small tile is level or
+    // ahead up to K = 128 whatever the grid (4096^2 x 64: 34 -> 31 us, 3000 x 5000 x 100: 49 -> 45, 10000 x 1000 x
+    // 100: 40 -> 33; 8192^2 x 128 and 2048 x 8192 x 128 level), and up to K = 384 where its rounds are the fuller
+    // ones (10000 x 1000 x 256: 73 -> 51, x 384: 96 -> 71; 33333 x 257 x 257: 84 -> 63); from K = 200 on a grid that
+    // fills its rounds either way the large tile is 2-7 % ahead and stays.
+    if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && !small_tile && tiles64 > slots64 && splits == 1 &&
+        spread_workers == 0) {
+      const size_t slots128 = (size_t)ctx->num_cu * 2;
+      const double fill128 = (double)tiles / (double)((tiles + slots128 - 1) / slots128 * slots128);
+      const double fill64 = (double)tiles64 / (double)((tiles64 + slots64 - 1) / slots64 * slots64);
+      if (K <= 128 || (K <= 384 && fill64 > 1.1 * fill128)) small_tile = true;
+    }
     if (small_tile) {
       tiles_m = (M + 63) / 64; tiles_n = (N + 63) / 64;
       tiles = tiles64;
