@@ -570,12 +570,17 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     // 100: 40 -> 33; 8192^2 x 128 and 2048 x 8192 x 128 level), and up to K = 384 where its rounds are the fuller
     // ones (10000 x 1000 x 256: 73 -> 51, x 384: 96 -> 71; 33333 x 257 x 257: 84 -> 63); from K = 200 on a grid that
     // fills its rounds either way the large tile is 2-7 % ahead and stays.
-    if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && !small_tile && tiles64 > slots64 && splits == 1 &&
-        spread_workers == 0) {
+    // And where the large tiles are a single round that is at most 85 % full (some CUs hold two workgroups,
+    // the others one, which finishes early and waits): up to K = 512 the small tiles are 10-28 % ahead of
+    // whatever the large-tile plans make of it (2304^2 x 512: 72 -> 57 us, 2000 x 3000 x 200: 38 -> 30, 1800 x 2600 x
+    // 256: 40 -> 32, 2500^2 x 512: 71 -> 63; 2816^2, a round 95 % full, level); at K = 1024 they are level to 14 %
+    // ahead, at 2048 level, and the large-tile plans stay.
+    if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && !small_tile && tiles64 > slots64) {
       const size_t slots128 = (size_t)ctx->num_cu * 2;
       const double fill128 = (double)tiles / (double)((tiles + slots128 - 1) / slots128 * slots128);
       const double fill64 = (double)tiles64 / (double)((tiles64 + slots64 - 1) / slots64 * slots64);
-      if (K <= 128 || (K <= 384 && fill64 > 1.1 * fill128)) small_tile = true;
+      if (splits == 1 && spread_workers == 0 && (K <= 128 || (K <= 384 && fill64 > 1.1 * fill128))) small_tile = true;
+      if (K <= 512 && tiles < slots128 && tiles * 100 <= slots128 * 85) small_tile = true;
     }
     if (small_tile) {
       tiles_m = (M + 63) / 64; tiles_n = (N + 63) / 64;
