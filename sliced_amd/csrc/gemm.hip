@@ -570,6 +570,10 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     // 100: 40 -> 33; 8192^2 x 128 and 2048 x 8192 x 128 level), and up to K = 384 where its rounds are the fuller
     // ones (10000 x 1000 x 256: 73 -> 51, x 384: 96 -> 71; 33333 x 257 x 257: 84 -> 63); from K = 200 on a grid that
     // fills its rounds either way the large tile is 2-7 % ahead and stays.
+    // Fewer than four k tiles (no large-tile plan is modelled that short) and small tiles that fit the chip
+    // at once: 2610 x 160 x 70 13 -> 8 us, 1080 x 578 x 69 13 -> 8, 586 x 1419 x 33 12 -> 7, 1104 x 1156 x 75 14 -> 10.
+    if (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && !small_tile && kt_total < 4 && tiles64 <= slots64)
+      small_tile = true;
     // And where the large tiles are a single round that is at most 85 % full (some CUs hold two workgroups,
     // the others one, which finishes early and waits): up to K = 512 the small tiles are 10-28 % ahead of
     // whatever the large-tile plans make of it (2304^2 x 512: 72 -> 57 us, 2000 x 3000 x 200: 38 -> 30, 1800 x 2600 x
@@ -580,7 +584,13 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       const double fill128 = (double)tiles / (double)((tiles + slots128 - 1) / slots128 * slots128);
       const double fill64 = (double)tiles64 / (double)((tiles64 + slots64 - 1) / slots64 * slots64);
       if (splits == 1 && spread_workers == 0 && (K <= 128 || (K <= 384 && fill64 > 1.1 * fill128))) small_tile = true;
-      if (K <= 512 && tiles < slots128 && tiles * 100 <= slots128 * 85) small_tile = true;
+      if (K <= 640 && tiles < slots128 && tiles * 100 <= slots128 * 85) small_tile = true;
+      // ragged grids: where the small tiles waste at least 4 % less of their area on the edges of C they are
+      // 12-19 % ahead up to K of about 1500 (3209 x 1809 x 1354: 161 -> 136 us, 6313 x 931 x 1164: 141 -> 120,
+      // 791 x 6880 x 1230: 145 -> 130); the large-tile plans for such grids pay a spread tail and its fix-up too
+      const double used128 = (double)M * (double)N / ((double)tiles * 128.0 * 128.0);
+      const double used64 = (double)M * (double)N / ((double)tiles64 * 64.0 * 64.0);
+      if (K <= 1536 && used64 >= 1.04 * used128) small_tile = true;
     }
     if (small_tile) {
       tiles_m = (M + 63) / 64; tiles_n = (N + 63) / 64;
