@@ -353,13 +353,13 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // shape the tall and narrow kernels stream - the large operand once, at 5-6 TB/s, where the wave-per-tile
   // kernel reads it in 128-byte pieces per row (16 x 16384 x 16384: 2.8-3.7 TB/s of B).  C^T goes to the top of
   // the workspace (the inner product sees a workspace that ends below it) and is transposed into C, which is
-  // where beta (0 or 1) is applied.  Up to 16 rows against a B stored K x N (the inner A^T * B kernels take
-  // at most 16 columns), up to 32 against one stored N x K; from 2^24 elements of B (2^25 where fewer than 8
+  // where beta (0 or 1) is applied.  Up to 32 rows (the inner kernels' columns); from 2^24 elements of B (2^25 where fewer than 8
   // rows are stored M x K: the inner kernels for fewer than 8 columns want them as K x M and turn them
   // round only beside an operand that large).  Measured, us before -> after, A*B / A*Bt / At*B:
   // 16 x 16384 x 16384 313 / 399 / 319 -> 237 / 193 / 187; 10 x 4096 x 32768 246 / 322 / 254 -> 104 / 111 / 94;
   // 2 x 10000 x 10000 161 / 190 / 171 -> 88 / 114 / 83; 32 x 16384 x 16384 A*Bt 468 -> 275; 8 x 2048 x 8192 34 / 36 / 36 -> 24 / 28 / 23.
-  if (M >= 2 && M <= (tb ? 32u : 16u) && N >= 512 && K >= 256 && N * K >= (size_t(1) << (!ta && M < 8 ? 25 : 24)) && !bias && !relu &&
+  // (17..32 rows against a B stored K x N only where N is a multiple of 32, which the inner kernel for that many columns needs)
+  if (M >= 2 && M <= 32 && (tb || M <= 16 || N % 32 == 0) && N >= 512 && K >= 256 && N * K >= (size_t(1) << (!ta && M < 8 ? 25 : 24)) && !bias && !relu &&
       !pre_act && !mask && (beta == 0.0f || beta == 1.0f)) {
     const size_t tmp_bytes = (M * N * sizeof(float) + 255) & ~(size_t)255;
     if (tmp_bytes <= ((size_t)16 << 20) && ctx->workspace_bytes >= tmp_bytes + ((size_t)128 << 20)) {

@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
   }
 }
 
-// C = At * B for an A stored K x M (the large operand: read once) and a B of at most 16 columns, stored
+// C = At * B for an A stored K x M (the large operand: read once) and a B of at most 32 columns, stored
 // K x N or N x K: the weight gradient of a narrow layer.  Both operands go from global memory straight into
 // the 16 x 16 x 4 instruction, no LDS on the way: lane (i, kk) = (lane % 16, lane / 16) loads the
 // float4 A[k0 + kk][m0 + 4 i .. + 3] - a wave's load instruction reads 256 contiguous bytes of four
@@ -214,8 +214,10 @@ __global__ __launch_bounds__(256) void gemm_tall_kernel(GemmArgs g, const float*
 // with one per wave.)
 constexpr int TT_STEPS = 8;  // loads in flight per wave: 8 KiB of A
 
+template <int NB>
 __global__ __launch_bounds__(256) void gemm_tall_t_kernel(GemmArgs g, size_t k_share, int tb) {
-  __shared__ __attribute__((aligned(16))) float part[3][64][17];  // waves 1..3: [lane][16 accumulators], padded
+  // NB = 1: at most 16 columns; NB = 2: 17..32, a second block of 16 columns on the same loads of A
+  __shared__ __attribute__((aligned(16))) float part[3][64][16 * NB + 1];  // waves 1..3: [lane][accumulators], padded
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int i = lane & 15, kk = lane >> 4;
   const size_t M = g.M, K = g.K;
@@ -225,24 +227,31 @@ __global__ __launch_bounds__(256) void gemm_tall_t_kernel(GemmArgs g, size_t k_s
   const size_t kend = kbeg + k_share < K ? kbeg + k_share : K;
   const size_t m = m0 + 4 * i;
   const bool m_ok = m < M;  // M is a multiple of 4: the vector lies inside the row or beyond it
-  const bool c_ok = i < N;
   const float* ap = g.A + (m_ok ? m : 0);
   // B stored K x N, or (tb) N x K: element (k, c) at k * bk + c * bc
   const size_t bk = tb ? 1 : (size_t)N, bc = tb ? K : 1;
-  const float* bp = g.B + (c_ok ? i * bc : 0);
+  bool c_ok[NB];
+  const float* bp[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    c_ok[nb] = i + 16 * nb < N;
+    bp[nb] = g.B + (c_ok[nb] ? (size_t)(i + 16 * nb) * bc : 0);
+  }
 
-  floatx4 acc[4];
+  floatx4 acc[NB][4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-    for (int v = 0; v < 4; ++v) acc[t][v] = 0.0f;
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[nb][t][v] = 0.0f;
 
   // wave w takes the steps w, w + 4, ... of its share; step s covers the rows kbeg + 4 s .. + 3
   const size_t steps = (kend - kbeg + 3) / 4;
   // One set of loads at a time: with a second set requested before the first is multiplied the
   // kernel needs 112 VGPRs instead of 74, holds half the waves and measured 3-20 % slower.
   float4 a[TT_STEPS];
-  float b[TT_STEPS];
+  float b[NB][TT_STEPS];
   for (size_t s0 = w; s0 < steps; s0 += 4 * TT_STEPS) {
 #pragma unroll
     for (int u = 0; u < TT_STEPS; ++u) {
@@ -250,23 +259,31 @@ __global__ __launch_bounds__(256) void gemm_tall_t_kernel(GemmArgs g, size_t k_s
       const bool k_ok = s0 + 4 * (size_t)u < steps && k < kend;
       const size_t kc = k_ok ? k : kbeg;
       a[u] = ld4s(ap + kc * M);
-      b[u] = bp[kc * bk];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) b[nb][u] = bp[nb][kc * bk];
       if (!k_ok || !m_ok) a[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (!k_ok || !c_ok) b[u] = 0.0f;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        if (!k_ok || !c_ok[nb]) b[nb][u] = 0.0f;
     }
 #pragma unroll
     for (int u = 0; u < TT_STEPS; ++u) {
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].x, b[u], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].y, b[u], acc[1], 0, 0, 0);
-      acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].z, b[u], acc[2], 0, 0, 0);
-      acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].w, b[u], acc[3], 0, 0, 0);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        acc[nb][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].x, b[nb][u], acc[nb][0], 0, 0, 0);
+        acc[nb][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].y, b[nb][u], acc[nb][1], 0, 0, 0);
+        acc[nb][2] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].z, b[nb][u], acc[nb][2], 0, 0, 0);
+        acc[nb][3] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u].w, b[nb][u], acc[nb][3], 0, 0, 0);
+      }
     }
   }
   if (w) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) part[w - 1][lane][4 * t + v] = acc[t][v];
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part[w - 1][lane][16 * nb + 4 * t + v] = acc[nb][t][v];
   }
   __syncthreads();
   const bool raw = gridDim.y > 1;
@@ -274,25 +291,30 @@ __global__ __launch_bounds__(256) void gemm_tall_t_kernel(GemmArgs g, size_t k_s
 #pragma unroll
     for (int o = 0; o < 3; ++o)
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[t][v] += part[o][lane][4 * t + v];
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[nb][t][v] += part[o][lane][16 * nb + 4 * t + v];
 
-    // register v of block t in lane (i, kk): row m0 + 4 * (4 kk + v) + t of C, column i
-    if (c_ok) {
-      float* dst = raw ? g.partial + (size_t)blockIdx.y * M * (size_t)N : g.C;
+    // register v of block t in lane (i, kk): row m0 + 4 * (4 kk + v) + t of C, column i (+ 16 for the second block)
+    float* dst = raw ? g.partial + (size_t)blockIdx.y * M * (size_t)N : g.C;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      if (!c_ok[nb]) continue;
+      const int col = i + 16 * nb;
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           const size_t row = m0 + 4 * (4 * kk + v) + t;
           if (row >= M) continue;
-          const size_t at = row * (size_t)N + i;
-          float x = acc[t][v];
+          const size_t at = row * (size_t)N + col;
+          float x = acc[nb][t][v];
           if (!raw) {
             if (g.mask) x = (g.mask[at] >= 0.0f ? 1.0f : 0.0f) * x;
             if (g.beta != 0.0f) x = g.beta * g.C[at] + x;
-            if (g.bias) x = x + g.bias[i];
+            if (g.bias) x = x + g.bias[col];
             if (g.pre_act) g.pre_act[at] = x;
             if (g.relu) x = (x >= 0.0f ? 1.0f : 0.0f) * x;
           }
@@ -310,7 +332,9 @@ int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc)
   // 2048 x 10 x 8192 24.5 -> 19.1 us, 16384 x 10 / 16 x 16384 220 / 234 -> 172 / 177 (6.3 / 6.1 TB/s),
   // 2048 x 16 x 2048 16.6 -> 10.1, 256 x 16 x 262144 94 -> 65, 65536 x 10 x 1024 60 -> 46; with 4..7
   // columns the two are level (ahead on some shapes, behind on others) and the other one stays.
-  if (ta && N <= 16 && N >= 8 && M % 32 == 0 && M >= 64 && K >= 64 && M * K >= (size_t(1) << 22)) {
+  // 17..32 columns: a second block of 16 columns on the same loads of A (4096 x 17 / 32 x 65536 502 -> 205 / 211 us,
+  // 16384 x 24 x 16384 276 -> 203, 65536 x 32 x 1024 87 -> 63, all on the wave-per-tile kernel before).
+  if (ta && N <= 32 && N >= 8 && M % 32 == 0 && M >= 64 && K >= 64 && M * K >= (size_t(1) << 22)) {
     const size_t gx = (M + 63) / 64;
     if (gx > 0x7fffffffu) return 0;
     // two workgroups per CU; every wave of a share gets at least 8 steps of four k
@@ -322,7 +346,8 @@ int gemm_tall_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* rc)
     const size_t share = ((K + splits - 1) / splits + 3) / 4 * 4;
     splits = (K + share - 1) / share;
     g.splits = (unsigned)splits;
-    hipLaunchKernelGGL(gemm_tall_t_kernel, dim3((unsigned)gx, (unsigned)splits), dim3(256), 0, ctx->stream, g, share, tb ? 1 : 0);
+    if (N <= 16) hipLaunchKernelGGL(gemm_tall_t_kernel<1>, dim3((unsigned)gx, (unsigned)splits), dim3(256), 0, ctx->stream, g, share, tb ? 1 : 0);
+    else hipLaunchKernelGGL(gemm_tall_t_kernel<2>, dim3((unsigned)gx, (unsigned)splits), dim3(256), 0, ctx->stream, g, share, tb ? 1 : 0);
     *rc = post_launch();
     return splits > 1 && *rc == SLHIP_OK ? 2 : 1;
   }

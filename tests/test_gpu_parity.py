@@ -257,12 +257,14 @@ def test_gemm_tall_kernel(hip, orc):
 
 
 def test_gemm_transposed_tall_operand_with_narrow_b(hip, orc):
-    """At * B and At * Bt with A stored K x M and 8..16 columns of B (the weight gradient of a narrow
+    """At * B and At * Bt with A stored K x M and 8..32 columns of B (the weight gradient of a narrow
     layer): the kernel that feeds both operands from global memory into the 16 x 16 x 4 instruction.
     M on and off the multiples of 64, K off the multiples of 4 and of a share, one share and many,
     beta and the mask epilogue; the same sums whichever way B is stored and on every run."""
     for (m, n, k) in [(2048, 10, 8192), (96, 16, 70001), (4096, 8, 1030), (64, 13, 65536), (65536, 9, 65), (8192, 12, 2048),
-                      (1056, 11, 4099)]:
+                      (1056, 11, 4099),
+                      # 17..32 columns: the second block of 16 on the same loads of A
+                      (2048, 17, 8192), (96, 32, 70001), (4096, 24, 1030), (64, 31, 65539), (8192, 20, 2048), (1056, 29, 4099)]:
         a, b = gemm_operands(1, 0, m, n, k)
         exact, bound = gemm_bound(1, 0, m, n, k, a, b)
         say("At*B, narrow B", m, n, k)
@@ -327,8 +329,8 @@ def test_gemm_few_rows_times_a_large_matrix(hip, orc):
     """2..32 rows times a matrix of 2^24 elements and more (a small batch through a wide layer): computed as
     C^T = op(B)^T * op(A)^T through the tall and narrow kernels and transposed into C.  All three forms and
     A^T * B^T, beta 0 and 1 (applied by the transpose), N and K off the vector and tile grids, the row
-    counts either side of the limits (16 against a B stored K x N, 32 against one stored N x K), and what
-    lies just outside the route (33 rows, a B just below 2^24 elements, another beta)."""
+    counts 2..32 either side of the kernels' limits of 8 and 16, and what lies just outside the route (33 rows,
+    a B just below 2^24 elements, another beta)."""
     cases = [(16, 4096, 4096, 0, 0), (10, 4099, 4100, 0, 0), (2, 8192, 4096, 0, 0), (7, 5000, 7001, 1, 0), (16, 2048, 8200, 1, 0),
              (3, 4096, 8192, 0, 1), (8, 4096, 4096, 0, 1), (17, 4099, 4101, 0, 1), (32, 2050, 8190, 0, 1), (5, 6000, 3000, 1, 1),
              (17, 4096, 4096, 0, 0), (33, 4096, 4096, 0, 1), (16, 4000, 4000, 0, 0), (2, 4096, 4096, 0, 1), (12, 16384, 1024, 0, 0)]
