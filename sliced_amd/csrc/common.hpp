@@ -29,6 +29,11 @@ struct slhip_ctx {
     bool ta = false, tb = false, only_fast = false, small_tile = false;
     unsigned splits = 1, waves = 4;
   } last_gemm;
+  // A product issued as its transpose (gemm_run): where the combine of the inner product's k shares may
+  // write the result, transposed, instead of leaving it to a transpose launch of its own.
+  float* swap_c = nullptr;   // the caller's C (N' x M' row-major for an inner M' x N' product), or null
+  float swap_beta = 0.0f;
+  bool swap_done = false;    // a combine has written swap_c
 };
 
 struct slhip_event {

@@ -296,7 +296,37 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(size_t mn, size_t N,
   }
 }
 
+// The same sums written transposed: C[n * M + r] = beta * C[n * M + r] + sum_z partial[z][r * N + n], for an
+// M x N product with a narrow N (at most 32) that stands for the N x M product the caller asked for.
+// Thread i takes element i of C (consecutive lanes: consecutive r of one n), so the stores are whole lines
+// and a wave's loads cover one contiguous run of 64 rows of the partial.
+__global__ __launch_bounds__(256) void splitk_reduce_t_kernel(size_t M, size_t N, unsigned splits, const float* __restrict__ partial,
+                                                              float* C, float beta) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= M * N) return;
+  const size_t n = i / M, r = i - n * M;
+  const float* p = partial + r * N + n;
+  const size_t step = M * N;
+  float s = p[0];
+  unsigned z = 1;
+  for (; z + 8 <= splits; z += 8) {  // eight loads in flight, added in the same order as one by one
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = p[(size_t)(z + u) * step];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += t[u];
+  }
+  for (; z < splits; ++z) s += p[(size_t)z * step];
+  C[i] = beta != 0.0f ? beta * C[i] + s : s;
+}
+
 static int32_t splitk_combine(slhip_ctx* ctx, const GemmArgs& g, size_t splits) {
+  if (ctx->swap_c && !g.bias && !g.relu && !g.pre_act && !g.mask && g.beta == 0.0f && g.M * g.N <= 0xffffffffu * (size_t)256) {
+    hipLaunchKernelGGL(splitk_reduce_t_kernel, dim3((unsigned)((g.M * g.N + 255) / 256)), dim3(256), 0, ctx->stream, g.M, g.N,
+                       (unsigned)splits, (const float*)ctx->workspace, ctx->swap_c, ctx->swap_beta);
+    ctx->swap_done = true;
+    return post_launch();
+  }
   const size_t mn = g.M * g.N;
   const int vec = mn % 4 == 0;  // the flat M x N array in whole vectors (each may run over a row end)
   size_t blocks = ((vec ? mn / 4 : mn) + 255) / 256;
@@ -353,22 +383,31 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // shape the tall and narrow kernels stream - the large operand once, at 5-6 TB/s, where the wave-per-tile
   // kernel reads it in 128-byte pieces per row (16 x 16384 x 16384: 2.8-3.7 TB/s of B).  C^T goes to the top of
   // the workspace (the inner product sees a workspace that ends below it) and is transposed into C, which is
-  // where beta (0 or 1) is applied.  Up to 32 rows (the inner kernels' columns); from 2^24 elements of B (2^25 where fewer than 8
-  // rows are stored M x K: the inner kernels for fewer than 8 columns want them as K x M and turn them
-  // round only beside an operand that large).  Measured, us before -> after, A*B / A*Bt / At*B:
+  // where beta (0 or 1) is applied - unless the inner product ends in a combine of k shares, which then writes
+  // C itself, transposed (one launch less: 10 x 2048 x 8192 24 -> 20 us).  Up to 32 rows (the inner kernels'
+  // columns).  Measured, us before -> after, A*B / A*Bt / At*B:
   // 16 x 16384 x 16384 313 / 399 / 319 -> 237 / 193 / 187; 10 x 4096 x 32768 246 / 322 / 254 -> 104 / 111 / 94;
   // 2 x 10000 x 10000 161 / 190 / 171 -> 88 / 114 / 83; 32 x 16384 x 16384 A*Bt 468 -> 275; 8 x 2048 x 8192 34 / 36 / 36 -> 24 / 28 / 23.
   // (17..32 rows against a B stored K x N only where N is a multiple of 32, which the inner kernel for that many columns needs)
-  if (M >= 2 && M <= 32 && (tb || M <= 16 || N % 32 == 0) && N >= 512 && K >= 256 && N * K >= (size_t(1) << (!ta && M < 8 ? 25 : 24)) && !bias && !relu &&
+  // From how many elements of B: 2^24; 2^23 for at most 16 rows against a B stored K x N (16 x 2048 x 4096 A*B 21.5 ->
+  // 16.1 us, At*B 22.1 -> 15.2; A*Bt loses there, 22.3 -> 24.0, and so do 32 rows); 2^22 for fewer than 8 rows stored
+  // K x M (4 x 2048 x 2048 At*B 19.9 -> 11.6); 2^25 for fewer than 8 rows stored M x K (the inner kernels for fewer
+  // than 8 columns want them as K x M and turn them round only beside an operand that large).
+  const int swap_from = !ta && M < 8 ? 25 : ta && !tb && M < 8 ? 22 : !tb && M <= 16 ? 23 : 24;
+  if (M >= 2 && M <= 32 && (tb || M <= 16 || N % 32 == 0) && N >= 512 && K >= 256 && N * K >= (size_t(1) << swap_from) && !bias && !relu &&
       !pre_act && !mask && (beta == 0.0f || beta == 1.0f)) {
     const size_t tmp_bytes = (M * N * sizeof(float) + 255) & ~(size_t)255;
     if (tmp_bytes <= ((size_t)16 << 20) && ctx->workspace_bytes >= tmp_bytes + ((size_t)128 << 20)) {
       const size_t whole = ctx->workspace_bytes;
       float* ct = (float*)((char*)ctx->workspace + whole - tmp_bytes);
       ctx->workspace_bytes = whole - tmp_bytes;
+      // (where the inner product ends in a combine of k shares, that combine writes C itself, transposed)
+      ctx->swap_c = C; ctx->swap_beta = beta; ctx->swap_done = false;
       const int32_t rc = gemm_run(ctx, !tb, !ta, N, M, K, B, A, ct, 0.0f, nullptr, 0, nullptr, nullptr);
+      const bool done = ctx->swap_done;
+      ctx->swap_c = nullptr; ctx->swap_done = false;
       ctx->workspace_bytes = whole;
-      if (rc != SLHIP_OK) return rc;
+      if (rc != SLHIP_OK || done) return rc;
       const auto inner = ctx->last_gemm;
       const int32_t rt = slhip_transpose(ctx, N, M, ct, C, beta);
       ctx->last_gemm = inner;

@@ -266,10 +266,11 @@ __global__ __launch_bounds__(64 * NARROW_WAVES) void gemm_narrow_n_kernel(size_t
 template <int NP>
 __global__ __launch_bounds__(256) void narrow_n_combine_kernel(size_t M, int N, unsigned splits, const float* __restrict__ partial,
                                                                float* C, float beta, const float* __restrict__ bias, int relu,
-                                                               float* pre_act, const float* __restrict__ mask) {
+                                                               float* pre_act, const float* __restrict__ mask, int transposed) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= M * (size_t)N) return;
-  const size_t row = i / N, n = i % N;
+  // (transposed: C is N x M, element i of it is column i / M of row i % M of the product; no epilogue then)
+  const size_t row = transposed ? i % M : i / N, n = transposed ? i / M : i % N;
   const float* p = partial + row * NP + n;
   const size_t step = M * NP;
   float s = p[0];
@@ -562,18 +563,22 @@ int gemm_skinny_launch(slhip_ctx* ctx, bool ta, bool tb, GemmArgs& g, int32_t* r
     const dim3 grid((unsigned)gx, (unsigned)splits);
     const size_t outs = M * N;
     const dim3 cgrid((unsigned)((outs + 255) / 256));
+    // (a product issued as its transpose: the combine writes the caller's C)
+    const bool swap = ctx->swap_c && !g.bias && !g.relu && !g.pre_act && !g.mask && g.beta == 0.0f;
 #define SL_NN(NP_)                                                                                                           \
   do {                                                                                                                       \
     hipLaunchKernelGGL((gemm_narrow_n_kernel<NP_>), grid, dim3(64 * NARROW_WAVES), 0, ctx->stream, M, (int)N, K, g.A, g.B,   \
                        g.partial, k_chunk);                                                                                  \
     hipLaunchKernelGGL((narrow_n_combine_kernel<NP_>), cgrid, dim3(256), 0, ctx->stream, M, (int)N, (unsigned)splits,        \
-                       (const float*)g.partial, g.C, g.beta, g.bias, g.relu, g.pre_act, g.mask);                             \
+                       (const float*)g.partial, swap ? ctx->swap_c : g.C, swap ? ctx->swap_beta : g.beta, g.bias, g.relu,    \
+                       g.pre_act, g.mask, swap ? 1 : 0);                                                                     \
   } while (0)
     if (NP == 4) SL_NN(4);
     else if (NP == 8) SL_NN(8);
     else if (NP == 12) SL_NN(12);
     else SL_NN(16);
 #undef SL_NN
+    if (swap) ctx->swap_done = true;
     *rc = post_launch();
     return 1;
   }

@@ -333,7 +333,9 @@ def test_gemm_few_rows_times_a_large_matrix(hip, orc):
     a B just below 2^24 elements, another beta)."""
     cases = [(16, 4096, 4096, 0, 0), (10, 4099, 4100, 0, 0), (2, 8192, 4096, 0, 0), (7, 5000, 7001, 1, 0), (16, 2048, 8200, 1, 0),
              (3, 4096, 8192, 0, 1), (8, 4096, 4096, 0, 1), (17, 4099, 4101, 0, 1), (32, 2050, 8190, 0, 1), (5, 6000, 3000, 1, 1),
-             (17, 4096, 4096, 0, 0), (33, 4096, 4096, 0, 1), (16, 4000, 4000, 0, 0), (2, 4096, 4096, 0, 1), (12, 16384, 1024, 0, 0)]
+             (17, 4096, 4096, 0, 0), (33, 4096, 4096, 0, 1), (16, 4000, 4000, 0, 0), (2, 4096, 4096, 0, 1), (12, 16384, 1024, 0, 0),
+             # the lower size limits of the forms: 2^23 elements of B for at most 16 rows against K x N, 2^22 for fewer than 8 stored K x M
+             (16, 2048, 4096, 0, 0), (9, 4100, 2050, 1, 0), (4, 2048, 2048, 1, 0), (7, 1028, 4099, 1, 0), (16, 2048, 4096, 0, 1), (4, 2048, 2048, 0, 0)]
     for (m, n, k, ta, tb) in cases:
         a, b = gemm_operands(ta, tb, m, n, k)
         exact, bound = gemm_bound(ta, tb, m, n, k, a, b)
