@@ -106,8 +106,11 @@ struct SumOp {
   static __device__ __forceinline__ float identity() { return 0.0f; }
   static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
 };
+// fmaxf returns its other operand when one is NaN, so NaN is its neutral element and -inf is not:
+// a row of nothing but NaN has NaN as its maximum (src/ops2/max/cpu.rs:11-13 folds `T::max` from the
+// row's first element), which an accumulator that starts at -inf would turn into -inf.
 struct MaxOp {
-  static __device__ __forceinline__ float identity() { return -__builtin_huge_valf(); }
+  static __device__ __forceinline__ float identity() { return __builtin_nanf(""); }
   static __device__ __forceinline__ float apply(float a, float b) { return fmaxf(a, b); }
 };
 

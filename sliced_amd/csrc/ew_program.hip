@@ -60,7 +60,8 @@ struct EwProgArgs {
 __device__ __forceinline__ float ewp_pow(float x, float p) {  // as pow_ref of the single-op kernels
   if (p == 2.0f) return x * x;
   if (p == 1.0f) return x;
-  if (p == 0.5f) return sqrtf(x);
+  // powf(-inf, 0.5) is +inf and powf(-0, 0.5) is +0 where the square root has NaN and -0
+  if (p == 0.5f) return x == -__builtin_huge_valf() ? __builtin_huge_valf() : sqrtf(x) + 0.0f;
   return powf(x, p);
 }
 

@@ -6,6 +6,7 @@
 // row); *_rows reduces along the strided axis (one value per column).
 #include <mutex>
 #include <numeric>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -251,8 +252,9 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, Src x,
 // out[r] = reduce over the contiguous axis.
 template <class Op, class Src>
 static int32_t reduce_cols_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin) {
-  // one column: every row is its own sum / max / mean (x/1 == x), i.e. a plain copy
-  if constexpr (Src::IS_PLAIN)
+  // one column: every row is its own maximum, i.e. a plain copy (not so for a sum or a mean: the
+  // reference's sum starts at +0, and 0 + -0 is +0 where a copy would leave -0)
+  if constexpr (Src::IS_PLAIN && std::is_same<Op, MaxOp>::value)
     if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, rows * sizeof(float));
   if (cols <= 128 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {  // many short rows
     // whole multiples of 256 rows while they fit (every lane of the second phase busy), else as many
@@ -526,8 +528,8 @@ template <class Op, class Src>
 static int32_t reduce_rows_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin, float* ws,
                            size_t ws_left) {
   if (cols == 1) return reduce_all_src<Op, Src>(ctx, rows, x, out, fin, ws);  // at most 4 partials per CU
-  // one row: the reduction over rows is that row itself
-  if constexpr (Src::IS_PLAIN)
+  // one row: the maximum over rows is that row itself (a sum starts at +0 and turns a -0 into +0)
+  if constexpr (Src::IS_PLAIN && std::is_same<Op, MaxOp>::value)
     if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, cols * sizeof(float));
   // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
   // about 512 per CU (measured optimum: 7.0 TB/s at 131072 threads on [16384 x 16384]; 5.4 TB/s at
