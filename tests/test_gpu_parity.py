@@ -1117,6 +1117,59 @@ def test_context_on_a_callers_stream(hip, orc):
     assert rt.hipStreamDestroy(stream) == 0
 
 
+def test_contexts_on_several_host_threads_do_not_disturb_each_other(hip):
+    """Three contexts, each driven by its own host thread at the same time (ctypes releases the
+    interpreter lock during a call), each with its own stream and workspace: a split-k product and
+    a strided-axis sum (both keep partials in the workspace), a softmax, a transpose and a fused
+    loss, thirty rounds each.  Every round of every thread equals, bit for bit, what one context
+    computes alone: nothing in the library is shared between contexts but the error string, which
+    is per thread."""
+    import threading
+    from sliced_amd.device import Context
+    m, n, k = 96, 40, 8192                      # few tiles, long k: split over the grid, partials in the workspace
+    rows, cols = 3000, 129
+
+    def work(ctx, seed, rounds, out):
+        a = ctx.array(rng.uniform(m * k, -1, 1, tag=0, seed=seed))
+        b = ctx.array(rng.uniform(k * n, -1, 1, tag=1, seed=seed))
+        x = ctx.array(rng.uniform(rows * cols, -4, 4, tag=2, seed=seed))
+        cmat, colsum, soft, tr = ctx.empty(m * n), ctx.empty(cols), ctx.empty(rows * cols), ctx.empty(rows * cols)
+        try:
+            for _ in range(rounds):
+                ctx.call("slhip_sgemm", 0, 0, m, n, k, a.ptr, b.ptr, cmat.ptr, 0.0)
+                ctx.call("slhip_sum_rows", rows, cols, x.ptr, colsum.ptr)
+                ctx.call("slhip_softmax", rows, cols, x.ptr, soft.ptr)
+                ctx.call("slhip_transpose", rows, cols, soft.ptr, tr.ptr, 0.0)
+                out.append((cmat.numpy(), colsum.numpy(), tr.numpy()))
+                ctx.call("slhip_ew_unary", 6, 0.999, 0.0, rows * cols, x.ptr, x.ptr)      # the input moves on
+        except Exception as e:                   # a failure in a thread has to reach the test
+            out.append(e)
+        for z in (a, b, x, cmat, colsum, soft, tr):
+            z.free()
+
+    seeds = [SEED + 1, SEED + 2, SEED + 3]
+    alone = []
+    for sd in seeds:
+        res = []
+        work(hip.ctx(), sd, 30, res)
+        alone.append(res)
+    ctxs = [Context(0) for _ in seeds]
+    together = [[] for _ in seeds]
+    threads = [threading.Thread(target=work, args=(c, sd, 30, res)) for c, sd, res in zip(ctxs, seeds, together)]
+    say("three contexts on three threads")
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for c in ctxs:
+        c.close()
+    for res, ref in zip(together, alone):
+        assert len(res) == len(ref) == 30 and not any(isinstance(r, Exception) for r in res + ref), [r for r in res if isinstance(r, Exception)]
+        for got, want in zip(res, ref):
+            for g, w in zip(got, want):
+                assert np.array_equal(g, w)
+
+
 # --------------------------------------------------------------------------- error behaviour
 def test_invalid_arguments_return_status_not_crash(hip):
     c = hip.ctx()

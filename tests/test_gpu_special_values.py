@@ -314,3 +314,25 @@ def test_softmax_gradient_and_losses_on_special_operands(hip, orc):
         targets.reshape(rows, cols)[np.arange(rows), rs.randint(0, cols, rows)] = 1.0
         assert_same_outcome(hip.cce(rows, cols, preds, targets), orc.cce(rows, cols, preds, targets), "cce", rel=2e-6)
         assert_same_outcome(hip.cce_grad(rows, cols, preds, targets), orc.cce_grad(rows, cols, preds, targets), "cce_grad", rel=2e-6)
+
+
+def test_fused_chains_on_special_operands_equal_the_ops_one_by_one(hip):
+    """A chain run as one launch keeps its intermediates in registers; NaN, inf, -0 and subnormals
+    have to come out of it exactly as out of the same ops launched one after the other."""
+    import test_gpu_fusion as fusion
+    rs = np.random.RandomState(11)
+    for name, (n_in, prog) in fusion.PROGRAMS.items():
+        for n in (11, 1000, 4099):
+            say("program", name, n)
+            inputs = [special_operand(rs, n) for _ in range(n_in)]
+            want = fusion.run_one_by_one(hip, inputs, prog)[4 + len(prog) - 1]
+            got = hip.ew_program(inputs, prog)
+            assert np.array_equal(got, want, equal_nan=True), name
+            ok = ~np.isnan(want)
+            assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32)), name      # the sign of a zero too
+            g = special_operand(rs, n)
+            grads0 = [np.zeros(n, np.float32) for _ in range(n_in)]
+            want_g = fusion.grads_one_by_one(hip, inputs, grads0, prog, g)
+            got_g = hip.ew_program_grad(inputs, grads0, prog, g)
+            for j in range(n_in):
+                assert np.array_equal(got_g[j], want_g[j], equal_nan=True), (name, j)
