@@ -336,3 +336,64 @@ def test_fused_chains_on_special_operands_equal_the_ops_one_by_one(hip):
             got_g = hip.ew_program_grad(inputs, grads0, prog, g)
             for j in range(n_in):
                 assert np.array_equal(got_g[j], want_g[j], equal_nan=True), (name, j)
+
+
+SET_SHAPES = [(1, 1, 1), (5, 10, 7), (64, 64, 64), (129, 127, 130), (300, 10, 2048), (1024, 64, 1), (1, 64, 1024),
+              (64, 1, 1024), (512, 512, 512), (32, 32, 100003), (16, 3000, 500), (257, 17, 3333), (40, 72, 15),
+              (96, 40, 8192), (16, 2048, 4096), (8, 4096, 2048), (4096, 16, 4096), (2048, 24, 8192), (1000, 1000, 256),
+              (1, 2048, 2048), (2048, 2048, 96), (1100, 1100, 700)]
+
+
+@pytest.mark.parametrize("shape", SET_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_beta_zero_overwrites_whatever_the_output_held(hip, shape):
+    """beta = 0 is the reference's SET (src/ops2/gemm/cpu_stack.rs:39 hands BLAS beta = 0, which by
+    the BLAS rule does not read C): an output full of NaN must come out as if it had held zeros,
+    on every product kernel and every split / combine / transposed route behind the entry point."""
+    m, n, k = shape
+    rs = np.random.RandomState(m + 3 * n + 5 * k)
+    a = rs.uniform(-1, 1, m * k).astype(np.float32)
+    b = rs.uniform(-1, 1, k * n).astype(np.float32)
+    nan_c = np.full(m * n, np.nan, np.float32)
+    for ta, tb in ((0, 0), (0, 1), (1, 0), (1, 1)):
+        say("sgemm", ta, tb, shape)
+        clean = hip.sgemm(ta, tb, m, n, k, a, b, c=np.zeros(m * n, np.float32), beta=0.0)
+        dirty = hip.sgemm(ta, tb, m, n, k, a, b, c=nan_c.copy(), beta=0.0)
+        say("   ", hip.ctx().last_gemm_plan())
+        assert np.isfinite(clean).all() and np.array_equal(clean, dirty)
+    pre = rs.uniform(-1, 1, m * n).astype(np.float32)
+    clean = hip.sgemm_relu_mask(0, 0, m, n, k, a, b, pre, c=np.zeros(m * n, np.float32))
+    dirty = hip.sgemm_relu_mask(0, 0, m, n, k, a, b, pre, c=nan_c.copy())
+    assert np.isfinite(clean).all() and np.array_equal(clean, dirty)
+    # the gradient pair of a product and of a Linear layer (trait order m, k, n)
+    g = rs.uniform(-1, 1, m * n).astype(np.float32)
+    lg0, rg0 = hip.gemm_grad(m, k, n, a, b, np.zeros(m * k, np.float32), np.zeros(k * n, np.float32), g)
+    lg1, rg1 = hip.gemm_grad(m, k, n, a, b, np.full(m * k, np.nan, np.float32), np.full(k * n, np.nan, np.float32), g)
+    assert np.array_equal(lg0, lg1) and np.array_equal(rg0, rg1) and np.isfinite(lg0).all() and np.isfinite(rg0).all()
+    z = lambda cnt: np.zeros(cnt, np.float32)
+    f = lambda cnt: np.full(cnt, np.nan, np.float32)
+    x0, w0, b0 = hip.linear_grad(m, k, n, a, b, g, x_grad=z(m * k), relu_pre=None, w_grad=z(k * n), bias_grad=z(n))
+    # (the bias gradient always accumulates, as add_row_mut_grad does in the reference: src/ops2/row_op/grad/cpu.rs:42-50)
+    x1, w1, b1 = hip.linear_grad(m, k, n, a, b, g, x_grad=f(m * k), relu_pre=None, w_grad=f(k * n), bias_grad=z(n))
+    assert np.array_equal(x0, x1) and np.array_equal(w0, w1) and np.array_equal(b0, b1)
+    assert np.isfinite(x0).all() and np.isfinite(w0).all() and np.isfinite(b0).all()
+
+
+def test_set_semantics_of_the_other_ops_with_an_output_full_of_nan(hip):
+    rs = np.random.RandomState(5)
+    for rows, cols in [(7, 5), (300, 129), (1000, 4099), (5000, 10), (8191, 1025), (64, 100003)]:
+        n = rows * cols
+        x = rs.uniform(-3, 3, n).astype(np.float32)
+        say("set semantics", rows, cols)
+        clean = hip.transpose(rows, cols, x, out=np.zeros(n, np.float32), assign=False)
+        dirty = hip.transpose(rows, cols, x, out=np.full(n, np.nan, np.float32), assign=False)
+        assert np.array_equal(clean, dirty) and np.array_equal(clean.reshape(cols, rows), x.reshape(rows, cols).T)
+        p = hip.softmax(rows, cols, x)
+        g = rs.uniform(-1, 1, n).astype(np.float32)
+        clean = hip.softmax_grad(rows, cols, p, g, x_grad=np.zeros(n, np.float32), beta=0.0)
+        dirty = hip.softmax_grad(rows, cols, p, g, x_grad=np.full(n, np.nan, np.float32), beta=0.0)
+        assert np.isfinite(clean).all() and np.array_equal(clean, dirty)
+        t = np.zeros(n, np.float32)
+        t.reshape(rows, cols)[np.arange(rows), rs.randint(0, cols, rows)] = 1.0
+        clean = hip.softmax_cce_grad(rows, cols, p, t, np.zeros(n, np.float32), beta=0.0)
+        dirty = hip.softmax_cce_grad(rows, cols, p, t, np.full(n, np.nan, np.float32), beta=0.0)
+        assert np.isfinite(clean).all() and np.array_equal(clean, dirty)
