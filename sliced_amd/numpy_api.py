@@ -30,6 +30,20 @@ def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32).ravel()
 
 
+_operand_offsets = None       # see operands_off_the_vector_grid()
+_next_offset = 0
+
+
+def operands_off_the_vector_grid(on):
+    """With on=True every device buffer this facade creates starts 1, 2 or 3 floats (in turn) into
+    its allocation instead of on the allocator's 256-byte grid: the library promises to take
+    pointers that are only float-aligned, and this lets any test that goes through the facade ask
+    for exactly that."""
+    global _operand_offsets, _next_offset
+    _operand_offsets = (1, 2, 3) if on else None
+    _next_offset = 0
+
+
 class _Scope:
     """Frees every device buffer created inside the with-block."""
 
@@ -44,22 +58,27 @@ class _Scope:
         for b in self.bufs:
             b.free()
 
+    def _alloc(self, n, zero):
+        global _next_offset
+        off = 0
+        if _operand_offsets:
+            off = _operand_offsets[_next_offset % len(_operand_offsets)]
+            _next_offset += 1
+        pool = (self.c.zeros if zero else self.c.empty)(n + off)
+        self.bufs.append(pool)
+        return pool.view(off, n) if off else pool
+
     def up(self, a):
         if a is None:
             return None
-        b = self.c.array(_f32(a))
-        self.bufs.append(b)
-        return b
+        a = _f32(a)
+        return self._alloc(a.size, False).upload(a)
 
     def zeros(self, n):
-        b = self.c.zeros(n)
-        self.bufs.append(b)
-        return b
+        return self._alloc(n, True)
 
     def empty(self, n):
-        b = self.c.empty(n)
-        self.bufs.append(b)
-        return b
+        return self._alloc(n, False)
 
 
 def _ptr(b):
