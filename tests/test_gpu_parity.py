@@ -1263,6 +1263,83 @@ def test_recorded_sequence_replays_like_eager_calls(hip, orc):
         z.free()
 
 
+def test_recording_holds_every_product_route_and_kernel_family(hip):
+    """One recording with the products that take the library's side routes (a few rows times a large
+    matrix, computed as the transposed product with a transposed combine; A^T B with 24 columns;
+    split k with its combine; a grid with a spread tail; tall A; the wave-per-tile kernel), the
+    transposes that stage more rows than they write, reductions that keep partials in the workspace,
+    softmax on short, medium and two-sweep rows, the fused losses and a fused elementwise chain:
+    three replays, eager work between them, each equal bit for bit to the same calls made eagerly.
+    State that a route keeps on the context between its launches must not leak into a recording."""
+    c = hip.ctx()
+    lib = c.lib
+    products = [(0, 0, 16, 2048, 4096), (0, 1, 8, 4096, 2048), (1, 0, 2048, 24, 8192), (0, 0, 96, 40, 8192),
+                (0, 0, 1100, 1100, 700), (0, 0, 16384, 16, 2048), (0, 0, 40, 72, 15), (1, 0, 300, 10, 2048), (0, 1, 1, 2048, 2048)]
+    mats = [(8191, 1025), (100003, 56), (64, 5000), (300, 129), (5000, 10), (9, 40000)]
+    bufs = []
+
+    def dev(n, tag):
+        b = c.array(rng.uniform(n, -1, 1, tag=tag, seed=SEED + n % 1000))
+        bufs.append(b)
+        return b
+
+    def out(n):
+        b = c.zeros(n)
+        bufs.append(b)
+        return b
+
+    P = [(ta, tb, m, n, k, dev(m * k, 0), dev(k * n, 1), out(m * n)) for ta, tb, m, n, k in products]
+    M = [(r, cl, dev(r * cl, 2), out(r * cl), out(r * cl), out(cl), out(r), out(r * cl), out(r)) for r, cl in mats]
+    outputs = [p[7] for p in P] + [b for mrow in M for b in mrow[3:]]
+
+    def sequence():
+        for ta, tb, m, n, k, a, b, cm in P:
+            c.call("slhip_sgemm", ta, tb, m, n, k, a.ptr, b.ptr, cm.ptr, 0.0)
+        for r, cl, x, tr, sm, colsum, rowmax, gr, loss in M:
+            c.call("slhip_transpose", r, cl, x.ptr, tr.ptr, 0.0)
+            c.call("slhip_softmax", r, cl, x.ptr, sm.ptr)
+            c.call("slhip_sum_rows", r, cl, sm.ptr, colsum.ptr)
+            c.call("slhip_max_cols", r, cl, x.ptr, rowmax.ptr)
+            c.call("slhip_softmax_grad", r, cl, gr.ptr, sm.ptr, tr.ptr, 0.0)         # tr: any tensor of that size as upstream gradient
+            c.call("slhip_softmax_cce", r, cl, x.ptr, sm.ptr, None, loss.ptr)        # sm as (soft) targets
+            c.call("slhip_ew_unary", 6, 0.75, 0.0, r * cl, x.ptr, x.ptr)             # the input moves on
+        for ta, tb, m, n, k, a, b, cm in P:
+            c.call("slhip_ew_unary", 6, 0.9, 0.0, m * k, a.ptr, a.ptr)
+
+    def snapshot():
+        return [b.numpy() for b in outputs]
+
+    inputs0 = [(p[5], p[5].numpy()) for p in P] + [(mrow[2], mrow[2].numpy()) for mrow in M]
+    eager = []
+    for _ in range(3):
+        sequence()
+        eager.append(snapshot())
+    for b, h in inputs0:
+        b.upload(h)
+    for b in outputs:
+        c.call("slhip_memset", b.ptr, 0, b.nbytes)
+    c.call("slhip_graph_begin")
+    sequence()
+    g = C.c_void_p()
+    c.call("slhip_graph_end", C.byref(g))
+    scratch = c.empty(1 << 16)
+    ea, eb, ec = dev(16 * 4096, 5), dev(4096 * 2048, 6), out(16 * 2048)
+    for i in range(3):
+        say("replay", i)
+        c.call("slhip_graph_launch", g)
+        c.call("slhip_fill", scratch.n, float(i), scratch.ptr)
+        # an eager product on the same context between the replays: its route leaves its own state behind
+        c.call("slhip_sgemm", 0, 0, 16, 2048, 4096, ea.ptr, eb.ptr, ec.ptr, 0.0)
+        c.sync()
+        got = snapshot()
+        for j, (gv, ev) in enumerate(zip(got, eager[i])):
+            assert np.array_equal(gv, ev, equal_nan=True), (i, j)
+    assert lib.slhip_graph_destroy(g) == 0
+    scratch.free()
+    for z in bufs:
+        z.free()
+
+
 def test_relu_mask_as_bits_equals_the_float_mask(hip, orc):
     """slhip_linear_fwd_bits / slhip_sgemm_relu_bits / slhip_relu_grad_bits against the float forms
     (linear_fwd with pre-activations, sgemm_relu_mask, the relu gradient): the same values within the
