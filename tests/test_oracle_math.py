@@ -299,3 +299,34 @@ def test_host_rng_is_reproducible_and_in_range():
     assert k.min() == 0 and k.max() == 9
     x = rng.inject_row_max_ties(rng.uniform(40 * 300, -10, 10, tag=0), 40, 300, 0.01).reshape(40, 300)
     assert np.all((x == x.max(1, keepdims=True)).sum(1) >= 3)
+
+
+def test_special_values_follow_ieee_and_the_documented_maximum(orc):
+    """What the oracle does with NaN, infinities and signed zeros, pinned by what fixes it outside
+    the oracle: `f32::max` is documented to return the other argument when one is NaN (so a maximum
+    skips NaNs and is NaN only over nothing but NaN: numpy's fmax has the same rule); a sum is a
+    chain of IEEE additions from +0 (NaN and inf - inf poison it, 0 + -0 is +0); softmax's shift by
+    the row maximum turns a row holding +inf, or nothing but -inf, into NaN."""
+    nan, inf = np.float32(np.nan), np.float32(np.inf)
+    x = np.array([[nan, 1, -inf, nan], [2, nan, -inf, nan], [-3, inf, -inf, nan]], np.float32)
+    rows, cols = x.shape
+    assert np.array_equal(orc.max_rows(cols, x.ravel()), np.fmax.reduce(x, axis=0), equal_nan=True)
+    assert np.array_equal(orc.max_cols(cols, x.ravel()), np.fmax.reduce(x, axis=1), equal_nan=True)
+    assert np.array_equal(orc.max_rows(cols, x.ravel()), np.array([2, inf, -inf, nan], np.float32), equal_nan=True)
+    assert np.array_equal(orc.max_cols(cols, x.ravel()), np.array([1, 2, inf], np.float32), equal_nan=True)
+    with np.errstate(invalid="ignore"):
+        assert np.array_equal(orc.sum_rows(cols, x.ravel()), x.sum(axis=0), equal_nan=True)
+        assert np.array_equal(orc.sum_cols(cols, x.ravel()), x.sum(axis=1), equal_nan=True)
+    y = np.array([[1, inf, -inf], [-inf, -inf, -inf], [inf, -inf, 0], [0, 1, -inf]], np.float32)
+    assert np.array_equal(orc.sum_cols(3, y.ravel()), np.array([nan, -inf, nan, -inf], np.float32), equal_nan=True)
+    z = np.array([-0.0, -0.0, -0.0, -0.0], np.float32)
+    for got in (orc.sum_rows(2, z), orc.sum_cols(2, z), orc.sum_rows(4, z), orc.sum_cols(1, z)):
+        assert not np.signbit(got).any() and np.all(got == 0)
+    s = orc.softmax(4, 3, y.ravel()).reshape(4, 3)
+    assert np.isnan(s[0]).all() and np.isnan(s[1]).all() and np.isnan(s[2]).all()
+    e = np.exp(np.float64(-1))
+    assert np.allclose(s[3], [e / (1 + e), 1 / (1 + e), 0.0], rtol=1e-6, atol=0)
+    # powf's corners, which a square root does not share
+    got = orc.unary(orc.POW, np.array([-inf, -0.0, 0.0, inf, 4.0, -4.0], np.float32), 0.5)
+    assert np.array_equal(got, np.array([inf, 0.0, 0.0, inf, 2.0, nan], np.float32), equal_nan=True)
+    assert not np.signbit(got[1])
