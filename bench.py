@@ -24,7 +24,8 @@ loops' variants, the CPU streaming ops) go to stderr as they are measured and, a
 named by --detail.  An untimed second of matrix-core load (`config.spin_up_s`) precedes the W
 declared warm-up launches of the headline.
 Bandwidth ops and sweep entries are timed as the median of per-launch HIP-event pairs over at least
-20 launches after at least 5 warm-ups; operands below 512 MiB have the caches swept (a read of a
+20 launches after at least 5 warm-ups and 25 ms of untimed launches of the same op
+(`config.op_warm_ms`); operands below 512 MiB have the caches swept (a read of a
 1 GiB scratch) between launches, outside the event pair.  A per-launch pair contains the launch gap
 (about 6 us: `fill of one element` in the list); the GEMM sweep therefore also reports the rate of
 launches queued back to back inside one pair.  Only one GPU is used; --gpus above 1 is refused.
@@ -52,6 +53,7 @@ HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 MIN_ITERS, MIN_WARMUP = 20, 5
 SPIN_UP_SECONDS = 1.0             # untimed load before the headline's declared warm-up launches
+OP_WARM_MS = 25.0                 # untimed launches of an op before its per-launch pairs, at least this long
 MAX_LINE_BYTES = 4096             # the result line stays well below what a log tail keeps
 DETAIL_DEFAULT = os.path.join(ROOT, "bench_detail.json")
 # the ops the metric names, as they appear in the one-line summary: (short key, entry of the suite)
@@ -101,6 +103,16 @@ def pair_times(ctx, fn, iters=MIN_ITERS, warmup=MIN_WARMUP, sweep=None):
     iters, warmup = max(iters, MIN_ITERS), max(warmup, MIN_WARMUP)
     for _ in range(warmup):
         fn()
+    # ... and more of them until OP_WARM_MS have passed: setting up an entry's operands (allocation,
+    # generation, a wait) lets the clocks drop, and five launches of a 0.1 ms kernel do not bring them
+    # back - whichever entry came first after a change of shape measured 1-4 % low (3584^3: 133 TFLOP/s
+    # as the first of the three forms, 137 as the last)
+    t0 = time.perf_counter()
+    ctx.sync()
+    while (time.perf_counter() - t0) * 1e3 < OP_WARM_MS:
+        for _ in range(8):
+            fn()
+        ctx.sync()
     ev = [(ctx.event(), ctx.event()) for _ in range(iters)]
     for a, b in ev:
         if sweep is not None:
@@ -495,7 +507,7 @@ def main():
     detail["notes"] = {
         "traffic_source": "profiles/hbm_traffic_gemm_and_bandwidth_suite.md (rocprofv3 --pmc of this program, not this run)",
         "timing": "achieved: average over the timed launches; *_median and every op: median of per-launch "
-                  "HIP-event pairs, >= %d launches after >= %d warm-ups" % (MIN_ITERS, MIN_WARMUP)}
+                  "HIP-event pairs, >= %d launches after >= %d warm-ups and %g ms of untimed launches of the same op" % (MIN_ITERS, MIN_WARMUP, OP_WARM_MS)}
     # the clock while the matrix cores are busy: queue 0.3 s of launches, sample, then wait
     a, b, c = ctx.uniform(M * K, -1, 1, 0, SEED), ctx.uniform(K * N, -1, 1, 1, SEED), ctx.zeros(M * N)
     for _ in range(min(200, int(300 / max(head["ms_kernel"], 0.01)) + 1)):
@@ -597,7 +609,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "C2 standalone sgemm, M=N=K=%d, C = A*B, A and B ~ U(-1,1) seeded, beta=0" % M,
-                   "kernel": kernel_name, "spin_up_s": SPIN_UP_SECONDS},
+                   "kernel": kernel_name, "spin_up_s": SPIN_UP_SECONDS, "op_warm_ms": OP_WARM_MS},
         "roofline": roof,
         "cpu_baseline": cpu,
     }
