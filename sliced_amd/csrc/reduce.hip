@@ -249,6 +249,25 @@ static int32_t rowreduce_launch(slhip_ctx* ctx, size_t rows, size_t cols, Src x,
   return post_launch();
 }
 
+// The sum (or mean) over an axis of length one: out[i] = 0 + x[i], the reference's fold from +0 -
+// a copy but for -0, which it turns into +0.  One streaming vector per thread.
+__global__ __launch_bounds__(64) void sum_of_one_kernel(size_t n, const float* __restrict__ x, float* __restrict__ out) {
+  const size_t i = 4 * ((size_t)blockIdx.x * 64 + threadIdx.x);
+  if (i + 3 < n) {
+    float4 v = ld4s(x + i);
+    v.x += 0.0f; v.y += 0.0f; v.z += 0.0f; v.w += 0.0f;
+    st4s(out + i, v);
+  } else {
+    for (size_t e = i; e < n; ++e) out[e] = x[e] + 0.0f;
+  }
+}
+static int32_t sum_of_one(slhip_ctx* ctx, size_t n, const float* x, float* out) {
+  const size_t blocks = ((n + 3) / 4 + 63) / 64;
+  SLHIP_REQUIRE(blocks <= 0x7fffffffu, "too many elements for one launch");
+  hipLaunchKernelGGL(sum_of_one_kernel, dim3((unsigned)blocks), dim3(64), 0, ctx->stream, n, x, out);
+  return post_launch();
+}
+
 // out[r] = reduce over the contiguous axis.
 template <class Op, class Src>
 static int32_t reduce_cols_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, float* out, Finalize fin) {
@@ -256,6 +275,8 @@ static int32_t reduce_cols_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, 
   // reference's sum starts at +0, and 0 + -0 is +0 where a copy would leave -0)
   if constexpr (Src::IS_PLAIN && std::is_same<Op, MaxOp>::value)
     if (cols == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, rows * sizeof(float));
+  if constexpr (Src::IS_PLAIN && std::is_same<Op, SumOp>::value)
+    if (cols == 1 && !fin.accumulate && fin.divide != 2 && x.x != out) return sum_of_one(ctx, rows, x.x, out);  // (a mean divides by 1)
   if (cols <= 128 && (cols <= 64 || (cols & (cols - 1)) != 0) && rows >= 1024) {  // many short rows
     // whole multiples of 256 rows while they fit (every lane of the second phase busy), else as many
     // rows as fit, rounded down so that every chunk starts on a 128-byte boundary
@@ -531,6 +552,8 @@ static int32_t reduce_rows_src(slhip_ctx* ctx, size_t rows, size_t cols, Src x, 
   // one row: the maximum over rows is that row itself (a sum starts at +0 and turns a -0 into +0)
   if constexpr (Src::IS_PLAIN && std::is_same<Op, MaxOp>::value)
     if (rows == 1 && !fin.accumulate) return slhip_memcpy_d2d(ctx, out, x.x, cols * sizeof(float));
+  if constexpr (Src::IS_PLAIN && std::is_same<Op, SumOp>::value)
+    if (rows == 1 && !fin.accumulate && fin.divide != 2 && x.x != out) return sum_of_one(ctx, cols, x.x, out);
   // Streaming stages until the matrix is short, then the one-kernel form.  Threads per stage:
   // about 512 per CU (measured optimum: 7.0 TB/s at 131072 threads on [16384 x 16384]; 5.4 TB/s at
   // four times as many), at least 16 vectors each, and a multiple of cols / gcd(cols, 4) so that
