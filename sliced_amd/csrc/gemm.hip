@@ -664,7 +664,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // One workgroup per CU at most (and the 128 x 128 tile): the eight-wave kernel
   const bool wide_fits = !small_tile && !(ta && tb);
   if (wide_fits && (ctx->gemm_tile == SLHIP_TILE_128X128_WIDE ||
-                    (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && tiles * splits <= (size_t)ctx->num_cu))) {
+                    (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO))) {
     ctx->last_gemm.kind = 3;
     ctx->last_gemm.waves = 8;
     int32_t rc = gemm_wide_launch(ctx, ta, tb, only_fast, g);

@@ -43,7 +43,7 @@ def check_line(out, steps, warmup):
         assert k in j, k
     assert j["n_gpus"] == 1 and j["steps"] == steps and j["warmup"] == warmup and j["dtype"] == "f32" and j["vs_baseline"] is None
     assert "workload" in j["config"] and "model" not in j["config"]
-    assert j["config"]["spin_up_s"] > 0 and "gemm_kernel<false,false,32,true,2,2>" in j["config"]["kernel"]
+    assert j["config"]["spin_up_s"] > 0 and "gemm_wide_kernel<false,false,true>" in j["config"]["kernel"]
     rf = j["roofline"]
     assert rf["bound"] == "mfma" and rf["unit"] == "TFLOP/s" and rf["peak"] == 157.3
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-9
