@@ -524,7 +524,9 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
         // workgroups are handed out as slots free up, so a partly filled last round costs about
         // half of what a strict round-by-round schedule would lose
         const double exact = (double)wgs / (double)slots, up = (double)(full_rounds + (rest ? 1 : 0));
-        t = (exact + 0.5 * (up - exact)) * kt * 4.35 + up * 6.0;
+        // (a last round more than half full puts two workgroups on some CUs, and those set its length:
+        // the eight-wave kernel's single workgroups finish in 0.525 of that time and wait)
+        t = (exact + (2 * rest > slots ? 0.75 : 0.5) * (up - exact)) * kt * 4.35 + up * 6.0;
       }
       if (sp > 1) t += 4.0 + 2.0 * (double)sp * (double)mn_bytes / 5.0e6;
       if (t < best) { best = t; splits = sp; }
@@ -550,7 +552,14 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       const double per_kt = (full == 0 && workers <= slots / 2) ? 2.43 : 4.35;
       const double t = (double)(full / slots) * ((double)kt_total * 4.35 + 6.0) + (double)units * per_kt + 6.0 + 4.0 +
                        2.0 * (double)runs * (double)(SPREAD_SLOT * sizeof(float)) / 5.0e6;
-      if (t < best || ctx->gemm_tail == SLHIP_TAIL_SPREAD) {
+      // A last round that is at most half full gives every tile a CU of its own, where the eight-wave
+      // kernel takes 0.525 of the time of a round of two workgroups per CU: spreading a tail of 0.4 to
+      // 0.5 rounds gains less than the spread's own overhead (fix-up launch, partial tiles) while K is
+      // short.  Measured at one to four whole rounds + 208..240 tiles: whole launches 3-17 % ahead up to
+      // K = 1024, the spread tail 0-6 % ahead from K = 1536; tails of 64..128 tiles: the spread tail at every K.
+      const bool whole_wide_wins = ctx->gemm_tail == SLHIP_TAIL_AUTO && ctx->gemm_tile == SLHIP_TILE_AUTO && !(ta && tb) &&
+                                   full > 0 && 2 * tail <= slots && 5 * tail >= 2 * slots && kt_total <= 40;
+      if (!whole_wide_wins && (t < best || ctx->gemm_tail == SLHIP_TAIL_SPREAD)) {
         best = t;
         splits = 1;
         sp.first = (unsigned)full;
@@ -659,7 +668,17 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // clamped loops (k_chunk is a multiple of BK, so only the end of K can leave a partial tile)
   const bool only_fast = g.a_vec && g.b_vec && g.m_fast && M % tile_m == 0 && N % tile_n == 0 && K % BK == 0;
   ctx->last_gemm = {spread_workers ? 4 : 2, ta, tb, only_fast, small_tile, (unsigned)splits, 4};
-  if (spread_workers) return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tiles - sp.first);
+  if (spread_workers) {
+    // On eight waves like the whole-tile launches (two workgroups put four waves on a SIMD: 3584^3 138 -> 143
+    // TFLOP/s, 4608^3 141 -> 146, 7168^3 144 -> 148), except where a short tail of an eighth to a quarter of a
+    // round follows whole rounds of a short K, which measured 3-5 % behind the four-wave form
+    // (10000 x 1000 x 1024: 178 against 170 us; 5000 x 2000 x 2048: 333 against 318)
+    const size_t tail = tiles - sp.first;
+    const bool four = ctx->gemm_tile == SLHIP_TILE_128X128 ||
+                      (ctx->gemm_tile == SLHIP_TILE_AUTO && sp.first > 0 && tail * 8 > slots && tail * 4 <= slots &&
+                       kt_total >= 12 && kt_total < 96);
+    return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tail, !four);
+  }
 
   // One workgroup per CU at most (and the 128 x 128 tile): the eight-wave kernel
   const bool wide_fits = !small_tile && !(ta && tb);
@@ -754,6 +773,11 @@ SLHIP_API int32_t slhip_gemm_plan_describe(slhip_ctx* ctx, char* buf, size_t len
       break;
     case 2:
     case 4:
+      if (p.kind == 4 && p.waves == 8) {
+        snprintf(buf, len, "gemm_spread_wide_kernel<%s,%s,%d,%s>: 128x128 tiles on 8 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32",
+                 tf[p.ta], tf[p.tb], GEMM_BK, tf[p.only_fast], GEMM_BK, p.splits);
+        break;
+      }
       snprintf(buf, len, "%s<%s,%s,%d,%s,%s>: %s tiles on 4 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32",
                p.kind == 4 ? "gemm_spread_kernel" : "gemm_kernel", tf[p.ta], tf[p.tb], GEMM_BK, tf[p.only_fast],
                p.small_tile ? "1,1" : "2,2", p.small_tile ? "64x64" : "128x128", GEMM_BK, p.splits);

@@ -11,13 +11,13 @@ namespace slhip {
 
 // A workgroup of the spread tail: up to two runs of k tiles, each inside one tile of C, each
 // written as a raw partial tile (row-major, the tile's own size) to workspace slot 2*w + run.
-template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
 __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const SpreadArgs& sp,
-                                                   float (*lds_a)[Cfg<BK, 64 * WM>::STAGE_FLOATS],
-                                                   float (*lds_b)[Cfg<BK, 64 * WN>::STAGE_FLOATS]) {
-  constexpr int TM = 64 * WM, TN = 64 * WN;
+                                                   float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
+                                                   float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS]) {
+  constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
   const unsigned w = blockIdx.x - sp.first;
   unsigned u = w * sp.units;
@@ -39,7 +39,7 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
+    gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN>(g, ka, kb, 0, g.K, m0, n0, lds_a, lds_b, acc);
 
     float* slot = g.partial + ((size_t)2 * w + run) * (TM * TN);
 #pragma unroll
@@ -48,7 +48,7 @@ __device__ __forceinline__ void gemm_spread_worker(const GemmArgs& g, const Spre
       for (int j = 0; j < WN; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          slot[(block_of<2>(wm, i) + 8 * (v / 4) + 4 * h + (v % 4)) * TN + block_of<2>(wn, j) + r] = acc[i][j][v];
+          slot[(block_of<WGM>(wm, i) + 8 * (v / 4) + 4 * h + (v % 4)) * TN + block_of<WGN>(wn, j) + r] = acc[i][j][v];
   }
 }
 
@@ -58,6 +58,16 @@ __global__ __launch_bounds__(256, 2) void gemm_spread_kernel(GemmArgs g, SpreadA
   __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 64 * WN>::STAGE_FLOATS];
   if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST, WM, WN>(g, sp, lds_a, lds_b);
   else gemm_whole_tile<TA, TB, BK, ONLY_FAST, WM, WN>(g, lds_a, lds_b);
+}
+
+// The same on eight waves (the 128 x 128 tile as 2 x 4 waves of 64 x 32 each, as gemm_wide_kernel): two
+// such workgroups put four waves on a SIMD.
+template <bool TA, bool TB, int BK, bool ONLY_FAST>
+__global__ __launch_bounds__(512, 2) void gemm_spread_wide_kernel(GemmArgs g, SpreadArgs sp) {
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<BK, 128>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 128>::STAGE_FLOATS];
+  if (blockIdx.x >= sp.first) gemm_spread_worker<TA, TB, BK, ONLY_FAST, 2, 1, 2, 4>(g, sp, lds_a, lds_b);
+  else gemm_whole_tile<TA, TB, BK, ONLY_FAST, 2, 1, 2, 4>(g, lds_a, lds_b);
 }
 
 // The tiles of a spread tail: C tile = sum of its partial tiles in ascending k order (workgroup
@@ -145,8 +155,26 @@ __global__ __launch_bounds__(256) void spread_fixup_kernel(GemmArgs g, SpreadArg
 }
 
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
-                           const SpreadArgs& sp, size_t workers, size_t tail_tiles) {
+                           const SpreadArgs& sp, size_t workers, size_t tail_tiles, bool wide) {
   const dim3 grid((unsigned)(sp.first + workers));
+  if (wide && !small_tile && !(ta && tb)) {
+#define SL_WIDE(TA_, TB_)                                                                                                     \
+  do {                                                                                                                        \
+    if (only_fast)                                                                                                            \
+      hipLaunchKernelGGL((gemm_spread_wide_kernel<TA_, TB_, GEMM_BK, true>), grid, dim3(512), 0, ctx->stream, g, sp);         \
+    else                                                                                                                      \
+      hipLaunchKernelGGL((gemm_spread_wide_kernel<TA_, TB_, GEMM_BK, false>), grid, dim3(512), 0, ctx->stream, g, sp);        \
+  } while (0)
+    if (!ta && !tb) SL_WIDE(false, false);
+    else if (!ta && tb) SL_WIDE(false, true);
+    else SL_WIDE(true, false);
+#undef SL_WIDE
+    ctx->last_gemm.waves = 8;
+    int32_t rcw = post_launch();
+    if (rcw) return rcw;
+    hipLaunchKernelGGL((spread_fixup_kernel<128, 128>), dim3((unsigned)(16 * tail_tiles)), dim3(256), 0, ctx->stream, g, sp);
+    return post_launch();
+  }
 #define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                          \
   do {                                                                                                                        \
     if (only_fast)                                                                                                            \

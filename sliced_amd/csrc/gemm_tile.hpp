@@ -607,6 +607,6 @@ int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, con
 int32_t gemm_wide_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
 
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
-                           const SpreadArgs& sp, size_t workers, size_t tail_tiles);
+                           const SpreadArgs& sp, size_t workers, size_t tail_tiles, bool wide);
 
 }  // namespace slhip
