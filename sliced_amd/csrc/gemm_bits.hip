@@ -23,10 +23,13 @@ namespace slhip {
 
 __host__ __device__ constexpr int bits_row_of(int v, int h) { return 8 * (v / 4) + 4 * h + v % 4; }
 
-template <bool TA, bool TB, bool ONLY_FAST>
-__global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uint32_t* __restrict__ bits_in,
+// WM x WN accumulator blocks per wave, WGM x WGN waves: 2, 2, 2, 2 is the four-wave tile; 2, 1, 2, 4 the eight-wave
+// one (as gemm_wide_kernel: two such workgroups put four waves on a SIMD).
+template <bool TA, bool TB, bool ONLY_FAST, int WM = 2, int WN = 2, int WGM = 2, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN, 2) void gemm_bits_kernel(GemmArgs g, const uint32_t* __restrict__ bits_in,
                                                            uint32_t* __restrict__ bits_out, size_t W) {
   constexpr int BK = GEMM_BK;
+  static_assert(32 * WM * WGM == 128 && 32 * WN * WGN == 128, "a 128 x 128 tile");
   __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<BK, 128>::STAGE_FLOATS];
   __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<BK, 128>::STAGE_FLOATS];
   unsigned tm, tn;
@@ -34,29 +37,33 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
   const size_t m0 = (size_t)tm * 128, n0 = (size_t)tn * 128;
   const int ktiles = (int)((g.K + BK - 1) / BK);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
 
   // the tile's mask words, in flight during the k loop
-  uint32_t mw[2][2] = {{0u, 0u}, {0u, 0u}};
+  uint32_t mw[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) mw[i][j] = 0u;
   if (bits_in) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const size_t row = m0 + block_of<2>(wm, i) + r, cw = (n0 + block_of<2>(wn, j)) >> 5;
+      for (int j = 0; j < WN; ++j) {
+        const size_t row = m0 + block_of<WGM>(wm, i) + r, cw = (n0 + block_of<WGN>(wn, j)) >> 5;
         if (h == 0 && row < g.M && cw < W) mw[i][j] = bits_in[row * W + cw];
       }
   }
 
-  floatx16 acc[2][2];
+  floatx16 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-  gemm_k_range<TA, TB, BK, ONLY_FAST, 2, 2>(g, 0, ktiles, 0, g.K, m0, n0, lds_a, lds_b, acc);
+  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN>(g, 0, ktiles, 0, g.K, m0, n0, lds_a, lds_b, acc);
 
   // Tiles inside the matrix with nothing to read back (every tile of a layer whose sides are multiples of
   // 128): no bounds, one scalar row pointer per accumulator register and one 32-bit lane offset for all of
@@ -67,21 +74,23 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
   // not in the caches yet and the stores set the pace, the same kernels gain 2 us each).
   if (m0 + 128 <= g.M && n0 + 128 <= g.N && g.beta == 0.0f && g.N < (size_t(1) << 28) && (bits_in == nullptr) != (bits_out == nullptr)) {
     const int uw = __builtin_amdgcn_readfirstlane(wave);
-    const int uwm = uw >> 1, uwn = uw & 1;
+    const int uwm = uw / WGN, uwn = uw % WGN;
     const unsigned lane_off = (unsigned)(4 * h) * (unsigned)g.N + (unsigned)r;
     auto run = [&](auto in_tag) {
       constexpr bool IN = decltype(in_tag)::value;  // the mask comes in (input gradient); else it goes out (forward)
-      float bias_of[2] = {0.0f, 0.0f};
+      float bias_of[WN];
+#pragma unroll
+      for (int j = 0; j < WN; ++j) bias_of[j] = 0.0f;
       if (!IN && g.bias) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) bias_of[j] = g.bias[n0 + block_of<2>(wn, j) + r];
+        for (int j = 0; j < WN; ++j) bias_of[j] = g.bias[n0 + block_of<WGN>(wn, j) + r];
       }
       const bool relu = g.relu != 0;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          float* const block = g.C + (m0 + block_of<2>(uwm, i)) * g.N + n0 + block_of<2>(uwn, j);  // wave-uniform
+        for (int j = 0; j < WN; ++j) {
+          float* const block = g.C + (m0 + block_of<WGM>(uwm, i)) * g.N + n0 + block_of<WGN>(uwn, j);  // wave-uniform
           uint32_t word = 0u;
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
             }
             (block + (size_t)(8 * (v / 4) + v % 4) * g.N)[lane_off] = val;
           }
-          if (!IN && h == 0) bits_out[(m0 + block_of<2>(wm, i) + r) * W + ((n0 + block_of<2>(wn, j)) >> 5)] = word;
+          if (!IN && h == 0) bits_out[(m0 + block_of<WGM>(wm, i) + r) * W + ((n0 + block_of<WGN>(wn, j)) >> 5)] = word;
         }
     };
     if (bits_in) run(std::true_type());
@@ -110,10 +119,10 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
 
   // every read (mask words, C for beta) before the first store
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + block_of<2>(wn, j) + r;
+    for (int j = 0; j < WN; ++j) {
+      const size_t col = n0 + block_of<WGN>(wn, j) + r;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         float val = acc[i][j][v];
@@ -123,25 +132,27 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
           val = ((((h ? hi : lo) >> r) & 1u) ? 1.0f : 0.0f) * val;
         }
         if (g.beta != 0.0f) {
-          const size_t row = m0 + block_of<2>(wm, i) + bits_row_of(v, h);
+          const size_t row = m0 + block_of<WGM>(wm, i) + bits_row_of(v, h);
           if (row < g.M && col < g.N) val = g.beta * g.C[row * g.N + col] + val;
         }
         acc[i][j][v] = val;
       }
     }
-  float bias_of[2] = {0.0f, 0.0f};
+  float bias_of[WN];
+#pragma unroll
+  for (int j = 0; j < WN; ++j) bias_of[j] = 0.0f;
   if (g.bias) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + block_of<2>(wn, j) + r;
+    for (int j = 0; j < WN; ++j) {
+      const size_t col = n0 + block_of<WGN>(wn, j) + r;
       if (col < g.N) bias_of[j] = g.bias[col];
     }
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const size_t col = n0 + block_of<2>(wn, j) + r;
+    for (int j = 0; j < WN; ++j) {
+      const size_t col = n0 + block_of<WGN>(wn, j) + r;
       const bool cin = col < g.N;
       const float bias = bias_of[j];
       uint32_t word = 0u;
@@ -155,11 +166,11 @@ __global__ __launch_bounds__(256, 2) void gemm_bits_kernel(GemmArgs g, const uin
           if (lane == bits_row_of(v, 1)) word = (uint32_t)(b >> 32);
         }
         if (g.relu) val = (val >= 0.0f ? 1.0f : 0.0f) * val;
-        const size_t row = m0 + block_of<2>(wm, i) + bits_row_of(v, h);
+        const size_t row = m0 + block_of<WGM>(wm, i) + bits_row_of(v, h);
         if (row < g.M && cin) g.C[row * g.N + col] = val;
       }
       if (bits_out) {
-        const size_t row = m0 + block_of<2>(wm, i) + r, cw = (n0 + block_of<2>(wn, j)) >> 5;
+        const size_t row = m0 + block_of<WGM>(wm, i) + r, cw = (n0 + block_of<WGN>(wn, j)) >> 5;
         if (h == 0 && row < g.M && cw < W) bits_out[row * W + cw] = word;
       }
     }
@@ -275,11 +286,20 @@ static int32_t gemm_bits_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t 
     if (only_fast) hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, true>), grid, dim3(256), 0, ctx->stream, g, bits_in, bits_out, W); \
     else hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, false>), grid, dim3(256), 0, ctx->stream, g, bits_in, bits_out, W);  \
   } while (0)
-  if (!ta && !tb) SL_GB(false, false);
-  else if (!ta && tb) SL_GB(false, true);
-  else if (ta && !tb) SL_GB(true, false);
+#define SL_GBW(TA_, TB_)                                                                                                     \
+  do {                                                                                                                       \
+    if (only_fast)                                                                                                           \
+      hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, true, 2, 1, 2, 4>), grid, dim3(512), 0, ctx->stream, g, bits_in, bits_out, W);  \
+    else                                                                                                                     \
+      hipLaunchKernelGGL((gemm_bits_kernel<TA_, TB_, false, 2, 1, 2, 4>), grid, dim3(512), 0, ctx->stream, g, bits_in, bits_out, W); \
+  } while (0)
+  const bool four = ctx->gemm_tile == SLHIP_TILE_128X128;  // the tile policy's four-wave form, for comparison
+  if (!ta && !tb) { if (four) SL_GB(false, false); else SL_GBW(false, false); }
+  else if (!ta && tb) { if (four) SL_GB(false, true); else SL_GBW(false, true); }
+  else if (ta && !tb) { if (four) SL_GB(true, false); else SL_GBW(true, false); }
   else SL_GB(true, true);
 #undef SL_GB
+#undef SL_GBW
   return post_launch();
 }
 
