@@ -148,10 +148,10 @@ enum { SLHIP_TAIL_AUTO = 0, SLHIP_TAIL_WHOLE = 1, SLHIP_TAIL_SPREAD = 2 };
 int32_t slhip_gemm_tail_policy(slhip_ctx* ctx, int32_t policy);
 /* The tile of C that one workgroup of the tiled kernel computes.  SLHIP_TILE_AUTO (the default)
  * chooses by a cost model (64 x 64, unsplit, for products of a few hundred such tiles and a
- * moderate K; 128 x 128 otherwise, on eight waves instead of four when the grid gives a CU at most
- * one workgroup); the others force a tile for every product that takes the tiled kernel
- * (SLHIP_TILE_128X128_WIDE: the eight-wave form; it has no doubly transposed instance and then
- * falls back to four waves).  Same results up to the summation order of k splits; a tuning and
+ * moderate K; 128 x 128 otherwise, on eight waves, two workgroups to a CU); the others force a
+ * tile for every product that takes the tiled kernel (SLHIP_TILE_128X128: the four-wave form of
+ * that tile; SLHIP_TILE_128X128_WIDE: the eight-wave form, which has no doubly transposed instance
+ * and then falls back to four waves).  Same results up to the summation order of k splits; a tuning and
  * testing knob with no counterpart in the reference. */
 enum { SLHIP_TILE_AUTO = 0, SLHIP_TILE_128X128 = 1, SLHIP_TILE_64X64 = 3, SLHIP_TILE_128X128_WIDE = 4 };
 int32_t slhip_gemm_tile_policy(slhip_ctx* ctx, int32_t policy);

@@ -8,9 +8,11 @@
 // k permutation inside every group of 8: instruction t (0..3) multiplies k = t for lanes 0..31
 // and k = 4 + t for lanes 32..63.
 //
-// Tiling (gemm_tile.hpp): 256 threads = 4 waves in a 2x2 grid, 128x128 macro tile, each wave
-// 64x64 = four 32x32 accumulators (64 VGPRs), BK = 32 per LDS stage, two LDS stages with register
-// prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead.
+// Tiling (gemm_tile.hpp): a 128x128 macro tile, BK = 32 per LDS stage, two LDS stages with register
+// prefetch of the next stage (one barrier per stage), MFMA fragments read one k-group ahead; on 512
+// threads = 8 waves in a 2x4 grid, each wave 64x32 = two 32x32 accumulators (gemm_wide.hip: the form
+// every whole-tile launch takes, two workgroups to a CU), or on 256 threads = 4 waves in a 2x2 grid,
+// each wave 64x64 (the kernel below: the doubly transposed form, the 64x64 tile, the tile policy).
 // Tiles are numbered so that each XCD (its own L2) works along one tile row at a time.
 //
 // This file: the plain kernel (one workgroup per tile and k chunk), the wave-per-tile kernel for
@@ -680,7 +682,7 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tail, !four);
   }
 
-  // One workgroup per CU at most (and the 128 x 128 tile): the eight-wave kernel
+  // The 128 x 128 tile on eight waves (gemm_wide.hip)
   const bool wide_fits = !small_tile && !(ta && tb);
   if (wide_fits && (ctx->gemm_tile == SLHIP_TILE_128X128_WIDE ||
                     (ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO))) {

@@ -1,12 +1,18 @@
 // The 128 x 128 tile on EIGHT waves (2 x 4, each 64 x 32 = two 32 x 32 accumulators) instead of
 // four.  Same staging, same k loop, same LDS footprint as the four-wave kernel (gemm.hip); what
-// changes is who shares a SIMD: a tile grid that gives every CU one workgroup leaves the four-wave
-// kernel with ONE wave per SIMD, whose LDS reads, stores and barriers then stall the matrix core
-// with nobody to fill in; here two waves of the same workgroup take turns (2048^3: 110 -> 117
-// TFLOP/s for A*B, 117 -> 124 for A*Bt; with two workgroups to a CU it is 6-10 % slower than the
-// four-wave kernel, so it only takes grids of at most one workgroup per CU).  A third LDS stage,
-// which lets the fragment reads run on across the k-tile barrier, measured the same.  A translation unit
-// of its own, like the spread-tail kernel: the four-wave kernel's speed moves with the code around it.
+// changes is who shares a SIMD.  With 124 vector registers a wave, two such workgroups fit a CU and
+// put FOUR waves on every SIMD where the four-wave kernel has two: while one wave reads fragments,
+// stores a stage or waits at the k-tile barrier, three others can issue to the matrix core
+// (4096^3 per launch: 142.2 -> 146.3 TFLOP/s, MFMA-busy share 0.93 -> 0.96; 8192^3 144.0 -> 150.4, 0.98;
+// 8192 x 2048 x 784 128.9 -> 133.1).  A grid that gives every CU ONE workgroup leaves the four-wave
+// kernel with one wave per SIMD and this one with two (2048^3: 118 -> 133), and a last round that is
+// at most half full runs in 0.525 of a full round's time.  It is the kernel of every whole-tile
+// launch of the 128 x 128 tile (the spread tail and the bit-mask kernels have their own eight-wave
+// forms); the four-wave kernel stays for the doubly transposed form and behind the tile policy.
+// Where the loop starts relative to a 32-byte boundary and where in the k tile the refill sits
+// measured within 0.5 % of each other on this kernel; a third LDS stage measured the same.
+// A translation unit of its own, like the spread-tail kernel: the four-wave kernel's speed moves
+// with the code around it.
 #include "gemm_tile.hpp"
 
 namespace slhip {
