@@ -242,14 +242,29 @@ __device__ __forceinline__ void read_frag(float (&out)[NI][4], const float* lds,
   }
 }
 
-// Linear workgroup id -> tile.  Tiles are walked in groups of 8 tile rows, row index fastest.
-// The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, so with a group
-// height of 8 every XCD (its own L2) keeps working along ONE tile row of the group: its A panel
-// stays put in that L2 while the B panels stream through.  Measured on 4096^3: an explicit
-// remap that instead gave each XCD a compact 8x8 block of tiles was no faster for A*B and
-// At*B and 25 % slower for A*Bt.
+// Linear workgroup id -> tile.  The hardware deals consecutive workgroup ids round-robin to the 8
+// XCDs, each with an L2 of its own and room for 64 workgroups of the 128 x 128 tile.
+// Grids that are whole 8 x 8 blocks of tiles, a multiple of eight of them (4096^3, 8192^3, the
+// 2048-wide layers at batch 8192): XCD x works through blocks x, x + 8, ..., one block at a time, so
+// the 64 tiles it holds share 8 panels of A and 8 of B.  FETCH_SIZE per 4096^3 launch of the eight-wave
+// kernel: 765 MiB, against 2.1 GiB for the walk below (there an XCD holds two tile rows of 32 tiles
+// each, which share a B panel only while the two rows stay within a few k tiles of each other, and
+// on eight waves they do not); 4096^3 140.3 -> 143.6 TFLOP/s, 8192^3 138.8 -> 141.1, 2048 x 8192 x 4096
+// 140.3 -> 143.7 on a box whose memory side is on the slow end of the pool.  (On the four-wave kernel of
+// an earlier build the same remap was no faster for A*B and At*B and 25 % slower for A*Bt.)
+// Any other grid: tiles are walked in groups of 8 tile rows, row index fastest, so that every XCD
+// keeps working along ONE tile row of the group: its A panel stays put in that L2 while the B
+// panels stream through.
 __device__ __forceinline__ void tile_of_block(unsigned bid, unsigned tiles_m, unsigned tiles_n, unsigned& tm,
                                               unsigned& tn) {
+  if (tiles_m % 8 == 0 && tiles_n % 8 == 0 && ((tiles_m / 8) * (tiles_n / 8)) % 8 == 0) {
+    const unsigned x = bid & 7, q = bid >> 3;
+    const unsigned blk = (q >> 6) * 8 + x, t = q & 63;
+    const unsigned bm = blk % (tiles_m / 8), bn = blk / (tiles_m / 8);
+    tm = bm * 8 + (t & 7);
+    tn = bn * 8 + (t >> 3);
+    return;
+  }
   constexpr unsigned GROUP_M = 8;
   const unsigned in_group = GROUP_M * tiles_n;
   const unsigned group = bid / in_group;
