@@ -48,7 +48,7 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 # the factors being what the same counters read for the 1 GiB device copy of known size.  The read
 # figure moves by +-15 % from run to run (557 000 to 768 000 KiB raw) with what the caches still hold.
 # A counter run cannot happen inside this program; the figure is that profile's, not this run's.
-GEMM_4096_TRAFFIC_BYTES = 2271295821  # (1076276.5 x 2.000 + 65536.0 x 1.000) KiB: FETCH_SIZE + WRITE_SIZE medians of the headline kernel, scaled by the 1 GiB copy
+GEMM_4096_TRAFFIC_BYTES = 868778845  # (391450.6 x 2.000 + 65536.0 x 1.000) KiB: FETCH_SIZE + WRITE_SIZE medians of the headline kernel, scaled by the 1 GiB copy
 HBM_PEAK_GBS = 8000.0             # MI355X HBM3E
 SEED = 0x51CED
 MIN_ITERS, MIN_WARMUP = 20, 5
