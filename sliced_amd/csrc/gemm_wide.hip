@@ -18,7 +18,7 @@
 namespace slhip {
 
 template <bool TA, bool TB, bool ONLY_FAST>
-__global__ __launch_bounds__(512) void gemm_wide_kernel(GemmArgs g) {
+__global__ __launch_bounds__(512, 2) void gemm_wide_kernel(GemmArgs g) {  // two workgroups to a CU: at most 128 VGPRs
   __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<GEMM_BK, 128>::STAGE_FLOATS];
   __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<GEMM_BK, 128>::STAGE_FLOATS];
   gemm_whole_tile<TA, TB, GEMM_BK, ONLY_FAST, 2, 1, 2, 4>(g, lds_a, lds_b);
