@@ -693,6 +693,14 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     return splitk_combine(ctx, g, splits);
   }
 
+  // The 64 x 64 tile with at most one workgroup per CU: on eight waves, two sets of four that split every k
+  // tile (gemm_wide.hip), which puts two waves on a SIMD where the four-wave form has one: 1024^3 A*Bt 25.2 ->
+  // 23.2 us, 896^3 21.7 -> 20.3, 1000^3 25.0 -> 23.6, 2048 x 512 x 1024 24.1 -> 22.5 per launch
+  if (small_tile && !(ta && tb) && splits == 1 && tiles <= (size_t)ctx->num_cu && ctx->gemm_tile == SLHIP_TILE_AUTO) {
+    ctx->last_gemm.waves = 8;
+    return gemm_small8_launch(ctx, ta, tb, only_fast, g);
+  }
+
   dim3 grid((unsigned)tiles, (unsigned)splits);
 #define SL_GEMM3(TA_, TB_, WM_, WN_)                                                                                  \
   do {                                                                                                                \
@@ -778,6 +786,11 @@ SLHIP_API int32_t slhip_gemm_plan_describe(slhip_ctx* ctx, char* buf, size_t len
       if (p.kind == 4 && p.waves == 8) {
         snprintf(buf, len, "gemm_spread_wide_kernel<%s,%s,%d,%s>: 128x128 tiles on 8 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32",
                  tf[p.ta], tf[p.tb], GEMM_BK, tf[p.only_fast], GEMM_BK, p.splits);
+        break;
+      }
+      if (p.kind == 2 && p.small_tile && p.waves == 8) {
+        snprintf(buf, len, "gemm_small8_kernel<%s,%s,%s>: 64x64 tiles on 8 waves (two sets of four, each half of every k tile), BK=%d, 1 k splits, v_mfma_f32_32x32x2_f32",
+                 tf[p.ta], tf[p.tb], tf[p.only_fast], GEMM_BK);
         break;
       }
       snprintf(buf, len, "%s<%s,%s,%d,%s,%s>: %s tiles on 4 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32",

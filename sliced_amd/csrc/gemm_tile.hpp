@@ -303,13 +303,17 @@ constexpr int PIN_SMALL[2][2] = {{1, 0}, {0, 0}};      // the 64 x 64 tile (1024
 // modes are separate loops on purpose: when vector and per-element loads sat behind a branch in
 // ONE loop body the compiler folded them into the per-element form, which cost 19 % of the
 // kernel's throughput.
-template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
+// KS = 2: two sets of WGM x WGN waves share the tile and split every k tile between them, the first
+// taking its k groups 0 and 1, the second 2 and 3 (the caller adds the two sets' accumulators): a
+// grid that gives a CU one workgroup then puts two waves on a SIMD instead of one.
+template <bool TA, bool TB, int BK, int MODE, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2, int KS = 1>
 __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int kt_end, size_t kbeg, size_t kend,
                                            size_t m0, size_t n0, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
                                            float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
   constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;  // the workgroup's tile of C
-  constexpr int NT = 64 * WGM * WGN;                      // its threads
+  constexpr int NT = 64 * WGM * WGN * KS;                 // its threads
   constexpr int KSTEPS = BK / 8;
+  static_assert(KS == 1 || (KS == 2 && KSTEPS == 4 && !(WM == 2 && WN == 2 && WGM == 2 && WGN == 2)), "k halves: the unrolled loop only");
   // The refill (LDS stores of tile kt+1, loads of tile kt+2) sits before the LAST k-group of a k
   // tile, as one run: store A, store B, load A, load B.  Measured at 4096^3 for the refill before
   // group 0 / 1 / 2 / 3 (TFLOP/s, launches back to back): A*B 133.7 / 137.1 / 136.2 / 142.8, A*Bt
@@ -321,9 +325,11 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   // load addresses and LDS row bases with vector instructions the optimum was group 1 for A*B and
   // A*Bt: where the memory instructions sit matters because, issued in one run, they hold the
   // wave's MFMA issue up behind them - and so did that arithmetic.)
-  constexpr int REFILL_AT = KSTEPS - 1;
+  constexpr int KG = KSTEPS / KS;        // k groups of a k tile that one wave multiplies
+  constexpr int REFILL_AT = KG - 1;
   if (kt_begin >= kt_end) return;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = (threadIdx.x >> 6) % (WGM * WGN), lane = threadIdx.x & 63;
+  const int g0 = KS == 1 ? 0 : ((threadIdx.x >> 6) / (WGM * WGN)) * KG;  // this wave's first k group
   const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
   // A is KC ([m][k], ld = K) unless transposed ([k][m], ld = M); B is XC ([k][n], ld = N)
@@ -390,14 +396,14 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
   auto k_tile = [&](int kt, auto stage) {
     constexpr int s = decltype(stage)::value;
     float a[2][WM][4], b[2][WN][4];
-    read_frag<!TA, BK, TM, WM, WGM>(a[0], lds_a[s], wm, 0, r, h);
-    read_frag<TB, BK, TN, WN, WGN>(b[0], lds_b[s], wn, 0, r, h);
+    read_frag<!TA, BK, TM, WM, WGM>(a[0], lds_a[s], wm, g0, r, h);
+    read_frag<TB, BK, TN, WN, WGN>(b[0], lds_b[s], wn, g0, r, h);
 #pragma unroll
-    for (int kk8 = 0; kk8 < KSTEPS; ++kk8) {
+    for (int kk8 = 0; kk8 < KG; ++kk8) {
       const int cur = kk8 & 1, nxt = cur ^ 1;
-      if (kk8 + 1 < KSTEPS) {
-        read_frag<!TA, BK, TM, WM, WGM>(a[nxt], lds_a[s], wm, kk8 + 1, r, h);
-        read_frag<TB, BK, TN, WN, WGN>(b[nxt], lds_b[s], wn, kk8 + 1, r, h);
+      if (kk8 + 1 < KG) {
+        read_frag<!TA, BK, TM, WM, WGM>(a[nxt], lds_a[s], wm, g0 + kk8 + 1, r, h);
+        read_frag<TB, BK, TN, WN, WGN>(b[nxt], lds_b[s], wn, g0 + kk8 + 1, r, h);
       }
       if (kk8 == REFILL_AT) {
         // stage s^1 was last read in the previous k tile, which ended with a barrier
@@ -474,12 +480,12 @@ __device__ __forceinline__ void gemm_tiles(const GemmArgs& g, int kt_begin, int 
 // ONLY_FAST: the host has checked that every k tile of every tile qualifies for LOAD_FAST (M and N
 // multiples of 128, every k chunk a multiple of BK, operands float4-loadable and 16-byte aligned);
 // the kernel then contains that one loop and nothing else.
-template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2, int KS = 1>
 __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, size_t kbeg, size_t kend, size_t m0,
                                              size_t n0, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
                                              float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS], floatx16 (&acc)[WM][WN]) {
   if (ONLY_FAST) {
-    gemm_tiles<TA, TB, BK, LOAD_FAST, true, WM, WN, WGM, WGN>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+    gemm_tiles<TA, TB, BK, LOAD_FAST, true, WM, WN, WGM, WGN, KS>(g, ka, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
     return;
   }
   const bool vec = g.a_vec && g.b_vec;
@@ -496,15 +502,15 @@ __device__ __forceinline__ void gemm_k_range(const GemmArgs& g, int ka, int kb, 
     if (e2 < e1) e2 = e1;
   }
   const int e3 = vec ? kb : e2;
-  gemm_tiles<TA, TB, BK, LOAD_FAST, false, WM, WN, WGM, WGN>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false, WM, WN, WGM, WGN>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false, WM, WN, WGM, WGN>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
-  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false, WM, WN, WGM, WGN>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_FAST, false, WM, WN, WGM, WGN, KS>(g, ka, e1, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_XCLAMP, false, WM, WN, WGM, WGN, KS>(g, e1, e2, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_VCLAMP, false, WM, WN, WGM, WGN, KS>(g, e2, e3, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_tiles<TA, TB, BK, LOAD_SCALAR, false, WM, WN, WGM, WGN, KS>(g, e3, kb, kbeg, kend, m0, n0, lds_a, lds_b, acc);
 }
 
 // A workgroup that computes one whole tile of C (or, with g.splits > 1, one k chunk of it as a raw
 // partial product): blockIdx.x = tile, blockIdx.y = k chunk.
-template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2>
+template <bool TA, bool TB, int BK, bool ONLY_FAST, int WM, int WN, int WGM = 2, int WGN = 2, int KS = 1>
 __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a)[Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS],
                                                 float (*lds_b)[Cfg<BK, 32 * WN * WGN>::STAGE_FLOATS]) {
   constexpr int TM = 32 * WM * WGM, TN = 32 * WN * WGN;
@@ -515,7 +521,7 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
   const size_t kend = kbeg + g.k_chunk < g.K ? kbeg + g.k_chunk : g.K;
   const int ktiles = (int)((kend - kbeg + BK - 1) / BK);
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = (threadIdx.x >> 6) % (WGM * WGN), lane = threadIdx.x & 63;
   const int wm = wave / WGN, wn = wave % WGN;
   const int r = lane & 31, h = lane >> 5;
 
@@ -527,7 +533,31 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+  gemm_k_range<TA, TB, BK, ONLY_FAST, WM, WN, WGM, WGN, KS>(g, 0, ktiles, kbeg, kend, m0, n0, lds_a, lds_b, acc);
+
+  if (KS == 2) {
+    // the second set of waves hands its accumulators over through LDS (every k loop ends with a barrier, so
+    // the stages are free) and is done; the first adds them - always in this order - and writes the tile
+    static_assert(KS == 1 || WM * WN * WGM * WGN * 1024 <= 2 * Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS, "the accumulators fit stage memory");
+    float* red = &lds_a[0][0];
+    const bool second = (threadIdx.x >> 6) >= WGM * WGN;
+    if (second) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) red[(((wave * WM + i) * WN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+    }
+    __syncthreads();
+    if (second) return;
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] += red[(((wave * WM + i) * WN + j) * 16 + v) * 64 + lane];
+  }
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
   //   row = 8*(v/4) + 4*h + v%4,  col = r   within the 32 x 32 block at (block_of(wm, i), block_of(wn, j)).
@@ -620,6 +650,8 @@ int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, con
 
 // gemm_wide.hip: the 128 x 128 tile on eight waves, g planned as for the four-wave kernel.
 int32_t gemm_wide_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
+// gemm_wide.hip: the 64 x 64 tile on eight waves, two sets of four that split every k tile; g planned for 64 x 64 tiles, no k split.
+int32_t gemm_small8_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
 
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
                            const SpreadArgs& sp, size_t workers, size_t tail_tiles, bool wide);

@@ -41,4 +41,29 @@ int32_t gemm_wide_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const
   return post_launch();
 }
 
+// The 64 x 64 tile on eight waves: two sets of 2 x 2 waves that split every k tile between them and add
+// their accumulators through LDS at the end.  For grids that give a CU one workgroup of the small tile
+// (1024^3: 256 tiles), where the four-wave form leaves each SIMD a single wave.
+template <bool TA, bool TB, bool ONLY_FAST>
+__global__ __launch_bounds__(512) void gemm_small8_kernel(GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<GEMM_BK, 64>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<GEMM_BK, 64>::STAGE_FLOATS];
+  gemm_whole_tile<TA, TB, GEMM_BK, ONLY_FAST, 1, 1, 2, 2, 2>(g, lds_a, lds_b);
+}
+
+int32_t gemm_small8_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g) {
+  if ((ta && tb) || g.splits != 1) return SLHIP_EINVAL;
+  const dim3 grid(g.tiles_m * g.tiles_n, 1);
+#define SL_S8(TA_, TB_)                                                                                       \
+  do {                                                                                                        \
+    if (only_fast) hipLaunchKernelGGL((gemm_small8_kernel<TA_, TB_, true>), grid, dim3(512), 0, ctx->stream, g); \
+    else hipLaunchKernelGGL((gemm_small8_kernel<TA_, TB_, false>), grid, dim3(512), 0, ctx->stream, g);        \
+  } while (0)
+  if (!ta && !tb) SL_S8(false, false);
+  else if (!ta && tb) SL_S8(false, true);
+  else SL_S8(true, false);
+#undef SL_S8
+  return post_launch();
+}
+
 }  // namespace slhip
