@@ -657,6 +657,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     }
   }
   const size_t tile_m = small_tile ? 64 : BM, tile_n = small_tile ? 64 : BN;
+  // More than half a round of large tiles and at most one per CU, whole or split in two: one workgroup of
+  // sixteen waves per tile, unsplit (gemm_wide.hip; 2048^3 129.2 -> 125.9 us per launch, 2048 x 2048 x 4096
+  // 252.5 -> 245.0, 2048 x 2048 x 8192 484.2 with two k splits and their combine -> 478.6 without)
+  const bool wide16 = ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && !small_tile && !(ta && tb) &&
+                      spread_workers == 0 && splits <= 2 && tiles <= (size_t)ctx->num_cu && 2 * tiles > (size_t)ctx->num_cu;
+  if (wide16) splits = 1;
 
   size_t k_chunk = (K + splits - 1) / splits;
   k_chunk = (k_chunk + BK - 1) / BK * BK;
@@ -682,6 +688,11 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     return gemm_spread_launch(ctx, ta, tb, only_fast, small_tile, g, sp, spread_workers, tail, !four);
   }
 
+  if (wide16) {
+    ctx->last_gemm.kind = 3;
+    ctx->last_gemm.waves = 16;
+    return gemm_wide16_launch(ctx, ta, tb, only_fast, g);
+  }
   // The 128 x 128 tile on eight waves (gemm_wide.hip)
   const bool wide_fits = !small_tile && !(ta && tb);
   if (wide_fits && (ctx->gemm_tile == SLHIP_TILE_128X128_WIDE ||
@@ -798,8 +809,12 @@ SLHIP_API int32_t slhip_gemm_plan_describe(slhip_ctx* ctx, char* buf, size_t len
                p.small_tile ? "1,1" : "2,2", p.small_tile ? "64x64" : "128x128", GEMM_BK, p.splits);
       break;
     case 3:
-      snprintf(buf, len, "gemm_wide_kernel<%s,%s,%s>: 128x128 tiles on 8 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32", tf[p.ta],
-               tf[p.tb], tf[p.only_fast], GEMM_BK, p.splits);
+      if (p.waves == 16)
+        snprintf(buf, len, "gemm_wide16_kernel<%s,%s,%s>: 128x128 tiles on 16 waves (two sets of eight, each half of every k tile), BK=%d, 1 k splits, v_mfma_f32_32x32x2_f32",
+                 tf[p.ta], tf[p.tb], tf[p.only_fast], GEMM_BK);
+      else
+        snprintf(buf, len, "gemm_wide_kernel<%s,%s,%s>: 128x128 tiles on 8 waves, BK=%d, %u k splits, v_mfma_f32_32x32x2_f32", tf[p.ta],
+                 tf[p.tb], tf[p.only_fast], GEMM_BK, p.splits);
       break;
     case 5:
       snprintf(buf, len, "tall-A kernel (at most 32 columns), form %s,%s", tf[p.ta], tf[p.tb]);

@@ -537,26 +537,29 @@ __device__ __forceinline__ void gemm_whole_tile(const GemmArgs& g, float (*lds_a
 
   if (KS == 2) {
     // the second set of waves hands its accumulators over through LDS (every k loop ends with a barrier, so
-    // the stages are free) and is done; the first adds them - always in this order - and writes the tile
-    static_assert(KS == 1 || WM * WN * WGM * WGN * 1024 <= 2 * Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS, "the accumulators fit stage memory");
+    // the stages are free), one of its WM block rows at a time, and is done; the first adds them - always
+    // in this order - and writes the tile
+    static_assert(KS == 1 || WN * WGM * WGN * 1024 <= 2 * Cfg<BK, 32 * WM * WGM>::STAGE_FLOATS, "a block row of accumulators fits stage memory");
     float* red = &lds_a[0][0];
     const bool second = (threadIdx.x >> 6) >= WGM * WGN;
-    if (second) {
 #pragma unroll
-      for (int i = 0; i < WM; ++i)
+    for (int i = 0; i < WM; ++i) {
+      if (second) {
 #pragma unroll
         for (int j = 0; j < WN; ++j)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) red[(((wave * WM + i) * WN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+          for (int v = 0; v < 16; ++v) red[((wave * WN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+      }
+      __syncthreads();
+      if (!second) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] += red[((wave * WN + j) * 16 + v) * 64 + lane];
+      }
+      if (i + 1 < WM) __syncthreads();
     }
-    __syncthreads();
     if (second) return;
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] += red[(((wave * WM + i) * WN + j) * 16 + v) * 64 + lane];
   }
 
   // Epilogue.  Accumulator register v of lane (r, h) in block (i, j) is
@@ -652,6 +655,8 @@ int gemm_short_k_launch(slhip_ctx* ctx, bool ta, bool tb, const GemmArgs& g, con
 int32_t gemm_wide_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
 // gemm_wide.hip: the 64 x 64 tile on eight waves, two sets of four that split every k tile; g planned for 64 x 64 tiles, no k split.
 int32_t gemm_small8_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
+// gemm_wide.hip: the 128 x 128 tile on sixteen waves, two sets of eight that split every k tile; g planned for 128 x 128 tiles, no k split.
+int32_t gemm_wide16_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g);
 
 int32_t gemm_spread_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, bool small_tile, const GemmArgs& g,
                            const SpreadArgs& sp, size_t workers, size_t tail_tiles, bool wide);

@@ -66,4 +66,30 @@ int32_t gemm_small8_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, con
   return post_launch();
 }
 
+// The 128 x 128 tile on SIXTEEN waves, two sets of 2 x 4 that split every k tile: one such workgroup puts four
+// waves on every SIMD, as two eight-wave workgroups do.  For grids of more than half a round and at most one
+// tile per CU (2048^3, 2048 x 2048 x 8192), where the eight-wave kernel leaves a SIMD two waves - or needs a
+// k split into two workgroups per tile and a combine launch to get four.
+template <bool TA, bool TB, bool ONLY_FAST>
+__global__ __launch_bounds__(1024) void gemm_wide16_kernel(GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) float lds_a[2][Cfg<GEMM_BK, 128>::STAGE_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][Cfg<GEMM_BK, 128>::STAGE_FLOATS];
+  gemm_whole_tile<TA, TB, GEMM_BK, ONLY_FAST, 2, 1, 2, 4, 2>(g, lds_a, lds_b);
+}
+
+int32_t gemm_wide16_launch(slhip_ctx* ctx, bool ta, bool tb, bool only_fast, const GemmArgs& g) {
+  if ((ta && tb) || g.splits != 1) return SLHIP_EINVAL;
+  const dim3 grid(g.tiles_m * g.tiles_n, 1);
+#define SL_W16(TA_, TB_)                                                                                       \
+  do {                                                                                                         \
+    if (only_fast) hipLaunchKernelGGL((gemm_wide16_kernel<TA_, TB_, true>), grid, dim3(1024), 0, ctx->stream, g); \
+    else hipLaunchKernelGGL((gemm_wide16_kernel<TA_, TB_, false>), grid, dim3(1024), 0, ctx->stream, g);        \
+  } while (0)
+  if (!ta && !tb) SL_W16(false, false);
+  else if (!ta && tb) SL_W16(false, true);
+  else SL_W16(true, false);
+#undef SL_W16
+  return post_launch();
+}
+
 }  // namespace slhip
