@@ -704,10 +704,11 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
     return splitk_combine(ctx, g, splits);
   }
 
-  // The 64 x 64 tile with at most one workgroup per CU: on eight waves, two sets of four that split every k
-  // tile (gemm_wide.hip), which puts two waves on a SIMD where the four-wave form has one: 1024^3 A*Bt 25.2 ->
-  // 23.2 us, 896^3 21.7 -> 20.3, 1000^3 25.0 -> 23.6, 2048 x 512 x 1024 24.1 -> 22.5 per launch
-  if (small_tile && !(ta && tb) && splits == 1 && tiles <= (size_t)ctx->num_cu && ctx->gemm_tile == SLHIP_TILE_AUTO) {
+  // The 64 x 64 tile with at most two workgroups per CU: on eight waves, two sets of four that split every k
+  // tile (gemm_wide.hip), which doubles the waves on a SIMD: with one workgroup per CU 1024^3 24.2 -> 22.4 us per
+  // launch, 896^3 21.7 -> 20.3, 1000^3 25.0 -> 23.6, 2048 x 512 x 1024 24.1 -> 22.5; with two 1536 x 1024 x 1024
+  // 38.4 -> 36.0, 1400 x 1200 x 1000 39.4 -> 37.4, 1408^2 x 768 30.5 -> 29.2; level at K of 256-300
+  if (small_tile && !(ta && tb) && splits == 1 && tiles <= 2 * (size_t)ctx->num_cu && ctx->gemm_tile == SLHIP_TILE_AUTO) {
     ctx->last_gemm.waves = 8;
     return gemm_small8_launch(ctx, ta, tb, only_fast, g);
   }
