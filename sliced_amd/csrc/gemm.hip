@@ -451,7 +451,12 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   // products whose K or bases are off the 8-float grid go to the tiled kernels from a lower size on: the
   // staged tiles absorb the misalignment that the wave kernel's direct loads pay for
   const bool wave_aligned = K % 8 == 0 && (ta || g.a_vec) && (!tb || g.b_vec);
-  if (flop <= (wave_aligned ? 6.0e8 : 33554432.0) || M <= 32 || N <= 32 || K <= 16) {
+  // ... unless the output is a hundred 64 x 64 tiles or more and K at least four k tiles: the eight-wave small
+  // tile then fills the chip and is ahead (per launch 1024^2 x 256 15.8 -> 10.3 us, 1024^2 x 128 10.0 -> 8.1,
+  // 768^2 x 448 16.8 -> 13.0, 640^3 17.1 -> 14.6, 600^3 16.4 -> 15.5), where up to 64 tiles it is behind
+  // (512^3 9.5 against 12.6, 448^3 9.3 / 12.8, 512^2 x 256 7.8 / 9.8)
+  const bool many_tiles = ((M + 63) / 64) * ((N + 63) / 64) >= 100 && K >= 128 && flop > 33554432.0 && !(ta && tb);
+  if (flop <= (wave_aligned && !many_tiles ? 6.0e8 : 33554432.0) || M <= 32 || N <= 32 || K <= 16) {
     const size_t wt_m = (M + 31) / 32, wt_n = (N + 31) / 32;
     if (wt_m * wt_n > 0x7fffffffu) {
       set_error("sgemm: %zu x %zu tiles exceed one launch", wt_m, wt_n);
