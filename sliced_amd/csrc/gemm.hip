@@ -591,6 +591,10 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
   if (!(ta && tb)) {  // the doubly transposed form is not instantiated for the small tile
     const size_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
     static const double per_kt[5] = {0.0, 0.75, 1.25, 1.8, 2.3};
+    // (on eight waves, which up to two workgroups per CU take: 0.69 and 1.18; that is what the choice between
+    // the tiles below counts with, while the choice between whole small tiles and their spread form keeps the
+    // four-wave figures it was measured with)
+    static const double per_kt8[3] = {0.0, 0.69, 1.18};
     const size_t slots64 = (size_t)ctx->num_cu * 4;
     const bool automatic = ctx->gemm_tile == SLHIP_TILE_AUTO && ctx->gemm_tail == SLHIP_TAIL_AUTO && best < 1e299;
     // plan 1: one workgroup per small tile
@@ -614,7 +618,9 @@ static int32_t gemm_run(slhip_ctx* ctx, bool ta, bool tb, size_t M, size_t N, si
       small_tile = true;
       spread64 = ctx->gemm_tail == SLHIP_TAIL_SPREAD && t_spread < 1e299;
     } else if (automatic) {
-      const double t64 = t_whole < t_spread ? t_whole : t_spread;
+      double t_whole8 = t_whole;
+      if (tiles64 <= 2 * (size_t)ctx->num_cu) t_whole8 = (double)kt_total * per_kt8[(tiles64 + ctx->num_cu - 1) / ctx->num_cu] + 5.0;
+      const double t64 = t_whole8 < t_spread ? t_whole8 : t_spread;
       small_tile = t64 < 0.92 * best;
       spread64 = small_tile && t_spread < t_whole;
     }
